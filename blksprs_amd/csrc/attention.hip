@@ -1,0 +1,57 @@
+// C ABI of block-sparse flash attention: argument checks and the choice between the
+// MFMA kernels (16-bit operands, sbs 32/64) and the generic kernels (everything else).
+#include "attn_common.h"
+
+namespace {
+
+int check_args(const char *who, const bsa_attn_args *a, bool backward) {
+  BSA_REQUIRE(a != nullptr, "%s: NULL argument block", who);
+  BSA_REQUIRE(a->sbs == 16 || a->sbs == 32 || a->sbs == 64, "%s: sbs must be 16, 32 or 64 (got %d)", who, a->sbs);
+  BSA_REQUIRE(a->dtype == BSA_F32 || a->dtype == BSA_F16 || a->dtype == BSA_BF16, "%s: unknown dtype %d", who,
+              a->dtype);
+  BSA_REQUIRE(a->B >= 0 && a->nq >= 0 && a->nk >= 0 && a->nh >= 0 && a->nhv >= 0, "%s: negative layout size", who);
+  BSA_REQUIRE(a->n_q_blocks >= 0 && a->n_k_blocks >= 0 && a->n_v_blocks >= 0 && a->n_o_blocks >= 0 &&
+                  a->n_mask_blocks >= 0 && a->n_bias_blocks >= 0,
+              "%s: negative block count", who);
+  BSA_REQUIRE(a->mask_kind == 0 || a->mask_kind == 1, "%s: mask_kind must be 0 or 1", who);
+  BSA_REQUIRE((a->mask != nullptr) == (a->mask_kind == 1), "%s: mask pointer and mask_kind disagree", who);
+  if (a->B * a->nq == 0 && a->B * a->nk == 0) return BSA_OK;
+  BSA_REQUIRE(a->key_offsets != nullptr, "%s: key_offsets is NULL", who);
+  BSA_REQUIRE(a->lse != nullptr || a->B * a->nq == 0, "%s: lse is NULL", who);
+  BSA_REQUIRE(a->nh == 0 || (a->pidx_q && a->pidx_k), "%s: pidx_q / pidx_k is NULL", who);
+  BSA_REQUIRE(a->nhv == 0 || (a->pidx_v && a->pidx_o), "%s: pidx_v / pidx_o is NULL", who);
+  BSA_REQUIRE(!a->mask || a->pidx_mask, "%s: mask without pidx_mask", who);
+  BSA_REQUIRE(!a->bias || a->pidx_bias, "%s: bias without pidx_bias", who);
+  BSA_REQUIRE(a->B * a->nq < 0x7fffffffLL && a->B * a->nk < 0x7fffffffLL, "%s: too many sequence blocks", who);
+  BSA_REQUIRE(a->nh < 65536 && a->nhv < 65536, "%s: too many head slices", who);
+  if (backward) {
+    BSA_REQUIRE(a->query_offsets != nullptr, "%s: query_offsets is NULL", who);
+    BSA_REQUIRE(a->delta != nullptr || a->B * a->nq == 0, "%s: delta is NULL", who);
+    BSA_REQUIRE(a->n_o_blocks == 0 || (a->o && a->d_o), "%s: o / d_o is NULL", who);
+    BSA_REQUIRE(a->n_q_blocks == 0 || a->dq, "%s: dq is NULL", who);
+    BSA_REQUIRE(a->n_k_blocks == 0 || a->dk, "%s: dk is NULL", who);
+    BSA_REQUIRE(a->n_v_blocks == 0 || a->dv, "%s: dv is NULL", who);
+    BSA_REQUIRE(!a->dbias || a->bias, "%s: dbias without bias", who);
+  } else {
+    BSA_REQUIRE(a->n_o_blocks == 0 || a->o, "%s: o is NULL", who);
+  }
+  return BSA_OK;
+}
+
+}  // namespace
+
+extern "C" int bsa_attn_fwd(const bsa_attn_args *args, bsa_stream_t stream) {
+  if (int rc = check_args("bsa_attn_fwd", args, false)) return rc;
+  hipStream_t s = bsa::as_stream(stream);
+  int rc = bsa::attn_fwd_mfma(*args, s);
+  if (rc == 1) rc = bsa::attn_fwd_generic(*args, s);
+  return rc;
+}
+
+extern "C" int bsa_attn_bwd(const bsa_attn_args *args, bsa_stream_t stream) {
+  if (int rc = check_args("bsa_attn_bwd", args, true)) return rc;
+  hipStream_t s = bsa::as_stream(stream);
+  int rc = bsa::attn_bwd_mfma(*args, s);
+  if (rc == 1) rc = bsa::attn_bwd_generic(*args, s);
+  return rc;
+}

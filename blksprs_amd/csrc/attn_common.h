@@ -1,0 +1,44 @@
+// Pieces shared by the attention kernels: element traits and the argument block.
+#pragma once
+#include "common.h"
+
+namespace bsa {
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+struct AttnBf16 {
+  using elem_t = uint16_t;
+  __device__ static float widen(uint16_t h) { return __builtin_bit_cast(float, (uint32_t)h << 16); }
+  __device__ static uint16_t round(float v) {
+    uint32_t u = __builtin_bit_cast(uint32_t, v);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+  }
+};
+
+struct AttnF16 {
+  using elem_t = uint16_t;
+  __device__ static float widen(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
+  __device__ static uint16_t round(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
+};
+
+struct AttnF32 {
+  using elem_t = float;
+  __device__ static float widen(float v) { return v; }
+  __device__ static float round(float v) { return v; }
+};
+
+// value of a mask element (any non-zero value masks the position)
+__device__ inline bool mask_set(const void *mask, int kind, int64_t idx) {
+  if (kind == 1) return static_cast<const uint8_t *>(mask)[idx] != 0;
+  return false;
+}
+
+int attn_fwd_generic(const bsa_attn_args &a, hipStream_t s);
+int attn_bwd_generic(const bsa_attn_args &a, hipStream_t s);
+// MFMA paths; return 1 if the configuration is not covered (caller falls back to the generic kernels)
+int attn_fwd_mfma(const bsa_attn_args &a, hipStream_t s);
+int attn_bwd_mfma(const bsa_attn_args &a, hipStream_t s);
+
+}  // namespace bsa

@@ -1,0 +1,116 @@
+// Dense <-> compressed conversion: 16-byte vector copies, one thread per vector.
+//
+// A block row is sbs * elem_size bytes, a multiple of 16 for every supported
+// (sbs >= 16, elem_size >= 1), so both directions move uint4 vectors and are
+// independent of the element type.  Traffic: to_sparse reads and writes
+// nnz*sbs*sbs*elem_size bytes; to_dense writes the whole dense array once and
+// reads the active blocks once.
+#include "common.h"
+
+namespace {
+
+// blocks[n][e][:] <- dense[b][r*sbs + e][c*sbs : (c+1)*sbs]
+__global__ __launch_bounds__(256) void to_sparse_kernel(const uint4 *__restrict__ dense,
+                                                        const int64_t *__restrict__ coords,
+                                                        uint4 *__restrict__ blocks, int64_t n_vec,
+                                                        int vec_per_row_log2, int sbs_log2, int64_t dense_row_vecs,
+                                                        int64_t dense_batch_vecs) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  const int vec_per_block_log2 = vec_per_row_log2 + sbs_log2;
+  for (int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; g < n_vec; g += stride) {
+    const int64_t n = g >> vec_per_block_log2;
+    const int64_t in_block = g & (((int64_t)1 << vec_per_block_log2) - 1);
+    const int64_t e = in_block >> vec_per_row_log2;
+    const int64_t q = in_block & (((int64_t)1 << vec_per_row_log2) - 1);
+    const int64_t b = coords[n * 3 + 0];
+    const int64_t r = coords[n * 3 + 1];
+    const int64_t c = coords[n * 3 + 2];
+    const int64_t src = b * dense_batch_vecs + ((r << sbs_log2) + e) * dense_row_vecs + (c << vec_per_row_log2) + q;
+    blocks[g] = dense[src];
+  }
+}
+
+// dense[b][row][:] <- blocks[packed[b, row/sbs, col/sbs]] or the fill pattern
+__global__ __launch_bounds__(256) void to_dense_kernel(const uint4 *__restrict__ blocks,
+                                                       const int64_t *__restrict__ packed,
+                                                       uint4 *__restrict__ dense, int64_t n_vec, int64_t nnz,
+                                                       int64_t R, int64_t C, int vec_per_row_log2, int sbs_log2,
+                                                       uint4 fill) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  const int64_t dense_row_vecs = C << vec_per_row_log2;
+  for (int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; g < n_vec; g += stride) {
+    const int64_t col_vec = g % dense_row_vecs;
+    const int64_t row_all = g / dense_row_vecs;  // b * R*sbs + row
+    const int64_t c = col_vec >> vec_per_row_log2;
+    const int64_t q = col_vec & (((int64_t)1 << vec_per_row_log2) - 1);
+    const int64_t e = row_all & (((int64_t)1 << sbs_log2) - 1);
+    const int64_t br = row_all >> sbs_log2;  // b * R + r
+    const int64_t idx = packed[br * C + c];
+    uint4 v = fill;
+    if (idx >= 0 && idx < nnz) v = blocks[(((idx << sbs_log2) + e) << vec_per_row_log2) + q];
+    dense[g] = v;
+  }
+}
+
+int ilog2(int64_t v) {
+  int l = 0;
+  while (((int64_t)1 << l) < v) ++l;
+  return l;
+}
+
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+int check_block_shape(const char *who, int sbs, int elem_size) {
+  BSA_REQUIRE(sbs >= 16 && bsa::is_pow2(sbs), "%s: sbs must be a power of two >= 16 (got %d)", who, sbs);
+  BSA_REQUIRE(elem_size == 1 || elem_size == 2 || elem_size == 4 || elem_size == 8,
+              "%s: element size %d not in {1,2,4,8}", who, elem_size);
+  return BSA_OK;
+}
+
+unsigned copy_grid(int64_t n_vec) {
+  // enough resident threads to cover the memory latency of 256 CUs; the grid-stride loop takes the rest
+  int64_t blocks = bsa::cdiv(n_vec, 256);
+  const int64_t cap = 256 * 32;
+  return (unsigned)(blocks < cap ? blocks : cap);
+}
+
+}  // namespace
+
+extern "C" int bsa_to_sparse(const void *dense, const int64_t *coords, void *blocks, int64_t nnz, int64_t rows,
+                             int64_t cols, int sbs, int elem_size, bsa_stream_t stream) {
+  if (int rc = check_block_shape("bsa_to_sparse", sbs, elem_size)) return rc;
+  BSA_REQUIRE(nnz >= 0 && rows >= 0 && cols >= 0, "bsa_to_sparse: negative size");
+  BSA_REQUIRE(rows % sbs == 0 && cols % sbs == 0, "bsa_to_sparse: dense sizes not divisible by sbs");
+  if (nnz == 0) return BSA_OK;
+  BSA_REQUIRE(dense && coords && blocks, "bsa_to_sparse: NULL pointer");
+  BSA_REQUIRE(aligned16(dense) && aligned16(blocks), "bsa_to_sparse: buffers must be 16-byte aligned");
+  const int vec_per_row = sbs * elem_size / 16;
+  const int64_t n_vec = nnz * sbs * vec_per_row;
+  const int64_t dense_row_vecs = cols * elem_size / 16;
+  to_sparse_kernel<<<copy_grid(n_vec), 256, 0, bsa::as_stream(stream)>>>(
+      static_cast<const uint4 *>(dense), coords, static_cast<uint4 *>(blocks), n_vec, ilog2(vec_per_row),
+      ilog2(sbs), dense_row_vecs, rows * dense_row_vecs);
+  return bsa::check_launch("to_sparse_kernel");
+}
+
+extern "C" int bsa_to_dense(const void *blocks, const int64_t *packed, void *dense, int64_t B, int64_t R, int64_t C,
+                            int64_t nnz, int sbs, int elem_size, uint64_t fill_bits, bsa_stream_t stream) {
+  if (int rc = check_block_shape("bsa_to_dense", sbs, elem_size)) return rc;
+  BSA_REQUIRE(B >= 0 && R >= 0 && C >= 0 && nnz >= 0, "bsa_to_dense: negative size");
+  const int vec_per_row = sbs * elem_size / 16;
+  const int64_t n_vec = B * R * sbs * C * vec_per_row;
+  if (n_vec == 0) return BSA_OK;
+  BSA_REQUIRE(packed && dense && (nnz == 0 || blocks), "bsa_to_dense: NULL pointer");
+  BSA_REQUIRE(aligned16(dense) && aligned16(blocks), "bsa_to_dense: buffers must be 16-byte aligned");
+  // replicate the element pattern across 16 bytes
+  uint64_t pat = fill_bits;
+  if (elem_size < 8) pat &= ((uint64_t)1 << (8 * elem_size)) - 1;
+  for (int w = elem_size; w < 8; w *= 2) pat |= pat << (8 * w);
+  uint4 fill;
+  fill.x = fill.z = (uint32_t)(pat & 0xffffffffu);
+  fill.y = fill.w = (uint32_t)(pat >> 32);
+  to_dense_kernel<<<copy_grid(n_vec), 256, 0, bsa::as_stream(stream)>>>(
+      static_cast<const uint4 *>(blocks), packed, static_cast<uint4 *>(dense), n_vec, nnz, R, C,
+      ilog2(vec_per_row), ilog2(sbs), fill);
+  return bsa::check_launch("to_dense_kernel");
+}

@@ -1,0 +1,242 @@
+// Row-wise softmax over the active blocks of a block row (fp32), forward and backward.
+//
+// The blocks of one block row are consecutive in the compressed tensor (row-major
+// block order), so a row is `count` whole blocks starting at row_offsets[r].  One
+// wavefront owns a group of element rows of one block row and reads them with one
+// float4 per lane: for sbs <= 256 the 64 lanes cover 256 consecutive floats of a
+// block (256/sbs element rows), so every wave load is one contiguous KiB.  The max /
+// sum reductions stay inside the sbs/4 lanes of an element row (xor shuffles).
+// Rows of up to 32 float4 units per lane stay in registers between the reduction
+// and the write (one HBM read + one write); longer rows make two read passes.
+#include "common.h"
+
+namespace {
+
+constexpr int kMaxUnits = 32;
+
+struct RowGeom {
+  int sbs_log2;
+  int lpr;       // lanes per element row = min(64, sbs/4)
+  int nq_log2;   // float4 units per lane per block = max(1, sbs/256), as log2
+  int groups;    // wave tasks per block row = sbs * lpr / 64
+};
+
+__device__ inline float lanes_max(float v, int lpr) {
+  for (int d = 1; d < lpr; d <<= 1) v = fmaxf(v, __shfl_xor(v, d));
+  return v;
+}
+__device__ inline float lanes_sum(float v, int lpr) {
+  for (int d = 1; d < lpr; d <<= 1) v += __shfl_xor(v, d);
+  return v;
+}
+
+// float offset of unit u of this lane, relative to the first block of the row
+__device__ inline int64_t unit_offset(int u, const RowGeom &g, int64_t lane_base) {
+  const int t = u >> g.nq_log2;
+  const int q = u & ((1 << g.nq_log2) - 1);
+  return ((int64_t)t << (2 * g.sbs_log2)) + lane_base + q * 256;
+}
+
+__device__ inline bool wave_task(const RowGeom &g, const int32_t *row_offsets, int64_t n_tasks, int64_t &first,
+                                 int &units, int64_t &lane_base) {
+  const int64_t wave = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+  if (wave >= n_tasks) return false;
+  const int lane = threadIdx.x & 63;
+  const int64_t r = wave / g.groups;
+  const int grp = (int)(wave % g.groups);
+  const int start = row_offsets[r];
+  const int count = row_offsets[r + 1] - start;
+  if (count <= 0) return false;
+  first = (int64_t)start << (2 * g.sbs_log2);
+  units = count << g.nq_log2;
+  const int rows_per_wave = 64 / g.lpr;
+  const int row_in_block = grp * rows_per_wave + lane / g.lpr;
+  lane_base = ((int64_t)row_in_block << g.sbs_log2) + (lane % g.lpr) * 4;
+  return true;
+}
+
+__device__ inline float max4(float4 v) { return fmaxf(fmaxf(v.x, v.y), fmaxf(v.z, v.w)); }
+
+__global__ __launch_bounds__(256) void softmax_fwd_kernel(const float *__restrict__ x, float *__restrict__ out,
+                                                          const int32_t *__restrict__ row_offsets, int64_t n_tasks,
+                                                          RowGeom g) {
+  int64_t first, lane_base;
+  int units;
+  if (!wave_task(g, row_offsets, n_tasks, first, units, lane_base)) return;
+  const float *xr = x + first;
+  float *orow = out + first;
+
+  if (units <= kMaxUnits) {
+    float4 v[kMaxUnits];
+    float m = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < kMaxUnits; ++u) {
+      if (u < units) {
+        v[u] = *reinterpret_cast<const float4 *>(xr + unit_offset(u, g, lane_base));
+        m = fmaxf(m, max4(v[u]));
+      }
+    }
+    m = lanes_max(m, g.lpr);
+    float s = 0.f;
+#pragma unroll
+    for (int u = 0; u < kMaxUnits; ++u) {
+      if (u < units) {
+        v[u].x = expf(v[u].x - m);
+        v[u].y = expf(v[u].y - m);
+        v[u].z = expf(v[u].z - m);
+        v[u].w = expf(v[u].w - m);
+        s += (v[u].x + v[u].y) + (v[u].z + v[u].w);
+      }
+    }
+    s = lanes_sum(s, g.lpr);
+#pragma unroll
+    for (int u = 0; u < kMaxUnits; ++u) {
+      if (u < units) {
+        float4 o;
+        o.x = v[u].x / s;
+        o.y = v[u].y / s;
+        o.z = v[u].z / s;
+        o.w = v[u].w / s;
+        *reinterpret_cast<float4 *>(orow + unit_offset(u, g, lane_base)) = o;
+      }
+    }
+    return;
+  }
+
+  // long rows: max pass, sum pass folded into one online pass, then the write pass
+  float m = -INFINITY, s = 0.f;
+  for (int u = 0; u < units; ++u) {
+    const float4 v = *reinterpret_cast<const float4 *>(xr + unit_offset(u, g, lane_base));
+    const float mn = fmaxf(m, max4(v));
+    if (mn != -INFINITY) {
+      s = s * expf(m - mn) + (expf(v.x - mn) + expf(v.y - mn)) + (expf(v.z - mn) + expf(v.w - mn));
+    } else if (v.x != v.x || v.y != v.y || v.z != v.z || v.w != v.w) {
+      s = NAN;  // fmaxf drops NaN; keep it visible in the sum
+    }
+    m = mn;
+  }
+  const float mall = lanes_max(m, g.lpr);
+  float part = (m == -INFINITY) ? ((s != s) ? s : 0.f) : s * expf(m - mall);
+  const float sall = lanes_sum(part, g.lpr);
+  for (int u = 0; u < units; ++u) {
+    const int64_t off = unit_offset(u, g, lane_base);
+    const float4 v = *reinterpret_cast<const float4 *>(xr + off);
+    float4 o;
+    o.x = expf(v.x - mall) / sall;
+    o.y = expf(v.y - mall) / sall;
+    o.z = expf(v.z - mall) / sall;
+    o.w = expf(v.w - mall) / sall;
+    *reinterpret_cast<float4 *>(orow + off) = o;
+  }
+}
+
+__global__ __launch_bounds__(256) void softmax_bwd_kernel(const float *__restrict__ grad_out,
+                                                          const float *__restrict__ y, float *__restrict__ grad_in,
+                                                          const int32_t *__restrict__ row_offsets, int64_t n_tasks,
+                                                          RowGeom g) {
+  int64_t first, lane_base;
+  int units;
+  if (!wave_task(g, row_offsets, n_tasks, first, units, lane_base)) return;
+  const float *gr = grad_out + first;
+  const float *yr = y + first;
+  float *dr = grad_in + first;
+
+  if (units <= kMaxUnits / 2) {
+    constexpr int kU = kMaxUnits / 2;
+    float4 yv[kU], gv[kU];
+    float s = 0.f;
+#pragma unroll
+    for (int u = 0; u < kU; ++u) {
+      if (u < units) {
+        const int64_t off = unit_offset(u, g, lane_base);
+        yv[u] = *reinterpret_cast<const float4 *>(yr + off);
+        gv[u] = *reinterpret_cast<const float4 *>(gr + off);
+        s += (yv[u].x * gv[u].x + yv[u].y * gv[u].y) + (yv[u].z * gv[u].z + yv[u].w * gv[u].w);
+      }
+    }
+    s = lanes_sum(s, g.lpr);
+#pragma unroll
+    for (int u = 0; u < kU; ++u) {
+      if (u < units) {
+        float4 o;
+        o.x = yv[u].x * (gv[u].x - s);
+        o.y = yv[u].y * (gv[u].y - s);
+        o.z = yv[u].z * (gv[u].z - s);
+        o.w = yv[u].w * (gv[u].w - s);
+        *reinterpret_cast<float4 *>(dr + unit_offset(u, g, lane_base)) = o;
+      }
+    }
+    return;
+  }
+
+  float s = 0.f;
+  for (int u = 0; u < units; ++u) {
+    const int64_t off = unit_offset(u, g, lane_base);
+    const float4 yv = *reinterpret_cast<const float4 *>(yr + off);
+    const float4 gv = *reinterpret_cast<const float4 *>(gr + off);
+    s += (yv.x * gv.x + yv.y * gv.y) + (yv.z * gv.z + yv.w * gv.w);
+  }
+  s = lanes_sum(s, g.lpr);
+  for (int u = 0; u < units; ++u) {
+    const int64_t off = unit_offset(u, g, lane_base);
+    const float4 yv = *reinterpret_cast<const float4 *>(yr + off);
+    const float4 gv = *reinterpret_cast<const float4 *>(gr + off);
+    float4 o;
+    o.x = yv.x * (gv.x - s);
+    o.y = yv.y * (gv.y - s);
+    o.z = yv.z * (gv.z - s);
+    o.w = yv.w * (gv.w - s);
+    *reinterpret_cast<float4 *>(dr + off) = o;
+  }
+}
+
+int make_geom(const char *who, int sbs, RowGeom &g) {
+  BSA_REQUIRE(sbs >= 16 && bsa::is_pow2(sbs), "%s: sbs must be a power of two >= 16 (got %d)", who, sbs);
+  int l = 0;
+  while ((1 << l) < sbs) ++l;
+  g.sbs_log2 = l;
+  g.lpr = sbs / 4 < 64 ? sbs / 4 : 64;
+  int nq = sbs / 256 > 1 ? sbs / 256 : 1;
+  g.nq_log2 = 0;
+  while ((1 << g.nq_log2) < nq) ++g.nq_log2;
+  g.groups = sbs * g.lpr / 64;
+  return BSA_OK;
+}
+
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+}  // namespace
+
+extern "C" int bsa_softmax_fwd(const float *x, float *out, const int32_t *row_offsets, int64_t n_rows, int64_t nnz,
+                               int sbs, bsa_stream_t stream) {
+  RowGeom g;
+  if (int rc = make_geom("bsa_softmax_fwd", sbs, g)) return rc;
+  BSA_REQUIRE(n_rows >= 0 && nnz >= 0, "bsa_softmax_fwd: negative size");
+  if (n_rows == 0 || nnz == 0) return BSA_OK;
+  BSA_REQUIRE(x && out && row_offsets, "bsa_softmax_fwd: NULL pointer");
+  BSA_REQUIRE(aligned16(x) && aligned16(out), "bsa_softmax_fwd: buffers must be 16-byte aligned");
+  if (nnz > 0x7fffffffLL) return bsa::fail(BSA_ELIMIT, "bsa_softmax_fwd: more than 2^31-1 blocks");
+  const int64_t n_tasks = n_rows * g.groups;
+  const int64_t blocks = bsa::cdiv(n_tasks, 4);
+  if (blocks > 0x7fffffffLL) return bsa::fail(BSA_ELIMIT, "bsa_softmax_fwd: too many rows");
+  softmax_fwd_kernel<<<(unsigned)blocks, 256, 0, bsa::as_stream(stream)>>>(x, out, row_offsets, n_tasks, g);
+  return bsa::check_launch("softmax_fwd_kernel");
+}
+
+extern "C" int bsa_softmax_bwd(const float *grad_out, const float *y, float *grad_in, const int32_t *row_offsets,
+                               int64_t n_rows, int64_t nnz, int sbs, bsa_stream_t stream) {
+  RowGeom g;
+  if (int rc = make_geom("bsa_softmax_bwd", sbs, g)) return rc;
+  BSA_REQUIRE(n_rows >= 0 && nnz >= 0, "bsa_softmax_bwd: negative size");
+  if (n_rows == 0 || nnz == 0) return BSA_OK;
+  BSA_REQUIRE(grad_out && y && grad_in && row_offsets, "bsa_softmax_bwd: NULL pointer");
+  BSA_REQUIRE(aligned16(grad_out) && aligned16(y) && aligned16(grad_in),
+              "bsa_softmax_bwd: buffers must be 16-byte aligned");
+  if (nnz > 0x7fffffffLL) return bsa::fail(BSA_ELIMIT, "bsa_softmax_bwd: more than 2^31-1 blocks");
+  const int64_t n_tasks = n_rows * g.groups;
+  const int64_t blocks = bsa::cdiv(n_tasks, 4);
+  if (blocks > 0x7fffffffLL) return bsa::fail(BSA_ELIMIT, "bsa_softmax_bwd: too many rows");
+  softmax_bwd_kernel<<<(unsigned)blocks, 256, 0, bsa::as_stream(stream)>>>(grad_out, y, grad_in, row_offsets,
+                                                                           n_tasks, g);
+  return bsa::check_launch("softmax_bwd_kernel");
+}

@@ -1,0 +1,429 @@
+"""Block-sparse flash attention on compressed tensors, forward and backward.
+
+Signatures, validation order and messages, default scale, optional mask / bias /
+output layout / native causal lengths and every observable cache key follow the
+reference (blksprs/ops/flash_attention.py:19-242 wrapper and length normalisation,
+:1736-1920 cache builder, :1923-1957 CSR metadata).  The arithmetic is done by
+``bsa_attn_fwd`` / ``bsa_attn_bwd``; the learned relative-embedding branches of the
+reference are not part of this package.
+"""
+
+import ctypes
+import math
+from numbers import Real
+
+import torch
+from torch import Tensor
+
+from .. import _capi
+from ..layouting.sparsity_layout import build_sparsity_layout_matmul
+from ..utils.blksprs_tensor import BlksprsTensor
+from ..utils.tools import (INT32_INDEX_MAX, as_base_tensor, cast_for_autocast, csr_indices_from_packed,
+                           finalize_layout_cache, pack_layout, prepare_layout_cache)
+from ..utils.validation import (ensure_contiguous, validate_binary, validate_contiguous, validate_device,
+                                validate_dimensions, validate_dtype_float, validate_shape, validate_sparsity,
+                                validate_sparsity_block_size, validate_sparsity_layout)
+
+
+def _select_segmented_index_dtype(n_active_blocks: int, n_blocks_col: int) -> torch.dtype:
+    """int32 unless the number of active blocks or the largest column id needs more."""
+    if n_active_blocks > INT32_INDEX_MAX or n_blocks_col - 1 > INT32_INDEX_MAX:
+        return torch.int64
+    return torch.int32
+
+
+def _build_segmented_indices(attention_layout: Tensor, n_batches: int, n_blocks_row: int,
+                             n_blocks_col: int) -> tuple[Tensor, Tensor, int]:
+    """CSR adjacency of a ``(B, rows, cols)`` layout: ``(indices, offsets, max_blocks_per_row)``.
+
+    ``offsets`` has ``B * rows + 1`` entries with a leading 0, ``indices`` lists the active columns of each row
+    in ascending order.  Empty and all-zero layouts yield ``(empty, zeros, 1)``.
+    """
+    device = attention_layout.device
+    n_rows = n_batches * n_blocks_row
+    if attention_layout.numel() == 0:
+        return (torch.empty(0, dtype=torch.int32, device=device),
+                torch.zeros(n_rows + 1, dtype=torch.int32, device=device), 1)
+    info = pack_layout(attention_layout, row_len=n_blocks_col)
+    if info.max_per_row == 0:
+        return (torch.empty(0, dtype=torch.int32, device=device),
+                torch.zeros(n_rows + 1, dtype=torch.int32, device=device), 1)
+    dtype = _select_segmented_index_dtype(info.count, n_blocks_col)
+    indices = csr_indices_from_packed(info.packed, n_blocks_col, info.count)
+    offsets = info.row_offsets
+    if dtype != torch.int32:
+        indices, offsets = indices.to(dtype), offsets.to(dtype)
+    return as_base_tensor(indices), as_base_tensor(offsets), info.max_per_row
+
+
+def flash_attention_build_layout_cache(attention_layout: Tensor,
+                                       sparsity_layout_q: Tensor | None = None,
+                                       sparsity_layout_k: Tensor | None = None,
+                                       sparsity_layout_v: Tensor | None = None,
+                                       n_seq_blocks_q: int | None = None,
+                                       n_seq_blocks_k: int | None = None,
+                                       n_head_blocks: int | None = None,
+                                       sparsity_layout_o: Tensor | None = None,
+                                       n_head_blocks_v: int | None = None,
+                                       layout_cache: dict | None = None,
+                                       sparsity_layout_mask: Tensor | None = None,
+                                       sparsity_layout_bias: Tensor | None = None) -> dict:
+    """Builds reusable layout metadata for block-sparse flash attention.
+
+    Args:
+        attention_layout (Tensor): The block attention pattern ``(n_batches, n_seq_blocks_q, n_seq_blocks_k)``.
+        sparsity_layout_q (Tensor, optional): The sparsity layout of Q (default ``None``).
+        sparsity_layout_k (Tensor, optional): The sparsity layout of K (default ``None``).
+        sparsity_layout_v (Tensor, optional): The sparsity layout of V (default ``None``).
+        n_seq_blocks_q (int, optional): The number of Q sequence blocks (default ``None``).
+        n_seq_blocks_k (int, optional): The number of K sequence blocks (default ``None``).
+        n_head_blocks (int, optional): The number of Q/K head-dimension blocks (default ``None``).
+        sparsity_layout_o (Tensor, optional): The output sparsity layout (default ``None``).
+        n_head_blocks_v (int, optional): The number of V/output head-dimension blocks (default ``None``).
+        layout_cache (dict, optional): An existing layout metadata cache to extend (default ``None``).
+        sparsity_layout_mask (Tensor, optional): The attention-mask sparsity layout (default ``None``).
+        sparsity_layout_bias (Tensor, optional): The attention-bias sparsity layout (default ``None``).
+
+    Returns:
+        dict: The populated layout metadata cache.
+
+    """
+    validate_dimensions(attention_layout)
+    validate_contiguous(attention_layout)
+    validate_sparsity_layout(attention_layout)
+
+    named = (("sparsity_layout_q", sparsity_layout_q), ("sparsity_layout_k", sparsity_layout_k),
+             ("sparsity_layout_v", sparsity_layout_v), ("sparsity_layout_o", sparsity_layout_o),
+             ("sparsity_layout_mask", sparsity_layout_mask), ("sparsity_layout_bias", sparsity_layout_bias))
+    given = tuple(layout for _, layout in named if layout is not None)
+    if given:
+        validate_dimensions(*given)
+        validate_contiguous(*given)
+        validate_device(attention_layout, *given)
+        validate_sparsity_layout(*given)
+    else:
+        validate_device(attention_layout)
+
+    n_batches, rows_q, rows_k = attention_layout.shape
+    if n_seq_blocks_q is None:
+        n_seq_blocks_q = rows_q
+    elif n_seq_blocks_q != rows_q:
+        raise ValueError("n_seq_blocks_q does not match attention_layout")
+    if n_seq_blocks_k is None:
+        n_seq_blocks_k = rows_k
+    elif n_seq_blocks_k != rows_k:
+        raise ValueError("n_seq_blocks_k does not match attention_layout")
+
+    if n_head_blocks is None:
+        source = sparsity_layout_q if sparsity_layout_q is not None else sparsity_layout_k
+        if source is not None:
+            n_head_blocks = source.size(2)
+    if n_head_blocks_v is None:
+        for source in (sparsity_layout_v, sparsity_layout_o, sparsity_layout_q):
+            if source is not None:
+                n_head_blocks_v = source.size(2)
+                break
+
+    expected = {
+        "sparsity_layout_q": (n_batches, n_seq_blocks_q, n_head_blocks),
+        "sparsity_layout_k": (n_batches, n_seq_blocks_k, n_head_blocks),
+        "sparsity_layout_v": (n_batches, n_seq_blocks_k, n_head_blocks_v),
+        "sparsity_layout_o": (n_batches, n_seq_blocks_q, n_head_blocks_v),
+        "sparsity_layout_mask": (n_batches, n_seq_blocks_q, n_seq_blocks_k),
+        "sparsity_layout_bias": (n_batches, n_seq_blocks_q, n_seq_blocks_k),
+    }
+    for name, layout in named:
+        if layout is not None:
+            validate_shape(layout, expected[name], name)
+
+    layout_cache = prepare_layout_cache(
+        layout_cache, "flash_attention",
+        attention_layout, sparsity_layout_q, sparsity_layout_k, sparsity_layout_v,
+        n_seq_blocks_q, n_seq_blocks_k, n_head_blocks, sparsity_layout_o, n_head_blocks_v,
+        sparsity_layout_mask, sparsity_layout_bias,
+    )
+
+    if "sparsity_layout_o" not in layout_cache:
+        if sparsity_layout_o is not None:
+            layout_cache["sparsity_layout_o"] = as_base_tensor(sparsity_layout_o)
+        elif sparsity_layout_v is not None:
+            layout_cache["sparsity_layout_o"] = build_sparsity_layout_matmul(attention_layout, sparsity_layout_v)
+    resolved_o = layout_cache.get("sparsity_layout_o")
+
+    if "key_indices" not in layout_cache:
+        indices, offsets, longest = _build_segmented_indices(attention_layout, n_batches, n_seq_blocks_q,
+                                                             n_seq_blocks_k)
+        layout_cache["key_indices"], layout_cache["key_offsets"] = indices, offsets
+        layout_cache["max_keys_per_query"] = longest
+
+    if "query_indices" not in layout_cache:
+        transposed = as_base_tensor(attention_layout.transpose(1, 2).contiguous())
+        indices, offsets, longest = _build_segmented_indices(transposed, n_batches, n_seq_blocks_k, n_seq_blocks_q)
+        layout_cache["query_indices"], layout_cache["query_offsets"] = indices, offsets
+        layout_cache["max_queries_per_key"] = longest
+
+    for name, layout in (("q", sparsity_layout_q), ("k", sparsity_layout_k), ("v", sparsity_layout_v),
+                         ("mask", sparsity_layout_mask), ("bias", sparsity_layout_bias)):
+        if layout is not None and f"packed_indices_{name}" not in layout_cache:
+            info = pack_layout(layout)
+            layout_cache[f"packed_indices_{name}"] = info.packed
+            if name == "q":
+                layout_cache["n_sparse_blocks_q"] = info.count
+
+    if "packed_indices_o" not in layout_cache and resolved_o is not None:
+        info = pack_layout(resolved_o)
+        layout_cache["packed_indices_o"] = info.packed
+        layout_cache["n_sparse_blocks_o"] = info.count
+
+    tensors = [v for v in layout_cache.values() if isinstance(v, Tensor)]
+    if tensors:
+        validate_contiguous(*tensors)
+
+    return finalize_layout_cache(layout_cache)
+
+
+def _normalise_causal_lengths(causal_lengths: Tensor | None, n_batches: int, q_length: int, k_length: int,
+                              device: torch.device) -> Tensor | None:
+    if causal_lengths is None:
+        return None
+    if not isinstance(causal_lengths, Tensor):
+        raise TypeError("causal_lengths must be a tensor or None")
+    if q_length != k_length:
+        raise ValueError("Native causal attention requires equal query and key lengths")
+    if causal_lengths.dim() != 1:
+        raise ValueError("causal_lengths must be one-dimensional")
+    if causal_lengths.dtype == torch.bool or torch.is_floating_point(causal_lengths):
+        raise TypeError("causal_lengths must use an integral dtype")
+    validate_device(causal_lengths, torch.empty(0, device=device))
+    validate_shape(causal_lengths, (n_batches,), "causal_lengths")
+    if torch.any(causal_lengths < 0) or torch.any(causal_lengths > q_length):
+        raise ValueError(f"causal_lengths values must be between zero and {q_length}")
+    return ensure_contiguous(causal_lengths.to(dtype=torch.int64))
+
+
+def _as_index(t: Tensor | None, dtype: torch.dtype) -> Tensor | None:
+    if t is None or t.dtype == dtype:
+        return t
+    return t.to(dtype)
+
+
+class _Meta:
+    """Everything the kernels need besides the differentiable tensors."""
+
+    __slots__ = ("cache", "dims", "sbs", "scale", "mask", "causal_lengths", "has_bias")
+
+
+def _fill_args(meta: "_Meta", q, k, v, bias) -> _capi.AttnArgs:
+    c = meta.cache
+    a = _capi.AttnArgs()
+    B, nq, nk, nh, nhv = meta.dims
+    a.B, a.nq, a.nk, a.nh, a.nhv = B, nq, nk, nh, nhv
+    a.q, a.k, a.v = _capi.ptr(q), _capi.ptr(k), _capi.ptr(v)
+    a.n_q_blocks, a.n_k_blocks, a.n_v_blocks = q.size(0), k.size(0), v.size(0)
+    a.n_o_blocks = c["n_sparse_blocks_o"]
+    a.pidx_q, a.pidx_k = _capi.ptr(c["packed_indices_q"]), _capi.ptr(c["packed_indices_k"])
+    a.pidx_v, a.pidx_o = _capi.ptr(c["packed_indices_v"]), _capi.ptr(c["packed_indices_o"])
+    # int64 CSR metadata only exists beyond 2**31 - 1 blocks; the kernels index with int32
+    a.key_offsets = c["key_offsets_i32"].data_ptr()
+    a.key_indices = _capi.ptr(c["key_indices_i32"])
+    a.query_offsets = c["query_offsets_i32"].data_ptr()
+    a.query_indices = _capi.ptr(c["query_indices_i32"])
+    if meta.mask is not None:
+        a.mask, a.pidx_mask = _capi.ptr(meta.mask), _capi.ptr(c["packed_indices_mask"])
+        a.n_mask_blocks = meta.mask.size(0)
+        a.mask_kind = 1 if meta.mask.numel() else 0
+    if meta.has_bias:
+        a.bias, a.pidx_bias = _capi.ptr(bias), _capi.ptr(c["packed_indices_bias"])
+        a.n_bias_blocks = bias.size(0)
+    if meta.causal_lengths is not None:
+        a.causal_lengths = meta.causal_lengths.data_ptr()
+    a.sbs = meta.sbs
+    a.dtype = _capi.DTYPE_CODES[q.dtype]
+    a.scale = meta.scale
+    return a
+
+
+class _FlashAttention(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, bias, meta: "_Meta"):
+        B, nq, nk, nh, nhv = meta.dims
+        sbs = meta.sbs
+        out = torch.empty((meta.cache["n_sparse_blocks_o"], sbs, sbs), dtype=q.dtype, device=q.device)
+        lse = torch.empty((B, nq, sbs), dtype=torch.float32, device=q.device)
+        args = _fill_args(meta, q, k, v, bias)
+        args.o, args.lse = _capi.ptr(out), _capi.ptr(lse)
+        with torch.cuda.device(q.device):
+            _capi.call("bsa_attn_fwd", ctypes.byref(args), _capi.stream(q.device))
+        ctx.save_for_backward(q, k, v, bias, out, lse)
+        ctx.meta = meta
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        grad_output = grad_output.contiguous()
+        q, k, v, bias, out, lse = ctx.saved_tensors
+        meta = ctx.meta
+        B, nq, nk, nh, nhv = meta.dims
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        delta = torch.empty((B, nq, meta.sbs), dtype=torch.float32, device=q.device)
+        dbias = torch.empty(bias.shape, dtype=torch.float32, device=q.device) if meta.has_bias else None
+        args = _fill_args(meta, q, k, v, bias)
+        args.o, args.d_o, args.lse, args.delta = _capi.ptr(out), _capi.ptr(grad_output), _capi.ptr(lse), _capi.ptr(delta)
+        args.dq, args.dk, args.dv, args.dbias = _capi.ptr(dq), _capi.ptr(dk), _capi.ptr(dv), _capi.ptr(dbias)
+        with torch.cuda.device(q.device):
+            _capi.call("bsa_attn_bwd", ctypes.byref(args), _capi.stream(q.device))
+        grad_bias = dbias.to(bias.dtype) if meta.has_bias else None
+        return dq, dk, dv, grad_bias, None
+
+
+@torch.compiler.disable
+@torch.amp.custom_fwd(device_type="cuda")
+def flash_attention(q: BlksprsTensor, sparsity_layout_q: Tensor,
+                    k: BlksprsTensor, sparsity_layout_k: Tensor,
+                    v: BlksprsTensor, sparsity_layout_v: Tensor,
+                    attention_layout: Tensor,
+                    sparsity_block_size: int,
+                    scale: float | None = None,
+                    attention_mask: BlksprsTensor | None = None, sparsity_layout_mask: Tensor | None = None,
+                    attention_bias: BlksprsTensor | None = None, sparsity_layout_bias: Tensor | None = None,
+                    layout_cache: dict | None = None,
+                    sparsity_layout_o: Tensor | None = None,
+                    causal_lengths: Tensor | None = None) -> BlksprsTensor:
+    """Computes block-sparse flash attention on compressed tensors.
+
+    All inputs use the compressed format ``(n_sparse_blocks, sbs, sbs)`` with an accompanying sparsity layout.
+    In ``attention_mask`` a non-zero value marks an **ignored** position (the ``masked_fill`` convention, the
+    opposite of ``scaled_dot_product_attention``'s boolean ``attn_mask``).  Supported block sizes are 16, 32
+    and 64.  Mask and bias each come with their own layout.
+
+    Args:
+        q (BlksprsTensor): Queries; layout ``(n_batches, seq_q // sbs, head_dim // sbs)``.
+        sparsity_layout_q (Tensor): The sparsity layout of ``q``.
+        k (BlksprsTensor): Keys; layout ``(n_batches, seq_k // sbs, head_dim // sbs)``.
+        sparsity_layout_k (Tensor): The sparsity layout of ``k``.
+        v (BlksprsTensor): Values.
+        sparsity_layout_v (Tensor): The sparsity layout of ``v``.
+        attention_layout (Tensor): Which (query block, key block) pairs attend, ``(n_batches, seq_q // sbs, seq_k // sbs)``.
+        sparsity_block_size (int): The size of the sparsity blocks.
+        scale (float, optional): Attention scale (default ``1/sqrt(head_dim)``).
+        attention_mask (BlksprsTensor, optional): Binary mask in compressed form, not differentiated.
+        sparsity_layout_mask (Tensor, optional): The sparsity layout of the mask.
+        attention_bias (BlksprsTensor, optional): Additive bias in compressed form, applied before softmax; differentiable.
+        sparsity_layout_bias (Tensor, optional): The sparsity layout of the bias.
+        layout_cache (dict, optional): Reusable layout metadata cache (default ``None``).
+        sparsity_layout_o (Tensor, optional): Output layout; defaults to the structural product of
+            ``attention_layout`` and ``sparsity_layout_v``.
+        causal_lengths (Tensor, optional): Integral valid lengths, one per batch, for native causal
+            self-attention: future keys and padded queries / keys are ignored without a mask tensor.
+
+    Returns:
+        BlksprsTensor: The attention output in compressed form.
+
+    """
+    q, k, v, attention_layout = ensure_contiguous(q, k, v, attention_layout)
+    q, k, v = cast_for_autocast(q, k, v)
+
+    validate_dimensions(q, k, v)
+    validate_contiguous(q, k, v)
+    validate_dtype_float(q, k, v)
+    validate_device(q, k, v)
+    validate_sparsity(sparsity_block_size, (q, sparsity_layout_q), (k, sparsity_layout_k), (v, sparsity_layout_v))
+    validate_sparsity_block_size(sparsity_block_size, q, k, v)
+    if sparsity_block_size > 64:
+        raise ValueError("Flash Attention sparsity block size must be at most 64")
+
+    validate_dimensions(attention_layout)
+    validate_contiguous(attention_layout)
+    validate_device(attention_layout, q)
+    validate_sparsity_layout(attention_layout)
+
+    n_batches = sparsity_layout_q.size(0)
+    n_seq_blocks_q = sparsity_layout_q.size(1)
+    n_head_blocks_qk = sparsity_layout_q.size(2)
+    n_seq_blocks_k = sparsity_layout_k.size(1)
+    n_head_blocks_v = sparsity_layout_v.size(2)
+
+    if sparsity_layout_k.size(0) != n_batches or sparsity_layout_k.size(2) != n_head_blocks_qk:
+        raise ValueError("K sparsity layout must be compatible with Q")
+    if sparsity_layout_v.size(0) != n_batches or sparsity_layout_v.size(1) != n_seq_blocks_k:
+        raise ValueError("V sparsity layout must be compatible with K")
+
+    attention_shape = (n_batches, n_seq_blocks_q, n_seq_blocks_k)
+    validate_shape(attention_layout, attention_shape, "attention_layout")
+    lengths = _normalise_causal_lengths(causal_lengths, n_batches, n_seq_blocks_q * sparsity_block_size,
+                                        n_seq_blocks_k * sparsity_block_size, q.device)
+
+    if sparsity_layout_o is not None:
+        sparsity_layout_o = ensure_contiguous(sparsity_layout_o)
+        validate_dimensions(sparsity_layout_o)
+        validate_contiguous(sparsity_layout_o)
+        validate_device(sparsity_layout_o, q)
+        validate_sparsity_layout(sparsity_layout_o)
+        validate_shape(sparsity_layout_o, (n_batches, n_seq_blocks_q, n_head_blocks_v), "sparsity_layout_o")
+
+    if scale is None:
+        head_dimension = n_head_blocks_qk * sparsity_block_size
+        scale = 1.0 if head_dimension == 0 else 1.0 / math.sqrt(head_dimension)
+    elif not isinstance(scale, Real):
+        raise TypeError("Attention scale must be a real number or None")
+    else:
+        scale = float(scale)
+
+    if (attention_mask is None) != (sparsity_layout_mask is None):
+        raise ValueError("attention_mask and sparsity_layout_mask must be provided together")
+    mask_bytes = None
+    if attention_mask is not None:
+        attention_mask = ensure_contiguous(attention_mask)
+        sparsity_layout_mask = ensure_contiguous(sparsity_layout_mask)
+        validate_dimensions(attention_mask, sparsity_layout_mask)
+        validate_contiguous(attention_mask, sparsity_layout_mask)
+        validate_device(attention_mask, sparsity_layout_mask, q)
+        if attention_mask.dtype != torch.bool:
+            validate_dtype_float(attention_mask)
+        validate_binary(attention_mask)
+        validate_sparsity(sparsity_block_size, (attention_mask, sparsity_layout_mask))
+        validate_shape(sparsity_layout_mask, attention_shape, "sparsity_layout_mask")
+        base = as_base_tensor(attention_mask.detach())
+        # the kernels read one byte per mask element
+        mask_bytes = (base if base.dtype == torch.bool else base != 0).view(torch.uint8)
+
+    if (attention_bias is None) != (sparsity_layout_bias is None):
+        raise ValueError("attention_bias and sparsity_layout_bias must be provided together")
+    has_bias = attention_bias is not None
+    if has_bias:
+        attention_bias = ensure_contiguous(attention_bias)
+        sparsity_layout_bias = ensure_contiguous(sparsity_layout_bias)
+        validate_dimensions(attention_bias, sparsity_layout_bias)
+        validate_contiguous(attention_bias, sparsity_layout_bias)
+        validate_device(attention_bias, sparsity_layout_bias, q)
+        validate_dtype_float(attention_bias)
+        validate_sparsity(sparsity_block_size, (attention_bias, sparsity_layout_bias))
+        validate_shape(sparsity_layout_bias, attention_shape, "sparsity_layout_bias")
+        if attention_bias.dtype != q.dtype:
+            attention_bias = attention_bias.to(q.dtype)
+    else:
+        attention_bias = torch.empty(0, device=q.device, dtype=q.dtype)
+
+    layout_cache = flash_attention_build_layout_cache(
+        attention_layout, sparsity_layout_q, sparsity_layout_k, sparsity_layout_v,
+        n_seq_blocks_q, n_seq_blocks_k, n_head_blocks_qk,
+        sparsity_layout_o=sparsity_layout_o, n_head_blocks_v=n_head_blocks_v,
+        sparsity_layout_mask=sparsity_layout_mask, sparsity_layout_bias=sparsity_layout_bias,
+        layout_cache=layout_cache,
+    )
+    if "key_offsets_i32" not in layout_cache:
+        for name in ("key_offsets", "key_indices", "query_offsets", "query_indices"):
+            layout_cache[name + "_i32"] = _as_index(layout_cache[name], torch.int32)
+        finalize_layout_cache(layout_cache)
+
+    meta = _Meta()
+    meta.cache = layout_cache
+    meta.dims = (int(n_batches), int(n_seq_blocks_q), int(n_seq_blocks_k), int(n_head_blocks_qk),
+                 int(n_head_blocks_v))
+    meta.sbs = sparsity_block_size
+    meta.scale = scale
+    meta.mask = mask_bytes
+    meta.causal_lengths = lengths
+    meta.has_bias = has_bias
+
+    return BlksprsTensor.wrap(_FlashAttention.apply(q, k, v, attention_bias, meta))

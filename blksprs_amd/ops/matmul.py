@@ -1,0 +1,159 @@
+"""Block-sparse matrix multiplication of two compressed tensors.
+
+Signature, validation order, error texts and the observable cache keys follow the
+reference (blksprs/ops/matmul.py:17-67 wrapper, :256-279 cache, :130-145 backward).
+The product itself walks per-output-block contraction lists built on the device
+and is computed by ``bsa_matmul``.  The backward pass reads the saved operands
+transposed inside the kernel instead of materialising transposed copies.
+"""
+
+import torch
+from torch import Tensor
+
+from .. import _capi
+from ..utils.blksprs_tensor import BlksprsTensor
+from ..utils.tools import (build_contraction_lists, cast_for_autocast, finalize_layout_cache, nonzero_from_packed,
+                           pack_layout, prepare_layout_cache)
+from ..utils.validation import (ensure_contiguous, validate_contiguous, validate_device, validate_dimensions,
+                                validate_dtype_float, validate_shape, validate_sparsity, validate_sparsity_block_size,
+                                validate_sparsity_layout)
+
+
+def _launch(x: Tensor, y: Tensor, pair_offsets: Tensor, pairs: Tensor, n_out: int, sbs: int,
+            trans_x: bool, trans_y: bool) -> Tensor:
+    out = torch.empty((n_out, sbs, sbs), dtype=x.dtype, device=x.device)
+    if n_out:
+        with torch.cuda.device(x.device):
+            _capi.call("bsa_matmul", _capi.ptr(x), _capi.ptr(y), out.data_ptr(), pair_offsets.data_ptr(),
+                       _capi.ptr(pairs), n_out, x.size(0), y.size(0), sbs, _capi.DTYPE_CODES[x.dtype],
+                       int(trans_x), int(trans_y), _capi.stream(x.device))
+    return out
+
+
+def _backward_lists(layout_cache: dict, shape_x, shape_y):
+    """Contraction lists of dX = dO Y^T and dY = X^T dO, built once per cache."""
+    if "grad_x_pair_offsets" not in layout_cache:
+        B, R, K = (int(s) for s in shape_x)
+        C = int(shape_y[2])
+        pidx_x = layout_cache["packed_indices_x"]
+        pidx_y = layout_cache["packed_indices_y"]
+        pidx_o = layout_cache["packed_indices_o"]
+        # operand layouts seen by the builder: dO (B,R,C) times Y^T (B,C,K) -> (B,R,K)
+        pidx_yt = pidx_y.view(B, K, C).transpose(1, 2).contiguous().view(-1)
+        gx = build_contraction_lists(pidx_o, pidx_yt, pidx_x, B, R, C, K, layout_cache["n_sparse_blocks_x"])
+        # X^T (B,K,R) times dO (B,R,C) -> (B,K,C)
+        pidx_xt = pidx_x.view(B, R, K).transpose(1, 2).contiguous().view(-1)
+        gy = build_contraction_lists(pidx_xt, pidx_o, pidx_y, B, K, R, C, layout_cache["n_sparse_blocks_y"])
+        layout_cache["grad_x_pair_offsets"], layout_cache["grad_x_pairs"] = gx.pair_offsets, gx.pairs
+        layout_cache["grad_y_pair_offsets"], layout_cache["grad_y_pairs"] = gy.pair_offsets, gy.pairs
+        finalize_layout_cache(layout_cache)
+    return (layout_cache["grad_x_pair_offsets"], layout_cache["grad_x_pairs"],
+            layout_cache["grad_y_pair_offsets"], layout_cache["grad_y_pairs"])
+
+
+class _Matmul(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, y, layout_cache, shape_x, shape_y, sparsity_block_size):
+        ctx.save_for_backward(x, y)
+        ctx.layout_cache = layout_cache
+        ctx.shapes = (shape_x, shape_y)
+        ctx.sparsity_block_size = sparsity_block_size
+        return _launch(x, y, layout_cache["contraction_offsets"], layout_cache["contraction_pairs"],
+                       layout_cache["n_sparse_blocks"], sparsity_block_size, False, False)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        grad_output = grad_output.contiguous()
+        x, y = ctx.saved_tensors
+        sbs = ctx.sparsity_block_size
+        gx_off, gx_pairs, gy_off, gy_pairs = _backward_lists(ctx.layout_cache, *ctx.shapes)
+        grad_x = grad_y = None
+        if ctx.needs_input_grad[0]:
+            grad_x = _launch(grad_output, y, gx_off, gx_pairs, x.size(0), sbs, False, True)
+        if ctx.needs_input_grad[1]:
+            grad_y = _launch(x, grad_output, gy_off, gy_pairs, y.size(0), sbs, True, False)
+        return grad_x, grad_y, None, None, None, None
+
+
+def matmul_build_layout_cache(layout_cache: dict | None, sparsity_layout_x: Tensor, sparsity_layout_y: Tensor,
+                              sparsity_layout_output: Tensor) -> dict:
+    """Fills the cache of one (x layout, y layout, output layout) triple.
+
+    Keys shared with the reference: ``packed_indices_x``, ``packed_indices_y`` (int64, flat),
+    ``layout_indices_o`` (int64 ``[n, 3]``), ``n_sparse_blocks``.  Additional keys hold the
+    contraction lists the kernel walks (``contraction_offsets`` int32 ``[n + 1]``,
+    ``contraction_pairs`` int32 ``[pairs, 2]``) and the counts they were sized with.
+    """
+    layout_cache = prepare_layout_cache(layout_cache, "matmul", sparsity_layout_x, sparsity_layout_y,
+                                        sparsity_layout_output)
+    if "contraction_pairs" not in layout_cache:
+        info_x, info_y = pack_layout(sparsity_layout_x), pack_layout(sparsity_layout_y)
+        info_o = pack_layout(sparsity_layout_output)
+        B, R, K = (int(s) for s in sparsity_layout_x.shape)
+        C = int(sparsity_layout_y.size(2))
+        lists = build_contraction_lists(info_x.packed, info_y.packed, info_o.packed, B, R, K, C, info_o.count)
+        layout_cache["packed_indices_x"] = info_x.packed
+        layout_cache["packed_indices_y"] = info_y.packed
+        layout_cache["packed_indices_o"] = info_o.packed
+        layout_cache["layout_indices_o"] = nonzero_from_packed(info_o.packed, sparsity_layout_output.shape,
+                                                               info_o.count)
+        layout_cache["n_sparse_blocks"] = info_o.count
+        layout_cache["n_sparse_blocks_x"] = info_x.count
+        layout_cache["n_sparse_blocks_y"] = info_y.count
+        layout_cache["contraction_offsets"] = lists.pair_offsets
+        layout_cache["contraction_pairs"] = lists.pairs
+
+    validate_contiguous(sparsity_layout_x, layout_cache["packed_indices_x"],
+                        sparsity_layout_y, layout_cache["packed_indices_y"],
+                        sparsity_layout_output, layout_cache["layout_indices_o"])
+    return finalize_layout_cache(layout_cache)
+
+
+@torch.compiler.disable
+@torch.amp.custom_fwd(device_type="cuda")
+def matmul(x: BlksprsTensor, sparsity_layout_x: Tensor,
+           y: BlksprsTensor, sparsity_layout_y: Tensor,
+           sparsity_layout_output: Tensor,
+           sparsity_block_size: int, layout_cache: dict | None = None) -> BlksprsTensor:
+    """Multiplies two compressed block-sparse tensors.
+
+    Only blocks marked active by ``sparsity_layout_output`` are calculated.
+
+    Args:
+        x (BlksprsTensor): The compressed left operand.
+        sparsity_layout_x (Tensor): The sparsity layout of ``x``.
+        y (BlksprsTensor): The compressed right operand.
+        sparsity_layout_y (Tensor): The sparsity layout of ``y``.
+        sparsity_layout_output (Tensor): The sparsity layout of the output tensor.
+        sparsity_block_size (int): The size of the sparsity blocks.
+        layout_cache (dict, optional): Reusable layout metadata cache (default ``None``).
+
+    Returns:
+        BlksprsTensor: The matrix product in compressed form.
+
+    """
+    x, y = ensure_contiguous(x, y)
+    x, y = cast_for_autocast(x, y)
+
+    validate_dimensions(x, y)
+    validate_contiguous(x, y, sparsity_layout_output)
+    validate_dtype_float(x, y)
+    validate_device(x, y, sparsity_layout_output)
+    validate_sparsity(sparsity_block_size, (x, sparsity_layout_x), (y, sparsity_layout_y))
+    validate_sparsity_layout(sparsity_layout_output)
+    if sparsity_layout_x.size(0) != sparsity_layout_y.size(0):
+        raise ValueError("Batch dimensions of tensors must match")
+    if sparsity_layout_x.size(-1) != sparsity_layout_y.size(-2):
+        raise ValueError("Inner dimensions of tensors must match")
+    validate_shape(
+        sparsity_layout_output,
+        (sparsity_layout_x.size(0), sparsity_layout_x.size(1), sparsity_layout_y.size(2)),
+        "Output sparsity layout",
+    )
+    validate_sparsity_block_size(sparsity_block_size, x, y)
+
+    layout_cache = matmul_build_layout_cache(layout_cache, sparsity_layout_x, sparsity_layout_y,
+                                             sparsity_layout_output)
+
+    return BlksprsTensor.wrap(_Matmul.apply(x, y, layout_cache, tuple(sparsity_layout_x.shape),
+                                            tuple(sparsity_layout_y.shape), sparsity_block_size))

@@ -1,0 +1,293 @@
+"""Layout -> lookup-table builders and the caller-owned layout cache.
+
+The lookup tables are computed on the device by the integer kernels of
+libblksprs_amd.so (``csrc/lut.hip``); this module sizes their outputs and keeps
+the observable results identical to the reference's torch formulations
+(blksprs/utils/tools.py:33-57 for the two basic tables, :60-156 for the cache,
+:159-287 for the shape and dtype helpers).
+"""
+
+from typing import Any
+
+import torch
+from torch import Tensor, Size
+
+from .. import _capi
+
+INT32_INDEX_MAX = 2_147_483_647
+
+LayoutCache = dict[str, Any]
+
+_KEY = "_blksprs_cache_key"
+_REFS = "_blksprs_cache_refs"
+_STATE = "_blksprs_cache_state"
+_PRIVATE = frozenset((_KEY, _REFS, _STATE))
+
+
+def as_base_tensor(value: Tensor) -> Tensor:
+    """Strips a tensor subclass (same storage) so metadata is always a plain ``torch.Tensor``."""
+    return value if type(value) is Tensor else Tensor(value)
+
+
+# --------------------------------------------------------------------------- device LUT builders
+
+def _layout_bytes(layout: Tensor) -> Tensor:
+    """The layout as contiguous 0/1 bytes on its device (a view for bool layouts)."""
+    layout = as_base_tensor(layout)
+    if not layout.is_contiguous():
+        layout = layout.contiguous()
+    if layout.dtype == torch.bool:
+        return layout.view(torch.uint8)
+    if layout.dtype == torch.uint8:
+        return layout
+    # numeric layouts hold exact 0/1 values (validated upstream)
+    return (layout != 0).view(torch.uint8)
+
+
+def _require_device(t: Tensor) -> None:
+    if t.device.type != "cuda":
+        raise RuntimeError(
+            "blksprs_amd builds lookup tables with HIP kernels and needs GPU tensors; "
+            f"got a layout on {t.device}")
+
+
+class PackedLayout:
+    """Result of one device pass over a layout.
+
+    Attributes:
+        packed: int64 reverse index over the flattened layout (``-1`` = inactive).
+        count: number of active blocks.
+        row_offsets: int32 CSR offsets over rows of length ``row_len`` (``None`` if not requested).
+        max_per_row: largest number of active blocks in one row (0 if not requested).
+    """
+
+    __slots__ = ("packed", "count", "row_offsets", "max_per_row")
+
+    def __init__(self, packed, count, row_offsets, max_per_row):
+        self.packed, self.count, self.row_offsets, self.max_per_row = packed, count, row_offsets, max_per_row
+
+
+def pack_layout(layout: Tensor, row_len: int = 0) -> PackedLayout:
+    """Scans a layout on the device: reverse index, block count and optional CSR row offsets.
+
+    One stream synchronisation (the count sizes the caller's next allocation).
+    """
+    _require_device(layout)
+    lay = _layout_bytes(layout)
+    n = lay.numel()
+    dev = lay.device
+    packed = torch.empty(n, dtype=torch.int64, device=dev)
+    n_rows = n // row_len if row_len > 0 else 0
+    row_offsets = torch.empty(n_rows + 1, dtype=torch.int32, device=dev) if row_len > 0 else None
+    stats_dev = torch.empty(2, dtype=torch.int64, device=dev)
+    stats_host = torch.empty(2, dtype=torch.int64, pin_memory=True)
+    lib = _capi.load()
+    ws_bytes = lib.bsa_lut_workspace_bytes(n)
+    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        _capi.call("bsa_lut_packed", _capi.ptr(lay), n, row_len, _capi.ptr(packed),
+                   row_offsets.data_ptr() if row_offsets is not None else 0,
+                   stats_dev.data_ptr(), stats_host.data_ptr(), _capi.ptr(workspace), ws_bytes, _capi.stream(dev))
+    return PackedLayout(packed, int(stats_host[0]), row_offsets, int(stats_host[1]))
+
+
+def build_packed_indices(sparsity_layout: Tensor) -> Tensor:
+    """int64 reverse index of a layout: position among the active blocks, ``-1`` for inactive ones."""
+    return pack_layout(sparsity_layout).packed
+
+
+def nonzero_from_packed(packed: Tensor, shape, count: int) -> Tensor:
+    """int64 ``[count, 3]`` coordinates of the active blocks in row-major order."""
+    B, R, C = (int(s) for s in shape)
+    coords = torch.empty((count, 3), dtype=torch.int64, device=packed.device)
+    if count:
+        with torch.cuda.device(packed.device):
+            _capi.call("bsa_lut_nonzero", packed.data_ptr(), B, R, C, coords.data_ptr(), _capi.stream(packed.device))
+    return coords
+
+
+def build_layout_indices(sparsity_layout: Tensor) -> Tensor:
+    """Coordinates of the active blocks, equal to ``torch.nonzero(sparsity_layout)``."""
+    info = pack_layout(sparsity_layout)
+    return nonzero_from_packed(info.packed, sparsity_layout.shape, info.count)
+
+
+def csr_indices_from_packed(packed: Tensor, n_cols: int, count: int) -> Tensor:
+    """int32 column ids of the active blocks, row by row."""
+    indices = torch.empty(count, dtype=torch.int32, device=packed.device)
+    if count:
+        with torch.cuda.device(packed.device):
+            _capi.call("bsa_lut_csr_indices", packed.data_ptr(), packed.numel(), n_cols, indices.data_ptr(),
+                       _capi.stream(packed.device))
+    return indices
+
+
+def sorted_rows_from_offsets(row_offsets: Tensor, n_rows: int, n_cols: int) -> Tensor:
+    """Per-row descending sort of the reverse index (active first), int64 flat."""
+    out = torch.empty(n_rows * n_cols, dtype=torch.int64, device=row_offsets.device)
+    if out.numel():
+        with torch.cuda.device(out.device):
+            _capi.call("bsa_lut_sorted_rows", row_offsets.data_ptr(), n_rows, n_cols, out.data_ptr(),
+                       _capi.stream(out.device))
+    return out
+
+
+class ContractionLists:
+    """Per-output-block lists of (x block, y block) index pairs of a block-sparse product."""
+
+    __slots__ = ("pair_offsets", "pairs", "n_pairs")
+
+    def __init__(self, pair_offsets, pairs, n_pairs):
+        self.pair_offsets, self.pairs, self.n_pairs = pair_offsets, pairs, n_pairs
+
+
+def build_contraction_lists(pidx_x: Tensor, pidx_y: Tensor, pidx_o: Tensor, B: int, R: int, K: int, C: int,
+                            nnz_o: int) -> ContractionLists:
+    """Builds, on the device, for every active output block the ascending-k list of block pairs to multiply."""
+    dev = pidx_o.device
+    n = B * R * C
+    W = (K + 63) // 64
+    mask_x = torch.empty(max(B * R * W, 1), dtype=torch.int64, device=dev)
+    mask_y = torch.empty(max(B * C * W, 1), dtype=torch.int64, device=dev)
+    pos_offsets = torch.empty(n + 1, dtype=torch.int32, device=dev)
+    stats_dev = torch.empty(2, dtype=torch.int64, device=dev)
+    stats_host = torch.empty(2, dtype=torch.int64, pin_memory=True)
+    lib = _capi.load()
+    ws_bytes = lib.bsa_lut_workspace_bytes(n)
+    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        st = _capi.stream(dev)
+        _capi.call("bsa_lut_contraction_offsets", _capi.ptr(pidx_x), _capi.ptr(pidx_y), _capi.ptr(pidx_o),
+                   B, R, K, C, mask_x.data_ptr(), mask_y.data_ptr(), pos_offsets.data_ptr(),
+                   stats_dev.data_ptr(), stats_host.data_ptr(), workspace.data_ptr(), ws_bytes, st)
+        total = int(stats_host[0])
+        if total > INT32_INDEX_MAX:
+            raise RuntimeError(f"block-sparse product has {total} block pairs; at most {INT32_INDEX_MAX} are supported")
+        pair_offsets = torch.empty(nnz_o + 1, dtype=torch.int32, device=dev)
+        pairs = torch.empty((total, 2), dtype=torch.int32, device=dev)
+        _capi.call("bsa_lut_contraction_pairs", _capi.ptr(pidx_x), _capi.ptr(pidx_y), _capi.ptr(pidx_o),
+                   B, R, K, C, mask_x.data_ptr(), mask_y.data_ptr(), pos_offsets.data_ptr(), nnz_o,
+                   pair_offsets.data_ptr(), _capi.ptr(pairs), st)
+    return ContractionLists(pair_offsets, pairs, total)
+
+
+# --------------------------------------------------------------------------- layout cache
+
+def _tensor_signature(value: Tensor, version):
+    return ("tensor", id(value), version, tuple(value.shape), tuple(value.stride()), value.dtype, value.device,
+            value.requires_grad)
+
+
+def prepare_layout_cache(layout_cache: LayoutCache | None, operation: str, *values: object) -> LayoutCache:
+    """Returns ``layout_cache`` ready for ``operation``, emptied first if it belongs to other inputs.
+
+    The cache is keyed on the operation name, on the identity / in-place version /
+    shape / stride / dtype / device / requires_grad of every tensor argument and on
+    every scalar argument, and it is also dropped when any derived entry changed
+    since it was finalized.  Inference tensors have no version counter, so a cache
+    keyed on one never hits.
+    """
+    if layout_cache is None:
+        layout_cache = {}
+
+    refs: list[Tensor] = []
+    never_equal = object()
+
+    def signature(value):
+        if isinstance(value, Tensor):
+            refs.append(value)
+            return _tensor_signature(value, never_equal if torch.is_inference(value) else int(value._version))
+        if isinstance(value, (tuple, list, Size)):
+            return tuple(signature(v) for v in value)
+        if isinstance(value, dict):
+            return tuple(sorted((k, signature(v)) for k, v in value.items()))
+        return value
+
+    key = (operation, tuple(signature(v) for v in values))
+    recorded = layout_cache.get(_STATE)
+    stale = (layout_cache.get(_KEY) != key or recorded is None or _snapshot(layout_cache) != recorded)
+    if stale:
+        layout_cache.clear()
+        layout_cache[_KEY] = key
+        # holding the sources keeps their ids from being reused by other tensors
+        layout_cache[_REFS] = tuple(refs)
+    return layout_cache
+
+
+def finalize_layout_cache(layout_cache: LayoutCache) -> LayoutCache:
+    """Records what the cache holds now; a later change of any entry invalidates it."""
+    layout_cache[_STATE] = _snapshot(layout_cache)
+    return layout_cache
+
+
+def _snapshot(layout_cache: LayoutCache) -> tuple:
+    return tuple((k, _entry_state(v)) for k, v in sorted(layout_cache.items()) if k not in _PRIVATE)
+
+
+def _entry_state(value):
+    if isinstance(value, Tensor):
+        return _tensor_signature(value, object() if torch.is_inference(value) else int(value._version))
+    if isinstance(value, dict):
+        return tuple((k, _entry_state(v)) for k, v in sorted(value.items()) if k not in _PRIVATE)
+    if isinstance(value, (tuple, list, Size)):
+        return tuple(_entry_state(v) for v in value)
+    if isinstance(value, (PackedLayout, ContractionLists)):
+        return tuple(_entry_state(getattr(value, s)) for s in value.__slots__)
+    return value
+
+
+# --------------------------------------------------------------------------- shape / dtype helpers
+
+def do_shape_blocksparse(x: Tensor) -> tuple[Tensor, Size]:
+    """Flattens all leading dimensions into one batch dimension; returns the 3-D tensor and the original shape."""
+    if x.dim() < 2:
+        raise ValueError("Tensor must have at least 2 dimensions")
+    if x.dim() == 3:
+        return x.contiguous(), x.size()
+    batch = 1
+    for s in x.shape[:-2]:
+        batch *= s
+    return x.reshape(batch, x.size(-2), x.size(-1)).contiguous(), x.size()
+
+
+def undo_shape_blocksparse(x: Tensor, shape: Size | tuple[int, ...]) -> Tensor:
+    """Restores the leading dimensions removed by :func:`do_shape_blocksparse` (last two taken from ``x``)."""
+    if x.dim() != 3:
+        raise ValueError("Tensor must have exactly 3 dimensions")
+    if len(shape) < 2:
+        raise ValueError("Original shape must have at least 2 dimensions")
+    batch = 1
+    for s in shape[:-2]:
+        batch *= s
+    if x.size(0) != batch:
+        raise ValueError("Tensor batch dimension does not match original shape")
+    if x.shape[:-2] == shape[:-2]:
+        return x
+    return x.reshape((*shape[:-2], *x.shape[-2:]))
+
+
+def ceil_pow2(x: int) -> int:
+    """Smallest power of two >= ``x``."""
+    if x <= 0:
+        raise ValueError("Input must be a positive integer.")
+    return 1 << (x - 1).bit_length()
+
+
+def can_use_int32_indexing(*values: Tensor | int | None) -> bool:
+    """Whether every given buffer (tensor or element count) has at most 2**31 - 1 elements."""
+    for v in values:
+        if v is None:
+            continue
+        n = v.numel() if isinstance(v, Tensor) else int(v)
+        if n > INT32_INDEX_MAX:
+            return False
+    return True
+
+
+def cast_for_autocast(*values: Tensor):
+    """Casts fp16 / bf16 / fp32 GPU tensors to the autocast dtype while autocast is on; others pass through."""
+    if torch.is_autocast_enabled():
+        target = torch.get_autocast_dtype("cuda")
+        eligible = (torch.float16, torch.bfloat16, torch.float32)
+        values = tuple(v.to(target) if v.is_cuda and v.dtype in eligible else v for v in values)
+    return values[0] if len(values) == 1 else values

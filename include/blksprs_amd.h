@@ -1,0 +1,231 @@
+/*
+ * C ABI of the MI355X (gfx950) block-sparse compute library, libblksprs_amd.so.
+ *
+ * Every entry point takes plain device pointers, sizes and a HIP stream and
+ * returns 0 on success or a negative BSA_E* code; bsa_last_error() then holds a
+ * message for the calling thread.  Nothing here allocates device memory: the
+ * caller owns every buffer, including the workspace of the LUT builder.  All
+ * kernels are enqueued on `stream` (a hipStream_t passed as void*); only
+ * bsa_lut_packed / bsa_lut_contraction_offsets with a non-NULL `stats_host`
+ * wait for the stream, because the caller needs the counts to size its outputs.
+ *
+ * A block-sparse tensor is the triple (blocks, layout, sbs): `layout` is a
+ * contiguous (B, R, C) array of 0/1 bytes, `blocks` is (nnz, sbs, sbs) holding
+ * the active blocks in row-major order of the layout.
+ *
+ * Each declaration names the reference interface it stands in for
+ * (paths relative to the FelixSchoen/blksprs checkout).
+ */
+#ifndef BLKSPRS_AMD_H
+#define BLKSPRS_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define BSA_ABI_VERSION 1
+
+/* error codes */
+#define BSA_OK 0
+#define BSA_EINVAL (-1)  /* bad argument (shape, dtype, alignment, NULL pointer) */
+#define BSA_ELAUNCH (-2) /* the HIP runtime refused a launch or copy */
+#define BSA_ELIMIT (-3)  /* a size exceeds what the kernels index */
+
+/* element types of matmul / attention operands */
+#define BSA_F32 0
+#define BSA_F16 1
+#define BSA_BF16 2
+
+typedef void *bsa_stream_t; /* hipStream_t */
+
+int bsa_abi_version(void);
+const char *bsa_last_error(void);
+
+/* ------------------------------------------------------------------ LUTs */
+
+/* Bytes of scratch bsa_lut_packed / bsa_lut_contraction_offsets need for n entries. */
+size_t bsa_lut_workspace_bytes(int64_t n);
+
+/*
+ * Reverse index of a layout: packed[i] = (number of ones before i) if
+ * layout[i] else -1, int64, over the flattened layout.
+ * Replaces build_packed_indices (blksprs/utils/tools.py:38-57) and the
+ * `layout.sum().item()` block counts (blksprs/ops/matmul.py:270-273,
+ * blksprs/ops/conversion.py:286-288).
+ *
+ * row_len > 0 additionally writes the CSR row offsets row_offsets[n/row_len+1]
+ * (int32; the cumsum of per-row counts with a leading 0 of
+ * _build_segmented_indices, blksprs/ops/flash_attention.py:1923-1949) and the
+ * largest row count.  stats_dev[0] = count, stats_dev[1] = max row count
+ * (0 when row_len == 0).  If stats_host != NULL the two values are copied to it
+ * and the stream is synchronised.
+ */
+int bsa_lut_packed(const uint8_t *layout, int64_t n, int64_t row_len, int64_t *packed,
+                   int32_t *row_offsets, int64_t *stats_dev, int64_t *stats_host,
+                   void *workspace, size_t workspace_bytes, bsa_stream_t stream);
+
+/*
+ * Coordinates of the active blocks, int64 [count, 3] = (b, r, c) in row-major
+ * order: torch.nonzero(layout) of build_layout_indices
+ * (blksprs/utils/tools.py:33-35), derived from the reverse index.
+ */
+int bsa_lut_nonzero(const int64_t *packed, int64_t B, int64_t R, int64_t C, int64_t *coords,
+                    bsa_stream_t stream);
+
+/*
+ * CSR column ids (int32 [count], ascending inside a row): the `indices` of
+ * _build_segmented_indices (blksprs/ops/flash_attention.py:1945-1947).
+ */
+int bsa_lut_csr_indices(const int64_t *packed, int64_t n, int64_t C, int32_t *indices,
+                        bsa_stream_t stream);
+
+/*
+ * Per-row descending sort of the reverse index (active blocks first, then -1):
+ * packed_indices_sorted of softmax_fused_build_layout_cache
+ * (blksprs/ops/softmax.py:652-657), int64 [n_rows * C].
+ */
+int bsa_lut_sorted_rows(const int32_t *row_offsets, int64_t n_rows, int64_t C, int64_t *sorted,
+                        bsa_stream_t stream);
+
+/*
+ * Boolean block product lo[b,i,j] = OR_k lx[b,i,k] & ly[b,k,j]:
+ * build_sparsity_layout_matmul (blksprs/layouting/sparsity_layout.py:244-258).
+ */
+int bsa_layout_matmul(const uint8_t *lx, const uint8_t *ly, int64_t B, int64_t R, int64_t K,
+                      int64_t C, uint8_t *lo, bsa_stream_t stream);
+
+/*
+ * Contraction lists of a block-sparse product, phase 1.  For every position
+ * (b,i,j) of the output layout that is active (pidx_o >= 0) counts the k with
+ * x(b,i,k) and y(b,k,j) both active and writes the exclusive prefix of those
+ * counts over positions to pos_offsets (int32 [B*R*C + 1]); stats_dev[0] = total
+ * number of (x block, y block) pairs.  The reference has no such list: its
+ * kernel scans every k of every output block (blksprs/ops/matmul.py:191-226).
+ * mask_x: uint64 [B*R*W], mask_y: uint64 [B*C*W], W = ceil(K/64) (scratch the
+ * caller provides; they are inputs of phase 2).
+ */
+int bsa_lut_contraction_offsets(const int64_t *pidx_x, const int64_t *pidx_y,
+                                const int64_t *pidx_o, int64_t B, int64_t R, int64_t K, int64_t C,
+                                uint64_t *mask_x, uint64_t *mask_y, int32_t *pos_offsets,
+                                int64_t *stats_dev, int64_t *stats_host, void *workspace,
+                                size_t workspace_bytes, bsa_stream_t stream);
+
+/*
+ * Phase 2: pair_offsets int32 [nnz_o + 1] and pairs int32 [total, 2] =
+ * (index of the x block, index of the y block), ascending k inside an output
+ * block (the accumulation order of blksprs/ops/matmul.py:191-242).
+ */
+int bsa_lut_contraction_pairs(const int64_t *pidx_x, const int64_t *pidx_y, const int64_t *pidx_o,
+                              int64_t B, int64_t R, int64_t K, int64_t C, const uint64_t *mask_x,
+                              const uint64_t *mask_y, const int32_t *pos_offsets, int64_t nnz_o,
+                              int32_t *pair_offsets, int32_t *pairs, bsa_stream_t stream);
+
+/* ------------------------------------------------------------ conversion */
+
+/*
+ * Gather the active sbs x sbs tiles of a dense (B, rows, cols) array into
+ * (nnz, sbs, sbs).  Bit-exact copy for any element size in {1,2,4,8}.
+ * Replaces to_sparse_forward / to_sparse_kernel (blksprs/ops/conversion.py:191-276).
+ */
+int bsa_to_sparse(const void *dense, const int64_t *coords, void *blocks, int64_t nnz, int64_t rows,
+                  int64_t cols, int sbs, int elem_size, bsa_stream_t stream);
+
+/*
+ * Scatter compressed blocks into a dense (B, R*sbs, C*sbs) array; inactive
+ * tiles receive the element whose bit pattern is the low elem_size bytes of
+ * fill_bits.  One pass over the output (the reference fills and then
+ * overwrites).  Replaces to_dense_forward / to_dense_kernel
+ * (blksprs/ops/conversion.py:463-557).
+ */
+int bsa_to_dense(const void *blocks, const int64_t *packed, void *dense, int64_t B, int64_t R,
+                 int64_t C, int64_t nnz, int sbs, int elem_size, uint64_t fill_bits,
+                 bsa_stream_t stream);
+
+/* --------------------------------------------------------------- softmax */
+
+/*
+ * Row-wise softmax over the active blocks of each block row, fp32.
+ * row_offsets: int32 [n_rows + 1] CSR offsets of the layout flattened to
+ * (B*R, C).  Replaces softmax_fused_forward / softmax_fused_kernel and the
+ * five-kernel softmax_forward (blksprs/ops/softmax.py:93-144, :437-570).
+ */
+int bsa_softmax_fwd(const float *x, float *out, const int32_t *row_offsets, int64_t n_rows,
+                    int64_t nnz, int sbs, bsa_stream_t stream);
+
+/*
+ * dx = y * (g - sum_row(y * g)).  Replaces softmax_fused_backward /
+ * softmax_backward (blksprs/ops/softmax.py:156-207, :478-513, :574-638).
+ */
+int bsa_softmax_bwd(const float *grad_out, const float *y, float *grad_in,
+                    const int32_t *row_offsets, int64_t n_rows, int64_t nnz, int sbs,
+                    bsa_stream_t stream);
+
+/* ---------------------------------------------------------------- matmul */
+
+/*
+ * out[n] = sum over the pairs of output block n of x[px] @ y[py], fp32
+ * accumulation, result rounded once to `dtype`; an output block with no pair is
+ * written as zeros.  Replaces matmul_forward / matmul_kernel
+ * (blksprs/ops/matmul.py:70-253).  trans_x / trans_y read the x / y blocks
+ * transposed (block[c][r] instead of block[r][c]); the reference materialises
+ * such operands with transpose() first (blksprs/ops/matmul.py:135-143).
+ */
+int bsa_matmul(const void *x, const void *y, void *out, const int32_t *pair_offsets,
+               const int32_t *pairs, int64_t nnz_o, int64_t nnz_x, int64_t nnz_y, int sbs, int dtype,
+               int trans_x, int trans_y, bsa_stream_t stream);
+
+/* ------------------------------------------------------------- attention */
+
+/*
+ * Arguments of the block-sparse flash-attention kernels.  Layout shapes:
+ * q/o (B, nq, nh) resp. (B, nq, nhv); k (B, nk, nh); v (B, nk, nhv); the
+ * attention layout, mask and bias layouts (B, nq, nk).  pidx_* are int64
+ * reverse indices of those layouts (-1 = inactive); NULL mask/bias = absent;
+ * NULL causal_lengths = no native causal predicate.  lse and delta are fp32
+ * (B, nq, sbs); lse is in the log2 domain.
+ */
+typedef struct bsa_attn_args {
+  const void *q, *k, *v;
+  void *o;            /* forward: output blocks (dtype); backward: the saved output */
+  const void *d_o;    /* backward: gradient of o */
+  void *dq, *dk, *dv; /* backward outputs (dtype) */
+  float *lse;         /* forward output / backward input */
+  float *delta;       /* backward scratch: rowsum(o * d_o) */
+  const void *mask;   /* compressed mask blocks, element type mask_kind */
+  const void *bias;   /* compressed bias blocks (dtype) */
+  float *dbias;       /* backward: fp32 (n_bias_blocks, sbs, sbs) or NULL */
+  const int64_t *pidx_q, *pidx_k, *pidx_v, *pidx_o, *pidx_mask, *pidx_bias;
+  const int32_t *key_offsets, *key_indices;     /* CSR of the attention layout rows */
+  const int32_t *query_offsets, *query_indices; /* CSR of its transpose */
+  const int64_t *causal_lengths;                /* int64 [B] or NULL */
+  int64_t B, nq, nk, nh, nhv;
+  int64_t n_q_blocks, n_k_blocks, n_v_blocks, n_o_blocks, n_mask_blocks, n_bias_blocks;
+  int32_t sbs;
+  int32_t dtype;     /* BSA_F32 / BSA_F16 / BSA_BF16 */
+  int32_t mask_kind; /* 0 = none, 1 = one byte per element (bool/uint8), 2 = same dtype as q */
+  float scale;
+} bsa_attn_args;
+
+/*
+ * o = softmax(scale * q k^T + bias, masked) v over the active key blocks of
+ * each query block, plus lse.  Replaces _FlashAttentionAutograd.forward /
+ * flash_attention_kernel (blksprs/ops/flash_attention.py:312-503, :994-1224).
+ * Every block of `o` that is active in the output layout is written.
+ */
+int bsa_attn_fwd(const bsa_attn_args *args, bsa_stream_t stream);
+
+/*
+ * dq, dk, dv (and dbias) from the saved lse.  Replaces
+ * _FlashAttentionAutograd.backward and its three kernels
+ * (blksprs/ops/flash_attention.py:505-787, :1228-1735).  Every block of dq, dk,
+ * dv (and dbias) is written, zeros where nothing contributes.
+ */
+int bsa_attn_bwd(const bsa_attn_args *args, bsa_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BLKSPRS_AMD_H */
