@@ -1,0 +1,278 @@
+"""Benchmark of the block-sparse compute path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2]
+
+A step is one pass of the hot path over one batch of synthetic, seeded input that is already resident in
+HBM, with the lookup tables built beforehand (their build time is reported separately).  The default
+workload is configuration 2 of BASELINE.json (bf16 block-sparse matmul, B=16, 4096^3, sbs 64, 25 % operand
+density, product output layout), the configuration the headline metric is quoted on; ``--config`` selects
+c1 (fp32 matmul 256^3), c3 (fp32 softmax), c4 / c4bwd (bf16 flash attention forward / forward+backward) or
+c5 (fp16 matmul, sbs 16) instead.  One JSON line is printed on stdout; everything else goes to stderr.
+
+The ``roofline`` object prices the dominant kernel against the roofline that bounds it, from the average
+launch duration measured with events on the launch stream; ``cpu_baseline`` times the CPU oracle on a
+bounded sample of the same workload on the host cores (reported, not a target).
+"""
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+import torch
+
+# MI355X published peaks (dense)
+PEAK_HBM_GBS = 8000.0
+PEAK_MFMA_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def _events(n):
+    return [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+
+
+def time_steps(step, steps, warmup):
+    """Returns (wall ms per step over exactly `steps` steps, mean per-launch ms from stream events)."""
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    ev = _events(steps)
+    for s, e in ev:
+        s.record()
+        step()
+        e.record()
+    torch.cuda.synchronize()
+    per = sorted(s.elapsed_time(e) for s, e in ev)
+    return wall_ms, sum(per) / len(per), per[len(per) // 2]
+
+
+# --------------------------------------------------------------------------- workloads
+
+
+def matmul_workload(name, B, n, sbs, dtype, density, ensure_rows, value_scale, dev, cpu_sample_batches):
+    import blksprs_amd as bs
+    from oracle import blksprs_oracle as orc
+
+    g = torch.Generator().manual_seed(0)
+    lx = orc.random_layout((B, n, n), density, g, ensure_rows=ensure_rows)
+    ly = orc.random_layout((B, n, n), density, g, ensure_rows=ensure_rows)
+    lxd, lyd = lx.to(dev), ly.to(dev)
+    lod = bs.layouting.build_sparsity_layout_matmul(lxd, lyd)
+    nnz_x, nnz_y, nnz_o = int(lx.sum()), int(ly.sum()), int(lod.sum())
+    gd = torch.Generator(device=dev).manual_seed(1)
+    x = (torch.randn((nnz_x, sbs, sbs), generator=gd, device=dev) * value_scale).to(dtype)
+    y = torch.randn((nnz_y, sbs, sbs), generator=gd, device=dev).to(dtype)
+
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    cache = {}
+    out = bs.ops.matmul(x, lxd, y, lyd, lod, sbs, layout_cache=cache)
+    torch.cuda.synchronize()
+    lut_ms = (time.perf_counter() - t0) * 1e3
+    pairs = int(cache["contraction_pairs"].size(0))
+    es = x.element_size()
+    flops = pairs * 2.0 * sbs ** 3
+    alg_bytes = (nnz_x + nnz_y + nnz_o) * sbs * sbs * es
+    log(f"[{name}] nnz_x={nnz_x} nnz_y={nnz_y} nnz_o={nnz_o} ({nnz_o / (B * n * n):.1%} of output) "
+        f"pairs={pairs} (mean {pairs / max(nnz_o, 1):.2f}/block) flops={flops / 1e9:.2f}G "
+        f"algorithmic bytes={alg_bytes / 1e6:.1f}MB; first call incl. LUT build {lut_ms:.2f} ms")
+
+    bs.utils.disable_validation()
+
+    def step():
+        return bs.ops.matmul(x, lxd, y, lyd, lod, sbs, layout_cache=cache)
+
+    def cpu_baseline():
+        nb = min(cpu_sample_batches, B)
+        sl = lambda lay, t: t[:int(lay[:nb].sum())].float().cpu()
+        lo = lod.cpu()
+        xs, ys = sl(lx, x), sl(ly, y)
+        t0 = time.perf_counter()
+        orc.matmul(xs, lx[:nb].numpy(), ys, ly[:nb].numpy(), lo[:nb].numpy(), sbs, acc_dtype=torch.float32)
+        dt = time.perf_counter() - t0
+        sample_pairs = int(torch.einsum("bik,bkj,bij->", lx[:nb].float(), ly[:nb].float(), lo[:nb].float()))
+        return {"value": sample_pairs * 2.0 * sbs ** 3 / dt / 1e12, "unit": "TFLOP/s",
+                "cores": torch.get_num_threads(), "kind": "port",
+                "sample": f"{nb} of {B} batches, dense-masked fp32 torch matmul + to_sparse, {dt:.2f} s"}
+
+    dt_name = {torch.bfloat16: "bf16", torch.float16: "f16", torch.float32: "f32"}[dtype]
+    return dict(step=step, flops=flops, alg_bytes=alg_bytes, dtype=dt_name, bound="hbm", cpu_baseline=cpu_baseline,
+                kernel="matmul_mfma_kernel" if sbs > 16 else "matmul_small_kernel",
+                config={"workload": name, "B": B, "M": n * sbs, "K": n * sbs, "N": n * sbs,
+                        "sparsity_block_size": sbs, "density": density, "nnz_x": nnz_x, "nnz_y": nnz_y,
+                        "nnz_o": nnz_o, "block_pairs": pairs, "lut_build_ms": round(lut_ms, 3)})
+
+
+def softmax_workload(dev):
+    import blksprs_amd as bs
+    from oracle import blksprs_oracle as orc
+
+    B, n, sbs = 32, 32, 64
+    g = torch.Generator().manual_seed(0)
+    tri = torch.tril(torch.ones((n, n), dtype=torch.bool))
+    layout = tri.unsqueeze(0) | ((torch.rand((B, n, n), generator=g) < 0.1) & ~tri)
+    ld = layout.to(dev)
+    nnz = int(layout.sum())
+    x = torch.randn((nnz, sbs, sbs), device=dev) * 2.0  # N(0, 4): sigma = 2
+    cache = {}
+    bs.ops.softmax(x, ld, sbs, layout_cache=cache)
+    alg_bytes = 2 * nnz * sbs * sbs * 4
+    log(f"[c3] nnz={nnz} algorithmic bytes={alg_bytes / 1e6:.1f}MB")
+    bs.utils.disable_validation()
+
+    def step():
+        return bs.ops.softmax(x, ld, sbs, layout_cache=cache)
+
+    def cpu_baseline():
+        nb = 8
+        cnt = int(layout[:nb].sum())
+        xs = x[:cnt].cpu()
+        t0 = time.perf_counter()
+        orc.softmax(xs, layout[:nb].numpy(), sbs)
+        dt = time.perf_counter() - t0
+        return {"value": 2 * cnt * sbs * sbs * 4 / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(),
+                "kind": "port", "sample": f"{nb} of {B} batches, dense -inf-masked torch softmax (fp64), {dt:.2f} s"}
+
+    return dict(step=step, flops=0.0, alg_bytes=alg_bytes, dtype="f32", bound="hbm", cpu_baseline=cpu_baseline,
+                kernel="softmax_fwd_kernel",
+                config={"workload": "c3_softmax_fp32", "B": B, "rows": n * sbs, "cols": n * sbs,
+                        "sparsity_block_size": sbs, "nnz": nnz})
+
+
+def attention_workload(dev, backward):
+    import blksprs_amd as bs
+    from oracle import blksprs_oracle as orc
+
+    BH, n, sbs, nh = 64, 128, 64, 2
+    g = torch.Generator().manual_seed(0)
+    la = orc.bigbird_layout(BH, n, g)
+    lmask = la & torch.ones((n, n), dtype=torch.bool).triu()
+    nnz = int(la.sum())
+    lad, lmd = la.to(dev), lmask.to(dev)
+    full = torch.ones((BH, n, nh), dtype=torch.bool, device=dev)
+    # causal mask inside every mask block (key position > query position), built on the device
+    midx = torch.nonzero(lmd)
+    r = torch.arange(sbs, device=dev)
+    qpos = midx[:, 1].view(-1, 1, 1) * sbs + r.view(1, -1, 1)
+    kpos = midx[:, 2].view(-1, 1, 1) * sbs + r.view(1, 1, -1)
+    mask = kpos > qpos
+    q, k, v = (torch.randn((BH * n * nh, sbs, sbs), device=dev).to(torch.bfloat16) for _ in range(3))
+    d_o = torch.randn((BH * n * nh, sbs, sbs), device=dev).to(torch.bfloat16)
+    cache = {}
+    if backward:
+        q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
+    bs.ops.flash_attention(q, full, k, full, v, full, lad, sbs, attention_mask=mask, sparsity_layout_mask=lmd,
+                           layout_cache=cache)
+    fwd_flops = nnz * 4.0 * sbs * sbs * (nh * sbs)
+    flops = fwd_flops * (3.5 if backward else 1.0)
+    alg_bytes = 4 * BH * n * nh * sbs * sbs * 2 + int(lmask.sum()) * sbs * sbs
+    log(f"[c4] layout blocks={nnz} ({nnz / (BH * n):.1f}/row) causal-useful={int((la & torch.ones((n, n), dtype=torch.bool).tril()).sum())} "
+        f"mask blocks={int(lmask.sum())} fwd flops={fwd_flops / 1e9:.1f}G")
+    bs.utils.disable_validation()
+
+    def step():
+        o = bs.ops.flash_attention(q, full, k, full, v, full, lad, sbs, attention_mask=mask,
+                                   sparsity_layout_mask=lmd, layout_cache=cache)
+        if backward:
+            q.grad = k.grad = v.grad = None
+            o.backward(d_o)
+        return o
+
+    def cpu_baseline():
+        heads = 1
+        qs, ks, vs = (t[:heads * n * nh].detach().float().cpu() for t in (q, k, v))
+        cnt = int(lmask[:heads].sum())
+        t0 = time.perf_counter()
+        orc.flash_attention(qs, full[:heads].cpu().numpy(), ks, full[:heads].cpu().numpy(), vs,
+                            full[:heads].cpu().numpy(), la[:heads].numpy(), sbs, mask=mask[:cnt].cpu(),
+                            layout_mask=lmask[:heads].numpy())
+        dt = time.perf_counter() - t0
+        return {"value": int(la[:heads].sum()) * 4.0 * sbs * sbs * nh * sbs / dt / 1e12, "unit": "TFLOP/s",
+                "cores": torch.get_num_threads(), "kind": "port",
+                "sample": f"forward of {heads} of {BH} heads, dense masked fp32 torch attention, {dt:.2f} s"}
+
+    return dict(step=step, flops=flops, alg_bytes=alg_bytes, dtype="bf16", bound="mfma", cpu_baseline=cpu_baseline,
+                kernel="attn_fwd",
+                config={"workload": "c4_flash_attention_bf16" + ("_fwd_bwd" if backward else "_fwd"),
+                        "batch_heads": BH, "seq": n * sbs, "head_dim": nh * sbs, "sparsity_block_size": sbs,
+                        "layout_blocks": nnz, "mask": "explicit causal blocks"})
+
+
+def make_workload(name, dev):
+    if name == "c1":
+        return matmul_workload("c1_matmul_fp32", 2, 8, 32, torch.float32, 0.5, True, 1.0, dev, 2)
+    if name == "c2":
+        return matmul_workload("c2_matmul_bf16", 16, 64, 64, torch.bfloat16, 0.25, False, 1.0 / 64.0, dev, 2)
+    if name == "c3":
+        return softmax_workload(dev)
+    if name == "c4":
+        return attention_workload(dev, backward=False)
+    if name == "c4bwd":
+        return attention_workload(dev, backward=True)
+    if name == "c5":
+        return matmul_workload("c5_matmul_fp16", 64, 128, 16, torch.float16, 0.05, True, 1.0, dev, 8)
+    raise SystemExit(f"unknown config {name}")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c4bwd", "c5"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        raise SystemExit("bench.py measures one GPU: the block-sparse path has no cross-GPU step in this build "
+                         "(it would shard on the batch dimension with no collective); run with --gpus 1")
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a GPU (the product has no CPU path)")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    w = make_workload(args.config, dev)
+    wall_ms, mean_ms, median_ms = time_steps(w["step"], args.steps, args.warmup)
+    tflops = w["flops"] / (wall_ms * 1e-3) / 1e12
+    gbs = w["alg_bytes"] / (mean_ms * 1e-3) / 1e9
+    if w["bound"] == "hbm":
+        roofline = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                    "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None}
+    else:
+        ach = w["flops"] / (mean_ms * 1e-3) / 1e12
+        peak = PEAK_MFMA_TFLOPS[w["dtype"]]
+        roofline = {"bound": "mfma", "achieved": round(ach, 1), "peak": peak, "unit": "TFLOP/s",
+                    "frac": round(ach / peak, 4), "traffic": None}
+    roofline["kernel"] = w["kernel"]
+    roofline["launch_ms_mean"] = round(mean_ms, 4)
+    roofline["launch_ms_median"] = round(median_ms, 4)
+    line = {
+        "metric": "effective TFLOP/s on nonzero blocks" if w["flops"] else "achieved GB/s on nonzero blocks",
+        "value": round(tflops, 3) if w["flops"] else round(gbs, 1),
+        "unit": "TFLOP/s" if w["flops"] else "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall_ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": w["dtype"], "data": "synthetic",
+        "config": w["config"], "roofline": roofline,
+    }
+    if w["flops"]:
+        line["pct_of_mfma_peak"] = round(100.0 * tflops / PEAK_MFMA_TFLOPS[w["dtype"]], 2)
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = w["cpu_baseline"]()
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

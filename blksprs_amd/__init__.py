@@ -10,7 +10,7 @@ import os as _os
 
 # Accepted for import-time compatibility with the reference's BLKSPRS_AUTOTUNE switch
 # (blksprs/utils/autotuning.py:5-9); tile shapes here are fixed per (block size, dtype) at compile time.
-if _os.environ.get("BLKSPRS_AUTOTUNE", "DEFAULT") not in ("DEFAULT", "TEST"):
+if _os.environ.get("BLKSPRS_AUTOTUNE", "DEFAULT").upper() not in ("DEFAULT", "TEST"):
     raise NotImplementedError(f"Unknown autotune mode: {_os.environ['BLKSPRS_AUTOTUNE']}")
 
 from .utils.blksprs_tensor import BlksprsTensor

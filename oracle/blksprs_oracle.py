@@ -1,0 +1,237 @@
+"""CPU restatement of the reference's block-sparse compute path.
+
+TEST INFRASTRUCTURE ONLY.  Imported by ``tests/``, ``__graft_entry__.smoke()`` and the
+``cpu_baseline`` leg of ``bench.py`` as the checker / reported baseline; the product
+(``blksprs_amd``) never imports, calls or falls back to anything in this file.
+
+Integer tables are numpy, floating-point operators are dense-masked torch on the CPU.
+Every function names the reference lines it restates (paths relative to the
+FelixSchoen/blksprs checkout).  How each one is pinned (brute force on tiny inputs,
+closed forms, torch library routines, known answers held by the reference's tests)
+is listed in ``tests/test_oracle_pins.py``; every function below has at least one
+such pin, none is "parity unpinned".
+"""
+
+import math
+
+import numpy as np
+import torch
+
+# --------------------------------------------------------------------------- lookup tables (integer, exact)
+
+
+def packed_indices(layout) -> np.ndarray:
+    """blksprs/utils/tools.py:38-57: ``where(l == 1, cumsum(l) - 1, -1)`` over the flattened layout, int64."""
+    flat = np.asarray(layout).reshape(-1).astype(np.int64)
+    return np.where(flat == 1, np.cumsum(flat) - 1, -1).astype(np.int64)
+
+
+def layout_indices(layout) -> np.ndarray:
+    """blksprs/utils/tools.py:33-35: ``nonzero(layout)`` as int64 ``[nnz, 3]`` in row-major order."""
+    return np.argwhere(np.asarray(layout) != 0).astype(np.int64).reshape(-1, 3)
+
+
+def n_sparse_blocks(layout) -> int:
+    """blksprs/ops/conversion.py:286-288: the block count, summed in int64."""
+    return int(np.asarray(layout).astype(np.int64).sum())
+
+
+def segmented_indices(layout):
+    """blksprs/ops/flash_attention.py:1923-1949: CSR adjacency ``(indices, offsets, max_per_row)``.
+
+    ``layout`` is ``(B, rows, cols)``; offsets has ``B * rows + 1`` int32 entries starting at 0; indices are
+    the active column ids row by row; empty or all-zero layouts give ``(empty, zeros, 1)``.
+    """
+    lay = np.asarray(layout).astype(np.int64)
+    B, R, C = lay.shape
+    counts = lay.sum(axis=2).reshape(-1)
+    zeros = np.zeros(B * R + 1, dtype=np.int32)
+    if counts.size == 0 or counts.max() == 0:
+        return np.empty(0, dtype=np.int32), zeros, 1
+    offsets = zeros.copy()
+    offsets[1:] = np.cumsum(counts)
+    indices = np.argwhere(lay.reshape(B * R, C) != 0)[:, 1].astype(np.int32)
+    return indices, offsets, int(counts.max())
+
+
+def segmented_index_dtype(n_active_blocks: int, n_blocks_col: int):
+    """blksprs/ops/flash_attention.py:1952-1957."""
+    limit = 2_147_483_647
+    return np.int64 if (n_active_blocks > limit or n_blocks_col - 1 > limit) else np.int32
+
+
+def sorted_packed_indices(layout):
+    """blksprs/ops/softmax.py:652-666: per-row descending sort of the packed indices and
+    ``max_blocks_line = ceil_pow2(max(longest row, 2))``."""
+    lay = np.asarray(layout)
+    packed = packed_indices(lay).reshape(lay.shape)
+    srt = -np.sort(-packed, axis=-1)
+    longest = int((srt.reshape(-1, lay.shape[-1]) != -1).sum(axis=-1).max()) if srt.size else 0
+    longest = max(longest, 2)
+    return srt.reshape(-1), 1 << (longest - 1).bit_length()
+
+
+def layout_matmul(layout_x, layout_y) -> np.ndarray:
+    """blksprs/layouting/sparsity_layout.py:244-258: boolean block product."""
+    lx = np.asarray(layout_x).astype(np.int64)
+    ly = np.asarray(layout_y).astype(np.int64)
+    return np.einsum("bik,bkj->bij", lx, ly) > 0
+
+
+def contraction_lists(layout_x, layout_y, layout_o):
+    """The work list implied by the reference kernel's scan (blksprs/ops/matmul.py:191-226): for every
+    active output block, in row-major order, the ``(packed x index, packed y index)`` of every k where both
+    operand blocks are active, ascending k.  Returns ``(pair_offsets int32 [nnz_o + 1], pairs int32 [T, 2])``.
+    """
+    lx, ly, lo = (np.asarray(a) != 0 for a in (layout_x, layout_y, layout_o))
+    px = packed_indices(lx).reshape(lx.shape)
+    py = packed_indices(ly).reshape(ly.shape)
+    offsets, pairs = [0], []
+    for b, i, j in np.argwhere(lo):
+        ks = np.nonzero(lx[b, i, :] & ly[b, :, j])[0]
+        pairs.extend((px[b, i, k], py[b, k, j]) for k in ks)
+        offsets.append(len(pairs))
+    return (np.asarray(offsets, dtype=np.int32),
+            np.asarray(pairs, dtype=np.int32).reshape(-1, 2))
+
+
+# --------------------------------------------------------------------------- conversion (bit exact)
+
+
+def to_sparse(x: torch.Tensor, layout, sbs: int) -> torch.Tensor:
+    """blksprs/ops/conversion.py:230-276: the active ``sbs x sbs`` tiles of dense ``(B, R*sbs, C*sbs)`` in
+    row-major block order (the reshape/permute identity of :127-138)."""
+    lay = torch.as_tensor(np.asarray(layout) != 0)
+    B, R, C = lay.shape
+    tiles = x.reshape(B, R, sbs, C, sbs).permute(0, 1, 3, 2, 4)
+    return tiles[lay].reshape(-1, sbs, sbs).clone()
+
+
+def to_dense(x: torch.Tensor, layout, sbs: int, fill_value=0) -> torch.Tensor:
+    """blksprs/ops/conversion.py:463-557: blocks scattered into a dense array pre-filled with ``fill_value``."""
+    lay = torch.as_tensor(np.asarray(layout) != 0)
+    B, R, C = lay.shape
+    tiles = torch.full((B, R, C, sbs, sbs), fill_value, dtype=x.dtype)
+    tiles[lay] = x
+    return tiles.permute(0, 1, 3, 2, 4).reshape(B, R * sbs, C * sbs).clone()
+
+
+# --------------------------------------------------------------------------- floating-point operators
+
+
+def matmul(x, layout_x, y, layout_y, layout_o, sbs: int, acc_dtype=torch.float32) -> torch.Tensor:
+    """blksprs/ops/matmul.py:186-253 via the recipe of test/cases/test_blocksparse.py:479-492:
+    ``to_sparse(to_dense(x) @ to_dense(y), layout_o)`` accumulated in ``acc_dtype``, rounded to the input dtype."""
+    xd = to_dense(x, layout_x, sbs).to(acc_dtype)
+    yd = to_dense(y, layout_y, sbs).to(acc_dtype)
+    return to_sparse(torch.matmul(xd, yd), layout_o, sbs).to(x.dtype)
+
+
+def softmax(x, layout, sbs: int) -> torch.Tensor:
+    """blksprs/ops/softmax.py:524-570: per element row, softmax over the concatenation of the row's active
+    blocks; inactive blocks act as ``-inf`` and rows without blocks do not exist in the output."""
+    dense = to_dense(x.to(torch.float64), layout, sbs, fill_value=float("-inf"))
+    lay = torch.as_tensor(np.asarray(layout) != 0)
+    row_has_block = lay.any(dim=-1).repeat_interleave(sbs, dim=1)  # (B, R*sbs)
+    out = torch.softmax(dense, dim=-1)
+    out = torch.where(row_has_block.unsqueeze(-1), out, torch.zeros_like(out))
+    return to_sparse(out, layout, sbs).to(x.dtype)
+
+
+def softmax_backward(grad_out, y, layout, sbs: int) -> torch.Tensor:
+    """blksprs/ops/softmax.py:581-638: ``dx = y * (g - sum_row(y * g))``."""
+    yd = to_dense(y.to(torch.float64), layout, sbs)
+    gd = to_dense(grad_out.to(torch.float64), layout, sbs)
+    s = (yd * gd).sum(dim=-1, keepdim=True)
+    return to_sparse(yd * (gd - s), layout, sbs).to(y.dtype)
+
+
+def attention_scores_mask(attention_layout, sbs: int, mask=None, layout_mask=None, causal_lengths=None):
+    """Boolean ``(B, Sq, Sk)`` array of ignored positions: outside the block layout
+    (blksprs/ops/flash_attention.py:1049-1057), native causal predicate (:1128-1142), explicit mask where a
+    mask block exists (:1146-1155)."""
+    lay = torch.as_tensor(np.asarray(attention_layout) != 0)
+    B, nq, nk = lay.shape
+    ignored = ~lay.repeat_interleave(sbs, dim=1).repeat_interleave(sbs, dim=2)
+    if causal_lengths is not None:
+        qpos = torch.arange(nq * sbs).view(1, -1, 1)
+        kpos = torch.arange(nk * sbs).view(1, 1, -1)
+        length = torch.as_tensor(causal_lengths).view(-1, 1, 1)
+        ignored = ignored | (kpos > qpos) | (qpos >= length) | (kpos >= length)
+    if mask is not None:
+        md = to_dense((mask != 0), layout_mask, sbs, fill_value=False)
+        ignored = ignored | md
+    return ignored
+
+
+def flash_attention(q, layout_q, k, layout_k, v, layout_v, attention_layout, sbs: int, scale=None,
+                    mask=None, layout_mask=None, bias=None, layout_bias=None, layout_o=None,
+                    causal_lengths=None, acc_dtype=torch.float32):
+    """blksprs/ops/flash_attention.py:1056-1224 restated densely, following the recipe of
+    test/cases/test_blocksparse.py:1796-1828: ``scale * q k^T`` -> ``+ bias`` -> causal / layout / mask to
+    ``-inf`` -> softmax -> NaN rows (nothing attended) to 0 -> ``@ v`` -> output layout.
+
+    Inactive q/k head slices contribute zeros to the scores (:1074), inactive v slices contribute nothing,
+    output slices inactive in ``layout_o`` are dropped.  Differentiable w.r.t. q, k, v, bias.
+    Returns the compressed output (in ``q.dtype``).
+    """
+    qd = to_dense_autograd(q, layout_q, sbs).to(acc_dtype)
+    kd = to_dense_autograd(k, layout_k, sbs).to(acc_dtype)
+    vd = to_dense_autograd(v, layout_v, sbs).to(acc_dtype)
+    head_dim = qd.shape[-1]
+    if scale is None:
+        scale = 1.0 if head_dim == 0 else 1.0 / math.sqrt(head_dim)
+    scores = torch.matmul(qd, kd.transpose(-1, -2)) * scale
+    if bias is not None:
+        scores = scores + to_dense_autograd(bias, layout_bias, sbs).to(acc_dtype)
+    ignored = attention_scores_mask(attention_layout, sbs, mask, layout_mask, causal_lengths)
+    scores = scores.masked_fill(ignored, float("-inf"))
+    all_ignored = ignored.all(dim=-1, keepdim=True)
+    probs = torch.softmax(scores, dim=-1)
+    probs = torch.where(all_ignored, torch.zeros_like(probs), probs)
+    out = torch.matmul(probs, vd)
+    if layout_o is None:
+        layout_o = layout_matmul(attention_layout, layout_v)
+    return to_sparse_autograd(out, layout_o, sbs).to(q.dtype)
+
+
+def to_dense_autograd(x, layout, sbs: int):
+    """``to_dense`` built from differentiable indexing (zeros outside the layout)."""
+    lay = torch.as_tensor(np.asarray(layout) != 0)
+    B, R, C = lay.shape
+    tiles = torch.zeros((B, R, C, sbs, sbs), dtype=x.dtype)
+    tiles = tiles.masked_scatter(lay.view(B, R, C, 1, 1).expand_as(tiles), x)
+    return tiles.permute(0, 1, 3, 2, 4).reshape(B, R * sbs, C * sbs)
+
+
+def to_sparse_autograd(x, layout, sbs: int):
+    lay = torch.as_tensor(np.asarray(layout) != 0)
+    B, R, C = lay.shape
+    return x.reshape(B, R, sbs, C, sbs).permute(0, 1, 3, 2, 4)[lay].reshape(-1, sbs, sbs)
+
+
+# --------------------------------------------------------------------------- seeded workloads
+
+
+def random_layout(shape, density: float, generator: torch.Generator, ensure_rows: bool = False) -> torch.Tensor:
+    """Bernoulli(density) block layout; with ``ensure_rows`` every row gets at least one block."""
+    lay = torch.rand(shape, generator=generator) < density
+    if ensure_rows and lay.numel():
+        B, R, C = shape
+        empty = ~lay.any(dim=-1)
+        cols = torch.randint(0, C, (B, R), generator=generator)
+        lay[empty, cols[empty]] = True
+    return lay
+
+
+def bigbird_layout(batch: int, n: int, generator: torch.Generator, window: int = 4, n_global: int = 2,
+                   n_random: int = 3) -> torch.Tensor:
+    """BigBird-style block layout: |i - j| <= window, the first ``n_global`` rows and columns, and
+    ``n_random`` random columns per row."""
+    i = torch.arange(n).view(-1, 1)
+    j = torch.arange(n).view(1, -1)
+    base = ((i - j).abs() <= window) | (j < n_global) | (i < n_global)
+    lay = base.unsqueeze(0).repeat(batch, 1, 1)
+    rnd = torch.rand((batch, n, n), generator=generator).argsort(dim=-1)[..., :n_random]
+    lay.scatter_(2, rnd, True)
+    return lay

@@ -1,0 +1,244 @@
+"""Parity of block-sparse flash attention (forward and backward) with the CPU oracle:
+rtol = atol = 1e-5 for fp32... the oracle is dense fp64 here, so fp32 is checked at 2e-5 absolute on
+O(1) values; 2e-2 for fp16 / bf16."""
+
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import blksprs_amd as bs
+from oracle import blksprs_oracle as orc
+from tests.helpers import assert_close, rand_blocks, rand_layout
+
+pytestmark = pytest.mark.gpu
+TOL = {torch.float32: 1e-5, torch.float16: 2e-2, torch.bfloat16: 2e-2}
+
+
+def _run_case(device, dtype, sbs, B, nq, nk, nh, nhv, density, seed, use_mask=False, use_bias=False,
+              use_causal=False, sparse_heads=False, custom_o=False, scale=None):
+    g = torch.Generator().manual_seed(seed)
+    la = orc.random_layout((B, nq, nk), density, g, ensure_rows=True)
+    full = lambda r, c: torch.ones((B, r, c), dtype=torch.bool)
+    lq, lk, lv = full(nq, nh), full(nk, nh), full(nk, nhv)
+    if sparse_heads:
+        lq = orc.random_layout((B, nq, nh), 0.7, g, ensure_rows=True)
+        lk = orc.random_layout((B, nk, nh), 0.7, g, ensure_rows=True)
+        lv = orc.random_layout((B, nk, nhv), 0.7, g, ensure_rows=True)
+    lo = orc.random_layout((B, nq, nhv), 0.8, g, ensure_rows=True) if custom_o else None
+    q = rand_blocks(int(lq.sum()), sbs, dtype, seed + 1)
+    k = rand_blocks(int(lk.sum()), sbs, dtype, seed + 2)
+    v = rand_blocks(int(lv.sum()), sbs, dtype, seed + 3)
+    mask = lmask = bias = lbias = lengths = None
+    if use_mask:
+        lmask = la & orc.random_layout((B, nq, nk), 0.7, g)
+        mask = torch.rand((int(lmask.sum()), sbs, sbs), generator=g) < 0.3
+    if use_bias:
+        lbias = la & orc.random_layout((B, nq, nk), 0.7, g)
+        bias = rand_blocks(int(lbias.sum()), sbs, dtype, seed + 4)
+    if use_causal:
+        lengths = torch.randint(1, nq * sbs + 1, (B,), generator=g)
+        lengths[0] = nq * sbs
+
+    to = lambda t: None if t is None else t.to(device)
+    qd, kd, vd = (t.to(device).requires_grad_(True) for t in (q, k, v))
+    bd = None if bias is None else bias.to(device).requires_grad_(True)
+    out = bs.ops.flash_attention(qd, to(lq), kd, to(lk), vd, to(lv), to(la), sbs, scale=scale,
+                                 attention_mask=to(mask), sparsity_layout_mask=to(lmask),
+                                 attention_bias=bd, sparsity_layout_bias=to(lbias),
+                                 sparsity_layout_o=to(lo), causal_lengths=to(lengths))
+    assert isinstance(out, bs.BlksprsTensor) and out.dtype == dtype
+
+    q64, k64, v64 = (t.double().requires_grad_(True) for t in (q, k, v))
+    b64 = None if bias is None else bias.double().requires_grad_(True)
+    ref = orc.flash_attention(q64, lq.numpy(), k64, lk.numpy(), v64, lv.numpy(), la.numpy(), sbs, scale=scale,
+                              mask=mask, layout_mask=None if lmask is None else lmask.numpy(),
+                              bias=b64, layout_bias=None if lbias is None else lbias.numpy(),
+                              layout_o=None if lo is None else lo.numpy(), causal_lengths=lengths,
+                              acc_dtype=torch.float64)
+    tol = TOL[dtype]
+    tag = f"{dtype} sbs={sbs} mask={use_mask} bias={use_bias} causal={use_causal}"
+    assert_close(out, ref, tol, "O " + tag)
+    go = rand_blocks(out.size(0), sbs, dtype, seed + 5)
+    out.backward(go.to(device))
+    ref.backward(go.double())
+    # gradients pass through probabilities rounded to the operand type: allow twice the forward tolerance
+    gtol = tol if dtype == torch.float32 else 2 * tol
+    assert_close(qd.grad, q64.grad, gtol, "dQ " + tag)
+    assert_close(kd.grad, k64.grad, gtol, "dK " + tag)
+    assert_close(vd.grad, v64.grad, gtol, "dV " + tag)
+    if bias is not None:
+        assert_close(bd.grad, b64.grad, gtol, "dBias " + tag)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("sbs", [16, 32, 64])
+def test_plain_layout(device, dtype, sbs):
+    _run_case(device, dtype, sbs, B=2, nq=4, nk=4, nh=2, nhv=2, density=0.5, seed=sbs)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("sbs", [16, 64])
+@pytest.mark.parametrize("use_mask,use_bias,use_causal", [(True, False, False), (False, True, False),
+                                                           (False, False, True), (True, True, True)])
+def test_mask_bias_causal(device, dtype, sbs, use_mask, use_bias, use_causal):
+    _run_case(device, dtype, sbs, B=2, nq=3, nk=3, nh=1, nhv=2, density=0.7, seed=3 * sbs + use_mask,
+              use_mask=use_mask, use_bias=use_bias, use_causal=use_causal)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_rectangular_sparse_heads_and_custom_output_layout(device, dtype):
+    _run_case(device, dtype, 32, B=2, nq=3, nk=5, nh=3, nhv=2, density=0.5, seed=77, sparse_heads=True,
+              custom_o=True, use_mask=True, use_bias=True, scale=0.37)
+
+
+def test_bigbird_layout_with_causal_mask_head_dim_128(device):
+    """Config 4's shape at reduced batch and length: bf16, sbs 64, head_dim 128, BigBird layout, causal mask."""
+    B, n, sbs, nh = 2, 16, 64, 2
+    g = torch.Generator().manual_seed(0)
+    la = orc.bigbird_layout(B, n, g)
+    lmask = la & torch.ones((n, n), dtype=torch.bool).triu()
+    pos = torch.arange(n * sbs)
+    dense_mask = (pos.view(1, -1) > pos.view(-1, 1)).unsqueeze(0).expand(B, -1, -1)
+    mask = orc.to_sparse(dense_mask, lmask.numpy(), sbs)
+    full = torch.ones((B, n, nh), dtype=torch.bool)
+    q, k, v = (rand_blocks(B * n * nh, sbs, torch.bfloat16, s) for s in (1, 2, 3))
+    qd, kd, vd = (t.to(device).requires_grad_(True) for t in (q, k, v))
+    out = bs.ops.flash_attention(qd, full.to(device), kd, full.to(device), vd, full.to(device), la.to(device), sbs,
+                                 attention_mask=mask.to(device), sparsity_layout_mask=lmask.to(device))
+    q64, k64, v64 = (t.double().requires_grad_(True) for t in (q, k, v))
+    ref = orc.flash_attention(q64, full.numpy(), k64, full.numpy(), v64, full.numpy(), la.numpy(), sbs,
+                              mask=mask, layout_mask=lmask.numpy(), acc_dtype=torch.float64)
+    assert_close(out, ref, 2e-2, "O bigbird")
+    # same result from the native causal predicate instead of the mask tensor
+    out2 = bs.ops.flash_attention(qd, full.to(device), kd, full.to(device), vd, full.to(device), la.to(device), sbs,
+                                  causal_lengths=torch.full((B,), n * sbs, device=device))
+    assert_close(out2, ref, 2e-2, "O bigbird, causal_lengths")
+    go = rand_blocks(out.size(0), sbs, torch.bfloat16, 5)
+    out.backward(go.to(device))
+    ref.backward(go.double())
+    assert_close(qd.grad, q64.grad, 4e-2, "dQ bigbird")
+    assert_close(kd.grad, k64.grad, 4e-2, "dK bigbird")
+    assert_close(vd.grad, v64.grad, 4e-2, "dV bigbird")
+
+
+def test_full_layout_equals_sdpa(device):
+    # reference: test_regressions.py:488-527
+    B, S, D, sbs = 2, 128, 64, 32
+    q, k, v = (torch.randn((B, S, D), device=device) for _ in range(3))
+    lay = torch.ones((B, S // sbs, D // sbs), dtype=torch.bool, device=device)
+    la = torch.ones((B, S // sbs, S // sbs), dtype=torch.bool, device=device)
+    out = bs.ops.flash_attention(bs.ops.to_sparse(q, lay, sbs), lay, bs.ops.to_sparse(k, lay, sbs), lay,
+                                 bs.ops.to_sparse(v, lay, sbs), lay, la, sbs)
+    expected = F.scaled_dot_product_attention(q.double().cpu(), k.double().cpu(), v.double().cpu())
+    assert_close(bs.ops.to_dense(out, lay, sbs), expected, 1e-5, "sdpa")
+
+
+@pytest.mark.parametrize("dtype,n_key_blocks", [(torch.bfloat16, 256), (torch.float16, 1024)])
+def test_uniform_attention_over_a_long_sequence_is_exact(device, dtype, n_key_blocks):
+    # reference: test_regressions.py:63-94 - q = k = 0, v = 1 must give exactly 1
+    sbs = 64
+    lq = torch.ones((1, 1, 1), dtype=torch.bool, device=device)
+    lk = torch.ones((1, n_key_blocks, 1), dtype=torch.bool, device=device)
+    la = torch.ones((1, 1, n_key_blocks), dtype=torch.bool, device=device)
+    q = torch.zeros((1, sbs, sbs), device=device, dtype=dtype)
+    k = torch.zeros((n_key_blocks, sbs, sbs), device=device, dtype=dtype)
+    v = torch.ones((n_key_blocks, sbs, sbs), device=device, dtype=dtype)
+    out = bs.ops.flash_attention(q, lq, k, lk, v, lk, la, sbs)
+    assert torch.all(out == 1)
+
+
+def test_uniform_gradient_over_many_queries_is_exact(device):
+    # reference: test_regressions.py:97-129 - dV = n_queries / n_keys exactly
+    sbs, nq = 64, 256
+    lq = torch.ones((1, nq, 1), dtype=torch.bool, device=device)
+    lk = torch.ones((1, 1, 1), dtype=torch.bool, device=device)
+    la = torch.ones((1, nq, 1), dtype=torch.bool, device=device)
+    q = torch.zeros((nq, sbs, sbs), device=device, dtype=torch.bfloat16)
+    k = torch.zeros((1, sbs, sbs), device=device, dtype=torch.bfloat16)
+    v = torch.ones((1, sbs, sbs), device=device, dtype=torch.bfloat16, requires_grad=True)
+    bs.ops.flash_attention(q, lq, k, lk, v, lk, la, sbs).sum().backward()
+    assert torch.all(v.grad == nq)
+
+
+def test_mask_beats_infinite_bias_and_fully_masked_rows_are_zero(device):
+    # reference: test_regressions.py:2075-2120
+    sbs = 16
+    lay = torch.ones((1, 1, 1), dtype=torch.bool, device=device)
+    q, k, v = (torch.randn((1, sbs, sbs), device=device, requires_grad=True) for _ in range(3))
+    bias = torch.zeros((1, sbs, sbs), device=device)
+    bias[0, :, 0] = float("inf")
+    bias.requires_grad_(True)
+    mask = torch.zeros((1, sbs, sbs), dtype=torch.bool, device=device)
+    mask[0, :, 0] = True
+    mask[0, 5, :] = True
+    out = bs.ops.flash_attention(q, lay, k, lay, v, lay, lay, sbs, attention_mask=mask, sparsity_layout_mask=lay,
+                                 attention_bias=bias, sparsity_layout_bias=lay)
+    assert torch.isfinite(out).all() and torch.all(out[0, 5] == 0)
+    out.sum().backward()
+    for t in (q, k, v, bias):
+        assert torch.isfinite(t.grad).all()
+    assert torch.all(bias.grad[0, :, 0] == 0) and torch.all(bias.grad[0, 5] == 0)
+
+
+def test_zero_width_qk_head_dimension(device):
+    # reference: test_regressions.py:1256-1283 - no q/k blocks: scores are zero, scale defaults to 1
+    sbs = 16
+    lq = torch.ones((1, 2, 0), dtype=torch.bool, device=device)
+    lv = torch.ones((1, 2, 1), dtype=torch.bool, device=device)
+    la = torch.ones((1, 2, 2), dtype=torch.bool, device=device)
+    e = torch.empty((0, sbs, sbs), device=device)
+    v = torch.randn((2, sbs, sbs), device=device)
+    out = bs.ops.flash_attention(e, lq, e, lq, v, lv, la, sbs)
+    mean = v.reshape(2 * sbs, sbs).mean(dim=0)
+    assert torch.isfinite(out).all()
+    assert_close(out, mean.expand(2, sbs, sbs), 1e-5, "zero head dim")
+    same = bs.ops.flash_attention(e, lq, e, lq, v, lv, la, sbs, scale=1.0)
+    assert torch.equal(out, same)
+
+
+def test_default_output_layout_and_cache_reuse(device):
+    # reference: test_regressions.py:450-532
+    sbs, B = 16, 1
+    la = torch.tensor([[[1, 0], [0, 0]]], dtype=torch.bool, device=device)
+    lay = torch.ones((B, 2, 1), dtype=torch.bool, device=device)
+    q, k, v = (torch.randn((2, sbs, sbs), device=device) for _ in range(3))
+    cache = bs.ops.flash_attention_build_layout_cache(la, lay, lay, lay)
+    assert torch.equal(cache["sparsity_layout_o"].cpu(), torch.tensor([[[True], [False]]]))
+    assert cache["key_indices"].dtype == torch.int32 and cache["query_offsets"].dtype == torch.int32
+    assert cache["max_keys_per_query"] == 1 and cache["n_sparse_blocks_o"] == 1 and cache["n_sparse_blocks_q"] == 2
+    kept = cache["key_indices"]
+    out = bs.ops.flash_attention(q, lay, k, lay, v, lay, la, sbs, layout_cache=cache)
+    assert cache["key_indices"] is kept and out.shape == (1, sbs, sbs)
+    # positional order of the builder's arguments (reference: test_regressions.py:477-485)
+    again = bs.ops.flash_attention_build_layout_cache(la, lay, lay, lay, 2, 2, 1, None, 1, cache)
+    assert again is cache
+
+
+def test_validation_errors(device):
+    sbs = 16
+    lay = torch.ones((1, 1, 1), dtype=torch.bool, device=device)
+    t = torch.randn((1, sbs, sbs), device=device)
+    with pytest.raises(ValueError, match="provided together"):
+        bs.ops.flash_attention(t, lay, t, lay, t, lay, lay, sbs, attention_mask=t)
+    with pytest.raises(ValueError, match="provided together"):
+        bs.ops.flash_attention(t, lay, t, lay, t, lay, lay, sbs, sparsity_layout_bias=lay)
+    with pytest.raises(TypeError, match="real number or None"):
+        bs.ops.flash_attention(t, lay, t, lay, t, lay, lay, sbs, scale="1")
+    with pytest.raises(ValueError, match="0 or 1"):
+        bs.ops.flash_attention(t, lay, t, lay, t, lay, lay, sbs, attention_mask=t * 3, sparsity_layout_mask=lay)
+    big = torch.randn((1, 128, 128), device=device)
+    with pytest.raises(ValueError, match="at most 64"):
+        bs.ops.flash_attention(big, lay, big, lay, big, lay, lay, 128)
+    with pytest.raises(ValueError, match="K sparsity layout must be compatible"):
+        bs.ops.flash_attention(t, lay, torch.randn((2, sbs, sbs), device=device),
+                               torch.ones((1, 1, 2), dtype=torch.bool, device=device), t, lay, lay, sbs)
+    with pytest.raises(TypeError, match="integral dtype"):
+        bs.ops.flash_attention(t, lay, t, lay, t, lay, lay, sbs, causal_lengths=torch.ones(1, device=device))
+    with pytest.raises(ValueError, match="between zero and 16"):
+        bs.ops.flash_attention(t, lay, t, lay, t, lay, lay, sbs,
+                               causal_lengths=torch.tensor([17], device=device))
+    import numpy as np
+    out = bs.ops.flash_attention(t, lay, t, lay, t, lay, lay, sbs, scale=np.float32(0.5))
+    assert out.shape == (1, sbs, sbs)

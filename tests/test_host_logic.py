@@ -1,0 +1,170 @@
+"""Host-side behaviour that needs no GPU: validation switches and messages, the layout cache rules, the
+shape helpers, and that the operators refuse CPU tensors instead of computing somewhere else."""
+
+import threading
+
+import pytest
+import torch
+
+import blksprs_amd as bs
+from blksprs_amd.utils import tools, validation
+
+
+def test_public_surface():
+    for name in ("matmul", "flash_attention", "flash_attention_build_layout_cache", "softmax", "softmax_fused",
+                 "to_sparse", "to_dense", "to_blksprs", "from_blksprs", "to_sparse_shaped", "to_dense_shaped"):
+        assert callable(getattr(bs.ops, name))
+    assert callable(bs.layouting.build_sparsity_layout_matmul)
+    for name in ("disable_validation", "enable_validation", "disable_contiguous", "enable_contiguous",
+                 "do_shape_blocksparse", "undo_shape_blocksparse"):
+        assert callable(getattr(bs.utils, name))
+
+
+def test_blksprs_tensor_wrap():
+    t = torch.zeros((1, 16, 16))
+    w = bs.BlksprsTensor.wrap(t)
+    assert isinstance(w, bs.BlksprsTensor) and w.data_ptr() == t.data_ptr()
+    assert repr(w).startswith("BlksprsTensor(tensor(")
+    assert type(tools.as_base_tensor(w)) is torch.Tensor
+
+
+def test_operators_refuse_cpu_tensors():
+    lay = torch.ones((1, 1, 1), dtype=torch.bool)
+    x = torch.zeros((1, 16, 16))
+    with pytest.raises(ValueError, match="Tensors must be on GPU"):
+        bs.ops.matmul(x, lay, x, lay, lay, 16)
+    with pytest.raises(ValueError, match="Tensors must be on GPU"):
+        bs.ops.softmax(x, lay, 16)
+    with pytest.raises(ValueError, match="Tensors must be on GPU"):
+        bs.ops.to_dense(x, lay, 16)
+    with pytest.raises(ValueError, match="Tensors must be on GPU"):
+        bs.ops.flash_attention(x, lay, x, lay, x, lay, lay, 16)
+    # with validation off there is still no CPU path: the LUT builder itself refuses
+    bs.utils.disable_validation()
+    try:
+        with pytest.raises(RuntimeError, match="needs GPU tensors"):
+            bs.ops.to_dense(x, torch.ones((1, 2, 1), dtype=torch.bool), 16)
+    finally:
+        bs.utils.enable_validation()
+
+
+def test_validation_messages():
+    v = validation
+    with pytest.raises(ValueError, match="Tensor must have 3 dimensions"):
+        v.validate_dimensions(torch.zeros(2, 2))
+    with pytest.raises(ValueError, match="Tensor must be contiguous"):
+        v.validate_contiguous(torch.zeros(4, 4).t())
+    with pytest.raises(ValueError, match="either float16, bfloat16, or float32"):
+        v.validate_dtype_float(torch.zeros(1, dtype=torch.float64))
+    with pytest.raises(ValueError, match="same dtype"):
+        v.validate_dtype_float(torch.zeros(1), torch.zeros(1, dtype=torch.float16))
+    with pytest.raises(ValueError, match="float32 dtype"):
+        v.validate_dtype_float_32(torch.zeros(1, dtype=torch.float16))
+    with pytest.raises(ValueError, match="0 or 1"):
+        v.validate_binary(torch.tensor([0.0, 2.0]))
+    with pytest.raises(TypeError, match="must be an integer"):
+        v.validate_sparsity_block_size(True)
+    with pytest.raises(TypeError, match="must be an integer"):
+        v.validate_sparsity_block_size(16.0)
+    with pytest.raises(ValueError, match="at least 16"):
+        v.validate_sparsity_block_size(8)
+    with pytest.raises(ValueError, match="power of 2"):
+        v.validate_sparsity_block_size(48)
+    with pytest.raises(ValueError, match="divisible by sparsity block size"):
+        v.validate_sparsity_block_size(32, torch.zeros(1, 48, 32))
+    with pytest.raises(ValueError, match=r"Output sparsity layout shape \(1, 2\) doesn't match expected \(2, 1\)"):
+        v.validate_shape(torch.zeros(1, 2), (2, 1), "Output sparsity layout")
+    with pytest.raises(ValueError, match="complex dtype"):
+        v.validate_sparsity(16, (torch.zeros(1, 16, 16), torch.ones((1, 1, 1), dtype=torch.complex64)))
+    with pytest.raises(ValueError, match="Blocks not conforming"):
+        v.validate_sparsity(16, (torch.zeros(1, 16, 32), torch.ones((1, 1, 1))))
+    with pytest.raises(ValueError, match="Mismatch between sparsity layout and blocks"):
+        v.validate_sparsity(16, (torch.zeros(2, 16, 16), torch.ones((1, 1, 1))))
+    with pytest.raises(ValueError, match="exactly 3 dimensions"):
+        v.validate_sparsity(16, (torch.zeros(1, 16, 16), torch.ones((1, 1))))
+    with pytest.raises(TypeError, match="must be an integer"):
+        v.validate_positive_integer(1.5, "Repeats")
+    with pytest.raises(ValueError, match="positive integer"):
+        v.validate_positive_integer(0, "Repeats")
+
+
+def test_switches_are_per_thread():
+    bs.utils.disable_validation()
+    bs.utils.disable_contiguous()
+    seen = {}
+
+    def worker():
+        seen["validation"] = validation._validation_enabled()
+        seen["contiguous"] = validation._contiguous_enabled()
+
+    t = threading.Thread(target=worker)
+    t.start()
+    t.join()
+    try:
+        assert seen == {"validation": True, "contiguous": True}
+        assert not validation._validation_enabled()
+        validation.validate_dimensions(torch.zeros(2))  # no-op while disabled
+        nc = torch.zeros(4, 4).t()
+        assert validation.ensure_contiguous(nc) is nc
+    finally:
+        bs.utils.enable_validation()
+        bs.utils.enable_contiguous()
+    assert validation.ensure_contiguous(torch.zeros(4, 4).t()).is_contiguous()
+
+
+def test_layout_cache_rules():
+    lay = torch.ones((1, 2, 2), dtype=torch.bool)
+    cache = tools.prepare_layout_cache(None, "op", lay, 3)
+    cache["table"] = torch.arange(4)
+    cache["count"] = 4
+    tools.finalize_layout_cache(cache)
+    assert tools.prepare_layout_cache(cache, "op", lay, 3).get("count") == 4      # hit
+    assert "count" not in tools.prepare_layout_cache(cache, "other", lay, 3)       # other operation
+    cache["count"] = 4
+    tools.finalize_layout_cache(cache)
+    assert "count" not in tools.prepare_layout_cache(cache, "other", lay, 4)       # other scalar
+    cache["count"] = 4
+    tools.finalize_layout_cache(cache)
+    lay[0, 0, 0] = False                                                            # source mutated in place
+    assert "count" not in tools.prepare_layout_cache(cache, "other", lay, 4)
+    cache["table"] = torch.arange(4)
+    tools.finalize_layout_cache(cache)
+    cache["table"].add_(1)                                                          # derived entry mutated
+    assert "table" not in tools.prepare_layout_cache(cache, "other", lay, 4)
+    cache["x"] = 1                                                                  # never finalized
+    assert "x" not in tools.prepare_layout_cache(cache, "other", lay, 4)
+    # sources are retained so their ids cannot be recycled
+    assert cache["_blksprs_cache_refs"][0] is lay
+    with torch.inference_mode():
+        inf = torch.ones((1, 1, 1))
+    c2 = tools.prepare_layout_cache(None, "op", inf)
+    c2["v"] = 1
+    tools.finalize_layout_cache(c2)
+    assert "v" not in tools.prepare_layout_cache(c2, "op", inf)                     # inference tensors never hit
+
+
+def test_shape_helpers():
+    x = torch.zeros((2, 3, 4, 5))
+    flat, shape = tools.do_shape_blocksparse(x)
+    assert flat.shape == (6, 4, 5) and shape == x.shape
+    assert tools.undo_shape_blocksparse(flat, shape).shape == x.shape
+    assert tools.undo_shape_blocksparse(torch.zeros((6, 4, 7)), shape).shape == (2, 3, 4, 7)
+    with pytest.raises(ValueError, match="at least 2 dimensions"):
+        tools.do_shape_blocksparse(torch.zeros(3))
+    with pytest.raises(ValueError, match="batch dimension does not match"):
+        tools.undo_shape_blocksparse(torch.zeros((5, 4, 5)), shape)
+    assert tools.ceil_pow2(1) == 1 and tools.ceil_pow2(5) == 8 and tools.ceil_pow2(8) == 8
+    with pytest.raises(ValueError):
+        tools.ceil_pow2(0)
+    assert tools.can_use_int32_indexing(torch.zeros(4), None, 2_147_483_647)
+    assert not tools.can_use_int32_indexing(2_147_483_648)
+
+
+def test_unknown_autotune_mode_is_rejected():
+    import os
+    import subprocess
+    import sys
+    env = dict(os.environ, BLKSPRS_AUTOTUNE="FAST")
+    proc = subprocess.run([sys.executable, "-c", "import blksprs_amd"], env=env, capture_output=True, text=True,
+                          cwd=str(__import__("pathlib").Path(__file__).resolve().parent.parent))
+    assert proc.returncode != 0 and "Unknown autotune mode" in proc.stderr

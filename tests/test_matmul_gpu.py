@@ -1,0 +1,165 @@
+"""Parity of the block-sparse matmul with the CPU oracle: rtol = atol = 1e-5 for fp32, 2e-2 for fp16 / bf16
+against an fp32-accumulated dense-masked product of the rounded inputs."""
+
+import math
+
+import pytest
+import torch
+
+import blksprs_amd as bs
+from oracle import blksprs_oracle as orc
+from tests.helpers import assert_close, rand_blocks, rand_layout
+
+pytestmark = pytest.mark.gpu
+TOL = {torch.float32: 1e-5, torch.float16: 2e-2, torch.bfloat16: 2e-2}
+
+
+def _problem(B, R, K, C, sbs, dtype, density, seed, product_layout=True):
+    lx = rand_layout((B, R, K), density, seed=seed, ensure_rows=True)
+    ly = rand_layout((B, K, C), density, seed=seed + 1, ensure_rows=True)
+    if product_layout:
+        lo = torch.from_numpy(orc.layout_matmul(lx.numpy(), ly.numpy()))
+    else:
+        lo = rand_layout((B, R, C), 0.6, seed=seed + 2)
+    scale = 1.0 / math.sqrt(K * sbs)
+    x = rand_blocks(int(lx.sum()), sbs, dtype, seed + 3, scale)
+    y = rand_blocks(int(ly.sum()), sbs, dtype, seed + 4)
+    return lx, ly, lo, x, y
+
+
+def _oracle(x, lx, y, ly, lo, sbs):
+    # fp64 accumulation of the (already rounded) inputs is the tightest statement of "fp32-accumulated"
+    return orc.matmul(x.double(), lx.numpy(), y.double(), ly.numpy(), lo.numpy(), sbs, acc_dtype=torch.float64)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("sbs,dims,density", [
+    (32, (2, 8, 8, 8), 0.5),      # config 1: B=2, 256^3, sbs 32, p = 0.5
+    (16, (3, 5, 9, 6), 0.4),
+    (16, (2, 16, 16, 16), 0.1),
+    (32, (2, 3, 7, 5), 0.6),
+    (64, (2, 4, 6, 5), 0.5),
+    (64, (1, 3, 20, 3), 0.9),
+    (128, (1, 2, 3, 2), 0.7),
+    (256, (1, 1, 2, 1), 1.0),
+])
+def test_forward_matches_oracle(device, dtype, sbs, dims, density):
+    B, R, K, C = dims
+    for product_layout in (True, False):
+        lx, ly, lo, x, y = _problem(B, R, K, C, sbs, dtype, density, seed=sbs + K, product_layout=product_layout)
+        out = bs.ops.matmul(x.to(device), lx.to(device), y.to(device), ly.to(device), lo.to(device), sbs)
+        assert isinstance(out, bs.BlksprsTensor) and out.dtype == dtype
+        assert out.shape == (int(lo.sum()), sbs, sbs)
+        assert_close(out, _oracle(x, lx, y, ly, lo, sbs), TOL[dtype], f"matmul {dtype} sbs={sbs} product={product_layout}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("sbs", [16, 32, 64, 128])
+def test_backward_matches_autograd_of_the_oracle(device, dtype, sbs):
+    B, R, K, C = 2, 3, 4, 5
+    lx, ly, lo, x, y = _problem(B, R, K, C, sbs, dtype, 0.6, seed=sbs)
+    xg = x.to(device).requires_grad_(True)
+    yg = y.to(device).requires_grad_(True)
+    cache = {}
+    out = bs.ops.matmul(xg, lx.to(device), yg, ly.to(device), lo.to(device), sbs, layout_cache=cache)
+    go = rand_blocks(out.size(0), sbs, dtype, seed=9)
+    out.backward(go.to(device))
+    x64 = x.double().requires_grad_(True)
+    y64 = y.double().requires_grad_(True)
+    xd = orc.to_dense_autograd(x64, lx.numpy(), sbs)
+    yd = orc.to_dense_autograd(y64, ly.numpy(), sbs)
+    ref = orc.to_sparse_autograd(xd @ yd, lo.numpy(), sbs)
+    ref.backward(go.double())
+    tol = TOL[dtype] if dtype == torch.float32 else 4e-2
+    assert_close(xg.grad, x64.grad, tol, f"dX {dtype} sbs={sbs}")
+    assert_close(yg.grad, y64.grad, tol, f"dY {dtype} sbs={sbs}")
+    # a second step reuses the forward and backward lists
+    offsets = cache["grad_x_pair_offsets"]
+    xg.grad = None
+    bs.ops.matmul(xg, lx.to(device), yg, ly.to(device), lo.to(device), sbs, layout_cache=cache).backward(go.to(device))
+    assert cache["grad_x_pair_offsets"] is offsets
+    assert_close(xg.grad, x64.grad, tol, "dX second step")
+
+
+def test_config1_fp32_unscaled_normal_values(device):
+    """Config 1 as stated: fp32, B=2, M=K=N=256, sbs 32, Bernoulli(0.5) layouts with one block per row
+    guaranteed, product output layout, N(0,1) values; rtol = atol = 1e-5 against the fp32-accumulated
+    dense-masked product (diagnosed against fp64 as well, at 2e-5)."""
+    sbs, B, n = 32, 2, 8
+    lx = rand_layout((B, n, n), 0.5, seed=0, ensure_rows=True)
+    ly = rand_layout((B, n, n), 0.5, seed=1, ensure_rows=True)
+    lo = torch.from_numpy(orc.layout_matmul(lx.numpy(), ly.numpy()))
+    x = rand_blocks(int(lx.sum()), sbs, torch.float32, 2)
+    y = rand_blocks(int(ly.sum()), sbs, torch.float32, 3)
+    out = bs.ops.matmul(x.to(device), lx.to(device), y.to(device), ly.to(device), lo.to(device), sbs)
+    fp32 = orc.matmul(x, lx.numpy(), y, ly.numpy(), lo.numpy(), sbs, acc_dtype=torch.float32)
+    assert_close(out, fp32, 1e-5, "config 1 vs fp32-accumulated oracle")
+    assert_close(out, _oracle(x, lx, y, ly, lo, sbs), 2e-5, "config 1 vs fp64 oracle")
+
+
+def test_output_blocks_without_contributions_are_zero(device):
+    sbs = 64
+    lx = torch.zeros((1, 2, 2), dtype=torch.bool)
+    lx[0, 0, 0] = True
+    ly = torch.zeros((1, 2, 2), dtype=torch.bool)
+    ly[0, 1, 1] = True
+    lo = torch.ones((1, 2, 2), dtype=torch.bool)
+    x = torch.randn((1, sbs, sbs), device=device, dtype=torch.bfloat16)
+    y = torch.randn((1, sbs, sbs), device=device, dtype=torch.bfloat16)
+    out = bs.ops.matmul(x, lx.to(device), y, ly.to(device), lo.to(device), sbs)
+    assert out.shape == (4, sbs, sbs) and torch.all(out == 0)
+
+
+def test_full_size_config2_linearity_and_sampled_parity(device):
+    """Config 2 (bf16, B=16, 4096^3, sbs 64, 25 % density, product layout) at full size: sampled output
+    blocks against the oracle, and exactness properties that need no oracle (x -> 2x doubles the result
+    bit for bit; zeroing y zeroes the output)."""
+    B, n, sbs = 16, 64, 64
+    lx = rand_layout((B, n, n), 0.25, seed=0)
+    ly = rand_layout((B, n, n), 0.25, seed=1)
+    lo = torch.from_numpy(orc.layout_matmul(lx.numpy(), ly.numpy()))
+    g = torch.Generator().manual_seed(2)
+    x = (torch.randn((int(lx.sum()), sbs, sbs), generator=g) / 64.0).to(torch.bfloat16)
+    y = torch.randn((int(ly.sum()), sbs, sbs), generator=g).to(torch.bfloat16)
+    xd, yd = x.to(device), y.to(device)
+    cache = {}
+    out = bs.ops.matmul(xd, lx.to(device), yd, ly.to(device), lo.to(device), sbs, layout_cache=cache)
+    assert out.shape[0] == int(lo.sum())
+    doubled = bs.ops.matmul(xd * 2, lx.to(device), yd, ly.to(device), lo.to(device), sbs, layout_cache=cache)
+    assert torch.equal(doubled, out * 2)
+    zero = bs.ops.matmul(xd, lx.to(device), torch.zeros_like(yd), ly.to(device), lo.to(device), sbs, layout_cache=cache)
+    assert torch.all(zero == 0)
+    # batch 3 against the oracle (one batch keeps the dense CPU product small)
+    b = 3
+    sl = lambda lay, t: t[int(lay[:b].sum()):int(lay[:b + 1].sum())]
+    exp = _oracle(sl(lx, x), lx[b:b + 1], sl(ly, y), ly[b:b + 1], lo[b:b + 1], sbs)
+    assert_close(sl(lo, out), exp, 2e-2, "config 2, batch 3")
+
+
+def test_autocast_and_validation(device):
+    sbs = 16
+    layout = torch.ones((1, 2, 2), dtype=torch.bool, device=device)
+    x = torch.randn((4, sbs, sbs), device=device)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        out = bs.ops.matmul(x, layout, x, layout, layout, sbs)
+    assert out.dtype == torch.bfloat16
+    # fp64 is not silently downcast (reference: test_regressions.py:694-722)
+    with torch.autocast("cuda", dtype=torch.float16):
+        with pytest.raises(ValueError, match="float16, bfloat16, or float32"):
+            bs.ops.matmul(x.double(), layout, x.double(), layout, layout, sbs)
+    with pytest.raises(ValueError, match="same dtype"):
+        bs.ops.matmul(x, layout, x.half(), layout, layout, sbs)
+    with pytest.raises(ValueError, match="Inner dimensions"):
+        bs.ops.matmul(x, layout, torch.randn((6, sbs, sbs), device=device),
+                      torch.ones((1, 3, 2), dtype=torch.bool, device=device), layout, sbs)
+    with pytest.raises(ValueError, match="Batch dimensions"):
+        bs.ops.matmul(x, layout, torch.randn((8, sbs, sbs), device=device),
+                      torch.ones((2, 2, 2), dtype=torch.bool, device=device), layout, sbs)
+    with pytest.raises(ValueError, match="Output sparsity layout shape"):
+        bs.ops.matmul(x, layout, x, layout, torch.ones((1, 2, 3), dtype=torch.bool, device=device), sbs)
+    bs.utils.disable_validation()
+    try:
+        out = bs.ops.matmul(x, layout, x, layout, layout, sbs)  # no checks, same result path
+        assert out.shape == (4, sbs, sbs)
+    finally:
+        bs.utils.enable_validation()

@@ -1,0 +1,274 @@
+"""Pins the CPU oracle: every oracle function is checked here against something that is not the
+oracle's own formula - brute-force loops on tiny inputs, closed forms, torch library routines, and the
+known answers the reference's own tests hold (test/cases/test_regressions.py, test_blocksparse.py).
+"""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import blksprs_oracle as orc
+
+
+def _layouts():
+    g = torch.Generator().manual_seed(7)
+    yield torch.zeros((1, 1, 1), dtype=torch.bool)
+    yield torch.ones((1, 1, 1), dtype=torch.bool)
+    yield torch.zeros((2, 3, 4), dtype=torch.bool)
+    yield torch.ones((2, 3, 4), dtype=torch.bool)
+    for shape, p in (((1, 4, 4), 0.5), ((3, 5, 7), 0.3), ((2, 8, 8), 0.8), ((4, 1, 9), 0.5)):
+        yield torch.rand(shape, generator=g) < p
+
+
+@pytest.mark.parametrize("layout", list(_layouts()))
+def test_packed_indices_bruteforce(layout):
+    flat = layout.reshape(-1).tolist()
+    expected, seen = [], 0
+    for v in flat:
+        expected.append(seen if v else -1)
+        seen += int(v)
+    got = orc.packed_indices(layout.numpy())
+    assert got.dtype == np.int64 and got.tolist() == expected
+
+
+@pytest.mark.parametrize("layout", list(_layouts()))
+def test_layout_indices_is_torch_nonzero(layout):
+    assert np.array_equal(orc.layout_indices(layout.numpy()), torch.nonzero(layout).numpy())
+    assert orc.n_sparse_blocks(layout.numpy()) == int(layout.sum())
+
+
+def test_block_count_is_exact_for_half_precision_layouts():
+    # test_regressions.py:1060-1075: 65536 ones in an fp16 layout must count exactly
+    layout = torch.ones((1, 256, 256), dtype=torch.float16)
+    assert orc.n_sparse_blocks(layout.numpy()) == 65536
+
+
+@pytest.mark.parametrize("layout", list(_layouts()))
+def test_segmented_indices_bruteforce(layout):
+    B, R, C = layout.shape
+    indices, offsets, longest = orc.segmented_indices(layout.numpy())
+    exp_idx, exp_off, exp_long = [], [0], 0
+    for b in range(B):
+        for r in range(R):
+            cols = [c for c in range(C) if layout[b, r, c]]
+            exp_idx += cols
+            exp_off.append(len(exp_idx))
+            exp_long = max(exp_long, len(cols))
+    if exp_long == 0:
+        # flash_attention.py:1928-1938: (empty, zeros, 1)
+        assert indices.size == 0 and offsets.tolist() == [0] * (B * R + 1) and longest == 1
+    else:
+        assert indices.tolist() == exp_idx and offsets.tolist() == exp_off and longest == exp_long
+    assert indices.dtype == np.int32 and offsets.dtype == np.int32
+
+
+def test_segmented_index_dtype_truth_table():
+    # test_regressions.py:1037-1047
+    assert orc.segmented_index_dtype(0, 1) == np.int32
+    assert orc.segmented_index_dtype(2_147_483_647, 2_147_483_648) == np.int32
+    assert orc.segmented_index_dtype(2_147_483_648, 1) == np.int64
+    assert orc.segmented_index_dtype(1, 2_147_483_649) == np.int64
+
+
+@pytest.mark.parametrize("layout", list(_layouts()))
+def test_sorted_packed_indices_against_torch_sort(layout):
+    packed = torch.from_numpy(orc.packed_indices(layout.numpy())).reshape(layout.shape)
+    expected = packed.sort(descending=True, dim=-1)[0].reshape(-1)
+    got, mbl = orc.sorted_packed_indices(layout.numpy())
+    assert np.array_equal(got, expected.numpy())
+    longest = int(layout.sum(dim=-1).max()) if layout.numel() else 0
+    assert mbl == max(2, 1 << max(longest - 1, 0).bit_length()) and mbl >= longest and (mbl & (mbl - 1)) == 0
+
+
+def test_layout_matmul_bruteforce_and_float_bmm():
+    g = torch.Generator().manual_seed(3)
+    lx = torch.rand((3, 5, 6), generator=g) < 0.3
+    ly = torch.rand((3, 6, 4), generator=g) < 0.3
+    got = orc.layout_matmul(lx.numpy(), ly.numpy())
+    brute = np.zeros((3, 5, 4), dtype=bool)
+    for b in range(3):
+        for i in range(5):
+            for j in range(4):
+                brute[b, i, j] = any(lx[b, i, k] and ly[b, k, j] for k in range(6))
+    assert np.array_equal(got, brute)
+    assert np.array_equal(got, torch.matmul(lx.float(), ly.float()).bool().numpy())
+    # empty inner dimension: nothing is active (test_regressions.py:1208-1217)
+    assert not orc.layout_matmul(np.ones((1, 2, 0)), np.ones((1, 0, 3))).any()
+
+
+def test_contraction_lists_reproduce_the_dense_product():
+    """The lists are a regrouping of a block matmul: summing x[px] @ y[py] per output block must equal the
+    dense masked product; and within a block k ascends."""
+    g = torch.Generator().manual_seed(11)
+    sbs = 4
+    lx = torch.rand((2, 3, 5), generator=g) < 0.5
+    ly = torch.rand((2, 5, 4), generator=g) < 0.5
+    lo = torch.rand((2, 3, 4), generator=g) < 0.7  # includes blocks with no contributing k
+    x = torch.randn((int(lx.sum()), sbs, sbs), generator=g, dtype=torch.float64)
+    y = torch.randn((int(ly.sum()), sbs, sbs), generator=g, dtype=torch.float64)
+    offsets, pairs = orc.contraction_lists(lx.numpy(), ly.numpy(), lo.numpy())
+    n_o = int(lo.sum())
+    assert offsets.shape == (n_o + 1,) and offsets[0] == 0 and offsets[-1] == len(pairs)
+    out = torch.zeros((n_o, sbs, sbs), dtype=torch.float64)
+    for n in range(n_o):
+        seg = pairs[offsets[n]:offsets[n + 1]]
+        assert np.all(np.diff(seg[:, 0]) > 0)  # x blocks of one row are stored in ascending k
+        for px, py in seg:
+            out[n] += x[px] @ y[py]
+    dense = orc.to_dense(x, lx.numpy(), sbs) @ orc.to_dense(y, ly.numpy(), sbs)
+    assert torch.allclose(out, orc.to_sparse(dense, lo.numpy(), sbs), atol=1e-12)
+    total = int(np.einsum("bik,bkj,bij->", lx.numpy().astype(int), ly.numpy().astype(int), lo.numpy().astype(int)))
+    assert len(pairs) == total
+
+
+def test_conversion_against_slice_loops():
+    # the loop form of test_blocksparse.py:1674-1699
+    g = torch.Generator().manual_seed(5)
+    sbs = 4
+    layout = torch.rand((2, 3, 5), generator=g) < 0.5
+    x = torch.randn((2, 3 * sbs, 5 * sbs), generator=g)
+    blocks = orc.to_sparse(x, layout.numpy(), sbs)
+    dense = orc.to_dense(blocks, layout.numpy(), sbs, fill_value=7.5)
+    n = 0
+    for b in range(2):
+        for r in range(3):
+            for c in range(5):
+                tile = x[b, r * sbs:(r + 1) * sbs, c * sbs:(c + 1) * sbs]
+                got = dense[b, r * sbs:(r + 1) * sbs, c * sbs:(c + 1) * sbs]
+                if layout[b, r, c]:
+                    assert torch.equal(blocks[n], tile) and torch.equal(got, tile)
+                    n += 1
+                else:
+                    assert torch.all(got == 7.5)
+    assert n == blocks.size(0)
+
+
+def test_matmul_full_layout_is_bmm_and_inactive_blocks_do_not_contribute():
+    g = torch.Generator().manual_seed(2)
+    sbs = 4
+    full = np.ones((2, 2, 2), dtype=bool)
+    a = torch.randn((2, 8, 8), generator=g, dtype=torch.float64)
+    b = torch.randn((2, 8, 8), generator=g, dtype=torch.float64)
+    out = orc.matmul(orc.to_sparse(a, full, sbs), full, orc.to_sparse(b, full, sbs), full, full, sbs,
+                     acc_dtype=torch.float64)
+    assert torch.allclose(orc.to_dense(out, full, sbs), torch.bmm(a, b), atol=1e-12)
+    # x with only block (0,0): output row 0 equals a00 @ b0*, row 1 is zero
+    lx = np.zeros((1, 2, 2), dtype=bool)
+    lx[0, 0, 0] = True
+    one = np.ones((1, 2, 2), dtype=bool)
+    out = orc.matmul(a[:1, :4, :4].clone(), lx, orc.to_sparse(b[:1], one, sbs), one, one, sbs,
+                     acc_dtype=torch.float64)
+    dense = orc.to_dense(out, one, sbs)
+    assert torch.allclose(dense[0, :4], a[0, :4, :4] @ b[0, :4, :], atol=1e-12)
+    assert torch.all(dense[0, 4:] == 0)
+
+
+def test_softmax_matches_per_row_softmax_over_concatenated_blocks():
+    g = torch.Generator().manual_seed(9)
+    sbs = 4
+    layout = torch.rand((2, 3, 4), generator=g) < 0.5
+    layout[0, 1] = False  # a row without blocks
+    x = torch.randn((int(layout.sum()), sbs, sbs), generator=g)
+    out = orc.softmax(x, layout.numpy(), sbs)
+    lidx = torch.nonzero(layout)
+    for b in range(2):
+        for r in range(3):
+            ids = [n for n, (bb, rr, _) in enumerate(lidx.tolist()) if bb == b and rr == r]
+            if not ids:
+                continue
+            for e in range(sbs):
+                row = torch.cat([x[n, e] for n in ids]).double()
+                expected = torch.softmax(row, dim=0)
+                got = torch.cat([out[n, e] for n in ids]).double()
+                assert torch.allclose(got, expected, atol=1e-6)
+    # backward formula against autograd
+    y = out.double().requires_grad_(False)
+    grad = torch.randn(x.shape, generator=g).double()
+    xd = orc.to_dense(x.double(), layout.numpy(), sbs, fill_value=float("-inf")).requires_grad_(True)
+    sm = torch.softmax(xd, dim=-1)
+    sm = torch.nan_to_num(sm, nan=0.0)
+    (sm * orc.to_dense(grad, layout.numpy(), sbs)).sum().backward()
+    expected = orc.to_sparse(torch.nan_to_num(xd.grad, nan=0.0), layout.numpy(), sbs)
+    assert torch.allclose(orc.softmax_backward(grad, y, layout.numpy(), sbs), expected, atol=1e-9)
+
+
+def _full(b, r, c):
+    return np.ones((b, r, c), dtype=bool)
+
+
+def test_attention_full_layout_is_sdpa():
+    # test_regressions.py:488-527: full layout without mask equals scaled_dot_product_attention
+    g = torch.Generator().manual_seed(4)
+    sbs, B, S, D = 4, 2, 8, 8
+    q, k, v = (torch.randn((B, S, D), generator=g, dtype=torch.float64) for _ in range(3))
+    lq = _full(B, S // sbs, D // sbs)
+    la = _full(B, S // sbs, S // sbs)
+    out = orc.flash_attention(orc.to_sparse(q, lq, sbs), lq, orc.to_sparse(k, lq, sbs), lq,
+                              orc.to_sparse(v, lq, sbs), lq, la, sbs, acc_dtype=torch.float64)
+    assert torch.allclose(orc.to_dense(out, lq, sbs), F.scaled_dot_product_attention(q, k, v), atol=1e-12)
+    # causal lengths equal an explicit is_causal mask when the length covers the sequence
+    out = orc.flash_attention(orc.to_sparse(q, lq, sbs), lq, orc.to_sparse(k, lq, sbs), lq,
+                              orc.to_sparse(v, lq, sbs), lq, la, sbs, causal_lengths=torch.full((B,), S),
+                              acc_dtype=torch.float64)
+    assert torch.allclose(orc.to_dense(out, lq, sbs), F.scaled_dot_product_attention(q, k, v, is_causal=True),
+                          atol=1e-12)
+
+
+def test_attention_known_answers_from_reference_tests():
+    sbs = 4
+    # uniform attention (test_regressions.py:63-94): q = k = 0, v = 1 -> output exactly 1
+    lq = _full(1, 1, 1)
+    lk = _full(1, 8, 1)
+    la = _full(1, 1, 8)
+    out = orc.flash_attention(torch.zeros((1, sbs, sbs)), lq, torch.zeros((8, sbs, sbs)), lk,
+                              torch.ones((8, sbs, sbs)), lk, la, sbs)
+    assert torch.all(out == 1)
+    # uniform gradient (test_regressions.py:97-129): many queries, one key block -> dV = n_query / n_key
+    lq = _full(1, 5, 1)
+    lk = _full(1, 1, 1)
+    la = _full(1, 5, 1)
+    v = torch.ones((1, sbs, sbs), requires_grad=True)
+    out = orc.flash_attention(torch.zeros((5, sbs, sbs)), lq, torch.zeros((1, sbs, sbs)), lk, v, lk, la, sbs)
+    out.sum().backward()
+    assert torch.all(v.grad == (5 * sbs) / sbs)
+    # zero-width QK head dimension: scores are 0, scale defaults to 1 (test_regressions.py:1256-1283)
+    lq0 = np.ones((1, 2, 0), dtype=bool)
+    lv = _full(1, 2, 1)
+    la = _full(1, 2, 2)
+    vv = torch.randn((2, sbs, sbs))
+    out = orc.flash_attention(torch.zeros((0, sbs, sbs)), lq0, torch.zeros((0, sbs, sbs)), lq0, vv, lv, la, sbs)
+    mean = orc.to_dense(vv, lv, sbs).mean(dim=1, keepdim=True).expand(1, 2 * sbs, sbs)
+    assert torch.allclose(orc.to_dense(out, lv, sbs), mean, atol=1e-6)
+
+
+def test_attention_mask_bias_order_and_fully_masked_rows():
+    g = torch.Generator().manual_seed(8)
+    sbs, S = 4, 8
+    lq = _full(1, 2, 1)
+    la = _full(1, 2, 2)
+    q, k, v = (orc.to_sparse(torch.randn((1, S, sbs), generator=g), lq, sbs) for _ in range(3))
+    # +inf bias under a mask stays ignored (test_regressions.py:2075-2120)
+    bias = torch.zeros((1, S, S))
+    bias[0, :, 0] = float("inf")
+    mask = torch.zeros((1, S, S), dtype=torch.bool)
+    mask[0, :, 0] = True
+    mask[0, 3, :] = True  # one fully masked query row -> output 0, no NaN
+    out = orc.flash_attention(q, lq, k, lq, v, lq, la, sbs, mask=orc.to_sparse(mask, la, sbs), layout_mask=la,
+                              bias=orc.to_sparse(bias, la, sbs), layout_bias=la)
+    dense = orc.to_dense(out, lq, sbs)
+    assert torch.isfinite(dense).all() and torch.all(dense[0, 3] == 0)
+    # brute force for one unmasked row
+    qd, kd, vd = (orc.to_dense(t, lq, sbs)[0] for t in (q, k, v))
+    s = (qd[1] @ kd.T) / math.sqrt(sbs)
+    w = torch.softmax(s[1:], dim=0)
+    assert torch.allclose(dense[0, 1], w @ vd[1:], atol=1e-6)
+    # block layout: a query block that attends nothing yields zeros and the default output layout follows
+    # attention (x) v (test_regressions.py:488-532)
+    la2 = np.array([[[1, 0], [0, 0]]], dtype=bool)
+    out = orc.flash_attention(q, lq, k, lq, v, lq, la2, sbs)
+    assert out.shape[0] == 1
+    w = torch.softmax((qd[:4] @ kd[:4].T) / math.sqrt(sbs), dim=-1)
+    assert torch.allclose(out[0], w @ vd[:4], atol=1e-6)
