@@ -54,7 +54,7 @@ SIGNATURES = {
                              c_uint64, c_void_p]),
     "bsa_softmax_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p]),
     "bsa_softmax_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p]),
-    "bsa_matmul": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int,
+    "bsa_matmul": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int,
                            c_int, c_int, c_int, c_void_p]),
     "bsa_attn_fwd": (c_int, [ctypes.POINTER(AttnArgs), c_void_p]),
     "bsa_attn_bwd": (c_int, [ctypes.POINTER(AttnArgs), c_void_p]),

@@ -37,28 +37,25 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+// native vector (not HIP's uint4 struct): arrays of it are always promoted to registers
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 struct Bf16Traits {
   static constexpr int kElem = 2;
   using store_t = uint16_t;
-  __device__ static f32x16 mfma(uint4 a, uint4 b, f32x16 c) {
+  __device__ static f32x16 mfma(u32x4 a, u32x4 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
                                                    0, 0, 0);
   }
-  __device__ static uint16_t round(float v) {
-    // round to nearest even, NaN kept quiet
-    uint32_t u = __builtin_bit_cast(uint32_t, v);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (uint16_t)(u >> 16);
-  }
+  // round to nearest even, NaN kept quiet (the hardware conversion of gfx950)
+  __device__ static uint16_t round(float v) { return __builtin_bit_cast(uint16_t, (__bf16)v); }
   __device__ static float widen(uint16_t h) { return __builtin_bit_cast(float, (uint32_t)h << 16); }
 };
 
 struct F16Traits {
   static constexpr int kElem = 2;
   using store_t = uint16_t;
-  __device__ static f32x16 mfma(uint4 a, uint4 b, f32x16 c) {
+  __device__ static f32x16 mfma(u32x4 a, u32x4 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0,
                                                   0, 0);
   }
@@ -69,16 +66,14 @@ struct F16Traits {
 struct F32Traits {
   static constexpr int kElem = 4;
   using store_t = float;
+  // by-value helper: __builtin_bit_cast applied directly to a vector component reads component 0
+  __device__ static float as_float(uint32_t v) { return __builtin_bit_cast(float, v); }
   // one fragment = 4 floats = 4 rank-2 updates
-  __device__ static f32x16 mfma(uint4 a, uint4 b, f32x16 c) {
-    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__builtin_bit_cast(float, a.x), __builtin_bit_cast(float, b.x), c, 0, 0,
-                                             0);
-    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__builtin_bit_cast(float, a.y), __builtin_bit_cast(float, b.y), c, 0, 0,
-                                             0);
-    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__builtin_bit_cast(float, a.z), __builtin_bit_cast(float, b.z), c, 0, 0,
-                                             0);
-    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__builtin_bit_cast(float, a.w), __builtin_bit_cast(float, b.w), c, 0, 0,
-                                             0);
+  __device__ static f32x16 mfma(u32x4 a, u32x4 b, f32x16 c) {
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(as_float(a[0]), as_float(b[0]), c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(as_float(a[1]), as_float(b[1]), c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(as_float(a[2]), as_float(b[2]), c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(as_float(a[3]), as_float(b[3]), c, 0, 0, 0);
     return c;
   }
   __device__ static float round(float v) { return v; }
@@ -116,32 +111,32 @@ __device__ inline int swizzle(int row, int chunk) {
 
 // k contiguous: element (row, k) at base[row * ld + k]
 template <typename G>
-__device__ inline void load_kcont(uint4 (&r)[G::LOADS], const char *base, int64_t ld_bytes, int lane) {
+__device__ inline void load_kcont(u32x4 (&r)[G::LOADS], const char *base, uint32_t ld_bytes, int lane) {
 #pragma unroll
   for (int i = 0; i < G::KCONT_LOADS; ++i) {
     const int q = i * 64 + lane;
     const int row = q / G::CPR, c = q % G::CPR;
-    r[i] = *reinterpret_cast<const uint4 *>(base + row * ld_bytes + c * 16);
+    r[i] = *reinterpret_cast<const u32x4 *>(base + (uint32_t)(row * ld_bytes + c * 16));
   }
 }
 
 // k strided: element (row, k) at base[k * ld + row]
 template <typename G, int TILE>
-__device__ inline void load_kstr(uint4 (&r)[G::LOADS], const char *base, int64_t ld_bytes, int lane) {
+__device__ inline void load_kstr(u32x4 (&r)[G::LOADS], const char *base, uint32_t ld_bytes, int lane) {
   if constexpr (G::ES == 2) {
 #pragma unroll
     for (int i = 0; i < G::KSTR_LOADS / 2; ++i) {
       const int q = i * 64 + lane;
       const int ro = q % (TILE / 8), kp = q / (TILE / 8);
-      r[2 * i] = *reinterpret_cast<const uint4 *>(base + (2 * kp) * ld_bytes + ro * 16);
-      r[2 * i + 1] = *reinterpret_cast<const uint4 *>(base + (2 * kp + 1) * ld_bytes + ro * 16);
+      r[2 * i] = *reinterpret_cast<const u32x4 *>(base + (uint32_t)((2 * kp) * ld_bytes + ro * 16));
+      r[2 * i + 1] = *reinterpret_cast<const u32x4 *>(base + (uint32_t)((2 * kp + 1) * ld_bytes + ro * 16));
     }
   } else {
 #pragma unroll
     for (int i = 0; i < G::KSTR_LOADS; ++i) {
       const int q = i * 64 + lane;
       const int rc = q % (TILE / 4), k = q / (TILE / 4);
-      r[i] = *reinterpret_cast<const uint4 *>(base + k * ld_bytes + rc * 16);
+      r[i] = *reinterpret_cast<const u32x4 *>(base + (uint32_t)(k * ld_bytes + rc * 16));
     }
   }
 }
@@ -149,25 +144,25 @@ __device__ inline void load_kstr(uint4 (&r)[G::LOADS], const char *base, int64_t
 // ---- registers -> LDS ----------------------------------------------------
 
 template <typename G>
-__device__ inline void stage_kcont(const uint4 (&r)[G::LOADS], char *lds, int lane) {
+__device__ inline void stage_kcont(const u32x4 (&r)[G::LOADS], char *lds, int lane) {
 #pragma unroll
   for (int i = 0; i < G::KCONT_LOADS; ++i) {
     const int q = i * 64 + lane;
     const int row = q / G::CPR, c = q % G::CPR;
-    *reinterpret_cast<uint4 *>(lds + row * (G::CPR * 16) + swizzle<G::CPR, G::RPL>(row, c) * 16) = r[i];
+    *reinterpret_cast<u32x4 *>(lds + row * (G::CPR * 16) + swizzle<G::CPR, G::RPL>(row, c) * 16) = r[i];
   }
 }
 
 template <typename G, int TILE>
-__device__ inline void stage_kstr(const uint4 (&r)[G::LOADS], char *lds, int lane) {
+__device__ inline void stage_kstr(const u32x4 (&r)[G::LOADS], char *lds, int lane) {
   if constexpr (G::ES == 2) {
 #pragma unroll
     for (int i = 0; i < G::KSTR_LOADS / 2; ++i) {
       const int q = i * 64 + lane;
       const int ro = q % (TILE / 8), kp = q / (TILE / 8);
-      const uint4 e = r[2 * i], o = r[2 * i + 1];  // rows 2kp and 2kp+1, 8 columns each
+      const u32x4 e = r[2 * i], o = r[2 * i + 1];  // rows 2kp and 2kp+1, 8 columns each
       // dword for column c = (even-row value, odd-row value)
-      uint4 lo, hi;
+      u32x4 lo, hi;
       lo.x = __builtin_amdgcn_perm(o.x, e.x, 0x05040100u);
       lo.y = __builtin_amdgcn_perm(o.x, e.x, 0x07060302u);
       lo.z = __builtin_amdgcn_perm(o.y, e.y, 0x05040100u);
@@ -177,15 +172,15 @@ __device__ inline void stage_kstr(const uint4 (&r)[G::LOADS], char *lds, int lan
       hi.z = __builtin_amdgcn_perm(o.w, e.w, 0x05040100u);
       hi.w = __builtin_amdgcn_perm(o.w, e.w, 0x07060302u);
       uint32_t *row = reinterpret_cast<uint32_t *>(lds) + kp * TILE + ro * 8;
-      *reinterpret_cast<uint4 *>(row) = lo;
-      *reinterpret_cast<uint4 *>(row + 4) = hi;
+      *reinterpret_cast<u32x4 *>(row) = lo;
+      *reinterpret_cast<u32x4 *>(row + 4) = hi;
     }
   } else {
 #pragma unroll
     for (int i = 0; i < G::KSTR_LOADS; ++i) {
       const int q = i * 64 + lane;
       const int rc = q % (TILE / 4), k = q / (TILE / 4);
-      *reinterpret_cast<uint4 *>(reinterpret_cast<uint32_t *>(lds) + k * TILE + rc * 4) = r[i];
+      *reinterpret_cast<u32x4 *>(reinterpret_cast<uint32_t *>(lds) + k * TILE + rc * 4) = r[i];
     }
   }
 }
@@ -194,17 +189,17 @@ __device__ inline void stage_kstr(const uint4 (&r)[G::LOADS], char *lds, int lan
 // fragment (block mb, step s) of lane (row = 32 mb + lane % 32, kg = lane / 32)
 
 template <typename G>
-__device__ inline uint4 frag_kcont(const char *lds, int mb, int s, int lane) {
+__device__ inline u32x4 frag_kcont(const char *lds, int mb, int s, int lane) {
   const int row = 32 * mb + (lane & 31), kg = lane >> 5;
-  return *reinterpret_cast<const uint4 *>(lds + row * (G::CPR * 16) + swizzle<G::CPR, G::RPL>(row, 2 * s + kg) * 16);
+  return *reinterpret_cast<const u32x4 *>(lds + row * (G::CPR * 16) + swizzle<G::CPR, G::RPL>(row, 2 * s + kg) * 16);
 }
 
 template <typename G, int TILE>
-__device__ inline uint4 frag_kstr(const char *lds, int mb, int s, int lane) {
+__device__ inline u32x4 frag_kstr(const char *lds, int mb, int s, int lane) {
   const int row = 32 * mb + (lane & 31), kg = lane >> 5;
   // 16-bit: (k,k+1) pair rows 8s + 4kg + t; fp32: k rows 8s + 4kg + t
   const uint32_t *p = reinterpret_cast<const uint32_t *>(lds) + (8 * s + 4 * kg) * TILE + row;
-  uint4 v;
+  u32x4 v;
   v.x = p[0];
   v.y = p[TILE];
   v.z = p[2 * TILE];
@@ -216,16 +211,28 @@ template <typename Tr, int TILE, bool XT, bool YT>
 __global__ __launch_bounds__(256, 2) void matmul_mfma_kernel(const char *__restrict__ x, const char *__restrict__ y,
                                                              char *__restrict__ out,
                                                              const int32_t *__restrict__ pair_offsets,
-                                                             const int32_t *__restrict__ pairs, int64_t n_tiles,
-                                                             int sbs, int side_log2, int64_t nnz_x, int64_t nnz_y) {
+                                                             const int32_t *__restrict__ pairs,
+                                                             const int32_t *__restrict__ block_order,
+                                                             int64_t n_tiles, int sbs, int side_log2, int64_t nnz_x,
+                                                             int64_t nnz_y) {
   using G = Geom<Tr, TILE>;
   constexpr int ES = G::ES;
   __shared__ __attribute__((aligned(16))) char smem[4 * G::WAVE_LDS];
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int64_t tile = (int64_t)blockIdx.x * 4 + wave;
-  if (tile >= n_tiles) return;
+  // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  Give XCD c the c-th contiguous
+  // eighth of the (ordered) work list, so that the tiles in flight on one L2 are neighbours in the list.
+  const int64_t per_xcd = gridDim.x >> 3;
+  const int64_t group = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  const int64_t item = group * 4 + wave;
+  if (item >= n_tiles) return;
+  int64_t tile = item;
+  if (block_order) {
+    const int64_t per_block = (int64_t)1 << (2 * side_log2);
+    tile = (int64_t)__builtin_amdgcn_readfirstlane(block_order[item >> (2 * side_log2)]) * per_block +
+           (item & (per_block - 1));
+  }
   char *lds_x = smem + wave * G::WAVE_LDS;
   char *lds_y = lds_x + G::REGION;
 
@@ -234,7 +241,7 @@ __global__ __launch_bounds__(256, 2) void matmul_mfma_kernel(const char *__restr
   const int ti = (int)(tile >> side_log2) & side_mask;
   const int tj = (int)tile & side_mask;
   const int64_t block_bytes = (int64_t)sbs * sbs * ES;
-  const int64_t ld_bytes = (int64_t)sbs * ES;
+  const uint32_t ld_bytes = (uint32_t)sbs * ES;
   const int n_chunks = sbs / G::KC;  // K-chunks per pair
 
   const int p_begin = __builtin_amdgcn_readfirstlane(pair_offsets[n]);
@@ -249,38 +256,43 @@ __global__ __launch_bounds__(256, 2) void matmul_mfma_kernel(const char *__restr
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
 
-  uint4 rx[G::LOADS], ry[G::LOADS];
+  u32x4 rx[G::LOADS], ry[G::LOADS];
 
-  auto fetch = [&](int it) {
-    const int p = p_begin + it / n_chunks;
-    const int kc = it % n_chunks;
-    int64_t px = __builtin_amdgcn_readfirstlane(pairs[2 * (int64_t)p]);
-    int64_t py = __builtin_amdgcn_readfirstlane(pairs[2 * (int64_t)p + 1]);
-    // a corrupt list must not turn into a wild read
-    if (px < 0 || px >= nnz_x) px = 0;
-    if (py < 0 || py >= nnz_y) py = 0;
-    const char *xb = x + px * block_bytes;
-    const char *yb = y + py * block_bytes;
-    // x tile: rows i = ti*TILE.., k = kc*KC..;  y tile: k rows, columns j = tj*TILE..
-    if constexpr (!XT)
-      load_kcont<G>(rx, xb + (int64_t)ti * TILE * ld_bytes + (int64_t)kc * G::KC * ES, ld_bytes, lane);
-    else  // block holds x^T: element (i, k) at blk[k][i]
-      load_kstr<G, TILE>(rx, xb + (int64_t)kc * G::KC * ld_bytes + (int64_t)ti * TILE * ES, ld_bytes, lane);
-    if constexpr (!YT)
-      load_kstr<G, TILE>(ry, yb + (int64_t)kc * G::KC * ld_bytes + (int64_t)tj * TILE * ES, ld_bytes, lane);
-    else  // block holds y^T: element (k, j) at blk[j][k]
-      load_kcont<G>(ry, yb + (int64_t)tj * TILE * ld_bytes + (int64_t)kc * G::KC * ES, ld_bytes, lane);
-  };
+  // Issues the global loads of iteration `it` (pair it / n_chunks, K-chunk it % n_chunks) into rx / ry.
+#define BSA_FETCH(it_)                                                                                           \
+  do {                                                                                                           \
+    const int p_ = p_begin + (it_) / n_chunks;                                                                   \
+    const int kc_ = (it_) % n_chunks;                                                                            \
+    int64_t px_ = __builtin_amdgcn_readfirstlane(pairs[2 * (int64_t)p_]);                                        \
+    int64_t py_ = __builtin_amdgcn_readfirstlane(pairs[2 * (int64_t)p_ + 1]);                                    \
+    /* a corrupt list must not turn into a wild read */                                                         \
+    px_ = (px_ < 0 || px_ >= nnz_x) ? 0 : px_;                                                                   \
+    py_ = (py_ < 0 || py_ >= nnz_y) ? 0 : py_;                                                                   \
+    const char *xb_ = x + px_ * block_bytes;                                                                     \
+    const char *yb_ = y + py_ * block_bytes;                                                                     \
+    /* x tile: rows i = ti*TILE.., k = kc*KC..;  y tile: k rows, columns j = tj*TILE.. */                        \
+    if constexpr (!XT)                                                                                           \
+      load_kcont<G>(rx, xb_ + (int64_t)ti * TILE * (int64_t)ld_bytes + (int64_t)kc_ * G::KC * ES, ld_bytes, lane);        \
+    else /* block holds x^T: element (i, k) at blk[k][i] */                                                      \
+      load_kstr<G, TILE>(rx, xb_ + (int64_t)kc_ * G::KC * (int64_t)ld_bytes + (int64_t)ti * TILE * ES, ld_bytes, lane);   \
+    if constexpr (!YT)                                                                                           \
+      load_kstr<G, TILE>(ry, yb_ + (int64_t)kc_ * G::KC * (int64_t)ld_bytes + (int64_t)tj * TILE * ES, ld_bytes, lane);   \
+    else /* block holds y^T: element (k, j) at blk[j][k] */                                                      \
+      load_kcont<G>(ry, yb_ + (int64_t)tj * TILE * (int64_t)ld_bytes + (int64_t)kc_ * G::KC * ES, ld_bytes, lane);        \
+  } while (0)
 
-  if (n_iter > 0) fetch(0);
+  if (n_iter > 0) BSA_FETCH(0);
   for (int it = 0; it < n_iter; ++it) {
     if constexpr (!XT) stage_kcont<G>(rx, lds_x, lane); else stage_kstr<G, TILE>(rx, lds_x, lane);
     if constexpr (!YT) stage_kstr<G, TILE>(ry, lds_y, lane); else stage_kcont<G>(ry, lds_y, lane);
-    if (it + 1 < n_iter) fetch(it + 1);
+    // prefetch the next chunk while this one is multiplied; the last iteration re-reads itself (cache hit)
+    // so that the loads stay unconditional and the staging registers never leave the register file
+    const int nxt = (it + 1 < n_iter) ? it + 1 : it;
+    BSA_FETCH(nxt);
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
 #pragma unroll
     for (int s = 0; s < G::STEPS; ++s) {
-      uint4 fx[G::NB], fy[G::NB];
+      u32x4 fx[G::NB], fy[G::NB];
 #pragma unroll
       for (int b = 0; b < G::NB; ++b) {
         if constexpr (!XT) fx[b] = frag_kcont<G>(lds_x, b, s, lane); else fx[b] = frag_kstr<G, TILE>(lds_x, b, s, lane);
@@ -293,6 +305,7 @@ __global__ __launch_bounds__(256, 2) void matmul_mfma_kernel(const char *__restr
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
   }
+#undef BSA_FETCH
 
   // epilogue: acc[bj][bi][r] = O[i = 32 bi + lane%32][j = 32 bj + 8 (r/4) + 4 (lane/32) + r%4]
   char *stage = lds_x;
@@ -322,7 +335,7 @@ __global__ __launch_bounds__(256, 2) void matmul_mfma_kernel(const char *__restr
         }
       }
   __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-  char *ob = out + n * block_bytes + (int64_t)ti * TILE * ld_bytes + (int64_t)tj * TILE * ES;
+  char *ob = out + n * block_bytes + (int64_t)ti * TILE * (int64_t)ld_bytes + (int64_t)tj * TILE * ES;
 #pragma unroll
   for (int t = 0; t < G::OUT_STORES; ++t) {
     const int q = t * 64 + lane;
@@ -380,19 +393,21 @@ __global__ __launch_bounds__(256) void matmul_small_kernel(const typename Tr::st
 
 template <typename Tr, int TILE>
 int launch_mfma(const void *x, const void *y, void *out, const int32_t *pair_offsets, const int32_t *pairs,
-                int64_t nnz_o, int64_t nnz_x, int64_t nnz_y, int sbs, int trans_x, int trans_y, hipStream_t s) {
+                const int32_t *block_order, int64_t nnz_o, int64_t nnz_x, int64_t nnz_y, int sbs, int trans_x,
+                int trans_y, hipStream_t s) {
   const int side = sbs / TILE;
   int side_log2 = 0;
   while ((1 << side_log2) < side) ++side_log2;
   const int64_t n_tiles = nnz_o * side * side;
-  const int64_t blocks = bsa::cdiv(n_tiles, 4);
+  // a multiple of 8 workgroups so that every XCD owns the same number of list positions
+  const int64_t blocks = bsa::cdiv(bsa::cdiv(n_tiles, 4), 8) * 8;
   if (blocks > 0x7fffffffLL) return bsa::fail(BSA_ELIMIT, "bsa_matmul: too many output tiles");
   const char *xc = static_cast<const char *>(x);
   const char *yc = static_cast<const char *>(y);
   char *oc = static_cast<char *>(out);
 #define BSA_MM_LAUNCH(XT, YT)                                                                                      \
-  matmul_mfma_kernel<Tr, TILE, XT, YT><<<(unsigned)blocks, 256, 0, s>>>(xc, yc, oc, pair_offsets, pairs, n_tiles, \
-                                                                        sbs, side_log2, nnz_x, nnz_y)
+  matmul_mfma_kernel<Tr, TILE, XT, YT><<<(unsigned)blocks, 256, 0, s>>>(xc, yc, oc, pair_offsets, pairs, block_order, \
+                                                                        n_tiles, sbs, side_log2, nnz_x, nnz_y)
   if (!trans_x && !trans_y) BSA_MM_LAUNCH(false, false);
   else if (!trans_x && trans_y) BSA_MM_LAUNCH(false, true);
   else if (trans_x && !trans_y) BSA_MM_LAUNCH(true, false);
@@ -403,7 +418,8 @@ int launch_mfma(const void *x, const void *y, void *out, const int32_t *pair_off
 
 template <typename Tr>
 int launch_any(const void *x, const void *y, void *out, const int32_t *pair_offsets, const int32_t *pairs,
-               int64_t nnz_o, int64_t nnz_x, int64_t nnz_y, int sbs, int trans_x, int trans_y, hipStream_t s) {
+               const int32_t *block_order, int64_t nnz_o, int64_t nnz_x, int64_t nnz_y, int sbs, int trans_x,
+               int trans_y, hipStream_t s) {
   if (sbs == 16) {
     using E = typename Tr::store_t;
     const int64_t blocks = bsa::cdiv(nnz_o, 4);
@@ -414,8 +430,8 @@ int launch_any(const void *x, const void *y, void *out, const int32_t *pair_offs
     return bsa::check_launch("matmul_small_kernel");
   }
   if (sbs == 32)
-    return launch_mfma<Tr, 32>(x, y, out, pair_offsets, pairs, nnz_o, nnz_x, nnz_y, sbs, trans_x, trans_y, s);
-  return launch_mfma<Tr, 64>(x, y, out, pair_offsets, pairs, nnz_o, nnz_x, nnz_y, sbs, trans_x, trans_y, s);
+    return launch_mfma<Tr, 32>(x, y, out, pair_offsets, pairs, block_order, nnz_o, nnz_x, nnz_y, sbs, trans_x, trans_y, s);
+  return launch_mfma<Tr, 64>(x, y, out, pair_offsets, pairs, block_order, nnz_o, nnz_x, nnz_y, sbs, trans_x, trans_y, s);
 }
 
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
@@ -423,7 +439,7 @@ bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 
 }  // namespace
 
 extern "C" int bsa_matmul(const void *x, const void *y, void *out, const int32_t *pair_offsets, const int32_t *pairs,
-                          int64_t nnz_o, int64_t nnz_x, int64_t nnz_y, int sbs, int dtype, int trans_x, int trans_y,
+                          const int32_t *block_order, int64_t nnz_o, int64_t nnz_x, int64_t nnz_y, int sbs, int dtype, int trans_x, int trans_y,
                           bsa_stream_t stream) {
   BSA_REQUIRE(sbs >= 16 && bsa::is_pow2(sbs), "bsa_matmul: sbs must be a power of two >= 16 (got %d)", sbs);
   BSA_REQUIRE(nnz_o >= 0 && nnz_x >= 0 && nnz_y >= 0, "bsa_matmul: negative size");
@@ -434,10 +450,10 @@ extern "C" int bsa_matmul(const void *x, const void *y, void *out, const int32_t
   hipStream_t s = bsa::as_stream(stream);
   switch (dtype) {
     case BSA_BF16:
-      return launch_any<Bf16Traits>(x, y, out, pair_offsets, pairs, nnz_o, nnz_x, nnz_y, sbs, trans_x, trans_y, s);
+      return launch_any<Bf16Traits>(x, y, out, pair_offsets, pairs, block_order, nnz_o, nnz_x, nnz_y, sbs, trans_x, trans_y, s);
     case BSA_F16:
-      return launch_any<F16Traits>(x, y, out, pair_offsets, pairs, nnz_o, nnz_x, nnz_y, sbs, trans_x, trans_y, s);
+      return launch_any<F16Traits>(x, y, out, pair_offsets, pairs, block_order, nnz_o, nnz_x, nnz_y, sbs, trans_x, trans_y, s);
     default:
-      return launch_any<F32Traits>(x, y, out, pair_offsets, pairs, nnz_o, nnz_x, nnz_y, sbs, trans_x, trans_y, s);
+      return launch_any<F32Traits>(x, y, out, pair_offsets, pairs, block_order, nnz_o, nnz_x, nnz_y, sbs, trans_x, trans_y, s);
   }
 }

@@ -19,15 +19,29 @@ from ..utils.validation import (ensure_contiguous, validate_contiguous, validate
                                 validate_sparsity_layout)
 
 
-def _launch(x: Tensor, y: Tensor, pair_offsets: Tensor, pairs: Tensor, n_out: int, sbs: int,
+def _launch(x: Tensor, y: Tensor, pair_offsets: Tensor, pairs: Tensor, order: Tensor | None, n_out: int, sbs: int,
             trans_x: bool, trans_y: bool) -> Tensor:
     out = torch.empty((n_out, sbs, sbs), dtype=x.dtype, device=x.device)
     if n_out:
         with torch.cuda.device(x.device):
             _capi.call("bsa_matmul", _capi.ptr(x), _capi.ptr(y), out.data_ptr(), pair_offsets.data_ptr(),
-                       _capi.ptr(pairs), n_out, x.size(0), y.size(0), sbs, _capi.DTYPE_CODES[x.dtype],
-                       int(trans_x), int(trans_y), _capi.stream(x.device))
+                       _capi.ptr(pairs), _capi.ptr(order), n_out, x.size(0), y.size(0), sbs,
+                       _capi.DTYPE_CODES[x.dtype], int(trans_x), int(trans_y), _capi.stream(x.device))
     return out
+
+
+_SUPER_TILE = 16
+
+
+def _block_order(layout_indices: Tensor) -> Tensor:
+    """Work order of the output blocks: 16 x 16 super-tiles of the block grid, columns of super-tiles
+    fastest, so that the blocks in flight on one L2 share x row panels and y column panels."""
+    b, i, j = layout_indices[:, 0], layout_indices[:, 1], layout_indices[:, 2]
+    t = _SUPER_TILE
+    n_i = int(i.max().item()) // t + 1 if i.numel() else 1
+    n_j = int(j.max().item()) // t + 1 if j.numel() else 1
+    key = ((b * n_i + i // t) * n_j + j // t) * (t * t) + (i % t) * t + (j % t)
+    return torch.argsort(key, stable=True).to(torch.int32)
 
 
 def _backward_lists(layout_cache: dict, shape_x, shape_y):
@@ -59,7 +73,8 @@ class _Matmul(torch.autograd.Function):
         ctx.shapes = (shape_x, shape_y)
         ctx.sparsity_block_size = sparsity_block_size
         return _launch(x, y, layout_cache["contraction_offsets"], layout_cache["contraction_pairs"],
-                       layout_cache["n_sparse_blocks"], sparsity_block_size, False, False)
+                       layout_cache["block_order"], layout_cache["n_sparse_blocks"], sparsity_block_size, False,
+                       False)
 
     @staticmethod
     def backward(ctx, grad_output):
@@ -69,9 +84,9 @@ class _Matmul(torch.autograd.Function):
         gx_off, gx_pairs, gy_off, gy_pairs = _backward_lists(ctx.layout_cache, *ctx.shapes)
         grad_x = grad_y = None
         if ctx.needs_input_grad[0]:
-            grad_x = _launch(grad_output, y, gx_off, gx_pairs, x.size(0), sbs, False, True)
+            grad_x = _launch(grad_output, y, gx_off, gx_pairs, None, x.size(0), sbs, False, True)
         if ctx.needs_input_grad[1]:
-            grad_y = _launch(x, grad_output, gy_off, gy_pairs, y.size(0), sbs, True, False)
+            grad_y = _launch(x, grad_output, gy_off, gy_pairs, None, y.size(0), sbs, True, False)
         return grad_x, grad_y, None, None, None, None
 
 
@@ -102,6 +117,7 @@ def matmul_build_layout_cache(layout_cache: dict | None, sparsity_layout_x: Tens
         layout_cache["n_sparse_blocks_y"] = info_y.count
         layout_cache["contraction_offsets"] = lists.pair_offsets
         layout_cache["contraction_pairs"] = lists.pairs
+        layout_cache["block_order"] = _block_order(layout_cache["layout_indices_o"])
 
     validate_contiguous(sparsity_layout_x, layout_cache["packed_indices_x"],
                         sparsity_layout_y, layout_cache["packed_indices_y"],

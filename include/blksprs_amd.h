@@ -172,9 +172,11 @@ int bsa_softmax_bwd(const float *grad_out, const float *y, float *grad_in,
  * (blksprs/ops/matmul.py:70-253).  trans_x / trans_y read the x / y blocks
  * transposed (block[c][r] instead of block[r][c]); the reference materialises
  * such operands with transpose() first (blksprs/ops/matmul.py:135-143).
+ * block_order (int32 [nnz_o], a permutation, or NULL for identity) is the order in
+ * which output blocks are worked on; it only affects cache behaviour, never results.
  */
 int bsa_matmul(const void *x, const void *y, void *out, const int32_t *pair_offsets,
-               const int32_t *pairs, int64_t nnz_o, int64_t nnz_x, int64_t nnz_y, int sbs, int dtype,
+               const int32_t *pairs, const int32_t *block_order, int64_t nnz_o, int64_t nnz_x, int64_t nnz_y, int sbs, int dtype,
                int trans_x, int trans_y, bsa_stream_t stream);
 
 /* ------------------------------------------------------------- attention */

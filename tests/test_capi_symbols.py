@@ -34,10 +34,10 @@ def test_argument_block_matches_the_header_layout():
 def test_bad_arguments_are_rejected_on_the_host():
     lib = _capi.load()
     # sbs = 24 is not a power of two; nothing is launched
-    rc = lib.bsa_matmul(0, 0, 0, 0, 0, 0, 0, 0, 24, 0, 0, 0, 0)
+    rc = lib.bsa_matmul(0, 0, 0, 0, 0, 0, 0, 0, 0, 24, 0, 0, 0, 0)
     assert rc == -1 and b"power of two" in lib.bsa_last_error()
     rc = lib.bsa_to_sparse(0, 0, 0, 0, 32, 32, 16, 3, 0)
     assert rc == -1 and b"element size" in lib.bsa_last_error()
     # empty problems are accepted without touching the device
-    assert lib.bsa_matmul(0, 0, 0, 0, 0, 0, 0, 0, 64, 2, 0, 0, 0) == 0
+    assert lib.bsa_matmul(0, 0, 0, 0, 0, 0, 0, 0, 0, 64, 2, 0, 0, 0) == 0
     assert lib.bsa_softmax_fwd(0, 0, 0, 0, 0, 32, 0) == 0

@@ -61,7 +61,8 @@ def test_backward_matches_autograd_of_the_oracle(device, dtype, sbs):
     xg = x.to(device).requires_grad_(True)
     yg = y.to(device).requires_grad_(True)
     cache = {}
-    out = bs.ops.matmul(xg, lx.to(device), yg, ly.to(device), lo.to(device), sbs, layout_cache=cache)
+    lxd, lyd, lod = lx.to(device), ly.to(device), lo.to(device)
+    out = bs.ops.matmul(xg, lxd, yg, lyd, lod, sbs, layout_cache=cache)
     go = rand_blocks(out.size(0), sbs, dtype, seed=9)
     out.backward(go.to(device))
     x64 = x.double().requires_grad_(True)
@@ -70,13 +71,15 @@ def test_backward_matches_autograd_of_the_oracle(device, dtype, sbs):
     yd = orc.to_dense_autograd(y64, ly.numpy(), sbs)
     ref = orc.to_sparse_autograd(xd @ yd, lo.numpy(), sbs)
     ref.backward(go.double())
-    tol = TOL[dtype] if dtype == torch.float32 else 4e-2
+    # the upstream gradient is unscaled N(0,1): fp32 sums of ~300 O(1) products differ by a few 1e-5 between
+    # accumulation orders, so fp32 gradients are held to 1e-4 here (the forward test holds 1e-5)
+    tol = 1e-4 if dtype == torch.float32 else 4e-2
     assert_close(xg.grad, x64.grad, tol, f"dX {dtype} sbs={sbs}")
     assert_close(yg.grad, y64.grad, tol, f"dY {dtype} sbs={sbs}")
     # a second step reuses the forward and backward lists
     offsets = cache["grad_x_pair_offsets"]
     xg.grad = None
-    bs.ops.matmul(xg, lx.to(device), yg, ly.to(device), lo.to(device), sbs, layout_cache=cache).backward(go.to(device))
+    bs.ops.matmul(xg, lxd, yg, lyd, lod, sbs, layout_cache=cache).backward(go.to(device))
     assert cache["grad_x_pair_offsets"] is offsets
     assert_close(xg.grad, x64.grad, tol, "dX second step")
 
@@ -123,11 +126,14 @@ def test_full_size_config2_linearity_and_sampled_parity(device):
     y = torch.randn((int(ly.sum()), sbs, sbs), generator=g).to(torch.bfloat16)
     xd, yd = x.to(device), y.to(device)
     cache = {}
-    out = bs.ops.matmul(xd, lx.to(device), yd, ly.to(device), lo.to(device), sbs, layout_cache=cache)
+    lxd, lyd, lod = lx.to(device), ly.to(device), lo.to(device)
+    out = bs.ops.matmul(xd, lxd, yd, lyd, lod, sbs, layout_cache=cache)
     assert out.shape[0] == int(lo.sum())
-    doubled = bs.ops.matmul(xd * 2, lx.to(device), yd, ly.to(device), lo.to(device), sbs, layout_cache=cache)
+    pairs = cache["contraction_pairs"]
+    doubled = bs.ops.matmul(xd * 2, lxd, yd, lyd, lod, sbs, layout_cache=cache)
+    assert cache["contraction_pairs"] is pairs
     assert torch.equal(doubled, out * 2)
-    zero = bs.ops.matmul(xd, lx.to(device), torch.zeros_like(yd), ly.to(device), lo.to(device), sbs, layout_cache=cache)
+    zero = bs.ops.matmul(xd, lxd, torch.zeros_like(yd), lyd, lod, sbs, layout_cache=cache)
     assert torch.all(zero == 0)
     # batch 3 against the oracle (one batch keeps the dense CPU product small)
     b = 3
