@@ -30,6 +30,19 @@ def _launch(x: Tensor, y: Tensor, pair_offsets: Tensor, pairs: Tensor, order: Te
     return out
 
 
+def _launch_rows(x: Tensor, y: Tensor, cache: dict, n_rows: int, sbs: int) -> Tensor:
+    """Forward product by output block row (fp16 / bf16, sbs 64): x row panels stay in LDS."""
+    n_out = cache["n_sparse_blocks"]
+    out = torch.empty((n_out, sbs, sbs), dtype=x.dtype, device=x.device)
+    if n_out:
+        with torch.cuda.device(x.device):
+            _capi.call("bsa_matmul_rows", _capi.ptr(x), _capi.ptr(y), out.data_ptr(),
+                       cache["contraction_offsets"].data_ptr(), _capi.ptr(cache["contraction_pairs"]),
+                       cache["row_offsets_x"].data_ptr(), cache["row_offsets_o"].data_ptr(), n_rows, n_out,
+                       x.size(0), y.size(0), sbs, _capi.DTYPE_CODES[x.dtype], _capi.stream(x.device))
+    return out
+
+
 _SUPER_TILE = 16
 
 
@@ -72,6 +85,9 @@ class _Matmul(torch.autograd.Function):
         ctx.layout_cache = layout_cache
         ctx.shapes = (shape_x, shape_y)
         ctx.sparsity_block_size = sparsity_block_size
+        if (sparsity_block_size == 64 and x.dtype in (torch.float16, torch.bfloat16)
+                and layout_cache["row_offsets_x"] is not None and layout_cache["row_offsets_o"] is not None):
+            return _launch_rows(x, y, layout_cache, shape_x[0] * shape_x[1], sparsity_block_size)
         return _launch(x, y, layout_cache["contraction_offsets"], layout_cache["contraction_pairs"],
                        layout_cache["block_order"], layout_cache["n_sparse_blocks"], sparsity_block_size, False,
                        False)
@@ -102,10 +118,10 @@ def matmul_build_layout_cache(layout_cache: dict | None, sparsity_layout_x: Tens
     layout_cache = prepare_layout_cache(layout_cache, "matmul", sparsity_layout_x, sparsity_layout_y,
                                         sparsity_layout_output)
     if "contraction_pairs" not in layout_cache:
-        info_x, info_y = pack_layout(sparsity_layout_x), pack_layout(sparsity_layout_y)
-        info_o = pack_layout(sparsity_layout_output)
         B, R, K = (int(s) for s in sparsity_layout_x.shape)
         C = int(sparsity_layout_y.size(2))
+        info_x, info_y = pack_layout(sparsity_layout_x, row_len=K), pack_layout(sparsity_layout_y)
+        info_o = pack_layout(sparsity_layout_output, row_len=C)
         lists = build_contraction_lists(info_x.packed, info_y.packed, info_o.packed, B, R, K, C, info_o.count)
         layout_cache["packed_indices_x"] = info_x.packed
         layout_cache["packed_indices_y"] = info_y.packed
@@ -118,6 +134,8 @@ def matmul_build_layout_cache(layout_cache: dict | None, sparsity_layout_x: Tens
         layout_cache["contraction_offsets"] = lists.pair_offsets
         layout_cache["contraction_pairs"] = lists.pairs
         layout_cache["block_order"] = _block_order(layout_cache["layout_indices_o"])
+        layout_cache["row_offsets_x"] = info_x.row_offsets
+        layout_cache["row_offsets_o"] = info_o.row_offsets
 
     validate_contiguous(sparsity_layout_x, layout_cache["packed_indices_x"],
                         sparsity_layout_y, layout_cache["packed_indices_y"],

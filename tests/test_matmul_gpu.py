@@ -169,3 +169,33 @@ def test_autocast_and_validation(device):
         assert out.shape == (4, sbs, sbs)
     finally:
         bs.utils.enable_validation()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("dims,dx,dy,do", [
+    ((2, 3, 40, 5), 0.9, 0.5, 0.8),     # rows with more than 16 x blocks: the part that does not fit in LDS
+    ((1, 2, 6, 600), 0.5, 0.5, 0.9),    # more than 64 output blocks per wave: boundary window reloads
+    ((1, 1, 30, 40), 1.0, 1.0, 1.0),    # more than 64 pairs per wave: pair window reloads
+    ((3, 9, 7, 11), 0.3, 0.3, 0.5),     # empty rows, output blocks without pairs
+])
+def test_row_panel_kernel_is_bit_identical_to_the_tile_kernel(device, dtype, dims, dx, dy, do):
+    """fp16 / bf16 with sbs 64 run the row-panel kernel; it must reproduce the per-tile kernel bit for bit
+    (same pairs, same ascending-k accumulation)."""
+    from blksprs_amd import _capi
+    B, R, K, C = dims
+    sbs = 64
+    lx = rand_layout((B, R, K), dx, seed=1).to(device)
+    ly = rand_layout((B, K, C), dy, seed=2).to(device)
+    lo = rand_layout((B, R, C), do, seed=3).to(device)
+    if dx < 0.5:
+        lx[0, 0] = False  # a row without x blocks
+    x = rand_blocks(int(lx.sum()), sbs, dtype, 4, 1.0 / math.sqrt(K * sbs)).to(device)
+    y = rand_blocks(int(ly.sum()), sbs, dtype, 5).to(device)
+    cache = {}
+    out = bs.ops.matmul(x, lx, y, ly, lo, sbs, layout_cache=cache)
+    ref = torch.empty_like(out)
+    _capi.call("bsa_matmul", x.data_ptr(), y.data_ptr(), ref.data_ptr(), cache["contraction_offsets"].data_ptr(),
+               _capi.ptr(cache["contraction_pairs"]), cache["block_order"].data_ptr(), out.size(0), x.size(0),
+               y.size(0), sbs, _capi.DTYPE_CODES[dtype], 0, 0, _capi.stream(device))
+    assert torch.equal(out, ref)
+    assert_close(out, _oracle(x.cpu(), lx.cpu(), y.cpu(), ly.cpu(), lo.cpu(), sbs), 2e-2, "row panel vs oracle")
