@@ -30,8 +30,11 @@ class AttnArgs(ctypes.Structure):
         + [(n, c_int64) for n in ("B", "nq", "nk", "nh", "nhv", "n_q_blocks", "n_k_blocks", "n_v_blocks",
                                   "n_o_blocks", "n_mask_blocks", "n_bias_blocks")]
         + [("sbs", ctypes.c_int32), ("dtype", ctypes.c_int32), ("mask_kind", ctypes.c_int32), ("scale", c_float)]
+        + [("group_offsets", c_void_p), ("group_records", c_void_p), ("group_size", ctypes.c_int32)]
     )
 
+
+ATTN_RECORD_INTS = 16  # BSA_ATTN_RECORD_INTS
 
 # name -> (restype, argtypes); must list every symbol of include/blksprs_amd.h
 SIGNATURES = {
@@ -58,6 +61,7 @@ SIGNATURES = {
                            c_int, c_int, c_int, c_void_p]),
     "bsa_matmul_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
                                 c_int64, c_int64, c_int64, c_int, c_int, c_void_p]),
+    "bsa_attn_fwd_records": (c_int, [ctypes.POINTER(AttnArgs), c_void_p, c_void_p, c_void_p]),
     "bsa_attn_fwd": (c_int, [ctypes.POINTER(AttnArgs), c_void_p]),
     "bsa_attn_bwd": (c_int, [ctypes.POINTER(AttnArgs), c_void_p]),
 }

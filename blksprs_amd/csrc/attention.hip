@@ -24,6 +24,8 @@ int check_args(const char *who, const bsa_attn_args *a, bool backward) {
   BSA_REQUIRE(!a->bias || a->pidx_bias, "%s: bias without pidx_bias", who);
   BSA_REQUIRE(a->B * a->nq < 0x7fffffffLL && a->B * a->nk < 0x7fffffffLL, "%s: too many sequence blocks", who);
   BSA_REQUIRE(a->nh < 65536 && a->nhv < 65536, "%s: too many head slices", who);
+  BSA_REQUIRE(a->group_size >= 0 && a->group_size <= 2, "%s: group_size must be 0, 1 or 2", who);
+  BSA_REQUIRE(a->group_size == 0 || a->group_offsets, "%s: group_size without group_offsets", who);
   if (backward) {
     BSA_REQUIRE(a->query_offsets != nullptr, "%s: query_offsets is NULL", who);
     BSA_REQUIRE(a->delta != nullptr || a->B * a->nq == 0, "%s: delta is NULL", who);
@@ -46,6 +48,23 @@ extern "C" int bsa_attn_fwd(const bsa_attn_args *args, bsa_stream_t stream) {
   int rc = bsa::attn_fwd_mfma(*args, s);
   if (rc == 1) rc = bsa::attn_fwd_generic(*args, s);
   return rc;
+}
+
+extern "C" int bsa_attn_fwd_records(const bsa_attn_args *a, const int32_t *group_entries, int32_t *records,
+                                    bsa_stream_t stream) {
+  const char *who = "bsa_attn_fwd_records";
+  BSA_REQUIRE(a != nullptr, "%s: NULL argument block", who);
+  BSA_REQUIRE(a->group_size == 1 || a->group_size == 2, "%s: group_size must be 1 or 2 (got %d)", who, a->group_size);
+  BSA_REQUIRE(a->B >= 0 && a->nq >= 0 && a->nk >= 0, "%s: negative layout size", who);
+  BSA_REQUIRE(a->nh >= 0 && a->nh <= 2 && a->nhv >= 0 && a->nhv <= 2, "%s: at most two head slices", who);
+  BSA_REQUIRE(a->nk < (1 << 28), "%s: too many key blocks for a list entry", who);
+  if (a->B * a->nq == 0) return BSA_OK;
+  BSA_REQUIRE(a->group_offsets != nullptr, "%s: group_offsets is NULL", who);
+  BSA_REQUIRE(a->nh == 0 || a->pidx_k, "%s: pidx_k is NULL", who);
+  BSA_REQUIRE(a->nhv == 0 || a->pidx_v, "%s: pidx_v is NULL", who);
+  BSA_REQUIRE(a->B * ((a->nq + a->group_size - 1) / a->group_size) < 0x7fffffffLL, "%s: too many groups", who);
+  if (group_entries == nullptr || records == nullptr) return BSA_OK;  // no entries
+  return bsa::attn_fwd_records(*a, group_entries, records, bsa::as_stream(stream));
 }
 
 extern "C" int bsa_attn_bwd(const bsa_attn_args *args, bsa_stream_t stream) {

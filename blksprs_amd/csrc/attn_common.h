@@ -35,7 +35,17 @@ __device__ inline bool mask_set(const void *mask, int kind, int64_t idx) {
   return false;
 }
 
+// One entry of a grouped forward list, 64 bytes (BSA_ATTN_RECORD_INTS int32): the list entry (key block in
+// the low 28 bits, bit 28 + g set if the key block is active for query block g of the group), the packed
+// indices of its K and V head slices (-1: inactive or no such slice) and of its mask and bias blocks for
+// either query block of the group (-1: none).
+struct AttnFwdRecord {
+  int32_t entry, pk[2], pv[2], pm[2], pb[2], pad[7];
+};
+static_assert(sizeof(AttnFwdRecord) == BSA_ATTN_RECORD_INTS * 4, "record layout");
+
 int attn_fwd_generic(const bsa_attn_args &a, hipStream_t s);
+int attn_fwd_records(const bsa_attn_args &a, const int32_t *entries, int32_t *records, hipStream_t s);
 int attn_bwd_generic(const bsa_attn_args &a, hipStream_t s);
 // MFMA paths; return 1 if the configuration is not covered (caller falls back to the generic kernels)
 int attn_fwd_mfma(const bsa_attn_args &a, hipStream_t s);

@@ -21,14 +21,36 @@
 //
 // The K / V tiles of key block e+1, the mask words of e+1, the packed indices of e+2
 // and the key index of e+3 are all fetched while block e is computed.  The index
-// fetches use vector loads on purpose: they complete in order with the tile loads, so
-// the one wait at the top of an iteration covers them and no scalar-load wait lands
-// in front of an LDS read.
+// fetches are one vector load (each index in its own lane) on purpose: it completes
+// in order with the tile loads, so the one wait at the top of an iteration covers it
+// and no scalar-load wait lands in front of an LDS read.  The vector memory pipeline
+// works per instruction, so the count of load instructions per tile is kept small.
 //
 // Score pipeline (log2 domain), in this order: scale * q k^T, + bias, native causal
 // predicate, explicit mask; probabilities are rounded to the operand type before they
 // multiply V; the row sum uses the unrounded values.
 #include "attn_common.h"
+
+// Phase clocks for an offline timing harness; compiled out of the library.
+#ifdef BSA_ATTN_PROBE
+__device__ unsigned long long bsa_attn_probe[8 * 4096];
+#define BSA_PROBE_DECL unsigned long long probe_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0}, probe_t = __builtin_readcyclecounter()
+#define BSA_PROBE(slot)                                            \
+  do {                                                             \
+    const unsigned long long now_ = __builtin_readcyclecounter();  \
+    probe_acc[slot] += now_ - probe_t;                             \
+    probe_t = now_;                                                \
+  } while (0)
+#define BSA_PROBE_FLUSH(wg, lane_)                                                                   \
+  do {                                                                                               \
+    if ((wg) < 4096 && (lane_) == 0)                                                                 \
+      for (int i_ = 0; i_ < 8; ++i_) bsa_attn_probe[(wg) * 8 + i_] = probe_acc[i_];                 \
+  } while (0)
+#else
+#define BSA_PROBE_DECL
+#define BSA_PROBE(slot)
+#define BSA_PROBE_FLUSH(wg, lane_)
+#endif
 
 namespace bsa {
 namespace {
@@ -68,6 +90,7 @@ struct MF16 {
 constexpr int kSbs = 64;
 constexpr int kBlockBytes = kSbs * kSbs * 2;  // one 16-bit block
 constexpr int kFwdThreads = 128;
+constexpr float kRescaleStep = 8.f;  // log2 units
 
 // dword offset of column c in a pair row of the (j, j+1)-packed V tile; the placement of the column
 // quads keeps both the 128-bit writes of the staging step and the 32-bit fragment reads conflict free
@@ -77,63 +100,35 @@ __device__ inline int pair_col_offset(int c) {
   return 4 * pos + (c & 3);
 }
 
-// keeps a wave-uniform value in a vector register so that loads addressed with it use the vector memory path
-__device__ inline int as_vector(int v) {
-  asm volatile("" : "+v"(v));
-  return v;
-}
-
 __device__ inline int first_lane(int v) { return __builtin_amdgcn_readfirstlane(v); }
-__device__ inline int64_t first_lane64(int64_t v) {
-  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
-  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)v >> 32));
-  return (int64_t)(((uint64_t)hi << 32) | lo);
-}
-
-// packed indices of one key block, as loaded (vector registers)
-template <int NH, int NHV>
-struct KeyIndices {
-  int kb;
-  int pk[NH];
-  int pv[NHV];
-  int pm, pb;
-};
-
-// Low half of a packed index.  Valid indices are below 2^31 (the block counts are), the marker of an
-// inactive block is -1, so the low half carries everything the kernels test.
-__device__ inline int low_half(const int64_t *p, int64_t i) { return reinterpret_cast<const int32_t *>(p)[2 * i]; }
-
-template <int NH, int NHV>
-__device__ inline KeyIndices<NH, NHV> load_key_indices(const bsa_attn_args &a, int64_t b, int64_t row, int kb) {
-  KeyIndices<NH, NHV> r;
-  r.kb = kb;
-  const int64_t krow = b * a.nk + kb;
-#pragma unroll
-  for (int h = 0; h < NH; ++h) r.pk[h] = low_half(a.pidx_k, krow * NH + h);
-#pragma unroll
-  for (int h = 0; h < NHV; ++h) r.pv[h] = low_half(a.pidx_v, krow * NHV + h);
-  r.pm = a.mask ? low_half(a.pidx_mask, row * a.nk + kb) : -1;
-  r.pb = a.bias ? low_half(a.pidx_bias, row * a.nk + kb) : -1;
-  return r;
-}
-
 typedef __attribute__((address_space(3))) void *lds_ptr_t;
 
 // Asynchronous copy of 64 x 16 bytes, global -> LDS: lane l's 16 bytes land at dst + 16 l (dst is wave
 // uniform).  Completion is counted by vmcnt like any vector load.  Written as inline assembly so that the
 // compiler's wait-count pass does not see it: it would otherwise wait for the copy in front of every later
-// LDS read, also reads of other LDS arrays.  The caller waits (vmcnt(0)) before the data is read.  Copies
+// LDS read, also reads of other LDS arrays.  m0 is reserved: the compiler sets it before each of its own
+// uses and keeps nothing in it across statements.  The caller waits (vmcnt(0)) before the data is read.  Copies
 // the compiler does not know about only make the waits it computes for its own loads longer, never shorter.
-__device__ inline void copy_1k_to_lds(const char *src, char *dst) {
+// The source is base (wave uniform) + off (per lane, 32 bits).
+__device__ inline void copy_1k_to_lds(const char *base, uint32_t off, char *dst) {
   const uint32_t lds_addr = (uint32_t)(uintptr_t)(lds_ptr_t)dst;
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                :
-               : "v"(src), "s"(lds_addr)
-               : "memory", "m0");
+               : "v"(off), "s"(base), "s"(lds_addr)
+               : "memory");
 }
 
-template <typename Tr, int NH, int NHV>
-__global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_args a) {
+// 16 bytes at base (wave uniform) + off (per lane): scalar base, 32-bit vector offset addressing
+__device__ inline u32x4 load16(const char *base, uint32_t off) {
+  return *reinterpret_cast<const u32x4 *>(base + off);
+}
+
+// G = query blocks per workgroup (1 or 2).  With G = 2 the workgroup has four waves and walks the union of
+// the key lists of two neighbouring query blocks, so that a K / V tile both of them need is fetched once;
+// bits 28 and 29 of a list entry say which of the two the key block is active for.
+template <typename Tr, int NH, int NHV, int G>
+__global__ __launch_bounds__(kFwdThreads *G, 2) void attn_fwd_mfma_kernel(bsa_attn_args a) {
+  constexpr int kThreads = kFwdThreads * G;
   // two arrays, not one: the compiler then knows that the asynchronous K copy never touches the V tile
   __shared__ __attribute__((aligned(1024))) char lds_k[NH * kBlockBytes];
   __shared__ __attribute__((aligned(16))) char lds_v[NHV * kBlockBytes];
@@ -142,13 +137,21 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
   const int lane = tid & 63;
   const int wave = first_lane(tid >> 6);
   const int li = lane & 31, kg = lane >> 5;
-  const int qi = 32 * wave + li;  // query row inside the block
+  const int qi = 32 * (wave & 1) + li;  // query row inside the block
   // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2: give every XCD a contiguous
   // range of rows, so that the query blocks in flight on one L2 share their batch entry's K and V.
-  const int64_t row = (int64_t)(blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
-  if (row >= a.B * a.nq) return;
-  const int64_t b = row / a.nq, qb = row % a.nq;
-  const int k_begin = a.key_offsets[row], k_end = a.key_offsets[row + 1];
+  const int64_t groups_per_batch = (a.nq + G - 1) / G;
+  const int64_t grp = (int64_t)(blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+  if (grp >= a.B * groups_per_batch) return;
+  const int64_t b = grp / groups_per_batch;
+  const int64_t qb_raw = (grp % groups_per_batch) * G + (wave >> 1);
+  // a group at the end of an odd sequence has one query block only: its second pair of waves only helps to copy
+  const bool has_q = qb_raw < a.nq;
+  const int64_t qb = has_q ? qb_raw : a.nq - 1;
+  const int64_t row = b * a.nq + qb;
+  const AttnFwdRecord *recs = reinterpret_cast<const AttnFwdRecord *>(a.group_records);
+  const int k_begin = a.group_offsets[grp], k_end = a.group_offsets[grp + 1];
+  const int my_bit = 28 + (wave >> 1);
 
   // Q fragments stay in registers for the whole row
   u32x4 qf[NH][4];
@@ -183,101 +186,112 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
   }
   const int qpos = (int)qb * kSbs + qi;
 
+  BSA_PROBE_DECL;
   if (k_begin < k_end) {
-    u32x4 vr[NHV][4];  // staging registers of the V tile in flight
-    uint32_t mask_nxt[8];
+    u32x4 vr[NHV][4 / G];  // staging registers of the V tile in flight
+    u32x4 mask_raw[2];
     // wave-uniform facts about the key block whose tiles are in flight
-    int kb_nxt, pk_nxt[NH], pm_nxt, pb_nxt;
+    int ent_nxt, pk_nxt[NH], pm_nxt, pb_nxt;
 
     // K tile: copied global -> LDS without passing through registers.  One instruction moves 1 KiB
     // (eight 128-byte rows); lane l supplies the 16-byte chunk that belongs at position l of that KiB,
-    // which is where the XOR swizzle of the chunk index is applied.  Wave w copies rows 32 w .. 32 w + 31.
+    // which is where the XOR swizzle of the chunk index is applied.  Wave w of W copies rows (64 / W) w .. (64 / W) (w + 1) - 1.
     auto copy_k = [&]() {
 #pragma unroll
       for (int h = 0; h < NH; ++h) {
         const int64_t pk = pk_nxt[h];
         if (pk >= 0) {
-          const char *kp = static_cast<const char *>(a.k) + pk * kBlockBytes;
+          // row r0 + lane / 8 of the block, chunk (lane % 8) ^ (row % 8); r0 is a multiple of 8
+          const uint32_t lane_off = (lane >> 3) * 128 + (((lane & 7) ^ ((lane >> 3) & 7)) << 4);
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int r0 = 32 * wave + 8 * i;
-            const int r = r0 + (lane >> 3);
-            const char *src = kp + r * 128 + (((lane & 7) ^ (r & 7)) << 4);
-            copy_1k_to_lds(src, lds_k + h * kBlockBytes + r0 * 128);
+          for (int i = 0; i < 4 / G; ++i) {
+            const int r0 = (32 / G) * wave + 8 * i;
+            const char *kp = static_cast<const char *>(a.k) + pk * kBlockBytes + r0 * 128;
+            copy_1k_to_lds(kp, lane_off, lds_k + h * kBlockBytes + r0 * 128);
           }
         } else {
           // inactive slice: zeros
 #pragma unroll
-          for (int i = 0; i < 4; ++i)
-            *reinterpret_cast<u32x4 *>(lds_k + h * kBlockBytes + (i * kFwdThreads + tid) * 16) = u32x4{0u, 0u, 0u, 0u};
+          for (int i = 0; i < 4 / G; ++i)
+            *reinterpret_cast<u32x4 *>(lds_k + h * kBlockBytes + (i * kThreads + tid) * 16) = u32x4{0u, 0u, 0u, 0u};
         }
       }
     };
 
     // facts and V tile of one key block
-    auto fetch_v = [&](const KeyIndices<NH, NHV> &kx) {
-      kb_nxt = first_lane(kx.kb);
+    auto fetch_v = [&](const AttnFwdRecord &r) {
+      ent_nxt = r.entry;
 #pragma unroll
       for (int h = 0; h < NH; ++h) {
-        pk_nxt[h] = first_lane(kx.pk[h]);
+        pk_nxt[h] = r.pk[h];
         if (pk_nxt[h] >= a.n_k_blocks) pk_nxt[h] = -1;
       }
-      pm_nxt = first_lane(kx.pm);
+      pm_nxt = a.mask ? ((wave >> 1) ? r.pm[1] : r.pm[0]) : -1;
       if (pm_nxt >= a.n_mask_blocks) pm_nxt = -1;
-      pb_nxt = first_lane(kx.pb);
+      pb_nxt = a.bias ? ((wave >> 1) ? r.pb[1] : r.pb[0]) : -1;
       if (pb_nxt >= a.n_bias_blocks) pb_nxt = -1;
 #pragma unroll
       for (int h = 0; h < NHV; ++h) {
-        const int64_t pv = first_lane(kx.pv[h]);
+        const int64_t pv = r.pv[h];
         const bool valid = pv >= 0 && pv < a.n_v_blocks;
         const char *vp = static_cast<const char *>(a.v) + (valid ? pv : 0) * kBlockBytes;
+        // thread tid stages rows 2 jp, 2 jp + 1 (jp = 16 G t + tid / 8), columns 8 (tid % 8) .. + 7
+        const uint32_t voff = (uint32_t)(tid >> 3) * 256u + (uint32_t)(tid & 7) * 16u;
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
-          const int q = t * kFwdThreads + tid;
-          const int ro = q & 7, jp = q >> 3;
+        for (int t = 0; t < 2 / G; ++t) {
           vr[h][2 * t] = u32x4{0u, 0u, 0u, 0u};
           vr[h][2 * t + 1] = u32x4{0u, 0u, 0u, 0u};
           if (valid) {
-            vr[h][2 * t] = *reinterpret_cast<const u32x4 *>(vp + (2 * jp) * 128 + ro * 16);
-            vr[h][2 * t + 1] = *reinterpret_cast<const u32x4 *>(vp + (2 * jp + 1) * 128 + ro * 16);
+            vr[h][2 * t] = load16(vp + 4096 * G * t, voff);
+            vr[h][2 * t + 1] = load16(vp + 4096 * G * t + 128, voff);
           }
         }
       }
     };
 
-    // bytes j = 32 jb + 8 q + 4 kg .. + 3 of mask row qi: dword 16 qi + 8 jb + 2 q + kg
+    // Mask words of the tile: lane (li, kg) needs bytes j = 32 jb + 8 q + 4 kg .. + 3 of mask row qi, that is
+    // dword 8 jb + 2 q + kg of the row, as word 4 jb + q.  It loads the 32 bytes [32 kg, 32 kg + 32) of the
+    // row (two 16-byte loads; the wave reads 2 KiB contiguously) and trades every other dword with lane
+    // (li, 1 - kg): one swap of the upper half of a register with the lower half of another per q.
     auto fetch_mask = [&]() {
       if (pm_nxt >= 0) {
-        const uint32_t *mp =
-            static_cast<const uint32_t *>(a.mask) + (int64_t)pm_nxt * (kSbs * kSbs / 4) + qi * 16 + kg;
-#pragma unroll
-        for (int w = 0; w < 8; ++w) mask_nxt[w] = mp[2 * w];
+        const char *mp = static_cast<const char *>(a.mask) + (int64_t)pm_nxt * (kSbs * kSbs);
+        const uint32_t moff = (uint32_t)qi * 64u + (uint32_t)kg * 32u;
+        mask_raw[0] = load16(mp, moff);
+        mask_raw[1] = load16(mp + 16, moff);
       }
+    };
+    auto mask_word = [&](int w) -> uint32_t {
+      // w = 4 jb + q: after the swap of (dword 2q, dword 2q + 1) the first holds the word of jb = 0, the second of jb = 1
+      const int q = w & 3;
+      const u32x2 sw = __builtin_amdgcn_permlane32_swap(mask_raw[q >> 1][2 * (q & 1)], mask_raw[q >> 1][2 * (q & 1) + 1],
+                                                        false, false);
+      return sw[w >> 2];
     };
 
     auto clamp_e = [&](int e) { return e < k_end ? e : k_end - 1; };
 
-    // prologue of the three-stage index pipeline
-    KeyIndices<NH, NHV> kx_nxt;
-    int kbv_nn;
+    // The record of a list entry (key block, packed indices of its K / V / mask / bias blocks) is read with
+    // scalar loads two iterations before its tile is used: r_next is the record of the tile after the one in flight.
+    AttnFwdRecord r_next;
     {
-      const int kb0 = a.key_indices[as_vector(k_begin)];
-      const int kb1 = a.key_indices[as_vector(clamp_e(k_begin + 1))];
-      kbv_nn = a.key_indices[as_vector(clamp_e(k_begin + 2))];
-      const KeyIndices<NH, NHV> kx0 = load_key_indices<NH, NHV>(a, b, row, kb0);
-      kx_nxt = load_key_indices<NH, NHV>(a, b, row, kb1);
-      fetch_v(kx0);
+      const AttnFwdRecord r0 = recs[k_begin];
+      r_next = recs[clamp_e(k_begin + 1)];
+      fetch_v(r0);
       copy_k();
       fetch_mask();
     }
 
     for (int e = k_begin; e < k_end; ++e) {
+      BSA_PROBE(0);
+      // issued first: the wait for the LDS writes below, which the barrier needs anyway, covers it
+      const AttnFwdRecord r_after = recs[clamp_e(e + 2)];
       // ---- V tile e: registers -> LDS as (j, j+1) pairs; the K tile of e has been copied by now ----
 #pragma unroll
       for (int h = 0; h < NHV; ++h)
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
-          const int q = t * kFwdThreads + tid;
+        for (int t = 0; t < 2 / G; ++t) {
+          const int q = t * kThreads + tid;
           const int ro = q & 7, jp = q >> 3;
           const u32x4 ev = vr[h][2 * t], od = vr[h][2 * t + 1];
           u32x4 lo, hi;
@@ -294,52 +308,48 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
           *reinterpret_cast<u32x4 *>(prow + pair_col_offset(ro * 8 + 4)) = hi;
         }
       const bool mask_on = pm_nxt >= 0;
-      const int kb = kb_nxt;
+      const int kb = ent_nxt & 0x0fffffff;
+      const bool mine = has_q && (G == 1 || ((ent_nxt >> my_bit) & 1));
       const int64_t pb = pb_nxt;
-      // mask words of tile e -> one bit per element (bit 4 w + t set: element masked); frees the word registers
+      // mask words of tile e (bytes are 0 or 1) -> one bit per element, which frees the word registers:
+      // bit 8 t + w is byte t of word w, the mask of score 4 w + t
       uint32_t mbits = 0;
       if (mask_on) {
 #pragma unroll
-        for (int w = 0; w < 8; ++w) {
-          // bit 7 of a byte of z is set where the mask byte is zero (exact per byte: no borrow crosses bytes)
-          const uint32_t x = mask_nxt[w];
-          const uint32_t z = ~(((x & 0x7f7f7f7fu) + 0x7f7f7f7fu) | x) & 0x80808080u;
-          // gather bits 7, 15, 23, 31 into a nibble
-          const uint32_t nib = ((z >> 7) * 0x00204081u) >> 21 & 0xfu;
-          mbits |= (nib ^ 0xfu) << (4 * w);
-        }
+        for (int w = 0; w < 8; ++w) mbits |= mask_word(w) << w;
       }
       // every outstanding copy of this wave (the K rows it moved) has to be in LDS before the barrier:
       // s_waitcnt vmcnt(0), other counters untouched
       __builtin_amdgcn_s_waitcnt(0x0F70);
+      BSA_PROBE(1);
       __syncthreads();
+      BSA_PROBE(2);
 
       // ---- prefetch: V tile of e+1, packed indices of e+2, key index of e+3 ----
       const bool more = e + 1 < k_end;
       if (more) {
-        fetch_v(kx_nxt);
+        fetch_v(r_next);
         fetch_mask();
       }
-      kx_nxt = load_key_indices<NH, NHV>(a, b, row, kbv_nn);
-      kbv_nn = a.key_indices[as_vector(clamp_e(e + 3))];
+      r_next = r_after;
 
       // A tile in which every score of this wave's 32 rows is masked changes nothing: m stays, alpha is 1,
       // every p is 0.  Such a tile is only fetched, not computed.
-      bool live = true;
-      if (mask_on) live = __any(mbits != 0xffffffffu);
+      bool live = mine;
+      if (mask_on && live) live = __any(mbits != 0xffffffffu);
       if (causal) {
-        const int q_last = (int)qb * kSbs + 32 * wave + 31, q_first = q_last - 31;
+        const int q_last = (int)qb * kSbs + 32 * (wave & 1) + 31, q_first = q_last - 31;
         if (kb * kSbs > q_last || q_first >= seq_len || kb * kSbs >= seq_len) live = false;
       }
 
       // ---- S^T = K Q^T ----
       // Fragments are read from LDS in batches of four, one batch ahead of the MFMAs that consume them.
       f32x16 sacc[2];
-#pragma unroll
-      for (int jb = 0; jb < 2; ++jb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) sacc[jb][r] = 0.f;
       if (live) {
+#pragma unroll
+        for (int jb = 0; jb < 2; ++jb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) sacc[jb][r] = 0.f;
         constexpr int kBatches = NH * 2;  // batch g: head slice g / 2, k steps 2 (g % 2) and 2 (g % 2) + 1, both key halves
         u32x4 kf[2][4];
         auto read_batch = [&](u32x4 (&dst)[4], int g) {
@@ -366,7 +376,9 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
       }
 
       // both waves are done with the K tile of e: start the copy of the K tile of e+1 into its place
+      BSA_PROBE(3);
       __syncthreads();
+      BSA_PROBE(4);
       if (more) copy_k();
 
       if (live) {
@@ -389,22 +401,33 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
       __builtin_amdgcn_sched_barrier(0);
 
       // ---- scores: scale, bias, causal predicate, mask ----
+      // sv holds the scores up to the positive factor cc: the raw dot products (cc = scale * log2 e), or, with
+      // a bias, the finished log2-domain scores (cc = 1).  The factor is applied inside the exponential.
       float sv[32];
+      float cc = qk_scale;
 #pragma unroll
       for (int jb = 0; jb < 2; ++jb)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) sv[16 * jb + r] = sacc[jb][r] * qk_scale;
+        for (int r = 0; r < 16; ++r) sv[16 * jb + r] = sacc[jb][r];
       if (pb >= 0) {
         // bias elements j = 32 jb + 8 q + 4 kg .. + 3 of row qi
-        const char *bp = static_cast<const char *>(a.bias) + pb * kBlockBytes + qi * 128 + kg * 8;
+        const char *bp0 = static_cast<const char *>(a.bias) + pb * kBlockBytes;
+        const uint32_t boff = (uint32_t)qi * 128u + (uint32_t)kg * 8u;
 #pragma unroll
-        for (int w = 0; w < 8; ++w) {
-          const u32x2 bw = *reinterpret_cast<const u32x2 *>(bp + 16 * w);
-          sv[4 * w + 0] += Tr::widen((uint16_t)(bw[0] & 0xffffu)) * kLog2e;
-          sv[4 * w + 1] += Tr::widen((uint16_t)(bw[0] >> 16)) * kLog2e;
-          sv[4 * w + 2] += Tr::widen((uint16_t)(bw[1] & 0xffffu)) * kLog2e;
-          sv[4 * w + 3] += Tr::widen((uint16_t)(bw[1] >> 16)) * kLog2e;
+        for (int w0 = 0; w0 < 8; w0 += 2) {
+          u32x2 bw[2];
+#pragma unroll
+          for (int w = 0; w < 2; ++w) bw[w] = *reinterpret_cast<const u32x2 *>(bp0 + 16 * (w0 + w) + boff);
+#pragma unroll
+          for (int w = 0; w < 2; ++w) {
+            float *d = sv + 4 * (w0 + w);
+            d[0] = d[0] * qk_scale + Tr::widen((uint16_t)(bw[w][0] & 0xffffu)) * kLog2e;
+            d[1] = d[1] * qk_scale + Tr::widen((uint16_t)(bw[w][0] >> 16)) * kLog2e;
+            d[2] = d[2] * qk_scale + Tr::widen((uint16_t)(bw[w][1] & 0xffffu)) * kLog2e;
+            d[3] = d[3] * qk_scale + Tr::widen((uint16_t)(bw[w][1] >> 16)) * kLog2e;
+          }
         }
+        cc = 1.f;
       }
       if (causal) {
         const int kbase = kb * kSbs + 4 * kg;
@@ -414,14 +437,14 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
 #pragma unroll
           for (int t = 0; t < 4; ++t) {
             const int kpos = kbase + 8 * w + t;
-            if (kpos > qpos || row_off || kpos >= seq_len) sv[4 * w + t] = -INFINITY;
+            sv[4 * w + t] = (kpos > qpos || row_off || kpos >= seq_len) ? -INFINITY : sv[4 * w + t];
           }
       }
       if (mask_on) {
         // most blocks of a mask mask nothing: one test for the wave skips the selects
         if (__any(mbits != 0)) {
 #pragma unroll
-          for (int x = 0; x < 32; ++x) sv[x] = ((mbits >> x) & 1u) ? -INFINITY : sv[x];
+          for (int x = 0; x < 32; ++x) sv[x] = ((mbits >> (8 * (x & 3) + (x >> 2))) & 1u) ? -INFINITY : sv[x];
         }
       }
 
@@ -429,21 +452,34 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
       float m_blk = sv[0];
 #pragma unroll
       for (int x = 1; x < 32; ++x) m_blk = fmaxf(m_blk, sv[x]);
-      m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 32));
-      const float m_new = fmaxf(m_i, m_blk);
-      const bool both_ninf = (m_i == -INFINITY) && (m_new == -INFINITY);
-      const float alpha = both_ninf ? 1.f : __builtin_amdgcn_exp2f(m_i - m_new);
-      // with m_new == -inf every score of the row is -inf (or NaN): subtracting 0 instead keeps p = 0
-      const float m_sub = (m_new == -INFINITY) ? 0.f : m_new;
+      m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 32)) * cc;
+      // The reference maximum m_i of the exponentials only follows the running maximum when that has grown by
+      // more than kRescaleStep since the last update (for some row of the wave): in between, probabilities may
+      // exceed 1 (by at most 2^kRescaleStep) and the accumulators need no rescaling.  o and lse do not depend on
+      // the reference maximum.  -inf - -inf is NaN and compares false: a row without a finite score keeps -inf.
+      const float m_cand = fmaxf(m_i, m_blk);
+      if (__any((m_cand - m_i) > kRescaleStep)) {
+        const bool both_ninf = (m_i == -INFINITY) && (m_cand == -INFINITY);
+        const float alpha = both_ninf ? 1.f : __builtin_amdgcn_exp2f(m_i - m_cand);
+        m_i = m_cand;
+        l_i *= alpha;
+#pragma unroll
+        for (int h = 0; h < NHV; ++h)
+#pragma unroll
+          for (int db = 0; db < 2; ++db)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) oacc[h][db][r] *= alpha;
+      }
+      // with m_i == -inf every score of the row so far is -inf (or NaN): subtracting 0 instead keeps p = 0
+      const float m_sub = (m_i == -INFINITY) ? 0.f : m_i;
       float sum = 0.f;
 #pragma unroll
       for (int x = 0; x < 32; ++x) {
-        sv[x] = __builtin_amdgcn_exp2f(sv[x] - m_sub);
+        sv[x] = __builtin_amdgcn_exp2f(fmaf(sv[x], cc, -m_sub));
         sum += sv[x];
       }
       sum += __shfl_xor(sum, 32);
-      l_i = l_i * alpha + sum;
-      m_i = m_new;
+      l_i += sum;
 
       u32x4 pf[2][2];
 #pragma unroll
@@ -454,16 +490,7 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
           for (int t = 0; t < 4; ++t)
             pf[jb][u][t] = Tr::pack2(sv[16 * jb + 8 * u + 2 * t], sv[16 * jb + 8 * u + 2 * t + 1]);
 
-      // ---- O^T = alpha O^T + V^T P^T ----
-      // once the running maximum has settled alpha is 1 for every row of the wave
-      if (__any(alpha != 1.f)) {
-#pragma unroll
-        for (int h = 0; h < NHV; ++h)
-#pragma unroll
-          for (int db = 0; db < 2; ++db)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) oacc[h][db][r] *= alpha;
-      }
+      // ---- O^T += V^T P^T ----
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int g = 0; g < kVBatches; ++g) {
@@ -475,11 +502,15 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
         __builtin_amdgcn_sched_barrier(0);
       }
       }  // live
+      BSA_PROBE(5);
       __syncthreads();
+      BSA_PROBE(6);
     }
   }
 
+  BSA_PROBE_FLUSH(blockIdx.x * 2 * G + wave, lane);
   // ---- epilogue: O = O^T^T / l, lse = m + log2(l) ----
+  if (!has_q) return;
 #pragma unroll
   for (int h = 0; h < NHV; ++h) {
     const int64_t po = a.pidx_o[row * NHV + h];
@@ -501,30 +532,78 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
   if (kg == 0) a.lse[row * kSbs + qi] = (l_i != 0.f) ? m_i + log2f(l_i) : -INFINITY;
 }
 
-template <typename Tr, int NH, int NHV>
+// One workgroup per group of query blocks: expands the group's list entries into records.
+__global__ __launch_bounds__(64) void attn_fwd_records_kernel(bsa_attn_args a, const int32_t *entries,
+                                                              AttnFwdRecord *records) {
+  const int64_t grp = blockIdx.x;
+  const int G = a.group_size;
+  const int64_t groups_per_batch = (a.nq + G - 1) / G;
+  const int64_t b = grp / groups_per_batch, q0 = (grp % groups_per_batch) * G;
+  const int begin = a.group_offsets[grp], end = a.group_offsets[grp + 1];
+  for (int e = begin + (int)threadIdx.x; e < end; e += 64) {
+    const int32_t ent = entries[e];
+    const int64_t kb = ent & 0x0fffffff;
+    AttnFwdRecord r;
+    r.entry = ent;
+    for (int h = 0; h < 2; ++h) {
+      r.pk[h] = h < a.nh ? (int32_t)a.pidx_k[(b * a.nk + kb) * a.nh + h] : -1;
+      r.pv[h] = h < a.nhv ? (int32_t)a.pidx_v[(b * a.nk + kb) * a.nhv + h] : -1;
+    }
+    for (int g = 0; g < 2; ++g) {
+      const int64_t qb = q0 + g;
+      const bool has = g < G && qb < a.nq && ((ent >> (28 + g)) & 1);
+      const int64_t pair = (b * a.nq + qb) * a.nk + kb;
+      r.pm[g] = has && a.pidx_mask ? (int32_t)a.pidx_mask[pair] : -1;
+      r.pb[g] = has && a.pidx_bias ? (int32_t)a.pidx_bias[pair] : -1;
+    }
+    for (int i = 0; i < 7; ++i) r.pad[i] = 0;
+    records[e] = r;
+  }
+}
+
+template <typename Tr, int NH, int NHV, int G>
 int launch_fwd(const bsa_attn_args &a, hipStream_t s) {
-  const int64_t rows = a.B * a.nq;
-  if (rows == 0) return BSA_OK;
-  attn_fwd_mfma_kernel<Tr, NH, NHV><<<(unsigned)(cdiv(rows, 8) * 8), kFwdThreads, 0, s>>>(a);
+  const int64_t groups = a.B * cdiv(a.nq, G);
+  if (groups == 0) return BSA_OK;
+  attn_fwd_mfma_kernel<Tr, NH, NHV, G><<<(unsigned)(cdiv(groups, 8) * 8), kFwdThreads * G, 0, s>>>(a);
   return check_launch("attn_fwd_mfma_kernel");
+}
+
+template <typename Tr, int G>
+int dispatch_fwd_g(const bsa_attn_args &a, hipStream_t s) {
+  if (a.nh == 1 && a.nhv == 1) return launch_fwd<Tr, 1, 1, G>(a, s);
+  if (a.nh == 2 && a.nhv == 2) return launch_fwd<Tr, 2, 2, G>(a, s);
+  if (a.nh == 1 && a.nhv == 2) return launch_fwd<Tr, 1, 2, G>(a, s);
+  if (a.nh == 2 && a.nhv == 1) return launch_fwd<Tr, 2, 1, G>(a, s);
+  return 1;
 }
 
 template <typename Tr>
 int dispatch_fwd(const bsa_attn_args &a, hipStream_t s) {
-  if (a.nh == 1 && a.nhv == 1) return launch_fwd<Tr, 1, 1>(a, s);
-  if (a.nh == 2 && a.nhv == 2) return launch_fwd<Tr, 2, 2>(a, s);
-  if (a.nh == 1 && a.nhv == 2) return launch_fwd<Tr, 1, 2>(a, s);
-  if (a.nh == 2 && a.nhv == 1) return launch_fwd<Tr, 2, 1>(a, s);
-  return 1;
+  if (a.group_size == 2) return dispatch_fwd_g<Tr, 2>(a, s);
+  return dispatch_fwd_g<Tr, 1>(a, s);
 }
 
 }  // namespace
 
 int attn_fwd_mfma(const bsa_attn_args &a, hipStream_t s) {
   if (a.sbs != kSbs || (a.dtype != BSA_BF16 && a.dtype != BSA_F16)) return 1;
-  // a query row without key_indices (an attention layout without active blocks) still writes o and lse
-  if (a.key_indices == nullptr && a.B * a.nq > 0) return 1;
+  // the kernels take the row maximum before the scale is applied
+  if (!(a.scale > 0.f) || a.scale > 3.0e38f) return 1;
+  // the matrix-core kernels walk the grouped record lists; without them the generic kernels run
+  if (a.group_offsets == nullptr || (a.group_size != 1 && a.group_size != 2)) return 1;
+  if (a.group_records == nullptr) {
+    // no list entry at all: every query block still writes o = 0 and lse = -inf
+    // (the caller passes NULL for an empty record array; the offsets then are all zero)
+  }
   return a.dtype == BSA_BF16 ? dispatch_fwd<MBf16>(a, s) : dispatch_fwd<MF16>(a, s);
+}
+
+int attn_fwd_records(const bsa_attn_args &a, const int32_t *entries, int32_t *records, hipStream_t s) {
+  const int64_t groups = a.B * cdiv(a.nq, a.group_size);
+  if (groups == 0) return BSA_OK;
+  attn_fwd_records_kernel<<<(unsigned)groups, 64, 0, s>>>(a, entries, reinterpret_cast<AttnFwdRecord *>(records));
+  return check_launch("attn_fwd_records_kernel");
 }
 
 int attn_bwd_mfma(const bsa_attn_args &, hipStream_t) { return 1; }

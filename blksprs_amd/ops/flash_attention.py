@@ -25,6 +25,11 @@ from ..utils.validation import (ensure_contiguous, validate_binary, validate_con
                                 validate_sparsity_block_size, validate_sparsity_layout)
 
 
+# Build the key lists of query block pairs (see _build_group_key_lists).  Off: the forward kernel walks one
+# list per query block, with the same results.
+_PAIR_QUERY_BLOCKS = True
+
+
 def _select_segmented_index_dtype(n_active_blocks: int, n_blocks_col: int) -> torch.dtype:
     """int32 unless the number of active blocks or the largest column id needs more."""
     if n_active_blocks > INT32_INDEX_MAX or n_blocks_col - 1 > INT32_INDEX_MAX:
@@ -54,6 +59,41 @@ def _build_segmented_indices(attention_layout: Tensor, n_batches: int, n_blocks_
     if dtype != torch.int32:
         indices, offsets = indices.to(dtype), offsets.to(dtype)
     return as_base_tensor(indices), as_base_tensor(offsets), info.max_per_row
+
+
+def _build_group_lists(attention_layout: Tensor, n_batches: int, n_blocks_row: int,
+                       n_blocks_col: int) -> tuple[Tensor, Tensor, int]:
+    """The attention layout as lists over groups of neighbouring query blocks: ``(offsets, entries, group_size)``.
+
+    With ``group_size == 2`` a group is the pair of query blocks ``(2p, 2p+1)`` and its list the union of their
+    key lists; with 1 it is one query block.  ``entries`` holds ``key_block | active_for_first << 28 |
+    active_for_second << 29`` (int32, key blocks ascending), ``offsets`` has ``B * ceil(rows / group_size) + 1``
+    int32 entries.  The forward kernel fetches a K / V block once per group; pairs are used when the two lists
+    of a pair overlap enough for that to save fetches.  These lists have no counterpart in the reference.
+    """
+    device = attention_layout.device
+    active = attention_layout.reshape(n_batches, n_blocks_row, n_blocks_col) != 0
+    padded = active
+    if n_blocks_row % 2:
+        padded = torch.cat([active, torch.zeros_like(active[:, :1])], dim=1)
+    even, odd = padded[:, 0::2], padded[:, 1::2]
+    union = even | odd
+    n_active, n_union = int(active.sum()), int(union.sum())
+    # a pair's workgroup is busy for the union of the two lists, a single block's for its own list
+    group_size = 2 if _PAIR_QUERY_BLOCKS and n_active >= 1.25 * n_union else 1
+    if group_size == 2:
+        where = torch.nonzero(union)
+        flags = even[where[:, 0], where[:, 1], where[:, 2]].to(torch.int32) \
+            | (odd[where[:, 0], where[:, 1], where[:, 2]].to(torch.int32) << 1)
+        counts = union.sum(dim=-1).reshape(-1)
+    else:
+        where = torch.nonzero(active)
+        flags = torch.ones(where.size(0), dtype=torch.int32, device=device)
+        counts = active.sum(dim=-1).reshape(-1)
+    entries = (where[:, 2].to(torch.int32) | (flags << 28)).contiguous()
+    offsets = torch.zeros(counts.numel() + 1, dtype=torch.int32, device=device)
+    offsets[1:] = torch.cumsum(counts, dim=0).to(torch.int32)
+    return as_base_tensor(offsets), as_base_tensor(entries), group_size
 
 
 def flash_attention_build_layout_cache(attention_layout: Tensor,
@@ -207,6 +247,27 @@ def _as_index(t: Tensor | None, dtype: torch.dtype) -> Tensor | None:
     return t.to(dtype)
 
 
+def _build_forward_records(layout_cache: dict, attention_layout: Tensor, n_batches: int, nq: int, nk: int,
+                           nh: int, nhv: int) -> None:
+    """Adds ``group_offsets`` / ``group_records`` / ``group_size`` (the lists the matrix-core forward kernel
+    walks) to a layout cache that already holds the packed indices."""
+    offsets, entries, group_size = _build_group_lists(attention_layout, n_batches, nq, nk)
+    records = torch.zeros(entries.numel() * _capi.ATTN_RECORD_INTS, dtype=torch.int32, device=entries.device)
+    a = _capi.AttnArgs()
+    a.B, a.nq, a.nk, a.nh, a.nhv = n_batches, nq, nk, nh, nhv
+    a.pidx_k, a.pidx_v = _capi.ptr(layout_cache["packed_indices_k"]), _capi.ptr(layout_cache["packed_indices_v"])
+    if "packed_indices_mask" in layout_cache:
+        a.pidx_mask = _capi.ptr(layout_cache["packed_indices_mask"])
+    if "packed_indices_bias" in layout_cache:
+        a.pidx_bias = _capi.ptr(layout_cache["packed_indices_bias"])
+    a.group_offsets, a.group_size = offsets.data_ptr(), group_size
+    with torch.cuda.device(entries.device):
+        _capi.check(_capi.load().bsa_attn_fwd_records(ctypes.byref(a), _capi.ptr(entries), _capi.ptr(records),
+                                                      _capi.stream(entries.device)), "bsa_attn_fwd_records")
+    layout_cache["group_offsets"], layout_cache["group_records"] = offsets, as_base_tensor(records)
+    layout_cache["group_size"] = group_size
+
+
 class _Meta:
     """Everything the kernels need besides the differentiable tensors."""
 
@@ -228,6 +289,10 @@ def _fill_args(meta: "_Meta", q, k, v, bias) -> _capi.AttnArgs:
     a.key_indices = _capi.ptr(c["key_indices_i32"])
     a.query_offsets = c["query_offsets_i32"].data_ptr()
     a.query_indices = _capi.ptr(c["query_indices_i32"])
+    if "group_offsets" in c:
+        a.group_offsets = c["group_offsets"].data_ptr()
+        a.group_records = _capi.ptr(c["group_records"])
+        a.group_size = c["group_size"]
     if meta.mask is not None:
         a.mask, a.pidx_mask = _capi.ptr(meta.mask), _capi.ptr(c["packed_indices_mask"])
         a.n_mask_blocks = meta.mask.size(0)
@@ -414,6 +479,10 @@ def flash_attention(q: BlksprsTensor, sparsity_layout_q: Tensor,
     if "key_offsets_i32" not in layout_cache:
         for name in ("key_offsets", "key_indices", "query_offsets", "query_indices"):
             layout_cache[name + "_i32"] = _as_index(layout_cache[name], torch.int32)
+        if (n_seq_blocks_k < (1 << 28) and layout_cache["key_indices"].numel() < INT32_INDEX_MAX
+                and n_head_blocks_qk <= 2 and n_head_blocks_v <= 2 and sparsity_block_size == 64):
+            _build_forward_records(layout_cache, attention_layout, int(n_batches), int(n_seq_blocks_q),
+                                   int(n_seq_blocks_k), int(n_head_blocks_qk), int(n_head_blocks_v))
         finalize_layout_cache(layout_cache)
 
     meta = _Meta()

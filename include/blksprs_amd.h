@@ -208,7 +208,7 @@ typedef struct bsa_attn_args {
   void *dq, *dk, *dv; /* backward outputs (dtype) */
   float *lse;         /* forward output / backward input */
   float *delta;       /* backward scratch: rowsum(o * d_o) */
-  const void *mask;   /* compressed mask blocks, element type mask_kind */
+  const void *mask;   /* compressed mask blocks, one byte per element: 1 = masked, 0 = kept */
   const void *bias;   /* compressed bias blocks (dtype) */
   float *dbias;       /* backward: fp32 (n_bias_blocks, sbs, sbs) or NULL */
   const int64_t *pidx_q, *pidx_k, *pidx_v, *pidx_o, *pidx_mask, *pidx_bias;
@@ -219,9 +219,30 @@ typedef struct bsa_attn_args {
   int64_t n_q_blocks, n_k_blocks, n_v_blocks, n_o_blocks, n_mask_blocks, n_bias_blocks;
   int32_t sbs;
   int32_t dtype;     /* BSA_F32 / BSA_F16 / BSA_BF16 */
-  int32_t mask_kind; /* 0 = none, 1 = one byte per element (bool/uint8), 2 = same dtype as q */
+  int32_t mask_kind; /* 0 = none, 1 = one byte per element (0 or 1) */
   float scale;
+  /* Optional, forward only (group_size 0: not used, the generic kernels run): the attention layout as lists
+   * over groups of group_size (1 or 2) neighbouring query blocks.  group_offsets has
+   * B * ceil(nq / group_size) + 1 entries; group_records holds BSA_ATTN_RECORD_INTS int32 per list entry, filled
+   * by bsa_attn_fwd_records.  With group_size 2 one workgroup fetches a K / V block once for both query blocks
+   * of a pair.  No counterpart in the reference. */
+  const int32_t *group_offsets, *group_records;
+  int32_t group_size;
 } bsa_attn_args;
+
+#define BSA_ATTN_RECORD_INTS 16
+
+/*
+ * Expands grouped list entries into the records bsa_attn_fwd walks (layout-to-LUT step, integer only).  Reads
+ * from args: B, nq, nk, nh (<= 2), nhv (<= 2), pidx_k, pidx_v, pidx_mask / pidx_bias (NULL: none),
+ * group_offsets, group_size.  group_entries[e] = key_block | active_for_first << 28 | active_for_second << 29,
+ * key blocks ascending within a group (the union of the key lists of the group's query blocks, in the order
+ * of _build_segmented_indices, blksprs/ops/flash_attention.py:1923-1950).  records receives
+ * BSA_ATTN_RECORD_INTS int32 per entry.  No counterpart in the reference: it resolves the packed indices
+ * there inside the kernel loop (blksprs/ops/flash_attention.py:1058-1175).
+ */
+int bsa_attn_fwd_records(const bsa_attn_args *args, const int32_t *group_entries, int32_t *records,
+                         bsa_stream_t stream);
 
 /*
  * o = softmax(scale * q k^T + bias, masked) v over the active key blocks of

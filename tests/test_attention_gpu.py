@@ -242,3 +242,42 @@ def test_validation_errors(device):
     import numpy as np
     out = bs.ops.flash_attention(t, lay, t, lay, t, lay, lay, sbs, scale=np.float32(0.5))
     assert out.shape == (1, sbs, sbs)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("nq,nh,nhv", [(7, 2, 2), (6, 1, 2), (5, 2, 1), (8, 1, 1)])
+def test_matrix_core_forward_odd_sequences_and_head_slice_counts(device, dtype, nq, nh, nhv):
+    _run_case(device, dtype, 64, 2, nq, 6, nh, nhv, 0.5, 70 + nq, use_mask=True, use_causal=(nq == 6))
+
+
+def test_paired_query_block_lists_give_the_same_bits_as_single_lists(device, monkeypatch):
+    """The forward kernel fetches K / V once per pair of query blocks when the cache holds the pair lists and
+    once per query block otherwise; both walk the key blocks in the same order, so the results are identical."""
+    g = torch.Generator().manual_seed(5)
+    B, nq, nk, nh, sbs = 3, 9, 11, 2, 64
+    la = orc.random_layout((B, nq, nk), 0.7, g, ensure_rows=True).to(device)
+    la[1, 4] = False  # a query block without keys
+    full = torch.ones((B, nq, nh), dtype=torch.bool, device=device)
+    fullk = torch.ones((B, nk, nh), dtype=torch.bool, device=device)
+    q = rand_blocks(B * nq * nh, sbs, torch.bfloat16, 1).to(device)
+    k = rand_blocks(B * nk * nh, sbs, torch.bfloat16, 2).to(device)
+    v = rand_blocks(B * nk * nh, sbs, torch.bfloat16, 3).to(device)
+    lmask = la.clone()
+    mask = (torch.rand((int(lmask.sum()), sbs, sbs), generator=g) < 0.5).to(device)
+    mask[::3] = True  # whole blocks masked: such tiles are fetched but not computed
+    cache = {}
+    paired = bs.ops.flash_attention(q, full, k, fullk, v, fullk, la, sbs, attention_mask=mask,
+                                    sparsity_layout_mask=lmask, layout_cache=cache)
+    assert cache["group_size"] == 2
+    entries = cache["group_records"].view(-1, 16)[:, 0]
+    assert int(((entries >> 28) & 1).sum() + ((entries >> 29) & 1).sum()) == int(la.sum())
+    import importlib
+    fa_module = importlib.import_module("blksprs_amd.ops.flash_attention")
+    monkeypatch.setattr(fa_module, "_PAIR_QUERY_BLOCKS", False)
+    plain = {}
+    single = bs.ops.flash_attention(q, full, k, fullk, v, fullk, la, sbs, attention_mask=mask,
+                                    sparsity_layout_mask=lmask, layout_cache=plain)
+    assert plain["group_size"] == 1 and plain["group_records"].size(0) == 16 * int(la.sum())
+    assert torch.equal(paired, single)
+    # the query block without keys has no output blocks
+    assert paired.size(0) == (B * nq - 1) * nh
