@@ -89,8 +89,13 @@ struct MF16 {
 
 constexpr int kSbs = 64;
 constexpr int kBlockBytes = kSbs * kSbs * 2;  // one 16-bit block
-constexpr int kFwdThreads = 128;
+constexpr int kFwdThreads = 256;
 constexpr float kRescaleStep = 8.f;  // log2 units
+
+// XOR applied to the 16-byte chunk index of K tile row r in LDS.  Two 128-byte rows span the 64 banks once, so
+// the 16 lanes a 128-bit read serves together (16 consecutive rows, one chunk each) are conflict free when
+// rows of equal parity get eight different values.
+__device__ inline int k_swizzle(int r) { return (r >> 1) & 7; }
 
 // dword offset of column c in a pair row of the (j, j+1)-packed V tile; the placement of the column
 // quads keeps both the 128-bit writes of the staging step and the 32-bit fragment reads conflict free
@@ -123,15 +128,21 @@ __device__ inline u32x4 load16(const char *base, uint32_t off) {
   return *reinterpret_cast<const u32x4 *>(base + off);
 }
 
-// G = query blocks per workgroup (1 or 2).  With G = 2 the workgroup has four waves and walks the union of
-// the key lists of two neighbouring query blocks, so that a K / V tile both of them need is fetched once;
-// bits 28 and 29 of a list entry say which of the two the key block is active for.
-template <typename Tr, int NH, int NHV, int G>
-__global__ __launch_bounds__(kFwdThreads *G, 2) void attn_fwd_mfma_kernel(bsa_attn_args a) {
-  constexpr int kThreads = kFwdThreads * G;
-  // two arrays, not one: the compiler then knows that the asynchronous K copy never touches the V tile
-  __shared__ __attribute__((aligned(1024))) char lds_k[NH * kBlockBytes];
-  __shared__ __attribute__((aligned(16))) char lds_v[NHV * kBlockBytes];
+// One workgroup (four waves) owns a PAIR of neighbouring query blocks and walks the union of their key lists,
+// so that a K / V tile both of them need is fetched once; bits 28 and 29 of a list entry say which of the
+// two the key block is active for.  Waves 0, 1 own the first query block, waves 2, 3 the second.
+//
+// The K and V tiles are double buffered in LDS: while tile e is computed from one buffer, the K tile of e+1 is
+// copied into the other and the V tile of e+1 travels through registers into it; ONE barrier per tile, at
+// its end, says both that the next tile is complete and that this one's buffer may be overwritten.
+template <typename Tr, int NH, int NHV>
+__global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_args a) {
+  constexpr int G = 2;
+  constexpr int kThreads = kFwdThreads;
+  constexpr int kKBytes = NH * kBlockBytes, kVBytes = NHV * kBlockBytes;
+  // two arrays, not one: the compiler then knows that the asynchronous K copy never touches the V tiles
+  __shared__ __attribute__((aligned(1024))) char lds_k[2 * kKBytes];
+  __shared__ __attribute__((aligned(16))) char lds_v[2 * kVBytes];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -139,7 +150,7 @@ __global__ __launch_bounds__(kFwdThreads *G, 2) void attn_fwd_mfma_kernel(bsa_at
   const int li = lane & 31, kg = lane >> 5;
   const int qi = 32 * (wave & 1) + li;  // query row inside the block
   // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2: give every XCD a contiguous
-  // range of rows, so that the query blocks in flight on one L2 share their batch entry's K and V.
+  // range of groups, so that the query blocks in flight on one L2 share their batch entry's K and V.
   const int64_t groups_per_batch = (a.nq + G - 1) / G;
   const int64_t grp = (int64_t)(blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
   if (grp >= a.B * groups_per_batch) return;
@@ -188,32 +199,32 @@ __global__ __launch_bounds__(kFwdThreads *G, 2) void attn_fwd_mfma_kernel(bsa_at
 
   BSA_PROBE_DECL;
   if (k_begin < k_end) {
-    u32x4 vr[NHV][4 / G];  // staging registers of the V tile in flight
+    u32x4 vr[NHV][2];  // staging registers of the V tile in flight
     u32x4 mask_raw[2];
     // wave-uniform facts about the key block whose tiles are in flight
-    int ent_nxt, pk_nxt[NH], pm_nxt, pb_nxt;
+    int ent_nxt, pm_nxt, pb_nxt;
 
     // K tile: copied global -> LDS without passing through registers.  One instruction moves 1 KiB
     // (eight 128-byte rows); lane l supplies the 16-byte chunk that belongs at position l of that KiB,
-    // which is where the XOR swizzle of the chunk index is applied.  Wave w of W copies rows (64 / W) w .. (64 / W) (w + 1) - 1.
-    auto copy_k = [&]() {
+    // which is where the XOR swizzle of the chunk index is applied.  Wave w copies rows 16 w .. 16 w + 15.
+    auto copy_k = [&](const AttnFwdRecord &r, int buf) {
 #pragma unroll
       for (int h = 0; h < NH; ++h) {
-        const int64_t pk = pk_nxt[h];
-        if (pk >= 0) {
-          // row r0 + lane / 8 of the block, chunk (lane % 8) ^ (row % 8); r0 is a multiple of 8
-          const uint32_t lane_off = (lane >> 3) * 128 + (((lane & 7) ^ ((lane >> 3) & 7)) << 4);
+        const int64_t pk = r.pk[h];
+        char *dst = lds_k + buf * kKBytes + h * kBlockBytes;
+        if (pk >= 0 && pk < a.n_k_blocks) {
 #pragma unroll
-          for (int i = 0; i < 4 / G; ++i) {
-            const int r0 = (32 / G) * wave + 8 * i;
+          for (int i = 0; i < 2; ++i) {
+            // row r0 + lane / 8 of the block, chunk (lane % 8) ^ k_swizzle(row); r0 is a multiple of 8
+            const int r0 = 16 * wave + 8 * i;
+            const uint32_t lane_off = (lane >> 3) * 128 + (((lane & 7) ^ k_swizzle(8 * i + (lane >> 3))) << 4);
             const char *kp = static_cast<const char *>(a.k) + pk * kBlockBytes + r0 * 128;
-            copy_1k_to_lds(kp, lane_off, lds_k + h * kBlockBytes + r0 * 128);
+            copy_1k_to_lds(kp, lane_off, dst + r0 * 128);
           }
         } else {
           // inactive slice: zeros
 #pragma unroll
-          for (int i = 0; i < 4 / G; ++i)
-            *reinterpret_cast<u32x4 *>(lds_k + h * kBlockBytes + (i * kThreads + tid) * 16) = u32x4{0u, 0u, 0u, 0u};
+          for (int i = 0; i < 2; ++i) *reinterpret_cast<u32x4 *>(dst + (i * kThreads + tid) * 16) = u32x4{0u, 0u, 0u, 0u};
         }
       }
     };
@@ -221,11 +232,6 @@ __global__ __launch_bounds__(kFwdThreads *G, 2) void attn_fwd_mfma_kernel(bsa_at
     // facts and V tile of one key block
     auto fetch_v = [&](const AttnFwdRecord &r) {
       ent_nxt = r.entry;
-#pragma unroll
-      for (int h = 0; h < NH; ++h) {
-        pk_nxt[h] = r.pk[h];
-        if (pk_nxt[h] >= a.n_k_blocks) pk_nxt[h] = -1;
-      }
       pm_nxt = a.mask ? ((wave >> 1) ? r.pm[1] : r.pm[0]) : -1;
       if (pm_nxt >= a.n_mask_blocks) pm_nxt = -1;
       pb_nxt = a.bias ? ((wave >> 1) ? r.pb[1] : r.pb[0]) : -1;
@@ -235,17 +241,35 @@ __global__ __launch_bounds__(kFwdThreads *G, 2) void attn_fwd_mfma_kernel(bsa_at
         const int64_t pv = r.pv[h];
         const bool valid = pv >= 0 && pv < a.n_v_blocks;
         const char *vp = static_cast<const char *>(a.v) + (valid ? pv : 0) * kBlockBytes;
-        // thread tid stages rows 2 jp, 2 jp + 1 (jp = 16 G t + tid / 8), columns 8 (tid % 8) .. + 7
+        // thread tid stages rows 2 jp, 2 jp + 1 (jp = tid / 8), columns 8 (tid % 8) .. + 7
         const uint32_t voff = (uint32_t)(tid >> 3) * 256u + (uint32_t)(tid & 7) * 16u;
-#pragma unroll
-        for (int t = 0; t < 2 / G; ++t) {
-          vr[h][2 * t] = u32x4{0u, 0u, 0u, 0u};
-          vr[h][2 * t + 1] = u32x4{0u, 0u, 0u, 0u};
-          if (valid) {
-            vr[h][2 * t] = load16(vp + 4096 * G * t, voff);
-            vr[h][2 * t + 1] = load16(vp + 4096 * G * t + 128, voff);
-          }
+        vr[h][0] = u32x4{0u, 0u, 0u, 0u};
+        vr[h][1] = u32x4{0u, 0u, 0u, 0u};
+        if (valid) {
+          vr[h][0] = load16(vp, voff);
+          vr[h][1] = load16(vp + 128, voff);
         }
+      }
+    };
+
+    // V tile in registers -> LDS as (j, j+1) pairs
+    auto stage_v = [&](int buf) {
+#pragma unroll
+      for (int h = 0; h < NHV; ++h) {
+        const int ro = tid & 7, jp = tid >> 3;
+        const u32x4 ev = vr[h][0], od = vr[h][1];
+        u32x4 lo, hi;
+        lo[0] = __builtin_amdgcn_perm(od[0], ev[0], 0x05040100u);
+        lo[1] = __builtin_amdgcn_perm(od[0], ev[0], 0x07060302u);
+        lo[2] = __builtin_amdgcn_perm(od[1], ev[1], 0x05040100u);
+        lo[3] = __builtin_amdgcn_perm(od[1], ev[1], 0x07060302u);
+        hi[0] = __builtin_amdgcn_perm(od[2], ev[2], 0x05040100u);
+        hi[1] = __builtin_amdgcn_perm(od[2], ev[2], 0x07060302u);
+        hi[2] = __builtin_amdgcn_perm(od[3], ev[3], 0x05040100u);
+        hi[3] = __builtin_amdgcn_perm(od[3], ev[3], 0x07060302u);
+        uint32_t *prow = reinterpret_cast<uint32_t *>(lds_v + buf * kVBytes + h * kBlockBytes) + jp * kSbs;
+        *reinterpret_cast<u32x4 *>(prow + pair_col_offset(ro * 8)) = lo;
+        *reinterpret_cast<u32x4 *>(prow + pair_col_offset(ro * 8 + 4)) = hi;
       }
     };
 
@@ -271,45 +295,48 @@ __global__ __launch_bounds__(kFwdThreads *G, 2) void attn_fwd_mfma_kernel(bsa_at
 
     auto clamp_e = [&](int e) { return e < k_end ? e : k_end - 1; };
 
-    // The record of a list entry (key block, packed indices of its K / V / mask / bias blocks) is read with
-    // scalar loads two iterations before its tile is used: r_next is the record of the tile after the one in flight.
-    AttnFwdRecord r_next;
+    // The record of a list entry (key block, packed indices of its K / V / mask / bias blocks) is read two
+    // tiles before its tile is used, by ONE vector load (field i in lane i): that load completes in order with
+    // the tile loads, so the wait at the end of a tile covers it, whereas a scalar load would put its full
+    // latency in front of the next LDS read.  rv_next is the record of the tile after the current one.
+    auto load_record = [&](int pos) -> int {
+      int v = 0;
+      if (lane < 9) v = reinterpret_cast<const int32_t *>(recs + pos)[lane];
+      return v;
+    };
+    auto unpack_record = [&](int rv) {
+      AttnFwdRecord r;
+      r.entry = __builtin_amdgcn_readlane(rv, 0);
+      r.pk[0] = __builtin_amdgcn_readlane(rv, 1);
+      r.pk[1] = __builtin_amdgcn_readlane(rv, 2);
+      r.pv[0] = __builtin_amdgcn_readlane(rv, 3);
+      r.pv[1] = __builtin_amdgcn_readlane(rv, 4);
+      r.pm[0] = __builtin_amdgcn_readlane(rv, 5);
+      r.pm[1] = __builtin_amdgcn_readlane(rv, 6);
+      r.pb[0] = __builtin_amdgcn_readlane(rv, 7);
+      r.pb[1] = __builtin_amdgcn_readlane(rv, 8);
+      return r;
+    };
+    int rv_next;
     {
-      const AttnFwdRecord r0 = recs[k_begin];
-      r_next = recs[clamp_e(k_begin + 1)];
+      const AttnFwdRecord r0 = unpack_record(load_record(k_begin));
+      rv_next = load_record(clamp_e(k_begin + 1));
       fetch_v(r0);
-      copy_k();
+      copy_k(r0, 0);
       fetch_mask();
+      stage_v(0);
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the K rows this wave copied are in LDS
+      __syncthreads();
     }
 
     for (int e = k_begin; e < k_end; ++e) {
       BSA_PROBE(0);
-      // issued first: the wait for the LDS writes below, which the barrier needs anyway, covers it
-      const AttnFwdRecord r_after = recs[clamp_e(e + 2)];
-      // ---- V tile e: registers -> LDS as (j, j+1) pairs; the K tile of e has been copied by now ----
-#pragma unroll
-      for (int h = 0; h < NHV; ++h)
-#pragma unroll
-        for (int t = 0; t < 2 / G; ++t) {
-          const int q = t * kThreads + tid;
-          const int ro = q & 7, jp = q >> 3;
-          const u32x4 ev = vr[h][2 * t], od = vr[h][2 * t + 1];
-          u32x4 lo, hi;
-          lo[0] = __builtin_amdgcn_perm(od[0], ev[0], 0x05040100u);
-          lo[1] = __builtin_amdgcn_perm(od[0], ev[0], 0x07060302u);
-          lo[2] = __builtin_amdgcn_perm(od[1], ev[1], 0x05040100u);
-          lo[3] = __builtin_amdgcn_perm(od[1], ev[1], 0x07060302u);
-          hi[0] = __builtin_amdgcn_perm(od[2], ev[2], 0x05040100u);
-          hi[1] = __builtin_amdgcn_perm(od[2], ev[2], 0x07060302u);
-          hi[2] = __builtin_amdgcn_perm(od[3], ev[3], 0x05040100u);
-          hi[3] = __builtin_amdgcn_perm(od[3], ev[3], 0x07060302u);
-          uint32_t *prow = reinterpret_cast<uint32_t *>(lds_v + h * kBlockBytes) + jp * kSbs;
-          *reinterpret_cast<u32x4 *>(prow + pair_col_offset(ro * 8)) = lo;
-          *reinterpret_cast<u32x4 *>(prow + pair_col_offset(ro * 8 + 4)) = hi;
-        }
+      const int buf = (e - k_begin) & 1;
+      const int rv_after = load_record(clamp_e(e + 2));
+      // facts of tile e, before the fetch of tile e+1 replaces them
       const bool mask_on = pm_nxt >= 0;
       const int kb = ent_nxt & 0x0fffffff;
-      const bool mine = has_q && (G == 1 || ((ent_nxt >> my_bit) & 1));
+      const bool mine = has_q && ((ent_nxt >> my_bit) & 1);
       const int64_t pb = pb_nxt;
       // mask words of tile e (bytes are 0 or 1) -> one bit per element, which frees the word registers:
       // bit 8 t + w is byte t of word w, the mask of score 4 w + t
@@ -318,20 +345,17 @@ __global__ __launch_bounds__(kFwdThreads *G, 2) void attn_fwd_mfma_kernel(bsa_at
 #pragma unroll
         for (int w = 0; w < 8; ++w) mbits |= mask_word(w) << w;
       }
-      // every outstanding copy of this wave (the K rows it moved) has to be in LDS before the barrier:
-      // s_waitcnt vmcnt(0), other counters untouched
-      __builtin_amdgcn_s_waitcnt(0x0F70);
-      BSA_PROBE(1);
-      __syncthreads();
-      BSA_PROBE(2);
 
-      // ---- prefetch: V tile of e+1, packed indices of e+2, key index of e+3 ----
+      // ---- prefetch of tile e+1: K copy into the other buffer, V and mask words into registers ----
       const bool more = e + 1 < k_end;
       if (more) {
+        const AttnFwdRecord r_next = unpack_record(rv_next);
         fetch_v(r_next);
+        copy_k(r_next, buf ^ 1);
         fetch_mask();
       }
-      r_next = r_after;
+      rv_next = rv_after;
+      BSA_PROBE(1);
 
       // A tile in which every score of this wave's 32 rows is masked changes nothing: m stays, alpha is 1,
       // every p is 0.  Such a tile is only fetched, not computed.
@@ -342,169 +366,171 @@ __global__ __launch_bounds__(kFwdThreads *G, 2) void attn_fwd_mfma_kernel(bsa_at
         if (kb * kSbs > q_last || q_first >= seq_len || kb * kSbs >= seq_len) live = false;
       }
 
-      // ---- S^T = K Q^T ----
-      // Fragments are read from LDS in batches of four, one batch ahead of the MFMAs that consume them.
-      f32x16 sacc[2];
       if (live) {
+        const char *kbuf = lds_k + buf * kKBytes;
+        const char *vbuf = lds_v + buf * kVBytes;
+        // ---- S^T = K Q^T ----
+        // Fragments are read from LDS in batches of four, one batch ahead of the MFMAs that consume them.
+        f32x16 sacc[2];
 #pragma unroll
         for (int jb = 0; jb < 2; ++jb)
 #pragma unroll
           for (int r = 0; r < 16; ++r) sacc[jb][r] = 0.f;
-        constexpr int kBatches = NH * 2;  // batch g: head slice g / 2, k steps 2 (g % 2) and 2 (g % 2) + 1, both key halves
-        u32x4 kf[2][4];
-        auto read_batch = [&](u32x4 (&dst)[4], int g) {
+        {
+          constexpr int kBatches = NH * 2;  // batch g: head slice g / 2, k steps 2 (g % 2), 2 (g % 2) + 1, both key halves
+          u32x4 kf[2][4];
+          auto read_batch = [&](u32x4 (&dst)[4], int g) {
 #pragma unroll
-          for (int t = 0; t < 4; ++t) {
-            const int h = g >> 1, st = 2 * (g & 1) + (t >> 1), jb = t & 1;
-            const int rj = 32 * jb + li;
-            dst[t] = *reinterpret_cast<const u32x4 *>(lds_k + h * kBlockBytes + rj * 128 +
-                                                      (((2 * st + kg) ^ (rj & 7)) << 4));
+            for (int t = 0; t < 4; ++t) {
+              const int h = g >> 1, st = 2 * (g & 1) + (t >> 1), jb = t & 1;
+              const int rj = 32 * jb + li;
+              dst[t] = *reinterpret_cast<const u32x4 *>(kbuf + h * kBlockBytes + rj * 128 +
+                                                        (((2 * st + kg) ^ k_swizzle(rj)) << 4));
+            }
+          };
+          read_batch(kf[0], 0);
+#pragma unroll
+          for (int g = 0; g < kBatches; ++g) {
+            if (g + 1 < kBatches) read_batch(kf[(g + 1) & 1], g + 1);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+              const int h = g >> 1, st = 2 * (g & 1) + (t >> 1), jb = t & 1;
+              sacc[jb] = Tr::mfma(kf[g & 1][t], qf[h][st], sacc[jb]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        }
+        BSA_PROBE(2);
+
+        // first batch of V fragments: in flight while the softmax runs
+        constexpr int kVBatches = NHV * 4;  // batch g: head slice g / 4, key quarter g % 4, both column halves
+        u32x4 vf[2][2];
+        auto read_vbatch = [&](u32x4 (&dst)[2], int g) {
+          const int h = g >> 2, jq = g & 3;
+#pragma unroll
+          for (int db = 0; db < 2; ++db) {
+            const uint32_t *vp = reinterpret_cast<const uint32_t *>(vbuf + h * kBlockBytes) +
+                                 pair_col_offset(32 * db + li) + (2 * kg + 8 * jq) * kSbs;
+            dst[db][0] = vp[0];
+            dst[db][1] = vp[kSbs];
+            dst[db][2] = vp[4 * kSbs];
+            dst[db][3] = vp[5 * kSbs];
           }
         };
-        read_batch(kf[0], 0);
-#pragma unroll
-        for (int g = 0; g < kBatches; ++g) {
-          if (g + 1 < kBatches) read_batch(kf[(g + 1) & 1], g + 1);
-          __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-          for (int t = 0; t < 4; ++t) {
-            const int h = g >> 1, st = 2 * (g & 1) + (t >> 1), jb = t & 1;
-            sacc[jb] = Tr::mfma(kf[g & 1][t], qf[h][st], sacc[jb]);
-          }
-          __builtin_amdgcn_sched_barrier(0);
-        }
-      }
-
-      // both waves are done with the K tile of e: start the copy of the K tile of e+1 into its place
-      BSA_PROBE(3);
-      __syncthreads();
-      BSA_PROBE(4);
-      if (more) copy_k();
-
-      if (live) {
-      // first batch of V fragments: in flight while the softmax runs
-      constexpr int kVBatches = NHV * 4;  // batch g: head slice g / 4, key quarter g % 4, both column halves
-      u32x4 vf[2][2];
-      auto read_vbatch = [&](u32x4 (&dst)[2], int g) {
-        const int h = g >> 2, jq = g & 3;
-#pragma unroll
-        for (int db = 0; db < 2; ++db) {
-          const uint32_t *vp = reinterpret_cast<const uint32_t *>(lds_v + h * kBlockBytes) +
-                               pair_col_offset(32 * db + li) + (2 * kg + 8 * jq) * kSbs;
-          dst[db][0] = vp[0];
-          dst[db][1] = vp[kSbs];
-          dst[db][2] = vp[4 * kSbs];
-          dst[db][3] = vp[5 * kSbs];
-        }
-      };
-      read_vbatch(vf[0], 0);
-      __builtin_amdgcn_sched_barrier(0);
-
-      // ---- scores: scale, bias, causal predicate, mask ----
-      // sv holds the scores up to the positive factor cc: the raw dot products (cc = scale * log2 e), or, with
-      // a bias, the finished log2-domain scores (cc = 1).  The factor is applied inside the exponential.
-      float sv[32];
-      float cc = qk_scale;
-#pragma unroll
-      for (int jb = 0; jb < 2; ++jb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) sv[16 * jb + r] = sacc[jb][r];
-      if (pb >= 0) {
-        // bias elements j = 32 jb + 8 q + 4 kg .. + 3 of row qi
-        const char *bp0 = static_cast<const char *>(a.bias) + pb * kBlockBytes;
-        const uint32_t boff = (uint32_t)qi * 128u + (uint32_t)kg * 8u;
-#pragma unroll
-        for (int w0 = 0; w0 < 8; w0 += 2) {
-          u32x2 bw[2];
-#pragma unroll
-          for (int w = 0; w < 2; ++w) bw[w] = *reinterpret_cast<const u32x2 *>(bp0 + 16 * (w0 + w) + boff);
-#pragma unroll
-          for (int w = 0; w < 2; ++w) {
-            float *d = sv + 4 * (w0 + w);
-            d[0] = d[0] * qk_scale + Tr::widen((uint16_t)(bw[w][0] & 0xffffu)) * kLog2e;
-            d[1] = d[1] * qk_scale + Tr::widen((uint16_t)(bw[w][0] >> 16)) * kLog2e;
-            d[2] = d[2] * qk_scale + Tr::widen((uint16_t)(bw[w][1] & 0xffffu)) * kLog2e;
-            d[3] = d[3] * qk_scale + Tr::widen((uint16_t)(bw[w][1] >> 16)) * kLog2e;
-          }
-        }
-        cc = 1.f;
-      }
-      if (causal) {
-        const int kbase = kb * kSbs + 4 * kg;
-        const bool row_off = qpos >= seq_len;
-#pragma unroll
-        for (int w = 0; w < 8; ++w)
-#pragma unroll
-          for (int t = 0; t < 4; ++t) {
-            const int kpos = kbase + 8 * w + t;
-            sv[4 * w + t] = (kpos > qpos || row_off || kpos >= seq_len) ? -INFINITY : sv[4 * w + t];
-          }
-      }
-      if (mask_on) {
-        // most blocks of a mask mask nothing: one test for the wave skips the selects
-        if (__any(mbits != 0)) {
-#pragma unroll
-          for (int x = 0; x < 32; ++x) sv[x] = ((mbits >> (8 * (x & 3) + (x >> 2))) & 1u) ? -INFINITY : sv[x];
-        }
-      }
-
-      // ---- online softmax of row qi ----
-      float m_blk = sv[0];
-#pragma unroll
-      for (int x = 1; x < 32; ++x) m_blk = fmaxf(m_blk, sv[x]);
-      m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 32)) * cc;
-      // The reference maximum m_i of the exponentials only follows the running maximum when that has grown by
-      // more than kRescaleStep since the last update (for some row of the wave): in between, probabilities may
-      // exceed 1 (by at most 2^kRescaleStep) and the accumulators need no rescaling.  o and lse do not depend on
-      // the reference maximum.  -inf - -inf is NaN and compares false: a row without a finite score keeps -inf.
-      const float m_cand = fmaxf(m_i, m_blk);
-      if (__any((m_cand - m_i) > kRescaleStep)) {
-        const bool both_ninf = (m_i == -INFINITY) && (m_cand == -INFINITY);
-        const float alpha = both_ninf ? 1.f : __builtin_amdgcn_exp2f(m_i - m_cand);
-        m_i = m_cand;
-        l_i *= alpha;
-#pragma unroll
-        for (int h = 0; h < NHV; ++h)
-#pragma unroll
-          for (int db = 0; db < 2; ++db)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) oacc[h][db][r] *= alpha;
-      }
-      // with m_i == -inf every score of the row so far is -inf (or NaN): subtracting 0 instead keeps p = 0
-      const float m_sub = (m_i == -INFINITY) ? 0.f : m_i;
-      float sum = 0.f;
-#pragma unroll
-      for (int x = 0; x < 32; ++x) {
-        sv[x] = __builtin_amdgcn_exp2f(fmaf(sv[x], cc, -m_sub));
-        sum += sv[x];
-      }
-      sum += __shfl_xor(sum, 32);
-      l_i += sum;
-
-      u32x4 pf[2][2];
-#pragma unroll
-      for (int jb = 0; jb < 2; ++jb)
-#pragma unroll
-        for (int u = 0; u < 2; ++u)
-#pragma unroll
-          for (int t = 0; t < 4; ++t)
-            pf[jb][u][t] = Tr::pack2(sv[16 * jb + 8 * u + 2 * t], sv[16 * jb + 8 * u + 2 * t + 1]);
-
-      // ---- O^T += V^T P^T ----
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int g = 0; g < kVBatches; ++g) {
-        if (g + 1 < kVBatches) read_vbatch(vf[(g + 1) & 1], g + 1);
+        read_vbatch(vf[0], 0);
         __builtin_amdgcn_sched_barrier(0);
-        const int h = g >> 2, jq = g & 3;
-#pragma unroll
-        for (int db = 0; db < 2; ++db) oacc[h][db] = Tr::mfma(vf[g & 1][db], pf[jq >> 1][jq & 1], oacc[h][db]);
+
+        // ---- scores: scale, bias, causal predicate, mask ----
+        // sv holds the scores up to the positive factor cc: the raw dot products (cc = scale * log2 e), or, with
+        // a bias, the finished log2-domain scores (cc = 1).  The factor is applied inside the exponential.
+        float sv[32];
+        float cc = qk_scale;
+  #pragma unroll
+        for (int jb = 0; jb < 2; ++jb)
+  #pragma unroll
+          for (int r = 0; r < 16; ++r) sv[16 * jb + r] = sacc[jb][r];
+        if (pb >= 0) {
+          // bias elements j = 32 jb + 8 q + 4 kg .. + 3 of row qi
+          const char *bp0 = static_cast<const char *>(a.bias) + pb * kBlockBytes;
+          const uint32_t boff = (uint32_t)qi * 128u + (uint32_t)kg * 8u;
+  #pragma unroll
+          for (int w0 = 0; w0 < 8; w0 += 2) {
+            u32x2 bw[2];
+  #pragma unroll
+            for (int w = 0; w < 2; ++w) bw[w] = *reinterpret_cast<const u32x2 *>(bp0 + 16 * (w0 + w) + boff);
+  #pragma unroll
+            for (int w = 0; w < 2; ++w) {
+              float *d = sv + 4 * (w0 + w);
+              d[0] = d[0] * qk_scale + Tr::widen((uint16_t)(bw[w][0] & 0xffffu)) * kLog2e;
+              d[1] = d[1] * qk_scale + Tr::widen((uint16_t)(bw[w][0] >> 16)) * kLog2e;
+              d[2] = d[2] * qk_scale + Tr::widen((uint16_t)(bw[w][1] & 0xffffu)) * kLog2e;
+              d[3] = d[3] * qk_scale + Tr::widen((uint16_t)(bw[w][1] >> 16)) * kLog2e;
+            }
+          }
+          cc = 1.f;
+        }
+        if (causal) {
+          const int kbase = kb * kSbs + 4 * kg;
+          const bool row_off = qpos >= seq_len;
+  #pragma unroll
+          for (int w = 0; w < 8; ++w)
+  #pragma unroll
+            for (int t = 0; t < 4; ++t) {
+              const int kpos = kbase + 8 * w + t;
+              sv[4 * w + t] = (kpos > qpos || row_off || kpos >= seq_len) ? -INFINITY : sv[4 * w + t];
+            }
+        }
+        if (mask_on) {
+          // most blocks of a mask mask nothing: one test for the wave skips the selects
+          if (__any(mbits != 0)) {
+  #pragma unroll
+            for (int x = 0; x < 32; ++x) sv[x] = ((mbits >> (8 * (x & 3) + (x >> 2))) & 1u) ? -INFINITY : sv[x];
+          }
+        }
+
+        // ---- online softmax of row qi ----
+        float m_blk = sv[0];
+  #pragma unroll
+        for (int x = 1; x < 32; ++x) m_blk = fmaxf(m_blk, sv[x]);
+        m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 32)) * cc;
+        // The reference maximum m_i of the exponentials only follows the running maximum when that has grown by
+        // more than kRescaleStep since the last update (for some row of the wave): in between, probabilities may
+        // exceed 1 (by at most 2^kRescaleStep) and the accumulators need no rescaling.  o and lse do not depend on
+        // the reference maximum.  -inf - -inf is NaN and compares false: a row without a finite score keeps -inf.
+        const float m_cand = fmaxf(m_i, m_blk);
+        if (__any((m_cand - m_i) > kRescaleStep)) {
+          const bool both_ninf = (m_i == -INFINITY) && (m_cand == -INFINITY);
+          const float alpha = both_ninf ? 1.f : __builtin_amdgcn_exp2f(m_i - m_cand);
+          m_i = m_cand;
+          l_i *= alpha;
+  #pragma unroll
+          for (int h = 0; h < NHV; ++h)
+  #pragma unroll
+            for (int db = 0; db < 2; ++db)
+  #pragma unroll
+              for (int r = 0; r < 16; ++r) oacc[h][db][r] *= alpha;
+        }
+        // with m_i == -inf every score of the row so far is -inf (or NaN): subtracting 0 instead keeps p = 0
+        const float m_sub = (m_i == -INFINITY) ? 0.f : m_i;
+        float sum = 0.f;
+  #pragma unroll
+        for (int x = 0; x < 32; ++x) {
+          sv[x] = __builtin_amdgcn_exp2f(fmaf(sv[x], cc, -m_sub));
+          sum += sv[x];
+        }
+        sum += __shfl_xor(sum, 32);
+        l_i += sum;
+
+        u32x4 pf[2][2];
+  #pragma unroll
+        for (int jb = 0; jb < 2; ++jb)
+  #pragma unroll
+          for (int u = 0; u < 2; ++u)
+  #pragma unroll
+            for (int t = 0; t < 4; ++t)
+              pf[jb][u][t] = Tr::pack2(sv[16 * jb + 8 * u + 2 * t], sv[16 * jb + 8 * u + 2 * t + 1]);
+
+        // ---- O^T += V^T P^T ----
         __builtin_amdgcn_sched_barrier(0);
-      }
+#pragma unroll
+        for (int g = 0; g < kVBatches; ++g) {
+          if (g + 1 < kVBatches) read_vbatch(vf[(g + 1) & 1], g + 1);
+          __builtin_amdgcn_sched_barrier(0);
+          const int h = g >> 2, jq = g & 3;
+#pragma unroll
+          for (int db = 0; db < 2; ++db) oacc[h][db] = Tr::mfma(vf[g & 1][db], pf[jq >> 1][jq & 1], oacc[h][db]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        BSA_PROBE(3);
       }  // live
-      BSA_PROBE(5);
+
+      // ---- tile e+1 into LDS; the barrier also ends the reads of tile e ----
+      if (more) stage_v(buf ^ 1);
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the K rows this wave copied are in LDS
+      BSA_PROBE(4);
       __syncthreads();
-      BSA_PROBE(6);
+      BSA_PROBE(5);
     }
   }
 
@@ -561,27 +587,21 @@ __global__ __launch_bounds__(64) void attn_fwd_records_kernel(bsa_attn_args a, c
   }
 }
 
-template <typename Tr, int NH, int NHV, int G>
+template <typename Tr, int NH, int NHV>
 int launch_fwd(const bsa_attn_args &a, hipStream_t s) {
-  const int64_t groups = a.B * cdiv(a.nq, G);
+  const int64_t groups = a.B * cdiv(a.nq, 2);
   if (groups == 0) return BSA_OK;
-  attn_fwd_mfma_kernel<Tr, NH, NHV, G><<<(unsigned)(cdiv(groups, 8) * 8), kFwdThreads * G, 0, s>>>(a);
+  attn_fwd_mfma_kernel<Tr, NH, NHV><<<(unsigned)(cdiv(groups, 8) * 8), kFwdThreads, 0, s>>>(a);
   return check_launch("attn_fwd_mfma_kernel");
-}
-
-template <typename Tr, int G>
-int dispatch_fwd_g(const bsa_attn_args &a, hipStream_t s) {
-  if (a.nh == 1 && a.nhv == 1) return launch_fwd<Tr, 1, 1, G>(a, s);
-  if (a.nh == 2 && a.nhv == 2) return launch_fwd<Tr, 2, 2, G>(a, s);
-  if (a.nh == 1 && a.nhv == 2) return launch_fwd<Tr, 1, 2, G>(a, s);
-  if (a.nh == 2 && a.nhv == 1) return launch_fwd<Tr, 2, 1, G>(a, s);
-  return 1;
 }
 
 template <typename Tr>
 int dispatch_fwd(const bsa_attn_args &a, hipStream_t s) {
-  if (a.group_size == 2) return dispatch_fwd_g<Tr, 2>(a, s);
-  return dispatch_fwd_g<Tr, 1>(a, s);
+  if (a.nh == 1 && a.nhv == 1) return launch_fwd<Tr, 1, 1>(a, s);
+  if (a.nh == 2 && a.nhv == 2) return launch_fwd<Tr, 2, 2>(a, s);
+  if (a.nh == 1 && a.nhv == 2) return launch_fwd<Tr, 1, 2>(a, s);
+  if (a.nh == 2 && a.nhv == 1) return launch_fwd<Tr, 2, 1>(a, s);
+  return 1;
 }
 
 }  // namespace
@@ -591,7 +611,7 @@ int attn_fwd_mfma(const bsa_attn_args &a, hipStream_t s) {
   // the kernels take the row maximum before the scale is applied
   if (!(a.scale > 0.f) || a.scale > 3.0e38f) return 1;
   // the matrix-core kernels walk the grouped record lists; without them the generic kernels run
-  if (a.group_offsets == nullptr || (a.group_size != 1 && a.group_size != 2)) return 1;
+  if (a.group_offsets == nullptr || a.group_size != 2) return 1;
   if (a.group_records == nullptr) {
     // no list entry at all: every query block still writes o = 0 and lse = -inf
     // (the caller passes NULL for an empty record array; the offsets then are all zero)

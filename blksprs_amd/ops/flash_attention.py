@@ -25,11 +25,6 @@ from ..utils.validation import (ensure_contiguous, validate_binary, validate_con
                                 validate_sparsity_block_size, validate_sparsity_layout)
 
 
-# Build the key lists of query block pairs (see _build_group_key_lists).  Off: the forward kernel walks one
-# list per query block, with the same results.
-_PAIR_QUERY_BLOCKS = True
-
-
 def _select_segmented_index_dtype(n_active_blocks: int, n_blocks_col: int) -> torch.dtype:
     """int32 unless the number of active blocks or the largest column id needs more."""
     if n_active_blocks > INT32_INDEX_MAX or n_blocks_col - 1 > INT32_INDEX_MAX:
@@ -63,37 +58,26 @@ def _build_segmented_indices(attention_layout: Tensor, n_batches: int, n_blocks_
 
 def _build_group_lists(attention_layout: Tensor, n_batches: int, n_blocks_row: int,
                        n_blocks_col: int) -> tuple[Tensor, Tensor, int]:
-    """The attention layout as lists over groups of neighbouring query blocks: ``(offsets, entries, group_size)``.
+    """The attention layout as lists over pairs of neighbouring query blocks: ``(offsets, entries, group_size)``.
 
-    With ``group_size == 2`` a group is the pair of query blocks ``(2p, 2p+1)`` and its list the union of their
-    key lists; with 1 it is one query block.  ``entries`` holds ``key_block | active_for_first << 28 |
-    active_for_second << 29`` (int32, key blocks ascending), ``offsets`` has ``B * ceil(rows / group_size) + 1``
-    int32 entries.  The forward kernel fetches a K / V block once per group; pairs are used when the two lists
-    of a pair overlap enough for that to save fetches.  These lists have no counterpart in the reference.
+    A group is the pair of query blocks ``(2p, 2p+1)`` and its list the union of their key lists.  ``entries``
+    holds ``key_block | active_for_first << 28 | active_for_second << 29`` (int32, key blocks ascending),
+    ``offsets`` has ``B * ceil(rows / 2) + 1`` int32 entries.  The forward kernel gives a pair to one workgroup,
+    which fetches a K / V block both query blocks need once.  These lists have no counterpart in the reference.
     """
     device = attention_layout.device
     active = attention_layout.reshape(n_batches, n_blocks_row, n_blocks_col) != 0
-    padded = active
     if n_blocks_row % 2:
-        padded = torch.cat([active, torch.zeros_like(active[:, :1])], dim=1)
-    even, odd = padded[:, 0::2], padded[:, 1::2]
+        active = torch.cat([active, torch.zeros_like(active[:, :1])], dim=1)
+    even, odd = active[:, 0::2], active[:, 1::2]
     union = even | odd
-    n_active, n_union = int(active.sum()), int(union.sum())
-    # a pair's workgroup is busy for the union of the two lists, a single block's for its own list
-    group_size = 2 if _PAIR_QUERY_BLOCKS and n_active >= 1.25 * n_union else 1
-    if group_size == 2:
-        where = torch.nonzero(union)
-        flags = even[where[:, 0], where[:, 1], where[:, 2]].to(torch.int32) \
-            | (odd[where[:, 0], where[:, 1], where[:, 2]].to(torch.int32) << 1)
-        counts = union.sum(dim=-1).reshape(-1)
-    else:
-        where = torch.nonzero(active)
-        flags = torch.ones(where.size(0), dtype=torch.int32, device=device)
-        counts = active.sum(dim=-1).reshape(-1)
+    where = torch.nonzero(union)
+    flags = even[where[:, 0], where[:, 1], where[:, 2]].to(torch.int32) \
+        | (odd[where[:, 0], where[:, 1], where[:, 2]].to(torch.int32) << 1)
     entries = (where[:, 2].to(torch.int32) | (flags << 28)).contiguous()
-    offsets = torch.zeros(counts.numel() + 1, dtype=torch.int32, device=device)
-    offsets[1:] = torch.cumsum(counts, dim=0).to(torch.int32)
-    return as_base_tensor(offsets), as_base_tensor(entries), group_size
+    offsets = torch.zeros(union.size(0) * union.size(1) + 1, dtype=torch.int32, device=device)
+    offsets[1:] = torch.cumsum(union.sum(dim=-1).reshape(-1), dim=0).to(torch.int32)
+    return as_base_tensor(offsets), as_base_tensor(entries), 2
 
 
 def flash_attention_build_layout_cache(attention_layout: Tensor,

@@ -250,34 +250,46 @@ def test_matrix_core_forward_odd_sequences_and_head_slice_counts(device, dtype, 
     _run_case(device, dtype, 64, 2, nq, 6, nh, nhv, 0.5, 70 + nq, use_mask=True, use_causal=(nq == 6))
 
 
-def test_paired_query_block_lists_give_the_same_bits_as_single_lists(device, monkeypatch):
-    """The forward kernel fetches K / V once per pair of query blocks when the cache holds the pair lists and
-    once per query block otherwise; both walk the key blocks in the same order, so the results are identical."""
+def test_pair_lists_cover_the_layout_and_masked_tiles_change_nothing(device):
+    """The forward kernel walks, per pair of query blocks, the union of their key lists.  Every active block of
+    the layout appears once with its flag; whole mask blocks that are set are fetched but not computed."""
     g = torch.Generator().manual_seed(5)
     B, nq, nk, nh, sbs = 3, 9, 11, 2, 64
-    la = orc.random_layout((B, nq, nk), 0.7, g, ensure_rows=True).to(device)
-    la[1, 4] = False  # a query block without keys
-    full = torch.ones((B, nq, nh), dtype=torch.bool, device=device)
-    fullk = torch.ones((B, nk, nh), dtype=torch.bool, device=device)
-    q = rand_blocks(B * nq * nh, sbs, torch.bfloat16, 1).to(device)
-    k = rand_blocks(B * nk * nh, sbs, torch.bfloat16, 2).to(device)
-    v = rand_blocks(B * nk * nh, sbs, torch.bfloat16, 3).to(device)
+    la = orc.random_layout((B, nq, nk), 0.6, g, ensure_rows=True)
+    full = torch.ones((B, nq, nh), dtype=torch.bool)
+    fullk = torch.ones((B, nk, nh), dtype=torch.bool)
+    q = rand_blocks(B * nq * nh, sbs, torch.bfloat16, 1)
+    k = rand_blocks(B * nk * nh, sbs, torch.bfloat16, 2)
+    v = rand_blocks(B * nk * nh, sbs, torch.bfloat16, 3)
     lmask = la.clone()
-    mask = (torch.rand((int(lmask.sum()), sbs, sbs), generator=g) < 0.5).to(device)
-    mask[::3] = True  # whole blocks masked: such tiles are fetched but not computed
+    mask = torch.rand((int(lmask.sum()), sbs, sbs), generator=g) < 0.5
+    mask[::3] = True
     cache = {}
-    paired = bs.ops.flash_attention(q, full, k, fullk, v, fullk, la, sbs, attention_mask=mask,
-                                    sparsity_layout_mask=lmask, layout_cache=cache)
+    out = bs.ops.flash_attention(q.to(device), full.to(device), k.to(device), fullk.to(device), v.to(device),
+                                 fullk.to(device), la.to(device), sbs, attention_mask=mask.to(device),
+                                 sparsity_layout_mask=lmask.to(device), layout_cache=cache)
     assert cache["group_size"] == 2
-    entries = cache["group_records"].view(-1, 16)[:, 0]
+    records = cache["group_records"].view(-1, 16).cpu()
+    entries = records[:, 0]
     assert int(((entries >> 28) & 1).sum() + ((entries >> 29) & 1).sum()) == int(la.sum())
-    import importlib
-    fa_module = importlib.import_module("blksprs_amd.ops.flash_attention")
-    monkeypatch.setattr(fa_module, "_PAIR_QUERY_BLOCKS", False)
-    plain = {}
-    single = bs.ops.flash_attention(q, full, k, fullk, v, fullk, la, sbs, attention_mask=mask,
-                                    sparsity_layout_mask=lmask, layout_cache=plain)
-    assert plain["group_size"] == 1 and plain["group_records"].size(0) == 16 * int(la.sum())
-    assert torch.equal(paired, single)
-    # the query block without keys has no output blocks
-    assert paired.size(0) == (B * nq - 1) * nh
+    # records against a host restatement: packed indices of K, V and of the mask block of either query block
+    offsets = cache["group_offsets"].cpu()
+    pidx_mask = (torch.cumsum(lmask.reshape(-1).long(), 0) - 1).masked_fill(~lmask.reshape(-1), -1).view(B, nq, nk)
+    for grp in range(B * ((nq + 1) // 2)):
+        b_, p_ = divmod(grp, (nq + 1) // 2)
+        keys = sorted(set(torch.nonzero(la[b_, 2 * p_]).flatten().tolist())
+                      | (set(torch.nonzero(la[b_, 2 * p_ + 1]).flatten().tolist()) if 2 * p_ + 1 < nq else set()))
+        got = records[offsets[grp]:offsets[grp + 1]]
+        assert (got[:, 0] & 0x0fffffff).tolist() == keys
+        for rec in got.tolist():
+            kb = rec[0] & 0x0fffffff
+            assert rec[1:5] == [(b_ * nk + kb) * nh, (b_ * nk + kb) * nh + 1] * 2
+            for half in range(2):
+                qb = 2 * p_ + half
+                active = qb < nq and bool(la[b_, qb, kb])
+                assert bool((rec[0] >> (28 + half)) & 1) == active
+                assert rec[5 + half] == (int(pidx_mask[b_, qb, kb]) if active else -1)
+                assert rec[7 + half] == -1
+    ref = orc.flash_attention(q.double(), full.numpy(), k.double(), fullk.numpy(), v.double(), fullk.numpy(),
+                              la.numpy(), sbs, mask=mask, layout_mask=lmask.numpy(), acc_dtype=torch.float64)
+    assert_close(out, ref, 2e-2, "O pair lists")
