@@ -1,0 +1,741 @@
+// Block-sparse flash attention backward on the matrix cores: fp16 / bf16 operands, sbs == 64, one or two
+// 64-wide head slices for q/k and for v/o.
+//
+// Three kernels, as in the reference (blksprs/ops/flash_attention.py:1235-1735): delta = rowsum(o * dO);
+// dK / dV (and dBias) per key block, walking the query blocks that attend to it; dQ per query block, walking
+// its key blocks.  The two main kernels recompute the scores and probabilities of a (query block, key block)
+// pair from the saved log-sum-exp, in the same order as the forward kernel: scale * q k^T, + bias, native causal
+// predicate, explicit mask.  Probabilities and dS are rounded to the operand type before they enter a product.
+//
+// Both main kernels have the same shape.  One workgroup of four waves owns the "stationary" block (a key block,
+// or a query block); each wave owns one 32 x 32 quadrant of the 64 x 64 score tile and keeps the fragments of
+// its half of the stationary operands in registers for the whole walk.  The blocks of the other side stream
+// through LDS, double buffered, one barrier per tile: row-major with XOR-swizzled 16-byte chunks where the head
+// dimension is contracted (scores, dP), and as (row, row + 1) pairs per column where the sequence index is
+// contracted (dV, dK, dQ), because a matrix-core operand wants eight consecutive contraction indices per lane.
+//
+//   dK / dV kernel, lane owns a key j, registers run over queries i:
+//     S[i][j]  = sum_d Q[i][d] K[j][d]        A = Q rows (LDS)     B = K (registers)
+//     dP[i][j] = sum_d dO[i][d] V[j][d]       A = dO rows (LDS)    B = V (registers)
+//     dV^T[d][j] += sum_i dO[i][d] P[i][j]    A = dO pairs (LDS)   B = P (registers, as computed)
+//     dK^T[d][j] += sum_i Q[i][d] dS[i][j]    A = Q pairs (LDS)    B = dS
+//   dQ kernel, lane owns a query i, registers run over keys j:
+//     S^T[j][i], dP^T[j][i] likewise with K, V rows from LDS and Q, dO in registers
+//     dQ^T[d][i] += sum_j K[j][d] dS^T[j][i]  A = K pairs (LDS)    B = dS^T
+//
+// The two waves that share a half of the stationary block hold partial sums over the two halves of the streamed
+// blocks; they are added through LDS once, at the end.  No atomics, fixed summation order.
+#include "attn_mfma_common.h"
+
+namespace bsa {
+namespace {
+
+using namespace mfma;
+
+constexpr int kBwdThreads = 256;
+constexpr int kStatBytes = 2 * kSbs * 4;  // lse and delta of the 64 queries of a tile
+
+// ---- one 64 x 64 16-bit block spread over 256 threads: thread t holds rows 2p, 2p + 1 (p = t / 8),
+// ---- columns 8 (t % 8) .. + 7
+struct TileRegs {
+  u32x4 ev, od;
+};
+
+__device__ inline TileRegs load_tile(const char *blk, bool valid, int tid) {
+  TileRegs t;
+  t.ev = u32x4{0u, 0u, 0u, 0u};
+  t.od = u32x4{0u, 0u, 0u, 0u};
+  if (valid) {
+    const uint32_t off = (uint32_t)(tid >> 3) * 256u + (uint32_t)(tid & 7) * 16u;
+    t.ev = load16(blk, off);
+    t.od = load16(blk + 128, off);
+  }
+  return t;
+}
+
+// row-major, chunk c of row r at position c ^ k_swizzle(r) (rows 2p and 2p + 1 share the swizzle value)
+__device__ inline void stage_rows(char *lds, const TileRegs &t, int tid) {
+  const int p = tid >> 3, c = tid & 7;
+  char *dst = lds + (2 * p) * 128 + ((c ^ (p & 7)) << 4);
+  *reinterpret_cast<u32x4 *>(dst) = t.ev;
+  *reinterpret_cast<u32x4 *>(dst + 128) = t.od;
+}
+
+// (row 2p, row 2p + 1) pairs per column
+__device__ inline void stage_pairs(char *lds, const TileRegs &t, int tid) {
+  const int p = tid >> 3, c = tid & 7;
+  u32x4 lo, hi;
+  lo[0] = __builtin_amdgcn_perm(t.od[0], t.ev[0], 0x05040100u);
+  lo[1] = __builtin_amdgcn_perm(t.od[0], t.ev[0], 0x07060302u);
+  lo[2] = __builtin_amdgcn_perm(t.od[1], t.ev[1], 0x05040100u);
+  lo[3] = __builtin_amdgcn_perm(t.od[1], t.ev[1], 0x07060302u);
+  hi[0] = __builtin_amdgcn_perm(t.od[2], t.ev[2], 0x05040100u);
+  hi[1] = __builtin_amdgcn_perm(t.od[2], t.ev[2], 0x07060302u);
+  hi[2] = __builtin_amdgcn_perm(t.od[3], t.ev[3], 0x05040100u);
+  hi[3] = __builtin_amdgcn_perm(t.od[3], t.ev[3], 0x07060302u);
+  uint32_t *prow = reinterpret_cast<uint32_t *>(lds) + p * kSbs;
+  *reinterpret_cast<u32x4 *>(prow + pair_col_offset(c * 8)) = lo;
+  *reinterpret_cast<u32x4 *>(prow + pair_col_offset(c * 8 + 4)) = hi;
+}
+
+// operand fragment with the head dimension contracted: 8 values of row `row`, 16-byte chunk `chunk`
+__device__ inline u32x4 frag_rows(const char *lds, int row, int chunk) {
+  return *reinterpret_cast<const u32x4 *>(lds + row * 128 + ((chunk ^ k_swizzle(row)) << 4));
+}
+
+// operand fragment with the row index contracted: column `col`, rows 2 pair0 .. + 3 and 2 pair0 + 8 .. + 11
+__device__ inline u32x4 frag_pairs(const char *lds, int col, int pair0) {
+  const uint32_t *p = reinterpret_cast<const uint32_t *>(lds) + pair0 * kSbs + pair_col_offset(col);
+  u32x4 v;
+  v[0] = p[0];
+  v[1] = p[kSbs];
+  v[2] = p[4 * kSbs];
+  v[3] = p[5 * kSbs];
+  return v;
+}
+
+// fragment of a block in global memory for the register-resident side: row `row`, chunks 2 s + kg
+__device__ inline void load_resident(u32x4 (&f)[4], const void *base, int64_t pidx, int64_t n_blocks, int row, int kg) {
+  const bool valid = pidx >= 0 && pidx < n_blocks;
+  const char *p = static_cast<const char *>(base) + (valid ? pidx : 0) * kBlockBytes + row * 128 + kg * 16;
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+    f[s] = u32x4{0u, 0u, 0u, 0u};
+    if (valid) f[s] = *reinterpret_cast<const u32x4 *>(p + 32 * s);
+  }
+}
+
+__device__ inline const int32_t *low_half_ptr(const int64_t *p, int64_t i) {
+  return reinterpret_cast<const int32_t *>(p) + 2 * i;
+}
+
+__device__ inline int as_vector(int v) {
+  asm volatile("" : "+v"(v));
+  return v;
+}
+
+// XCD-aware row of a workgroup: every XCD gets a contiguous range of rows, so that the blocks in flight on one
+// L2 belong to the same batch entries
+__device__ inline int64_t xcd_row() { return (int64_t)(blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3); }
+
+// sum of the accumulators of wave pairs (w, w ^ partner_bit): the wave with the bit set writes, the other adds
+template <int N>
+__device__ inline void reduce_partner(f32x16 (&acc)[N], float *lds, bool writer, int slot, int lane) {
+  // slot: which pair of waves (0 or 1); layout [slot][n][r][lane]
+  float *base = lds + (size_t)slot * N * 16 * 64 + lane;
+  __syncthreads();  // the tile buffers are free
+  if (writer) {
+#pragma unroll
+    for (int n = 0; n < N; ++n)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) base[(n * 16 + r) * 64] = acc[n][r];
+  }
+  __syncthreads();
+  if (!writer) {
+#pragma unroll
+    for (int n = 0; n < N; ++n)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[n][r] += base[(n * 16 + r) * 64];
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// delta[b, qb, i] = sum over active output slices of rowsum(o * dO); four lanes per query row
+template <typename Tr>
+__global__ __launch_bounds__(kBwdThreads) void attn_bwd_delta_kernel(bsa_attn_args a) {
+  const int64_t row = blockIdx.x;  // b * nq + qb
+  const int tid = threadIdx.x;
+  const int i = tid >> 2, part = tid & 3;
+  float acc = 0.f;
+  for (int64_t h = 0; h < a.nhv; ++h) {
+    const int64_t po = a.pidx_o[row * a.nhv + h];
+    if (po < 0 || po >= a.n_o_blocks) continue;
+    const char *ob = static_cast<const char *>(a.o) + po * kBlockBytes + i * 128 + part * 32;
+    const char *gb = static_cast<const char *>(a.d_o) + po * kBlockBytes + i * 128 + part * 32;
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      const u32x4 ov = *reinterpret_cast<const u32x4 *>(ob + 16 * c);
+      const u32x4 gv = *reinterpret_cast<const u32x4 *>(gb + 16 * c);
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        acc = fmaf(Tr::widen((uint16_t)(ov[t] & 0xffffu)), Tr::widen((uint16_t)(gv[t] & 0xffffu)), acc);
+        acc = fmaf(Tr::widen((uint16_t)(ov[t] >> 16)), Tr::widen((uint16_t)(gv[t] >> 16)), acc);
+      }
+    }
+  }
+  acc += __shfl_xor(acc, 1);
+  acc += __shfl_xor(acc, 2);
+  if (part == 0) a.delta[row * kSbs + i] = acc;
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// dK, dV and dBias of one key block
+template <typename Tr, int NH, int NHV>
+__global__ __launch_bounds__(kBwdThreads, 1) void attn_bwd_kv_kernel(bsa_attn_args a) {
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  constexpr int kQRows = 0, kQPairs = NH * kBlockBytes, kDoRows = 2 * NH * kBlockBytes,
+                kDoPairs = (2 * NH + NHV) * kBlockBytes, kStats = 2 * (NH + NHV) * kBlockBytes;
+  constexpr int kBufBytes = kStats + kStatBytes;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = first_lane(tid >> 6);
+  const int li = lane & 31, kg = lane >> 5;
+  const int wi = wave & 1, wj = wave >> 1;  // query half and key half of this wave's quadrant
+  const int64_t krow = xcd_row();
+  if (krow >= a.B * a.nk) return;
+  const int64_t b = krow / a.nk, kb = krow % a.nk;
+
+  int64_t pk[NH], pv[NHV];
+  bool any = a.dbias != nullptr;
+#pragma unroll
+  for (int h = 0; h < NH; ++h) {
+    pk[h] = a.pidx_k[krow * NH + h];
+    if (pk[h] >= a.n_k_blocks) pk[h] = -1;
+    any = any || pk[h] >= 0;
+  }
+#pragma unroll
+  for (int h = 0; h < NHV; ++h) {
+    pv[h] = a.pidx_v[krow * NHV + h];
+    if (pv[h] >= a.n_v_blocks) pv[h] = -1;
+    any = any || pv[h] >= 0;
+  }
+  if (!any) return;
+
+  // this wave's keys: B operands K[j][.], V[j][.] with j = 32 wj + li
+  u32x4 kfr[NH][4], vfr[NHV][4];
+#pragma unroll
+  for (int h = 0; h < NH; ++h) load_resident(kfr[h], a.k, pk[h], a.n_k_blocks, 32 * wj + li, kg);
+#pragma unroll
+  for (int h = 0; h < NHV; ++h) load_resident(vfr[h], a.v, pv[h], a.n_v_blocks, 32 * wj + li, kg);
+
+  // accumulators [slice][column half db]: D[m = d][n = j]
+  f32x16 dkacc[NH * 2], dvacc[NHV * 2];
+#pragma unroll
+  for (int n = 0; n < NH * 2; ++n)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) dkacc[n][r] = 0.f;
+#pragma unroll
+  for (int n = 0; n < NHV * 2; ++n)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) dvacc[n][r] = 0.f;
+
+  const float qk_scale = a.scale * kLog2e;
+  const bool causal = a.causal_lengths != nullptr;
+  int seq_len = 0;
+  if (causal) {
+    const int64_t len = a.causal_lengths[b];
+    seq_len = len < 0 ? 0 : (len > 0x7fffffffLL ? 0x7fffffff : (int)len);
+  }
+  const int kpos = (int)kb * kSbs + 32 * wj + li;
+
+  const int q_begin = a.query_offsets[krow], q_end = a.query_offsets[krow + 1];
+  if (q_begin < q_end) {
+    // lanes 0 .. NH-1: packed Q indices of a query block, next NHV lanes: packed O (= dO) indices, then its mask and
+    // bias block for this key block; lane 7: the list entry at `pos`
+    constexpr int kLaneMask = NH + NHV, kLaneBias = NH + NHV + 1, kLaneEntry = 7;
+    auto gather = [&](int qb, int pos) -> int {
+      const int64_t qrow = b * a.nq + qb;
+      const int32_t *p = a.query_indices + pos;
+      bool on = lane == kLaneEntry;
+      if (lane < NH) {
+        p = low_half_ptr(a.pidx_q, qrow * NH + lane);
+        on = true;
+      } else if (lane < NH + NHV) {
+        p = low_half_ptr(a.pidx_o, qrow * NHV + (lane - NH));
+        on = true;
+      } else if (lane == kLaneMask && a.mask) {
+        p = low_half_ptr(a.pidx_mask, qrow * a.nk + kb);
+        on = true;
+      } else if (lane == kLaneBias && a.bias) {
+        p = low_half_ptr(a.pidx_bias, qrow * a.nk + kb);
+        on = true;
+      }
+      int v = -1;
+      if (on) v = *p;
+      return v;
+    };
+    auto clamp_e = [&](int e) { return e < q_end ? e : q_end - 1; };
+
+    // registers of the tile in flight
+    TileRegs qt[NH], dot[NHV];
+    float stat = 0.f;           // thread t < 64: lse of query t; 64 <= t < 128: delta of query t - 64
+    uint32_t mask_b[16];        // mask bytes of this lane's 16 score elements
+    uint32_t bias_b[16];        // bias elements likewise
+    int qb_nxt, pm_nxt, pb_nxt;
+
+    auto fetch = [&](int rec, int qb) {
+      qb_nxt = qb;
+#pragma unroll
+      for (int h = 0; h < NH; ++h) {
+        const int64_t pq = __builtin_amdgcn_readlane(rec, h);
+        const bool valid = pq >= 0 && pq < a.n_q_blocks;
+        qt[h] = load_tile(static_cast<const char *>(a.q) + (valid ? pq : 0) * kBlockBytes, valid, tid);
+      }
+#pragma unroll
+      for (int h = 0; h < NHV; ++h) {
+        const int64_t po = __builtin_amdgcn_readlane(rec, NH + h);
+        const bool valid = po >= 0 && po < a.n_o_blocks;
+        dot[h] = load_tile(static_cast<const char *>(a.d_o) + (valid ? po : 0) * kBlockBytes, valid, tid);
+      }
+      const int64_t qrow = b * a.nq + qb;
+      if (tid < 64) stat = a.lse[qrow * kSbs + tid];
+      else if (tid < 128) stat = a.delta[qrow * kSbs + tid - 64];
+      pm_nxt = __builtin_amdgcn_readlane(rec, kLaneMask);
+      if (pm_nxt >= a.n_mask_blocks) pm_nxt = -1;
+      pb_nxt = __builtin_amdgcn_readlane(rec, kLaneBias);
+      if (pb_nxt >= a.n_bias_blocks) pb_nxt = -1;
+      // element r of this lane: query 32 wi + 8 (r / 4) + 4 kg + r % 4, key 32 wj + li
+      if (pm_nxt >= 0) {
+        const uint8_t *mp = static_cast<const uint8_t *>(a.mask) + (int64_t)pm_nxt * (kSbs * kSbs) +
+                            (32 * wi + 4 * kg) * kSbs + 32 * wj + li;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mask_b[r] = mp[(8 * (r >> 2) + (r & 3)) * kSbs];
+      }
+      if (pb_nxt >= 0) {
+        const uint16_t *bp = static_cast<const uint16_t *>(a.bias) + (int64_t)pb_nxt * (kSbs * kSbs) +
+                             (32 * wi + 4 * kg) * kSbs + 32 * wj + li;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) bias_b[r] = bp[(8 * (r >> 2) + (r & 3)) * kSbs];
+      }
+    };
+    auto stage = [&](int buf) {
+      char *base = smem + buf * kBufBytes;
+#pragma unroll
+      for (int h = 0; h < NH; ++h) {
+        stage_rows(base + kQRows + h * kBlockBytes, qt[h], tid);
+        stage_pairs(base + kQPairs + h * kBlockBytes, qt[h], tid);
+      }
+#pragma unroll
+      for (int h = 0; h < NHV; ++h) {
+        stage_rows(base + kDoRows + h * kBlockBytes, dot[h], tid);
+        stage_pairs(base + kDoPairs + h * kBlockBytes, dot[h], tid);
+      }
+      if (tid < 128) reinterpret_cast<float *>(base + kStats)[tid] = stat;
+    };
+
+    // index pipeline: `rec` holds the indices of query block qb_rec (the entry after the tile in flight) and, in
+    // lane 7, the entry after that
+    int rec, qb_rec;
+    {
+      const int qb0 = first_lane(a.query_indices[as_vector(q_begin)]);
+      const int rec0 = gather(qb0, clamp_e(q_begin + 1));
+      qb_rec = __builtin_amdgcn_readlane(rec0, kLaneEntry);
+      rec = gather(qb_rec, clamp_e(q_begin + 2));
+      fetch(rec0, qb0);
+      stage(0);
+      __syncthreads();
+    }
+
+    for (int e = q_begin; e < q_end; ++e) {
+      const int buf = (e - q_begin) & 1;
+      const char *base = smem + buf * kBufBytes;
+      // facts and per-element inputs of tile e, before the fetch of tile e+1 replaces them
+      const int qb = qb_nxt;
+      const int64_t pm = pm_nxt, pb = pb_nxt;
+      uint32_t mask_c[16], bias_c[16];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        mask_c[r] = mask_b[r];
+        bias_c[r] = bias_b[r];
+      }
+      const bool more = e + 1 < q_end;
+      if (more) fetch(rec, qb_rec);
+      qb_rec = __builtin_amdgcn_readlane(rec, kLaneEntry);
+      rec = gather(qb_rec, clamp_e(e + 3));
+
+      // ---- S and dP of this wave's quadrant ----
+      f32x16 sacc, dpacc;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sacc[r] = dpacc[r] = 0.f;
+#pragma unroll
+      for (int h = 0; h < NH; ++h)
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+          sacc = Tr::mfma(frag_rows(base + kQRows + h * kBlockBytes, 32 * wi + li, 2 * s + kg), kfr[h][s], sacc);
+#pragma unroll
+      for (int h = 0; h < NHV; ++h)
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+          dpacc = Tr::mfma(frag_rows(base + kDoRows + h * kBlockBytes, 32 * wi + li, 2 * s + kg), vfr[h][s], dpacc);
+
+      // ---- P and dS; element r: query 32 wi + 8 (r / 4) + 4 kg + r % 4 ----
+      const float *stats = reinterpret_cast<const float *>(base + kStats);
+      float p[16], ds[16];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int i0 = 32 * wi + 8 * q + 4 * kg;
+        const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(stats + i0);
+        const f32x4 del4 = *reinterpret_cast<const f32x4 *>(stats + kSbs + i0);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const int r = 4 * q + t;
+          float s = sacc[r] * qk_scale;
+          if (pb >= 0) s = s + Tr::widen((uint16_t)bias_c[r]) * kLog2e;
+          if (causal) {
+            const int qpos = qb * kSbs + i0 + t;
+            s = (kpos > qpos || qpos >= seq_len || kpos >= seq_len) ? -INFINITY : s;
+          }
+          if (pm >= 0) s = mask_c[r] ? -INFINITY : s;
+          const float lse = lse4[t];
+          p[r] = (lse == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(s - lse);
+          ds[r] = p[r] * (dpacc[r] - del4[t]);
+        }
+      }
+      if (a.dbias != nullptr && pb >= 0) {
+        // every (query block, key block) pair is visited once, so this is a plain store
+        float *dbp = a.dbias + pb * (kSbs * kSbs) + (32 * wi + 4 * kg) * kSbs + 32 * wj + li;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dbp[(8 * (r >> 2) + (r & 3)) * kSbs] = ds[r];
+      }
+      u32x4 pf[2], dsf[2];
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          pf[u][t] = Tr::pack2(p[8 * u + 2 * t], p[8 * u + 2 * t + 1]);
+          dsf[u][t] = Tr::pack2(ds[8 * u + 2 * t], ds[8 * u + 2 * t + 1]);
+        }
+
+      // ---- dV^T += dO^T P, dK^T += Q^T dS over this wave's 32 queries ----
+#pragma unroll
+      for (int h = 0; h < NHV; ++h)
+#pragma unroll
+        for (int db = 0; db < 2; ++db)
+#pragma unroll
+          for (int u = 0; u < 2; ++u)
+            dvacc[2 * h + db] = Tr::mfma(frag_pairs(base + kDoPairs + h * kBlockBytes, 32 * db + li, 16 * wi + 8 * u + 2 * kg),
+                                         pf[u], dvacc[2 * h + db]);
+#pragma unroll
+      for (int h = 0; h < NH; ++h)
+#pragma unroll
+        for (int db = 0; db < 2; ++db)
+#pragma unroll
+          for (int u = 0; u < 2; ++u)
+            dkacc[2 * h + db] = Tr::mfma(frag_pairs(base + kQPairs + h * kBlockBytes, 32 * db + li, 16 * wi + 8 * u + 2 * kg),
+                                         dsf[u], dkacc[2 * h + db]);
+
+      // ---- tile e+1 into the other buffer; the barrier also ends the reads of tile e ----
+      if (more) stage(buf ^ 1);
+      __syncthreads();
+    }
+  }
+
+  // ---- add the two query halves, scale, store ----
+  reduce_partner(dkacc, reinterpret_cast<float *>(smem), wi == 1, wj, lane);
+  reduce_partner(dvacc, reinterpret_cast<float *>(smem), wi == 1, wj, lane);
+  if (wi == 1) return;
+  // lane: key 32 wj + li; register 4 q + t of half db: column 32 db + 8 q + 4 kg + t
+#pragma unroll
+  for (int h = 0; h < NH; ++h) {
+    if (pk[h] < 0) continue;
+    char *op = static_cast<char *>(a.dk) + pk[h] * kBlockBytes + (32 * wj + li) * 128 + kg * 8;
+#pragma unroll
+    for (int db = 0; db < 2; ++db)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const f32x16 &acc = dkacc[2 * h + db];
+        u32x2 w;
+        w[0] = Tr::pack2(acc[4 * q] * a.scale, acc[4 * q + 1] * a.scale);
+        w[1] = Tr::pack2(acc[4 * q + 2] * a.scale, acc[4 * q + 3] * a.scale);
+        *reinterpret_cast<u32x2 *>(op + 64 * db + 16 * q) = w;
+      }
+  }
+#pragma unroll
+  for (int h = 0; h < NHV; ++h) {
+    if (pv[h] < 0) continue;
+    char *op = static_cast<char *>(a.dv) + pv[h] * kBlockBytes + (32 * wj + li) * 128 + kg * 8;
+#pragma unroll
+    for (int db = 0; db < 2; ++db)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const f32x16 &acc = dvacc[2 * h + db];
+        u32x2 w;
+        w[0] = Tr::pack2(acc[4 * q], acc[4 * q + 1]);
+        w[1] = Tr::pack2(acc[4 * q + 2], acc[4 * q + 3]);
+        *reinterpret_cast<u32x2 *>(op + 64 * db + 16 * q) = w;
+      }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// dQ of one query block
+template <typename Tr, int NH, int NHV>
+__global__ __launch_bounds__(kBwdThreads, 1) void attn_bwd_q_kernel(bsa_attn_args a) {
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  constexpr int kKRows = 0, kKPairs = NH * kBlockBytes, kVRows = 2 * NH * kBlockBytes;
+  constexpr int kBufBytes = (2 * NH + NHV) * kBlockBytes;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = first_lane(tid >> 6);
+  const int li = lane & 31, kg = lane >> 5;
+  const int wi = wave & 1, wj = wave >> 1;
+  const int64_t qrow = xcd_row();
+  if (qrow >= a.B * a.nq) return;
+  const int64_t b = qrow / a.nq, qb = qrow % a.nq;
+
+  int64_t pq[NH];
+  bool any = false;
+#pragma unroll
+  for (int h = 0; h < NH; ++h) {
+    pq[h] = a.pidx_q[qrow * NH + h];
+    if (pq[h] >= a.n_q_blocks) pq[h] = -1;
+    any = any || pq[h] >= 0;
+  }
+  if (!any) return;
+
+  // this wave's queries: B operands Q[i][.], dO[i][.] with i = 32 wi + li
+  const int qi = 32 * wi + li;
+  u32x4 qfr[NH][4], dofr[NHV][4];
+#pragma unroll
+  for (int h = 0; h < NH; ++h) load_resident(qfr[h], a.q, pq[h], a.n_q_blocks, qi, kg);
+#pragma unroll
+  for (int h = 0; h < NHV; ++h) load_resident(dofr[h], a.d_o, a.pidx_o[qrow * NHV + h], a.n_o_blocks, qi, kg);
+  const float lse = a.lse[qrow * kSbs + qi];
+  const float delta = a.delta[qrow * kSbs + qi];
+
+  f32x16 dqacc[NH * 2];
+#pragma unroll
+  for (int n = 0; n < NH * 2; ++n)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) dqacc[n][r] = 0.f;
+
+  const float qk_scale = a.scale * kLog2e;
+  const bool causal = a.causal_lengths != nullptr;
+  int seq_len = 0;
+  if (causal) {
+    const int64_t len = a.causal_lengths[b];
+    seq_len = len < 0 ? 0 : (len > 0x7fffffffLL ? 0x7fffffff : (int)len);
+  }
+  const int qpos = (int)qb * kSbs + qi;
+
+  const int k_begin = a.key_offsets[qrow], k_end = a.key_offsets[qrow + 1];
+  if (k_begin < k_end) {
+    constexpr int kLaneMask = NH + NHV, kLaneBias = NH + NHV + 1, kLaneEntry = 7;
+    auto gather = [&](int kb, int pos) -> int {
+      const int64_t krow = b * a.nk + kb;
+      const int32_t *p = a.key_indices + pos;
+      bool on = lane == kLaneEntry;
+      if (lane < NH) {
+        p = low_half_ptr(a.pidx_k, krow * NH + lane);
+        on = true;
+      } else if (lane < NH + NHV) {
+        p = low_half_ptr(a.pidx_v, krow * NHV + (lane - NH));
+        on = true;
+      } else if (lane == kLaneMask && a.mask) {
+        p = low_half_ptr(a.pidx_mask, qrow * a.nk + kb);
+        on = true;
+      } else if (lane == kLaneBias && a.bias) {
+        p = low_half_ptr(a.pidx_bias, qrow * a.nk + kb);
+        on = true;
+      }
+      int v = -1;
+      if (on) v = *p;
+      return v;
+    };
+    auto clamp_e = [&](int e) { return e < k_end ? e : k_end - 1; };
+
+    TileRegs kt[NH], vt[NHV];
+    uint32_t mask_w[4];  // mask bytes of keys 32 wj + 8 q + 4 kg .. + 3 of this lane's query, one word per q
+    u32x2 bias_w[4];     // bias elements likewise
+    int kb_nxt, pm_nxt, pb_nxt;
+
+    auto fetch = [&](int rec, int kb) {
+      kb_nxt = kb;
+#pragma unroll
+      for (int h = 0; h < NH; ++h) {
+        const int64_t pk = __builtin_amdgcn_readlane(rec, h);
+        const bool valid = pk >= 0 && pk < a.n_k_blocks;
+        kt[h] = load_tile(static_cast<const char *>(a.k) + (valid ? pk : 0) * kBlockBytes, valid, tid);
+      }
+#pragma unroll
+      for (int h = 0; h < NHV; ++h) {
+        const int64_t pv = __builtin_amdgcn_readlane(rec, NH + h);
+        const bool valid = pv >= 0 && pv < a.n_v_blocks;
+        vt[h] = load_tile(static_cast<const char *>(a.v) + (valid ? pv : 0) * kBlockBytes, valid, tid);
+      }
+      pm_nxt = __builtin_amdgcn_readlane(rec, kLaneMask);
+      if (pm_nxt >= a.n_mask_blocks) pm_nxt = -1;
+      pb_nxt = __builtin_amdgcn_readlane(rec, kLaneBias);
+      if (pb_nxt >= a.n_bias_blocks) pb_nxt = -1;
+      if (pm_nxt >= 0) {
+        const char *mp = static_cast<const char *>(a.mask) + (int64_t)pm_nxt * (kSbs * kSbs);
+        const uint32_t off = (uint32_t)qi * 64u + 32u * wj + 4u * kg;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) mask_w[q] = *reinterpret_cast<const uint32_t *>(mp + off + 8 * q);
+      }
+      if (pb_nxt >= 0) {
+        const char *bp = static_cast<const char *>(a.bias) + (int64_t)pb_nxt * kBlockBytes;
+        const uint32_t off = (uint32_t)qi * 128u + 64u * wj + 8u * kg;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) bias_w[q] = *reinterpret_cast<const u32x2 *>(bp + off + 16 * q);
+      }
+    };
+    auto stage = [&](int buf) {
+      char *base = smem + buf * kBufBytes;
+#pragma unroll
+      for (int h = 0; h < NH; ++h) {
+        stage_rows(base + kKRows + h * kBlockBytes, kt[h], tid);
+        stage_pairs(base + kKPairs + h * kBlockBytes, kt[h], tid);
+      }
+#pragma unroll
+      for (int h = 0; h < NHV; ++h) stage_rows(base + kVRows + h * kBlockBytes, vt[h], tid);
+    };
+
+    int rec, kb_rec;
+    {
+      const int kb0 = first_lane(a.key_indices[as_vector(k_begin)]);
+      const int rec0 = gather(kb0, clamp_e(k_begin + 1));
+      kb_rec = __builtin_amdgcn_readlane(rec0, kLaneEntry);
+      rec = gather(kb_rec, clamp_e(k_begin + 2));
+      fetch(rec0, kb0);
+      stage(0);
+      __syncthreads();
+    }
+
+    for (int e = k_begin; e < k_end; ++e) {
+      const int buf = (e - k_begin) & 1;
+      const char *base = smem + buf * kBufBytes;
+      const int kb = kb_nxt;
+      const int64_t pm = pm_nxt, pb = pb_nxt;
+      uint32_t mask_c[4];
+      u32x2 bias_c[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        mask_c[q] = mask_w[q];
+        bias_c[q] = bias_w[q];
+      }
+      const bool more = e + 1 < k_end;
+      if (more) fetch(rec, kb_rec);
+      kb_rec = __builtin_amdgcn_readlane(rec, kLaneEntry);
+      rec = gather(kb_rec, clamp_e(e + 3));
+
+      // ---- S^T and dP^T of this wave's quadrant: lane owns query qi, register r key 32 wj + 8 (r / 4) + 4 kg + r % 4 ----
+      f32x16 sacc, dpacc;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sacc[r] = dpacc[r] = 0.f;
+#pragma unroll
+      for (int h = 0; h < NH; ++h)
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+          sacc = Tr::mfma(frag_rows(base + kKRows + h * kBlockBytes, 32 * wj + li, 2 * s + kg), qfr[h][s], sacc);
+#pragma unroll
+      for (int h = 0; h < NHV; ++h)
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+          dpacc = Tr::mfma(frag_rows(base + kVRows + h * kBlockBytes, 32 * wj + li, 2 * s + kg), dofr[h][s], dpacc);
+
+      float ds[16];
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const int r = 4 * q + t;
+          float s = sacc[r] * qk_scale;
+          if (pb >= 0) {
+            const uint32_t bw = bias_c[q][t >> 1];
+            s = s + Tr::widen((uint16_t)((t & 1) ? (bw >> 16) : (bw & 0xffffu))) * kLog2e;
+          }
+          if (causal) {
+            const int kpos = kb * kSbs + 32 * wj + 8 * q + 4 * kg + t;
+            s = (kpos > qpos || qpos >= seq_len || kpos >= seq_len) ? -INFINITY : s;
+          }
+          if (pm >= 0) s = ((mask_c[q] >> (8 * t)) & 0xffu) ? -INFINITY : s;
+          const float p = (lse == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(s - lse);
+          ds[r] = p * (dpacc[r] - delta);
+        }
+      u32x4 dsf[2];
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) dsf[u][t] = Tr::pack2(ds[8 * u + 2 * t], ds[8 * u + 2 * t + 1]);
+
+      // ---- dQ^T += K^T dS^T over this wave's 32 keys ----
+#pragma unroll
+      for (int h = 0; h < NH; ++h)
+#pragma unroll
+        for (int db = 0; db < 2; ++db)
+#pragma unroll
+          for (int u = 0; u < 2; ++u)
+            dqacc[2 * h + db] = Tr::mfma(frag_pairs(base + kKPairs + h * kBlockBytes, 32 * db + li, 16 * wj + 8 * u + 2 * kg),
+                                         dsf[u], dqacc[2 * h + db]);
+
+      if (more) stage(buf ^ 1);
+      __syncthreads();
+    }
+  }
+
+  // ---- add the two key halves, scale, store ----
+  reduce_partner(dqacc, reinterpret_cast<float *>(smem), wj == 1, wi, lane);
+  if (wj == 1) return;
+#pragma unroll
+  for (int h = 0; h < NH; ++h) {
+    if (pq[h] < 0) continue;
+    char *op = static_cast<char *>(a.dq) + pq[h] * kBlockBytes + qi * 128 + kg * 8;
+#pragma unroll
+    for (int db = 0; db < 2; ++db)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const f32x16 &acc = dqacc[2 * h + db];
+        u32x2 w;
+        w[0] = Tr::pack2(acc[4 * q] * a.scale, acc[4 * q + 1] * a.scale);
+        w[1] = Tr::pack2(acc[4 * q + 2] * a.scale, acc[4 * q + 3] * a.scale);
+        *reinterpret_cast<u32x2 *>(op + 64 * db + 16 * q) = w;
+      }
+  }
+}
+
+__global__ void fill_zero_f32_kernel(float *p, int64_t n) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) p[i] = 0.f;
+}
+
+template <typename Tr, int NH, int NHV>
+int launch_bwd(const bsa_attn_args &a, hipStream_t s) {
+  const int64_t qrows = a.B * a.nq, krows = a.B * a.nk;
+  if (a.dbias && a.n_bias_blocks > 0) {
+    // bias blocks outside the attention layout get no gradient
+    const int64_t n = a.n_bias_blocks * kSbs * kSbs;
+    int64_t blocks = cdiv(n, 1024);
+    if (blocks > 65536) blocks = 65536;
+    fill_zero_f32_kernel<<<(unsigned)blocks, 256, 0, s>>>(a.dbias, n);
+    if (int rc = check_launch("fill_zero_f32_kernel")) return rc;
+  }
+  if (qrows > 0) {
+    attn_bwd_delta_kernel<Tr><<<(unsigned)qrows, kBwdThreads, 0, s>>>(a);
+    if (int rc = check_launch("attn_bwd_delta_kernel")) return rc;
+  }
+  if (krows > 0) {
+    constexpr int lds = 2 * (2 * (NH + NHV) * kBlockBytes + kStatBytes);
+    BSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_bwd_kv_kernel<Tr, NH, NHV>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    attn_bwd_kv_kernel<Tr, NH, NHV><<<(unsigned)(cdiv(krows, 8) * 8), kBwdThreads, lds, s>>>(a);
+    if (int rc = check_launch("attn_bwd_kv_kernel")) return rc;
+  }
+  if (qrows > 0) {
+    constexpr int lds = 2 * (2 * NH + NHV) * kBlockBytes;
+    BSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_bwd_q_kernel<Tr, NH, NHV>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    attn_bwd_q_kernel<Tr, NH, NHV><<<(unsigned)(cdiv(qrows, 8) * 8), kBwdThreads, lds, s>>>(a);
+    if (int rc = check_launch("attn_bwd_q_kernel")) return rc;
+  }
+  return BSA_OK;
+}
+
+template <typename Tr>
+int dispatch_bwd(const bsa_attn_args &a, hipStream_t s) {
+  if (a.nh == 1 && a.nhv == 1) return launch_bwd<Tr, 1, 1>(a, s);
+  if (a.nh == 2 && a.nhv == 2) return launch_bwd<Tr, 2, 2>(a, s);
+  if (a.nh == 1 && a.nhv == 2) return launch_bwd<Tr, 1, 2>(a, s);
+  if (a.nh == 2 && a.nhv == 1) return launch_bwd<Tr, 2, 1>(a, s);
+  return 1;
+}
+
+}  // namespace
+
+int attn_bwd_mfma(const bsa_attn_args &a, hipStream_t s) {
+  if (a.sbs != kSbs || (a.dtype != BSA_BF16 && a.dtype != BSA_F16)) return 1;
+  if ((a.B * a.nq > 0 && a.key_indices == nullptr) || (a.B * a.nk > 0 && a.query_indices == nullptr)) return 1;
+  return a.dtype == BSA_BF16 ? dispatch_bwd<MBf16>(a, s) : dispatch_bwd<MF16>(a, s);
+}
+
+}  // namespace bsa

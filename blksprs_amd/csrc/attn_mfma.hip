@@ -29,7 +29,7 @@
 // Score pipeline (log2 domain), in this order: scale * q k^T, + bias, native causal
 // predicate, explicit mask; probabilities are rounded to the operand type before they
 // multiply V; the row sum uses the unrounded values.
-#include "attn_common.h"
+#include "attn_mfma_common.h"
 
 // Phase clocks for an offline timing harness; compiled out of the library.
 #ifdef BSA_ATTN_PROBE
@@ -55,78 +55,10 @@ __device__ unsigned long long bsa_attn_probe[8 * 4096];
 namespace bsa {
 namespace {
 
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+using namespace mfma;
 
-struct MBf16 {
-  __device__ static f32x16 mfma(u32x4 a, u32x4 b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
-                                                   0, 0, 0);
-  }
-  __device__ static uint32_t pack2(float lo, float hi) {
-    bf16x2 v = {(__bf16)lo, (__bf16)hi};
-    return __builtin_bit_cast(uint32_t, v);
-  }
-  __device__ static float widen(uint16_t h) { return __builtin_bit_cast(float, (uint32_t)h << 16); }
-};
-
-struct MF16 {
-  __device__ static f32x16 mfma(u32x4 a, u32x4 b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0,
-                                                  0, 0);
-  }
-  __device__ static uint32_t pack2(float lo, float hi) {
-    f16x2 v = {(_Float16)lo, (_Float16)hi};
-    return __builtin_bit_cast(uint32_t, v);
-  }
-  __device__ static float widen(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
-};
-
-constexpr int kSbs = 64;
-constexpr int kBlockBytes = kSbs * kSbs * 2;  // one 16-bit block
 constexpr int kFwdThreads = 256;
 constexpr float kRescaleStep = 8.f;  // log2 units
-
-// XOR applied to the 16-byte chunk index of K tile row r in LDS.  Two 128-byte rows span the 64 banks once, so
-// the 16 lanes a 128-bit read serves together (16 consecutive rows, one chunk each) are conflict free when
-// rows of equal parity get eight different values.
-__device__ inline int k_swizzle(int r) { return (r >> 1) & 7; }
-
-// dword offset of column c in a pair row of the (j, j+1)-packed V tile; the placement of the column
-// quads keeps both the 128-bit writes of the staging step and the 32-bit fragment reads conflict free
-__device__ inline int pair_col_offset(int c) {
-  const int q = c >> 2, a = q >> 1, h = q & 1;
-  const int pos = ((a + 4 * h) & 7) + 8 * h;
-  return 4 * pos + (c & 3);
-}
-
-__device__ inline int first_lane(int v) { return __builtin_amdgcn_readfirstlane(v); }
-typedef __attribute__((address_space(3))) void *lds_ptr_t;
-
-// Asynchronous copy of 64 x 16 bytes, global -> LDS: lane l's 16 bytes land at dst + 16 l (dst is wave
-// uniform).  Completion is counted by vmcnt like any vector load.  Written as inline assembly so that the
-// compiler's wait-count pass does not see it: it would otherwise wait for the copy in front of every later
-// LDS read, also reads of other LDS arrays.  m0 is reserved: the compiler sets it before each of its own
-// uses and keeps nothing in it across statements.  The caller waits (vmcnt(0)) before the data is read.  Copies
-// the compiler does not know about only make the waits it computes for its own loads longer, never shorter.
-// The source is base (wave uniform) + off (per lane, 32 bits).
-__device__ inline void copy_1k_to_lds(const char *base, uint32_t off, char *dst) {
-  const uint32_t lds_addr = (uint32_t)(uintptr_t)(lds_ptr_t)dst;
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-               :
-               : "v"(off), "s"(base), "s"(lds_addr)
-               : "memory");
-}
-
-// 16 bytes at base (wave uniform) + off (per lane): scalar base, 32-bit vector offset addressing
-__device__ inline u32x4 load16(const char *base, uint32_t off) {
-  return *reinterpret_cast<const u32x4 *>(base + off);
-}
 
 // One workgroup (four waves) owns a PAIR of neighbouring query blocks and walks the union of their key lists,
 // so that a K / V tile both of them need is fetched once; bits 28 and 29 of a list entry say which of the
@@ -626,6 +558,5 @@ int attn_fwd_records(const bsa_attn_args &a, const int32_t *entries, int32_t *re
   return check_launch("attn_fwd_records_kernel");
 }
 
-int attn_bwd_mfma(const bsa_attn_args &, hipStream_t) { return 1; }
 
 }  // namespace bsa
