@@ -332,87 +332,102 @@ __global__ __launch_bounds__(kBwdThreads, 1) void attn_bwd_kv_kernel(bsa_attn_ar
       // facts and per-element inputs of tile e, before the fetch of tile e+1 replaces them
       const int qb = qb_nxt;
       const int64_t pm = pm_nxt, pb = pb_nxt;
-      uint32_t mask_c[16], bias_c[16];
+      // mask bytes (0 or 1) of the 16 elements -> one bit each, which frees their registers for the next tile
+      uint32_t mbits = 0;
+      if (pm >= 0) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        mask_c[r] = mask_b[r];
-        bias_c[r] = bias_b[r];
+        for (int r = 0; r < 16; ++r) mbits |= mask_b[r] << r;
+      }
+      uint32_t bias_c[16];
+      if (pb >= 0) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) bias_c[r] = bias_b[r];
       }
       const bool more = e + 1 < q_end;
       if (more) fetch(rec, qb_rec);
       qb_rec = __builtin_amdgcn_readlane(rec, kLaneEntry);
       rec = gather(qb_rec, clamp_e(e + 3));
 
-      // ---- S and dP of this wave's quadrant ----
-      f32x16 sacc, dpacc;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) sacc[r] = dpacc[r] = 0.f;
-#pragma unroll
-      for (int h = 0; h < NH; ++h)
-#pragma unroll
-        for (int s = 0; s < 4; ++s)
-          sacc = Tr::mfma(frag_rows(base + kQRows + h * kBlockBytes, 32 * wi + li, 2 * s + kg), kfr[h][s], sacc);
-#pragma unroll
-      for (int h = 0; h < NHV; ++h)
-#pragma unroll
-        for (int s = 0; s < 4; ++s)
-          dpacc = Tr::mfma(frag_rows(base + kDoRows + h * kBlockBytes, 32 * wi + li, 2 * s + kg), vfr[h][s], dpacc);
+      // A quadrant whose every score is masked has P = dS = 0: nothing to add, nothing to compute.
+      bool live = true;
+      if (pm >= 0) live = !__all(mbits == 0xffffu);
+      if (causal) {
+        const int k_first = (int)kb * kSbs + 32 * wj, q_first = qb * kSbs + 32 * wi;
+        if (k_first > q_first + 31 || q_first >= seq_len || k_first >= seq_len) live = false;
+      }
+      if (live) {
+        // ---- S and dP of this wave's quadrant ----
+        f32x16 sacc, dpacc;
+  #pragma unroll
+        for (int r = 0; r < 16; ++r) sacc[r] = dpacc[r] = 0.f;
+  #pragma unroll
+        for (int h = 0; h < NH; ++h)
+  #pragma unroll
+          for (int s = 0; s < 4; ++s)
+            sacc = Tr::mfma(frag_rows(base + kQRows + h * kBlockBytes, 32 * wi + li, 2 * s + kg), kfr[h][s], sacc);
+  #pragma unroll
+        for (int h = 0; h < NHV; ++h)
+  #pragma unroll
+          for (int s = 0; s < 4; ++s)
+            dpacc = Tr::mfma(frag_rows(base + kDoRows + h * kBlockBytes, 32 * wi + li, 2 * s + kg), vfr[h][s], dpacc);
 
-      // ---- P and dS; element r: query 32 wi + 8 (r / 4) + 4 kg + r % 4 ----
-      const float *stats = reinterpret_cast<const float *>(base + kStats);
-      float p[16], ds[16];
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int i0 = 32 * wi + 8 * q + 4 * kg;
-        const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(stats + i0);
-        const f32x4 del4 = *reinterpret_cast<const f32x4 *>(stats + kSbs + i0);
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          const int r = 4 * q + t;
-          float s = sacc[r] * qk_scale;
-          if (pb >= 0) s = s + Tr::widen((uint16_t)bias_c[r]) * kLog2e;
-          if (causal) {
-            const int qpos = qb * kSbs + i0 + t;
-            s = (kpos > qpos || qpos >= seq_len || kpos >= seq_len) ? -INFINITY : s;
+        // ---- P and dS; element r: query 32 wi + 8 (r / 4) + 4 kg + r % 4 ----
+        const float *stats = reinterpret_cast<const float *>(base + kStats);
+        float p[16], ds[16];
+  #pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int i0 = 32 * wi + 8 * q + 4 * kg;
+          const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(stats + i0);
+          const f32x4 del4 = *reinterpret_cast<const f32x4 *>(stats + kSbs + i0);
+  #pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            const int r = 4 * q + t;
+            float s = sacc[r] * qk_scale;
+            if (pb >= 0) s = s + Tr::widen((uint16_t)bias_c[r]) * kLog2e;
+            if (causal) {
+              const int qpos = qb * kSbs + i0 + t;
+              s = (kpos > qpos || qpos >= seq_len || kpos >= seq_len) ? -INFINITY : s;
+            }
+            if (pm >= 0) s = ((mbits >> r) & 1u) ? -INFINITY : s;
+            const float lse = lse4[t];
+            p[r] = (lse == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(s - lse);
+            ds[r] = p[r] * (dpacc[r] - del4[t]);
           }
-          if (pm >= 0) s = mask_c[r] ? -INFINITY : s;
-          const float lse = lse4[t];
-          p[r] = (lse == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(s - lse);
-          ds[r] = p[r] * (dpacc[r] - del4[t]);
         }
-      }
-      if (a.dbias != nullptr && pb >= 0) {
-        // every (query block, key block) pair is visited once, so this is a plain store
-        float *dbp = a.dbias + pb * (kSbs * kSbs) + (32 * wi + 4 * kg) * kSbs + 32 * wj + li;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) dbp[(8 * (r >> 2) + (r & 3)) * kSbs] = ds[r];
-      }
-      u32x4 pf[2], dsf[2];
-#pragma unroll
-      for (int u = 0; u < 2; ++u)
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          pf[u][t] = Tr::pack2(p[8 * u + 2 * t], p[8 * u + 2 * t + 1]);
-          dsf[u][t] = Tr::pack2(ds[8 * u + 2 * t], ds[8 * u + 2 * t + 1]);
+        if (a.dbias != nullptr && pb >= 0) {
+          // every (query block, key block) pair is visited once, so this is a plain store
+          float *dbp = a.dbias + pb * (kSbs * kSbs) + (32 * wi + 4 * kg) * kSbs + 32 * wj + li;
+  #pragma unroll
+          for (int r = 0; r < 16; ++r) dbp[(8 * (r >> 2) + (r & 3)) * kSbs] = ds[r];
         }
+        u32x4 pf[2], dsf[2];
+  #pragma unroll
+        for (int u = 0; u < 2; ++u)
+  #pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            pf[u][t] = Tr::pack2(p[8 * u + 2 * t], p[8 * u + 2 * t + 1]);
+            dsf[u][t] = Tr::pack2(ds[8 * u + 2 * t], ds[8 * u + 2 * t + 1]);
+          }
 
-      // ---- dV^T += dO^T P, dK^T += Q^T dS over this wave's 32 queries ----
-#pragma unroll
-      for (int h = 0; h < NHV; ++h)
-#pragma unroll
-        for (int db = 0; db < 2; ++db)
-#pragma unroll
-          for (int u = 0; u < 2; ++u)
-            dvacc[2 * h + db] = Tr::mfma(frag_pairs(base + kDoPairs + h * kBlockBytes, 32 * db + li, 16 * wi + 8 * u + 2 * kg),
-                                         pf[u], dvacc[2 * h + db]);
-#pragma unroll
-      for (int h = 0; h < NH; ++h)
-#pragma unroll
-        for (int db = 0; db < 2; ++db)
-#pragma unroll
-          for (int u = 0; u < 2; ++u)
-            dkacc[2 * h + db] = Tr::mfma(frag_pairs(base + kQPairs + h * kBlockBytes, 32 * db + li, 16 * wi + 8 * u + 2 * kg),
-                                         dsf[u], dkacc[2 * h + db]);
+        // ---- dV^T += dO^T P, dK^T += Q^T dS over this wave's 32 queries ----
+  #pragma unroll
+        for (int h = 0; h < NHV; ++h)
+  #pragma unroll
+          for (int db = 0; db < 2; ++db)
+  #pragma unroll
+            for (int u = 0; u < 2; ++u)
+              dvacc[2 * h + db] = Tr::mfma(frag_pairs(base + kDoPairs + h * kBlockBytes, 32 * db + li, 16 * wi + 8 * u + 2 * kg),
+                                           pf[u], dvacc[2 * h + db]);
+  #pragma unroll
+        for (int h = 0; h < NH; ++h)
+  #pragma unroll
+          for (int db = 0; db < 2; ++db)
+  #pragma unroll
+            for (int u = 0; u < 2; ++u)
+              dkacc[2 * h + db] = Tr::mfma(frag_pairs(base + kQPairs + h * kBlockBytes, 32 * db + li, 16 * wi + 8 * u + 2 * kg),
+                                           dsf[u], dkacc[2 * h + db]);
+
+      }  // live
 
       // ---- tile e+1 into the other buffer; the barrier also ends the reads of tile e ----
       if (more) stage(buf ^ 1);
@@ -600,64 +615,74 @@ __global__ __launch_bounds__(kBwdThreads, 1) void attn_bwd_q_kernel(bsa_attn_arg
       uint32_t mask_c[4];
       u32x2 bias_c[4];
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        mask_c[q] = mask_w[q];
-        bias_c[q] = bias_w[q];
+      for (int q = 0; q < 4; ++q) mask_c[q] = mask_w[q];
+      if (pb >= 0) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) bias_c[q] = bias_w[q];
       }
       const bool more = e + 1 < k_end;
       if (more) fetch(rec, kb_rec);
       kb_rec = __builtin_amdgcn_readlane(rec, kLaneEntry);
       rec = gather(kb_rec, clamp_e(e + 3));
 
-      // ---- S^T and dP^T of this wave's quadrant: lane owns query qi, register r key 32 wj + 8 (r / 4) + 4 kg + r % 4 ----
-      f32x16 sacc, dpacc;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) sacc[r] = dpacc[r] = 0.f;
-#pragma unroll
-      for (int h = 0; h < NH; ++h)
-#pragma unroll
-        for (int s = 0; s < 4; ++s)
-          sacc = Tr::mfma(frag_rows(base + kKRows + h * kBlockBytes, 32 * wj + li, 2 * s + kg), qfr[h][s], sacc);
-#pragma unroll
-      for (int h = 0; h < NHV; ++h)
-#pragma unroll
-        for (int s = 0; s < 4; ++s)
-          dpacc = Tr::mfma(frag_rows(base + kVRows + h * kBlockBytes, 32 * wj + li, 2 * s + kg), dofr[h][s], dpacc);
+      bool live = true;
+      if (pm >= 0) live = !__all((mask_c[0] & mask_c[1] & mask_c[2] & mask_c[3]) == 0x01010101u);
+      if (causal) {
+        const int k_first = kb * kSbs + 32 * wj, q_first = (int)qb * kSbs + 32 * wi;
+        if (k_first > q_first + 31 || q_first >= seq_len || k_first >= seq_len) live = false;
+      }
+      if (live) {
+        // ---- S^T and dP^T of this wave's quadrant: lane owns query qi, register r key 32 wj + 8 (r / 4) + 4 kg + r % 4 ----
+        f32x16 sacc, dpacc;
+  #pragma unroll
+        for (int r = 0; r < 16; ++r) sacc[r] = dpacc[r] = 0.f;
+  #pragma unroll
+        for (int h = 0; h < NH; ++h)
+  #pragma unroll
+          for (int s = 0; s < 4; ++s)
+            sacc = Tr::mfma(frag_rows(base + kKRows + h * kBlockBytes, 32 * wj + li, 2 * s + kg), qfr[h][s], sacc);
+  #pragma unroll
+        for (int h = 0; h < NHV; ++h)
+  #pragma unroll
+          for (int s = 0; s < 4; ++s)
+            dpacc = Tr::mfma(frag_rows(base + kVRows + h * kBlockBytes, 32 * wj + li, 2 * s + kg), dofr[h][s], dpacc);
 
-      float ds[16];
-#pragma unroll
-      for (int q = 0; q < 4; ++q)
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          const int r = 4 * q + t;
-          float s = sacc[r] * qk_scale;
-          if (pb >= 0) {
-            const uint32_t bw = bias_c[q][t >> 1];
-            s = s + Tr::widen((uint16_t)((t & 1) ? (bw >> 16) : (bw & 0xffffu))) * kLog2e;
+        float ds[16];
+  #pragma unroll
+        for (int q = 0; q < 4; ++q)
+  #pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            const int r = 4 * q + t;
+            float s = sacc[r] * qk_scale;
+            if (pb >= 0) {
+              const uint32_t bw = bias_c[q][t >> 1];
+              s = s + Tr::widen((uint16_t)((t & 1) ? (bw >> 16) : (bw & 0xffffu))) * kLog2e;
+            }
+            if (causal) {
+              const int kpos = kb * kSbs + 32 * wj + 8 * q + 4 * kg + t;
+              s = (kpos > qpos || qpos >= seq_len || kpos >= seq_len) ? -INFINITY : s;
+            }
+            if (pm >= 0) s = ((mask_c[q] >> (8 * t)) & 0xffu) ? -INFINITY : s;
+            const float p = (lse == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(s - lse);
+            ds[r] = p * (dpacc[r] - delta);
           }
-          if (causal) {
-            const int kpos = kb * kSbs + 32 * wj + 8 * q + 4 * kg + t;
-            s = (kpos > qpos || qpos >= seq_len || kpos >= seq_len) ? -INFINITY : s;
-          }
-          if (pm >= 0) s = ((mask_c[q] >> (8 * t)) & 0xffu) ? -INFINITY : s;
-          const float p = (lse == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(s - lse);
-          ds[r] = p * (dpacc[r] - delta);
-        }
-      u32x4 dsf[2];
-#pragma unroll
-      for (int u = 0; u < 2; ++u)
-#pragma unroll
-        for (int t = 0; t < 4; ++t) dsf[u][t] = Tr::pack2(ds[8 * u + 2 * t], ds[8 * u + 2 * t + 1]);
+        u32x4 dsf[2];
+  #pragma unroll
+        for (int u = 0; u < 2; ++u)
+  #pragma unroll
+          for (int t = 0; t < 4; ++t) dsf[u][t] = Tr::pack2(ds[8 * u + 2 * t], ds[8 * u + 2 * t + 1]);
 
-      // ---- dQ^T += K^T dS^T over this wave's 32 keys ----
-#pragma unroll
-      for (int h = 0; h < NH; ++h)
-#pragma unroll
-        for (int db = 0; db < 2; ++db)
-#pragma unroll
-          for (int u = 0; u < 2; ++u)
-            dqacc[2 * h + db] = Tr::mfma(frag_pairs(base + kKPairs + h * kBlockBytes, 32 * db + li, 16 * wj + 8 * u + 2 * kg),
-                                         dsf[u], dqacc[2 * h + db]);
+        // ---- dQ^T += K^T dS^T over this wave's 32 keys ----
+  #pragma unroll
+        for (int h = 0; h < NH; ++h)
+  #pragma unroll
+          for (int db = 0; db < 2; ++db)
+  #pragma unroll
+            for (int u = 0; u < 2; ++u)
+              dqacc[2 * h + db] = Tr::mfma(frag_pairs(base + kKPairs + h * kBlockBytes, 32 * db + li, 16 * wj + 8 * u + 2 * kg),
+                                           dsf[u], dqacc[2 * h + db]);
+
+      }  // live
 
       if (more) stage(buf ^ 1);
       __syncthreads();
