@@ -112,7 +112,7 @@ def matmul_workload(name, B, n, sbs, dtype, density, ensure_rows, value_scale, d
 
     dt_name = {torch.bfloat16: "bf16", torch.float16: "f16", torch.float32: "f32"}[dtype]
     return dict(step=step, flops=flops, alg_bytes=alg_bytes, dtype=dt_name, bound="hbm", cpu_baseline=cpu_baseline,
-                kernel="matmul_mfma_kernel" if sbs > 16 else "matmul_small_kernel",
+                kernel=("matmul_panel_kernel" if sbs == 64 and dtype != torch.float32 else "matmul_mfma_kernel") if sbs > 16 else "matmul_small_kernel",
                 config={"workload": name, "B": B, "M": n * sbs, "K": n * sbs, "N": n * sbs,
                         "sparsity_block_size": sbs, "density": density, "nnz_x": nnz_x, "nnz_y": nnz_y,
                         "nnz_o": nnz_o, "block_pairs": pairs, "lut_build_ms": round(lut_ms, 3)})
