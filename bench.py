@@ -33,6 +33,26 @@ PEAK_HBM_GBS = 8000.0
 PEAK_MFMA_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}
 
 
+# HBM bytes per launch of the dominant kernel: FETCH_SIZE and WRITE_SIZE (KiB per dispatch) from the rocprofv3
+# --pmc runs summarised under profiles/ (one file per kernel and configuration), scaled by what the same
+# counters read for a plain copy kernel of known size (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).  FETCH_SIZE counts
+# what leaves an L2, so reads served by the memory-side cache are included.  Not re-measured by this script.
+TRAFFIC_KIB = {  # config: (FETCH_SIZE, WRITE_SIZE)
+    "c1": (616.2, 476.0),
+    "c2": (592501.7, 514960.0),
+    "c3": (148346.4, 296128.0),
+    "c4": (548540.2, 133281.6),
+    "c5": (127107.7, 143960.0),
+}
+
+
+def traffic_bytes(config):
+    if config not in TRAFFIC_KIB:
+        return None
+    fetch, write = TRAFFIC_KIB[config]
+    return int((2.0 * fetch + 1.0 * write) * 1024)
+
+
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
@@ -207,7 +227,8 @@ def attention_workload(dev, backward):
                 "sample": f"forward of {heads} of {BH} heads, dense masked fp32 torch attention, {dt:.2f} s"}
 
     return dict(step=step, flops=flops, alg_bytes=alg_bytes, dtype="bf16", bound="mfma", cpu_baseline=cpu_baseline,
-                kernel="attn_fwd",
+                kernel="attn_fwd_mfma_kernel" if not backward else
+                "attn_fwd_mfma_kernel + attn_bwd_delta_kernel + attn_bwd_kv_kernel + attn_bwd_q_kernel (one step)",
                 config={"workload": "c4_flash_attention_bf16" + ("_fwd_bwd" if backward else "_fwd"),
                         "batch_heads": BH, "seq": n * sbs, "head_dim": nh * sbs, "sparsity_block_size": sbs,
                         "layout_blocks": nnz, "mask": "explicit causal blocks"})
@@ -256,6 +277,8 @@ def main():
         peak = PEAK_MFMA_TFLOPS[w["dtype"]]
         roofline = {"bound": "mfma", "achieved": round(ach, 1), "peak": peak, "unit": "TFLOP/s",
                     "frac": round(ach / peak, 4), "traffic": None}
+    roofline["traffic"] = traffic_bytes(args.config)
+    roofline["algorithmic_bytes"] = int(w["alg_bytes"])
     roofline["kernel"] = w["kernel"]
     roofline["launch_ms_mean"] = round(mean_ms, 4)
     roofline["launch_ms_median"] = round(median_ms, 4)
