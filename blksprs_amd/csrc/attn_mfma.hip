@@ -14,10 +14,10 @@
 // and the probabilities of S^T are, as they sit in registers, the B operand of the
 // second product: registers 8u .. 8u+7 of key half jb cover keys
 // 32 jb + 16 u + {4 kg .. 4 kg + 3, 8 + 4 kg .. 8 + 4 kg + 3} (kg = l / 32), and the V
-// fragment is gathered from LDS for exactly that key set.  V is kept in LDS as
-// (j, j+1) pairs per column (interleaved in registers with v_perm_b32 before the LDS
-// write) so that its fragment is four conflict-free 32-bit reads; K is kept row-major
-// with XOR-swizzled 16-byte chunks and its fragment is one 128-bit read.
+// fragment is gathered from LDS for exactly that key set.  K and V are both kept
+// row-major in LDS with XOR-swizzled 16-byte chunks: a K fragment (head dimension
+// contracted) is one 128-bit read, a V fragment (key index contracted) is two
+// transposing 64-bit reads (ds_read_b64_tr_b16), so neither tile passes through registers.
 //
 // The K / V tiles of key block e+1, the mask words of e+1, the packed indices of e+2
 // and the key index of e+3 are all fetched while block e is computed.  The index
@@ -131,7 +131,6 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
 
   BSA_PROBE_DECL;
   if (k_begin < k_end) {
-    u32x4 vr[NHV][2];  // staging registers of the V tile in flight
     u32x4 mask_raw[2];
     // wave-uniform facts about the key block whose tiles are in flight
     int ent_nxt, pm_nxt, pb_nxt;
@@ -161,47 +160,34 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
       }
     };
 
-    // facts and V tile of one key block
-    auto fetch_v = [&](const AttnFwdRecord &r) {
+    // facts of one key block
+    auto fetch_facts = [&](const AttnFwdRecord &r) {
       ent_nxt = r.entry;
       pm_nxt = a.mask ? ((wave >> 1) ? r.pm[1] : r.pm[0]) : -1;
       if (pm_nxt >= a.n_mask_blocks) pm_nxt = -1;
       pb_nxt = a.bias ? ((wave >> 1) ? r.pb[1] : r.pb[0]) : -1;
       if (pb_nxt >= a.n_bias_blocks) pb_nxt = -1;
+    };
+
+    // V tile: copied like the K tile, row-major, with the chunk swizzle of the transposing LDS load that
+    // turns its rows into matrix-core operands later
+    auto copy_v = [&](const AttnFwdRecord &r, int buf) {
 #pragma unroll
       for (int h = 0; h < NHV; ++h) {
         const int64_t pv = r.pv[h];
-        const bool valid = pv >= 0 && pv < a.n_v_blocks;
-        const char *vp = static_cast<const char *>(a.v) + (valid ? pv : 0) * kBlockBytes;
-        // thread tid stages rows 2 jp, 2 jp + 1 (jp = tid / 8), columns 8 (tid % 8) .. + 7
-        const uint32_t voff = (uint32_t)(tid >> 3) * 256u + (uint32_t)(tid & 7) * 16u;
-        vr[h][0] = u32x4{0u, 0u, 0u, 0u};
-        vr[h][1] = u32x4{0u, 0u, 0u, 0u};
-        if (valid) {
-          vr[h][0] = load16(vp, voff);
-          vr[h][1] = load16(vp + 128, voff);
-        }
-      }
-    };
-
-    // V tile in registers -> LDS as (j, j+1) pairs
-    auto stage_v = [&](int buf) {
+        char *dst = lds_v + buf * kVBytes + h * kBlockBytes;
+        if (pv >= 0 && pv < a.n_v_blocks) {
 #pragma unroll
-      for (int h = 0; h < NHV; ++h) {
-        const int ro = tid & 7, jp = tid >> 3;
-        const u32x4 ev = vr[h][0], od = vr[h][1];
-        u32x4 lo, hi;
-        lo[0] = __builtin_amdgcn_perm(od[0], ev[0], 0x05040100u);
-        lo[1] = __builtin_amdgcn_perm(od[0], ev[0], 0x07060302u);
-        lo[2] = __builtin_amdgcn_perm(od[1], ev[1], 0x05040100u);
-        lo[3] = __builtin_amdgcn_perm(od[1], ev[1], 0x07060302u);
-        hi[0] = __builtin_amdgcn_perm(od[2], ev[2], 0x05040100u);
-        hi[1] = __builtin_amdgcn_perm(od[2], ev[2], 0x07060302u);
-        hi[2] = __builtin_amdgcn_perm(od[3], ev[3], 0x05040100u);
-        hi[3] = __builtin_amdgcn_perm(od[3], ev[3], 0x07060302u);
-        uint32_t *prow = reinterpret_cast<uint32_t *>(lds_v + buf * kVBytes + h * kBlockBytes) + jp * kSbs;
-        *reinterpret_cast<u32x4 *>(prow + pair_col_offset(ro * 8)) = lo;
-        *reinterpret_cast<u32x4 *>(prow + pair_col_offset(ro * 8 + 4)) = hi;
+          for (int i = 0; i < 2; ++i) {
+            const int r0 = 16 * wave + 8 * i;
+            const uint32_t lane_off = (lane >> 3) * 128 + (((lane & 7) ^ t_swizzle(8 * i + (lane >> 3))) << 4);
+            const char *vp = static_cast<const char *>(a.v) + pv * kBlockBytes + r0 * 128;
+            copy_1k_to_lds(vp, lane_off, dst + r0 * 128);
+          }
+        } else {
+#pragma unroll
+          for (int i = 0; i < 2; ++i) *reinterpret_cast<u32x4 *>(dst + (i * kThreads + tid) * 16) = u32x4{0u, 0u, 0u, 0u};
+        }
       }
     };
 
@@ -253,10 +239,10 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
     {
       const AttnFwdRecord r0 = unpack_record(load_record(k_begin));
       rv_next = load_record(clamp_e(k_begin + 1));
-      fetch_v(r0);
+      fetch_facts(r0);
       copy_k(r0, 0);
+      copy_v(r0, 0);
       fetch_mask();
-      stage_v(0);
       __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the K rows this wave copied are in LDS
       __syncthreads();
     }
@@ -282,8 +268,9 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
       const bool more = e + 1 < k_end;
       if (more) {
         const AttnFwdRecord r_next = unpack_record(rv_next);
-        fetch_v(r_next);
+        fetch_facts(r_next);
         copy_k(r_next, buf ^ 1);
+        copy_v(r_next, buf ^ 1);
         fetch_mask();
       }
       rv_next = rv_after;
@@ -341,14 +328,9 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
         auto read_vbatch = [&](u32x4 (&dst)[2], int g) {
           const int h = g >> 2, jq = g & 3;
 #pragma unroll
-          for (int db = 0; db < 2; ++db) {
-            const uint32_t *vp = reinterpret_cast<const uint32_t *>(vbuf + h * kBlockBytes) +
-                                 pair_col_offset(32 * db + li) + (2 * kg + 8 * jq) * kSbs;
-            dst[db][0] = vp[0];
-            dst[db][1] = vp[kSbs];
-            dst[db][2] = vp[4 * kSbs];
-            dst[db][3] = vp[5 * kSbs];
-          }
+          for (int db = 0; db < 2; ++db)
+            // keys 16 jq + 4 kg .. + 3 and + 8 .. + 11, column 32 db + lane % 32
+            dst[db] = frag_cols_t(vbuf + h * kBlockBytes, 16 * jq + 4 * kg, 32 * db + 16 * ((lane >> 4) & 1), lane);
         };
         read_vbatch(vf[0], 0);
         __builtin_amdgcn_sched_barrier(0);
@@ -457,9 +439,8 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
         BSA_PROBE(3);
       }  // live
 
-      // ---- tile e+1 into LDS; the barrier also ends the reads of tile e ----
-      if (more) stage_v(buf ^ 1);
-      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the K rows this wave copied are in LDS
+      // ---- the barrier ends the reads of tile e and publishes tile e+1 ----
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the K and V rows this wave copied are in LDS
       BSA_PROBE(4);
       __syncthreads();
       BSA_PROBE(5);

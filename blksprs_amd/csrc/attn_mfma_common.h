@@ -47,6 +47,29 @@ constexpr int kBlockBytes = kSbs * kSbs * 2;  // one 16-bit block
 // rows of equal parity get eight different values.
 __device__ static inline int k_swizzle(int r) { return (r >> 1) & 7; }
 
+// XOR applied to the 16-byte chunk index of row r of a tile that is read with the transposing LDS load: one
+// such load serves 16 lanes with four rows r .. r + 3 and two neighbouring chunks of each, so rows two apart
+// must be shifted by two chunks.
+__device__ static inline int t_swizzle(int r) { return ((r >> 1) & 3) << 1; }
+
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+
+// Operand fragment whose eight contraction indices run over the ROWS of a row-major 64 x 64 16-bit tile
+// (chunks swizzled with t_swizzle): lane l gets column col0 + l % 16 of rows row0 .. + 3 and row0 + 8 .. + 11,
+// where col0 and row0 may differ between the four 16-lane groups.  The transposing load gives lane i of a
+// group element t = tile[row0 + t][col0 + i] when lane s of the group points at tile[row0 + s / 4][col0 + 4 (s % 4)].
+__device__ static inline u32x4 frag_cols_t(const char *lds, int row0, int col0, int lane) {
+  const int s = lane & 15;
+  const int r = row0 + (s >> 2), c = col0 + 4 * (s & 3);
+  const char *p0 = lds + r * 128 + ((((c >> 3) ^ t_swizzle(r))) << 4) + ((c & 4) << 1);
+  const int r8 = r + 8;
+  const char *p1 = lds + r8 * 128 + ((((c >> 3) ^ t_swizzle(r8))) << 4) + ((c & 4) << 1);
+  const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4 *)p0);
+  const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4 *)p1);
+  const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+  return u32x4{l2[0], l2[1], h2[0], h2[1]};
+}
+
 // dword offset of column c in a pair row of the (j, j+1)-packed V tile; the placement of the column
 // quads keeps both the 128-bit writes of the staging step and the 32-bit fragment reads conflict free
 __device__ static inline int pair_col_offset(int c) {
