@@ -132,8 +132,16 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
   BSA_PROBE_DECL;
   if (k_begin < k_end) {
     u32x4 mask_raw[2];
-    // wave-uniform facts about the key block whose tiles are in flight
-    int ent_nxt, pm_nxt, pb_nxt;
+    // Per-tile facts travel through a short pipeline.  For tile j: its record is loaded while tile j-3 is
+    // computed, its mask words while j-2 is computed; at the end of j-2 every wave says whether the tile is
+    // dead for it (nothing of its 32 rows survives the mask, or its query block does not have the key block),
+    // and only a tile that is live for some wave is copied to LDS while j-1 is computed.
+    struct Facts {
+      int entry, pm, pb;    // list entry, mask block, bias block (of this wave's query block)
+      uint32_t mbits;       // per lane: mask of its 32 scores of the tile, bit 8 t + w = byte t of word w
+      bool dead;            // for this wave
+    };
+    __shared__ int dead_votes[2][4];
 
     // K tile: copied global -> LDS without passing through registers.  One instruction moves 1 KiB
     // (eight 128-byte rows); lane l supplies the 16-byte chunk that belongs at position l of that KiB,
@@ -160,13 +168,17 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
       }
     };
 
-    // facts of one key block
-    auto fetch_facts = [&](const AttnFwdRecord &r) {
-      ent_nxt = r.entry;
-      pm_nxt = a.mask ? ((wave >> 1) ? r.pm[1] : r.pm[0]) : -1;
-      if (pm_nxt >= a.n_mask_blocks) pm_nxt = -1;
-      pb_nxt = a.bias ? ((wave >> 1) ? r.pb[1] : r.pb[0]) : -1;
-      if (pb_nxt >= a.n_bias_blocks) pb_nxt = -1;
+    // facts of one key block (without the mask, which arrives later)
+    auto make_facts = [&](const AttnFwdRecord &r) {
+      Facts f;
+      f.entry = r.entry;
+      f.pm = a.mask ? ((wave >> 1) ? r.pm[1] : r.pm[0]) : -1;
+      if (f.pm >= a.n_mask_blocks) f.pm = -1;
+      f.pb = a.bias ? ((wave >> 1) ? r.pb[1] : r.pb[0]) : -1;
+      if (f.pb >= a.n_bias_blocks) f.pb = -1;
+      f.mbits = 0;
+      f.dead = false;
+      return f;
     };
 
     // V tile: copied like the K tile, row-major, with the chunk swizzle of the transposing LDS load that
@@ -195,9 +207,9 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
     // dword 8 jb + 2 q + kg of the row, as word 4 jb + q.  It loads the 32 bytes [32 kg, 32 kg + 32) of the
     // row (two 16-byte loads; the wave reads 2 KiB contiguously) and trades every other dword with lane
     // (li, 1 - kg): one swap of the upper half of a register with the lower half of another per q.
-    auto fetch_mask = [&]() {
-      if (pm_nxt >= 0) {
-        const char *mp = static_cast<const char *>(a.mask) + (int64_t)pm_nxt * (kSbs * kSbs);
+    auto fetch_mask = [&](int pm) {
+      if (pm >= 0) {
+        const char *mp = static_cast<const char *>(a.mask) + (int64_t)pm * (kSbs * kSbs);
         const uint32_t moff = (uint32_t)qi * 64u + (uint32_t)kg * 32u;
         mask_raw[0] = load16(mp, moff);
         mask_raw[1] = load16(mp + 16, moff);
@@ -209,6 +221,33 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
       const u32x2 sw = __builtin_amdgcn_permlane32_swap(mask_raw[q >> 1][2 * (q & 1)], mask_raw[q >> 1][2 * (q & 1) + 1],
                                                         false, false);
       return sw[w >> 2];
+    };
+
+    // mask words (bytes 0 or 1) -> one bit per score, then this wave's verdict on the tile
+    auto finish_facts = [&](Facts &f) {
+      f.mbits = 0;
+      if (f.pm >= 0) {
+#pragma unroll
+        for (int w = 0; w < 8; ++w) f.mbits |= mask_word(w) << w;
+      }
+      bool live = has_q && ((f.entry >> my_bit) & 1);
+      if (f.pm >= 0 && live) live = __any(f.mbits != 0xffffffffu);
+      if (causal) {
+        const int kb = f.entry & 0x0fffffff;
+        const int q_last = (int)qb * kSbs + 32 * (wave & 1) + 31, q_first = q_last - 31;
+        if (kb * kSbs > q_last || q_first >= seq_len || kb * kSbs >= seq_len) live = false;
+      }
+      f.dead = !live;
+    };
+    // without a mask or a causal predicate some wave always has work on a tile
+    const bool may_skip = a.mask != nullptr || causal;
+    auto vote = [&](const Facts &f, int pos) {
+      if (may_skip && lane == 0) dead_votes[pos & 1][wave] = f.dead ? 1 : 0;
+    };
+    auto all_dead = [&](int pos) {
+      if (!may_skip) return false;
+      const int *v = dead_votes[pos & 1];
+      return first_lane(v[0] & v[1] & v[2] & v[3]) != 0;
     };
 
     auto clamp_e = [&](int e) { return e < k_end ? e : k_end - 1; };
@@ -235,55 +274,51 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
       r.pb[1] = __builtin_amdgcn_readlane(rv, 8);
       return r;
     };
-    int rv_next;
+    // prologue: tile k_begin copied and judged, tile k_begin + 1 judged, record of k_begin + 2 in flight
+    Facts f0, f1;
+    AttnFwdRecord r1;
+    int rv2;
     {
       const AttnFwdRecord r0 = unpack_record(load_record(k_begin));
-      rv_next = load_record(clamp_e(k_begin + 1));
-      fetch_facts(r0);
+      const int rv1 = load_record(clamp_e(k_begin + 1));
+      rv2 = load_record(clamp_e(k_begin + 2));
+      f0 = make_facts(r0);
       copy_k(r0, 0);
       copy_v(r0, 0);
-      fetch_mask();
-      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the K rows this wave copied are in LDS
+      fetch_mask(f0.pm);
+      r1 = unpack_record(rv1);
+      f1 = make_facts(r1);
+      finish_facts(f0);
+      fetch_mask(f1.pm);
+      finish_facts(f1);
+      vote(f1, k_begin + 1);
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the rows this wave copied are in LDS
       __syncthreads();
     }
 
     for (int e = k_begin; e < k_end; ++e) {
       BSA_PROBE(0);
       const int buf = (e - k_begin) & 1;
-      const int rv_after = load_record(clamp_e(e + 2));
-      // facts of tile e, before the fetch of tile e+1 replaces them
-      const bool mask_on = pm_nxt >= 0;
-      const int kb = ent_nxt & 0x0fffffff;
-      const bool mine = has_q && ((ent_nxt >> my_bit) & 1);
-      const int64_t pb = pb_nxt;
-      // mask words of tile e (bytes are 0 or 1) -> one bit per element, which frees the word registers:
-      // bit 8 t + w is byte t of word w, the mask of score 4 w + t
-      uint32_t mbits = 0;
-      if (mask_on) {
-#pragma unroll
-        for (int w = 0; w < 8; ++w) mbits |= mask_word(w) << w;
-      }
-
-      // ---- prefetch of tile e+1: K copy into the other buffer, V and mask words into registers ----
+      const int rv3 = load_record(clamp_e(e + 3));
+      // tile e+2: facts from its record, mask words on their way
+      const AttnFwdRecord r2 = unpack_record(rv2);
+      Facts f2 = make_facts(r2);
+      fetch_mask(f2.pm);
+      // tile e+1: copied unless no wave has anything to compute on it
       const bool more = e + 1 < k_end;
-      if (more) {
-        const AttnFwdRecord r_next = unpack_record(rv_next);
-        fetch_facts(r_next);
-        copy_k(r_next, buf ^ 1);
-        copy_v(r_next, buf ^ 1);
-        fetch_mask();
+      if (more && !all_dead(e + 1)) {
+        copy_k(r1, buf ^ 1);
+        copy_v(r1, buf ^ 1);
       }
-      rv_next = rv_after;
       BSA_PROBE(1);
 
-      // A tile in which every score of this wave's 32 rows is masked changes nothing: m stays, alpha is 1,
-      // every p is 0.  Such a tile is only fetched, not computed.
-      bool live = mine;
-      if (mask_on && live) live = __any(mbits != 0xffffffffu);
-      if (causal) {
-        const int q_last = (int)qb * kSbs + 32 * (wave & 1) + 31, q_first = q_last - 31;
-        if (kb * kSbs > q_last || q_first >= seq_len || kb * kSbs >= seq_len) live = false;
-      }
+      // tile e.  A tile in which every score of this wave's 32 rows is masked changes nothing: m stays, alpha
+      // is 1, every p is 0.
+      const bool mask_on = f0.pm >= 0;
+      const int kb = f0.entry & 0x0fffffff;
+      const int64_t pb = f0.pb;
+      const uint32_t mbits = f0.mbits;
+      const bool live = !f0.dead;
 
       if (live) {
         const char *kbuf = lds_k + buf * kKBytes;
@@ -439,8 +474,14 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
         BSA_PROBE(3);
       }  // live
 
-      // ---- the barrier ends the reads of tile e and publishes tile e+1 ----
-      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the K and V rows this wave copied are in LDS
+      // ---- the barrier ends the reads of tile e and publishes tile e+1 and the verdicts on tile e+2 ----
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the rows this wave copied are in LDS, the mask words here
+      finish_facts(f2);
+      vote(f2, e + 2);
+      f0 = f1;
+      f1 = f2;
+      r1 = r2;
+      rv2 = rv3;
       BSA_PROBE(4);
       __syncthreads();
       BSA_PROBE(5);
