@@ -131,7 +131,7 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
 
   BSA_PROBE_DECL;
   if (k_begin < k_end) {
-    u32x4 mask_raw[2];
+    u32x4 mask_a[2], mask_b[2];  // mask words of a tile as loaded: a = arrived, being judged; b = in flight
     // Per-tile facts travel through a short pipeline.  For tile j: its record is loaded while tile j-3 is
     // computed, its mask words while j-2 is computed; at the end of j-2 every wave says whether the tile is
     // dead for it (nothing of its 32 rows survives the mask, or its query block does not have the key block),
@@ -207,7 +207,7 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
     // dword 8 jb + 2 q + kg of the row, as word 4 jb + q.  It loads the 32 bytes [32 kg, 32 kg + 32) of the
     // row (two 16-byte loads; the wave reads 2 KiB contiguously) and trades every other dword with lane
     // (li, 1 - kg): one swap of the upper half of a register with the lower half of another per q.
-    auto fetch_mask = [&](int pm) {
+    auto fetch_mask = [&](int pm, u32x4 (&mask_raw)[2]) {
       if (pm >= 0) {
         const char *mp = static_cast<const char *>(a.mask) + (int64_t)pm * (kSbs * kSbs);
         const uint32_t moff = (uint32_t)qi * 64u + (uint32_t)kg * 32u;
@@ -215,7 +215,7 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
         mask_raw[1] = load16(mp + 16, moff);
       }
     };
-    auto mask_word = [&](int w) -> uint32_t {
+    auto mask_word = [&](const u32x4 (&mask_raw)[2], int w) -> uint32_t {
       // w = 4 jb + q: after the swap of (dword 2q, dword 2q + 1) the first holds the word of jb = 0, the second of jb = 1
       const int q = w & 3;
       const u32x2 sw = __builtin_amdgcn_permlane32_swap(mask_raw[q >> 1][2 * (q & 1)], mask_raw[q >> 1][2 * (q & 1) + 1],
@@ -224,11 +224,11 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
     };
 
     // mask words (bytes 0 or 1) -> one bit per score, then this wave's verdict on the tile
-    auto finish_facts = [&](Facts &f) {
+    auto finish_facts = [&](Facts &f, const u32x4 (&mask_raw)[2]) {
       f.mbits = 0;
       if (f.pm >= 0) {
 #pragma unroll
-        for (int w = 0; w < 8; ++w) f.mbits |= mask_word(w) << w;
+        for (int w = 0; w < 8; ++w) f.mbits |= mask_word(mask_raw, w) << w;
       }
       bool live = has_q && ((f.entry >> my_bit) & 1);
       if (f.pm >= 0 && live) live = __any(f.mbits != 0xffffffffu);
@@ -274,24 +274,29 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
       r.pb[1] = __builtin_amdgcn_readlane(rv, 8);
       return r;
     };
-    // prologue: tile k_begin copied and judged, tile k_begin + 1 judged, record of k_begin + 2 in flight
-    Facts f0, f1;
-    AttnFwdRecord r1;
-    int rv2;
+    // prologue: tile k_begin copied and judged, tile k_begin + 1 judged, mask words of k_begin + 2 and the
+    // record of k_begin + 3 in flight
+    Facts f0, f1, f2;
+    AttnFwdRecord r1, r2;
+    int rv3;
     {
       const AttnFwdRecord r0 = unpack_record(load_record(k_begin));
       const int rv1 = load_record(clamp_e(k_begin + 1));
-      rv2 = load_record(clamp_e(k_begin + 2));
+      const int rv2 = load_record(clamp_e(k_begin + 2));
+      rv3 = load_record(clamp_e(k_begin + 3));
       f0 = make_facts(r0);
       copy_k(r0, 0);
       copy_v(r0, 0);
-      fetch_mask(f0.pm);
+      fetch_mask(f0.pm, mask_a);
       r1 = unpack_record(rv1);
       f1 = make_facts(r1);
-      finish_facts(f0);
-      fetch_mask(f1.pm);
-      finish_facts(f1);
+      finish_facts(f0, mask_a);
+      fetch_mask(f1.pm, mask_a);
+      r2 = unpack_record(rv2);
+      f2 = make_facts(r2);
+      finish_facts(f1, mask_a);
       vote(f1, k_begin + 1);
+      fetch_mask(f2.pm, mask_b);
       __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the rows this wave copied are in LDS
       __syncthreads();
     }
@@ -299,17 +304,21 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
     for (int e = k_begin; e < k_end; ++e) {
       BSA_PROBE(0);
       const int buf = (e - k_begin) & 1;
-      const int rv3 = load_record(clamp_e(e + 3));
-      // tile e+2: facts from its record, mask words on their way
-      const AttnFwdRecord r2 = unpack_record(rv2);
-      Facts f2 = make_facts(r2);
-      fetch_mask(f2.pm);
-      // tile e+1: copied unless no wave has anything to compute on it
+      // mask words of tile e+2, requested one tile ago
+      mask_a[0] = mask_b[0];
+      mask_a[1] = mask_b[1];
+      // tile e+1: copied unless no wave has anything to compute on it.  Issued before this tile's other loads, so
+      // that the wait at the end of the tile can leave those outstanding.
       const bool more = e + 1 < k_end;
       if (more && !all_dead(e + 1)) {
         copy_k(r1, buf ^ 1);
         copy_v(r1, buf ^ 1);
       }
+      // tile e+3: facts from its record, mask words requested; record of tile e+4 requested
+      const AttnFwdRecord r3 = unpack_record(rv3);
+      Facts f3 = make_facts(r3);
+      const int rv4 = load_record(clamp_e(e + 4));
+      fetch_mask(f3.pm, mask_b);
       BSA_PROBE(1);
 
       // tile e.  A tile in which every score of this wave's 32 rows is masked changes nothing: m stays, alpha
@@ -475,13 +484,18 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
       }  // live
 
       // ---- the barrier ends the reads of tile e and publishes tile e+1 and the verdicts on tile e+2 ----
-      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the rows this wave copied are in LDS, the mask words here
-      finish_facts(f2);
+      finish_facts(f2, mask_a);
       vote(f2, e + 2);
+      // The rows this wave copied have to be in LDS; the loads issued after the copies (a record, two mask
+      // loads if the tile has a mask block) may stay in flight.  vmcnt(3) / vmcnt(1), other counters untouched.
+      if (f3.pm >= 0) __builtin_amdgcn_s_waitcnt(0x0F73);
+      else __builtin_amdgcn_s_waitcnt(0x0F71);
       f0 = f1;
       f1 = f2;
+      f2 = f3;
       r1 = r2;
-      rv2 = rv3;
+      r2 = r3;
+      rv3 = rv4;
       BSA_PROBE(4);
       __syncthreads();
       BSA_PROBE(5);
