@@ -10,18 +10,19 @@
 // Both main kernels have the same shape.  One workgroup of four waves owns the "stationary" block (a key block,
 // or a query block); each wave owns one 32 x 32 quadrant of the 64 x 64 score tile and keeps the fragments of
 // its half of the stationary operands in registers for the whole walk.  The blocks of the other side stream
-// through LDS, double buffered, one barrier per tile: row-major with XOR-swizzled 16-byte chunks where the head
-// dimension is contracted (scores, dP), and as (row, row + 1) pairs per column where the sequence index is
-// contracted (dV, dK, dQ), because a matrix-core operand wants eight consecutive contraction indices per lane.
+// through LDS, double buffered, one barrier per tile, copied global -> LDS asynchronously, row-major with
+// XOR-swizzled 16-byte chunks.  A matrix-core operand wants eight consecutive contraction indices per lane:
+// where the head dimension is contracted (scores, dP) a fragment is one 128-bit read of a row, where the
+// sequence index is contracted (dV, dK, dQ) it is two transposing 64-bit reads (ds_read_b64_tr_b16).
 //
 //   dK / dV kernel, lane owns a key j, registers run over queries i:
 //     S[i][j]  = sum_d Q[i][d] K[j][d]        A = Q rows (LDS)     B = K (registers)
 //     dP[i][j] = sum_d dO[i][d] V[j][d]       A = dO rows (LDS)    B = V (registers)
-//     dV^T[d][j] += sum_i dO[i][d] P[i][j]    A = dO pairs (LDS)   B = P (registers, as computed)
-//     dK^T[d][j] += sum_i Q[i][d] dS[i][j]    A = Q pairs (LDS)    B = dS
+//     dV^T[d][j] += sum_i dO[i][d] P[i][j]    A = dO columns (LDS) B = P (registers, as computed)
+//     dK^T[d][j] += sum_i Q[i][d] dS[i][j]    A = Q columns (LDS)  B = dS
 //   dQ kernel, lane owns a query i, registers run over keys j:
 //     S^T[j][i], dP^T[j][i] likewise with K, V rows from LDS and Q, dO in registers
-//     dQ^T[d][i] += sum_j K[j][d] dS^T[j][i]  A = K pairs (LDS)    B = dS^T
+//     dQ^T[d][i] += sum_j K[j][d] dS^T[j][i]  A = K columns (LDS)  B = dS^T
 //
 // The two waves that share a half of the stationary block hold partial sums over the two halves of the streamed
 // blocks; they are added through LDS once, at the end.  No atomics, fixed summation order.
@@ -35,63 +36,26 @@ using namespace mfma;
 constexpr int kBwdThreads = 256;
 constexpr int kStatBytes = 2 * kSbs * 4;  // lse and delta of the 64 queries of a tile
 
-// ---- one 64 x 64 16-bit block spread over 256 threads: thread t holds rows 2p, 2p + 1 (p = t / 8),
-// ---- columns 8 (t % 8) .. + 7
-struct TileRegs {
-  u32x4 ev, od;
-};
-
-__device__ inline TileRegs load_tile(const char *blk, bool valid, int tid) {
-  TileRegs t;
-  t.ev = u32x4{0u, 0u, 0u, 0u};
-  t.od = u32x4{0u, 0u, 0u, 0u};
+// One 64 x 64 16-bit block, global -> LDS, by the four waves of a workgroup: wave w copies rows 16 w .. + 15
+// with two asynchronous 1 KiB copies; lane l supplies the chunk that belongs at position l of the KiB, which
+// is where the chunk swizzle is applied.  An inactive block becomes zeros.
+__device__ inline void copy_block(const char *blk, bool valid, char *dst, int wave, int lane, int tid) {
   if (valid) {
-    const uint32_t off = (uint32_t)(tid >> 3) * 256u + (uint32_t)(tid & 7) * 16u;
-    t.ev = load16(blk, off);
-    t.od = load16(blk + 128, off);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int r0 = 16 * wave + 8 * i;
+      const uint32_t lane_off = (lane >> 3) * 128 + (((lane & 7) ^ t_swizzle(8 * i + (lane >> 3))) << 4);
+      copy_1k_to_lds(blk + r0 * 128, lane_off, dst + r0 * 128);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) *reinterpret_cast<u32x4 *>(dst + (i * kBwdThreads + tid) * 16) = u32x4{0u, 0u, 0u, 0u};
   }
-  return t;
-}
-
-// row-major, chunk c of row r at position c ^ k_swizzle(r) (rows 2p and 2p + 1 share the swizzle value)
-__device__ inline void stage_rows(char *lds, const TileRegs &t, int tid) {
-  const int p = tid >> 3, c = tid & 7;
-  char *dst = lds + (2 * p) * 128 + ((c ^ (p & 7)) << 4);
-  *reinterpret_cast<u32x4 *>(dst) = t.ev;
-  *reinterpret_cast<u32x4 *>(dst + 128) = t.od;
-}
-
-// (row 2p, row 2p + 1) pairs per column
-__device__ inline void stage_pairs(char *lds, const TileRegs &t, int tid) {
-  const int p = tid >> 3, c = tid & 7;
-  u32x4 lo, hi;
-  lo[0] = __builtin_amdgcn_perm(t.od[0], t.ev[0], 0x05040100u);
-  lo[1] = __builtin_amdgcn_perm(t.od[0], t.ev[0], 0x07060302u);
-  lo[2] = __builtin_amdgcn_perm(t.od[1], t.ev[1], 0x05040100u);
-  lo[3] = __builtin_amdgcn_perm(t.od[1], t.ev[1], 0x07060302u);
-  hi[0] = __builtin_amdgcn_perm(t.od[2], t.ev[2], 0x05040100u);
-  hi[1] = __builtin_amdgcn_perm(t.od[2], t.ev[2], 0x07060302u);
-  hi[2] = __builtin_amdgcn_perm(t.od[3], t.ev[3], 0x05040100u);
-  hi[3] = __builtin_amdgcn_perm(t.od[3], t.ev[3], 0x07060302u);
-  uint32_t *prow = reinterpret_cast<uint32_t *>(lds) + p * kSbs;
-  *reinterpret_cast<u32x4 *>(prow + pair_col_offset(c * 8)) = lo;
-  *reinterpret_cast<u32x4 *>(prow + pair_col_offset(c * 8 + 4)) = hi;
 }
 
 // operand fragment with the head dimension contracted: 8 values of row `row`, 16-byte chunk `chunk`
 __device__ inline u32x4 frag_rows(const char *lds, int row, int chunk) {
-  return *reinterpret_cast<const u32x4 *>(lds + row * 128 + ((chunk ^ k_swizzle(row)) << 4));
-}
-
-// operand fragment with the row index contracted: column `col`, rows 2 pair0 .. + 3 and 2 pair0 + 8 .. + 11
-__device__ inline u32x4 frag_pairs(const char *lds, int col, int pair0) {
-  const uint32_t *p = reinterpret_cast<const uint32_t *>(lds) + pair0 * kSbs + pair_col_offset(col);
-  u32x4 v;
-  v[0] = p[0];
-  v[1] = p[kSbs];
-  v[2] = p[4 * kSbs];
-  v[3] = p[5 * kSbs];
-  return v;
+  return *reinterpret_cast<const u32x4 *>(lds + row * 128 + ((chunk ^ t_swizzle(row)) << 4));
 }
 
 // fragment of a block in global memory for the register-resident side: row `row`, chunks 2 s + kg
@@ -173,8 +137,7 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_delta_kernel(bsa_attn_ar
 template <typename Tr, int NH, int NHV>
 __global__ __launch_bounds__(kBwdThreads, 1) void attn_bwd_kv_kernel(bsa_attn_args a) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  constexpr int kQRows = 0, kQPairs = NH * kBlockBytes, kDoRows = 2 * NH * kBlockBytes,
-                kDoPairs = (2 * NH + NHV) * kBlockBytes, kStats = 2 * (NH + NHV) * kBlockBytes;
+  constexpr int kQRows = 0, kDoRows = NH * kBlockBytes, kStats = (NH + NHV) * kBlockBytes;
   constexpr int kBufBytes = kStats + kStatBytes;
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -256,26 +219,28 @@ __global__ __launch_bounds__(kBwdThreads, 1) void attn_bwd_kv_kernel(bsa_attn_ar
     };
     auto clamp_e = [&](int e) { return e < q_end ? e : q_end - 1; };
 
-    // registers of the tile in flight
-    TileRegs qt[NH], dot[NHV];
+    // registers of the tile in flight (the blocks themselves go straight to LDS)
     float stat = 0.f;           // thread t < 64: lse of query t; 64 <= t < 128: delta of query t - 64
     uint32_t mask_b[16];        // mask bytes of this lane's 16 score elements
     uint32_t bias_b[16];        // bias elements likewise
     int qb_nxt, pm_nxt, pb_nxt;
 
-    auto fetch = [&](int rec, int qb) {
+    auto fetch = [&](int rec, int qb, int buf) {
       qb_nxt = qb;
+      char *base = smem + buf * kBufBytes;
 #pragma unroll
       for (int h = 0; h < NH; ++h) {
         const int64_t pq = __builtin_amdgcn_readlane(rec, h);
         const bool valid = pq >= 0 && pq < a.n_q_blocks;
-        qt[h] = load_tile(static_cast<const char *>(a.q) + (valid ? pq : 0) * kBlockBytes, valid, tid);
+        copy_block(static_cast<const char *>(a.q) + (valid ? pq : 0) * kBlockBytes, valid,
+                   base + kQRows + h * kBlockBytes, wave, lane, tid);
       }
 #pragma unroll
       for (int h = 0; h < NHV; ++h) {
         const int64_t po = __builtin_amdgcn_readlane(rec, NH + h);
         const bool valid = po >= 0 && po < a.n_o_blocks;
-        dot[h] = load_tile(static_cast<const char *>(a.d_o) + (valid ? po : 0) * kBlockBytes, valid, tid);
+        copy_block(static_cast<const char *>(a.d_o) + (valid ? po : 0) * kBlockBytes, valid,
+                   base + kDoRows + h * kBlockBytes, wave, lane, tid);
       }
       const int64_t qrow = b * a.nq + qb;
       if (tid < 64) stat = a.lse[qrow * kSbs + tid];
@@ -298,19 +263,11 @@ __global__ __launch_bounds__(kBwdThreads, 1) void attn_bwd_kv_kernel(bsa_attn_ar
         for (int r = 0; r < 16; ++r) bias_b[r] = bp[(8 * (r >> 2) + (r & 3)) * kSbs];
       }
     };
+    // the statistics of the tile go to LDS through a register; then every copy of this wave has to have landed
     auto stage = [&](int buf) {
       char *base = smem + buf * kBufBytes;
-#pragma unroll
-      for (int h = 0; h < NH; ++h) {
-        stage_rows(base + kQRows + h * kBlockBytes, qt[h], tid);
-        stage_pairs(base + kQPairs + h * kBlockBytes, qt[h], tid);
-      }
-#pragma unroll
-      for (int h = 0; h < NHV; ++h) {
-        stage_rows(base + kDoRows + h * kBlockBytes, dot[h], tid);
-        stage_pairs(base + kDoPairs + h * kBlockBytes, dot[h], tid);
-      }
       if (tid < 128) reinterpret_cast<float *>(base + kStats)[tid] = stat;
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     };
 
     // index pipeline: `rec` holds the indices of query block qb_rec (the entry after the tile in flight) and, in
@@ -321,7 +278,7 @@ __global__ __launch_bounds__(kBwdThreads, 1) void attn_bwd_kv_kernel(bsa_attn_ar
       const int rec0 = gather(qb0, clamp_e(q_begin + 1));
       qb_rec = __builtin_amdgcn_readlane(rec0, kLaneEntry);
       rec = gather(qb_rec, clamp_e(q_begin + 2));
-      fetch(rec0, qb0);
+      fetch(rec0, qb0, 0);
       stage(0);
       __syncthreads();
     }
@@ -344,7 +301,7 @@ __global__ __launch_bounds__(kBwdThreads, 1) void attn_bwd_kv_kernel(bsa_attn_ar
         for (int r = 0; r < 16; ++r) bias_c[r] = bias_b[r];
       }
       const bool more = e + 1 < q_end;
-      if (more) fetch(rec, qb_rec);
+      if (more) fetch(rec, qb_rec, buf ^ 1);
       qb_rec = __builtin_amdgcn_readlane(rec, kLaneEntry);
       rec = gather(qb_rec, clamp_e(e + 3));
 
@@ -416,7 +373,8 @@ __global__ __launch_bounds__(kBwdThreads, 1) void attn_bwd_kv_kernel(bsa_attn_ar
           for (int db = 0; db < 2; ++db)
   #pragma unroll
             for (int u = 0; u < 2; ++u)
-              dvacc[2 * h + db] = Tr::mfma(frag_pairs(base + kDoPairs + h * kBlockBytes, 32 * db + li, 16 * wi + 8 * u + 2 * kg),
+              dvacc[2 * h + db] = Tr::mfma(frag_cols_t(base + kDoRows + h * kBlockBytes, 32 * wi + 16 * u + 4 * kg,
+                                                       32 * db + 16 * ((lane >> 4) & 1), lane),
                                            pf[u], dvacc[2 * h + db]);
   #pragma unroll
         for (int h = 0; h < NH; ++h)
@@ -424,7 +382,8 @@ __global__ __launch_bounds__(kBwdThreads, 1) void attn_bwd_kv_kernel(bsa_attn_ar
           for (int db = 0; db < 2; ++db)
   #pragma unroll
             for (int u = 0; u < 2; ++u)
-              dkacc[2 * h + db] = Tr::mfma(frag_pairs(base + kQPairs + h * kBlockBytes, 32 * db + li, 16 * wi + 8 * u + 2 * kg),
+              dkacc[2 * h + db] = Tr::mfma(frag_cols_t(base + kQRows + h * kBlockBytes, 32 * wi + 16 * u + 4 * kg,
+                                                       32 * db + 16 * ((lane >> 4) & 1), lane),
                                            dsf[u], dkacc[2 * h + db]);
 
       }  // live
@@ -477,8 +436,8 @@ __global__ __launch_bounds__(kBwdThreads, 1) void attn_bwd_kv_kernel(bsa_attn_ar
 template <typename Tr, int NH, int NHV>
 __global__ __launch_bounds__(kBwdThreads, 1) void attn_bwd_q_kernel(bsa_attn_args a) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  constexpr int kKRows = 0, kKPairs = NH * kBlockBytes, kVRows = 2 * NH * kBlockBytes;
-  constexpr int kBufBytes = (2 * NH + NHV) * kBlockBytes;
+  constexpr int kKRows = 0, kVRows = NH * kBlockBytes;
+  constexpr int kBufBytes = (NH + NHV) * kBlockBytes;
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = first_lane(tid >> 6);
@@ -549,24 +508,26 @@ __global__ __launch_bounds__(kBwdThreads, 1) void attn_bwd_q_kernel(bsa_attn_arg
     };
     auto clamp_e = [&](int e) { return e < k_end ? e : k_end - 1; };
 
-    TileRegs kt[NH], vt[NHV];
     uint32_t mask_w[4];  // mask bytes of keys 32 wj + 8 q + 4 kg .. + 3 of this lane's query, one word per q
     u32x2 bias_w[4];     // bias elements likewise
     int kb_nxt, pm_nxt, pb_nxt;
 
-    auto fetch = [&](int rec, int kb) {
+    auto fetch = [&](int rec, int kb, int buf) {
       kb_nxt = kb;
+      char *base = smem + buf * kBufBytes;
 #pragma unroll
       for (int h = 0; h < NH; ++h) {
         const int64_t pk = __builtin_amdgcn_readlane(rec, h);
         const bool valid = pk >= 0 && pk < a.n_k_blocks;
-        kt[h] = load_tile(static_cast<const char *>(a.k) + (valid ? pk : 0) * kBlockBytes, valid, tid);
+        copy_block(static_cast<const char *>(a.k) + (valid ? pk : 0) * kBlockBytes, valid,
+                   base + kKRows + h * kBlockBytes, wave, lane, tid);
       }
 #pragma unroll
       for (int h = 0; h < NHV; ++h) {
         const int64_t pv = __builtin_amdgcn_readlane(rec, NH + h);
         const bool valid = pv >= 0 && pv < a.n_v_blocks;
-        vt[h] = load_tile(static_cast<const char *>(a.v) + (valid ? pv : 0) * kBlockBytes, valid, tid);
+        copy_block(static_cast<const char *>(a.v) + (valid ? pv : 0) * kBlockBytes, valid,
+                   base + kVRows + h * kBlockBytes, wave, lane, tid);
       }
       pm_nxt = __builtin_amdgcn_readlane(rec, kLaneMask);
       if (pm_nxt >= a.n_mask_blocks) pm_nxt = -1;
@@ -585,16 +546,8 @@ __global__ __launch_bounds__(kBwdThreads, 1) void attn_bwd_q_kernel(bsa_attn_arg
         for (int q = 0; q < 4; ++q) bias_w[q] = *reinterpret_cast<const u32x2 *>(bp + off + 16 * q);
       }
     };
-    auto stage = [&](int buf) {
-      char *base = smem + buf * kBufBytes;
-#pragma unroll
-      for (int h = 0; h < NH; ++h) {
-        stage_rows(base + kKRows + h * kBlockBytes, kt[h], tid);
-        stage_pairs(base + kKPairs + h * kBlockBytes, kt[h], tid);
-      }
-#pragma unroll
-      for (int h = 0; h < NHV; ++h) stage_rows(base + kVRows + h * kBlockBytes, vt[h], tid);
-    };
+    // every copy of this wave has to have landed before the barrier
+    auto stage = [&](int) { __builtin_amdgcn_s_waitcnt(0x0F70); };
 
     int rec, kb_rec;
     {
@@ -602,7 +555,7 @@ __global__ __launch_bounds__(kBwdThreads, 1) void attn_bwd_q_kernel(bsa_attn_arg
       const int rec0 = gather(kb0, clamp_e(k_begin + 1));
       kb_rec = __builtin_amdgcn_readlane(rec0, kLaneEntry);
       rec = gather(kb_rec, clamp_e(k_begin + 2));
-      fetch(rec0, kb0);
+      fetch(rec0, kb0, 0);
       stage(0);
       __syncthreads();
     }
@@ -621,7 +574,7 @@ __global__ __launch_bounds__(kBwdThreads, 1) void attn_bwd_q_kernel(bsa_attn_arg
         for (int q = 0; q < 4; ++q) bias_c[q] = bias_w[q];
       }
       const bool more = e + 1 < k_end;
-      if (more) fetch(rec, kb_rec);
+      if (more) fetch(rec, kb_rec, buf ^ 1);
       kb_rec = __builtin_amdgcn_readlane(rec, kLaneEntry);
       rec = gather(kb_rec, clamp_e(e + 3));
 
@@ -679,7 +632,8 @@ __global__ __launch_bounds__(kBwdThreads, 1) void attn_bwd_q_kernel(bsa_attn_arg
           for (int db = 0; db < 2; ++db)
   #pragma unroll
             for (int u = 0; u < 2; ++u)
-              dqacc[2 * h + db] = Tr::mfma(frag_pairs(base + kKPairs + h * kBlockBytes, 32 * db + li, 16 * wj + 8 * u + 2 * kg),
+              dqacc[2 * h + db] = Tr::mfma(frag_cols_t(base + kKRows + h * kBlockBytes, 32 * wj + 16 * u + 4 * kg,
+                                                       32 * db + 16 * ((lane >> 4) & 1), lane),
                                            dsf[u], dqacc[2 * h + db]);
 
       }  // live
@@ -730,14 +684,14 @@ int launch_bwd(const bsa_attn_args &a, hipStream_t s) {
     if (int rc = check_launch("attn_bwd_delta_kernel")) return rc;
   }
   if (krows > 0) {
-    constexpr int lds = 2 * (2 * (NH + NHV) * kBlockBytes + kStatBytes);
+    constexpr int lds = 2 * ((NH + NHV) * kBlockBytes + kStatBytes);
     BSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_bwd_kv_kernel<Tr, NH, NHV>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, lds));
     attn_bwd_kv_kernel<Tr, NH, NHV><<<(unsigned)(cdiv(krows, 8) * 8), kBwdThreads, lds, s>>>(a);
     if (int rc = check_launch("attn_bwd_kv_kernel")) return rc;
   }
   if (qrows > 0) {
-    constexpr int lds = 2 * (2 * NH + NHV) * kBlockBytes;
+    constexpr int lds = 2 * (NH + NHV) * kBlockBytes;
     BSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_bwd_q_kernel<Tr, NH, NHV>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, lds));
     attn_bwd_q_kernel<Tr, NH, NHV><<<(unsigned)(cdiv(qrows, 8) * 8), kBwdThreads, lds, s>>>(a);

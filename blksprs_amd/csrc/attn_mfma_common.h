@@ -47,10 +47,11 @@ constexpr int kBlockBytes = kSbs * kSbs * 2;  // one 16-bit block
 // rows of equal parity get eight different values.
 __device__ static inline int k_swizzle(int r) { return (r >> 1) & 7; }
 
-// XOR applied to the 16-byte chunk index of row r of a tile that is read with the transposing LDS load: one
-// such load serves 16 lanes with four rows r .. r + 3 and two neighbouring chunks of each, so rows two apart
-// must be shifted by two chunks.
-__device__ static inline int t_swizzle(int r) { return ((r >> 1) & 3) << 1; }
+// XOR applied to the 16-byte chunk index of row r of a tile that is read both ways: by rows (128-bit reads,
+// 16 lanes = 16 consecutive rows, one chunk each: rows of equal parity need eight different values) and with
+// the transposing LDS load (16 lanes = four rows r .. r + 3, two neighbouring chunks of each: rows two apart
+// must land in different chunk pairs).
+__device__ static inline int t_swizzle(int r) { return (((r >> 1) & 3) << 1) | ((r >> 3) & 1); }
 
 typedef short i16x4 __attribute__((ext_vector_type(4)));
 
