@@ -434,7 +434,7 @@ __global__ __launch_bounds__(kBwdThreads, 1) void attn_bwd_kv_kernel(bsa_attn_ar
 // ---------------------------------------------------------------------------------------------------------
 // dQ of one query block
 template <typename Tr, int NH, int NHV>
-__global__ __launch_bounds__(kBwdThreads, 1) void attn_bwd_q_kernel(bsa_attn_args a) {
+__global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_q_kernel(bsa_attn_args a) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   constexpr int kKRows = 0, kVRows = NH * kBlockBytes;
   constexpr int kBufBytes = (NH + NHV) * kBlockBytes;
