@@ -35,6 +35,9 @@ using namespace mfma;
 
 constexpr int kBwdThreads = 256;
 constexpr int kStatBytes = 2 * kSbs * 4;  // lse and delta of the 64 queries of a tile
+// dK and dV in one pass over the query blocks (one workgroup per CU) or in two passes (two workgroups per CU,
+// scores computed twice): measured equal within 3 % on the BigBird configuration; one pass reads less
+constexpr bool kSplitKeyPass = false;
 
 // One 64 x 64 16-bit block, global -> LDS, by the four waves of a workgroup: wave w copies rows 16 w .. + 15
 // with two asynchronous 1 KiB copies; lane l supplies the chunk that belongs at position l of the KiB, which
@@ -133,12 +136,15 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_delta_kernel(bsa_attn_ar
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// dK, dV and dBias of one key block
-template <typename Tr, int NH, int NHV>
-__global__ __launch_bounds__(kBwdThreads, 1) void attn_bwd_kv_kernel(bsa_attn_args a) {
+// dK and dBias (DK) and / or dV (DV) of one key block.  The two are launched as separate passes: each then fits
+// two workgroups per CU (the combined kernel needs more than 256 registers per lane), which more than pays
+// for computing the scores twice.
+template <typename Tr, int NH, int NHV, bool DK, bool DV>
+__global__ __launch_bounds__(kBwdThreads, (DK &&DV) ? 1 : 2) void attn_bwd_kv_kernel(bsa_attn_args a) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  constexpr int kQRows = 0, kDoRows = NH * kBlockBytes, kStats = (NH + NHV) * kBlockBytes;
-  constexpr int kBufBytes = kStats + kStatBytes;
+  constexpr int kQRows = 0, kDoRows = NH * kBlockBytes, kStats = (NH + NHV) * kBlockBytes,
+                kMask = kStats + kStatBytes;  // the tile's mask block, row-major bytes
+  constexpr int kBufBytes = kMask + kSbs * kSbs;
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = first_lane(tid >> 6);
@@ -149,18 +155,18 @@ __global__ __launch_bounds__(kBwdThreads, 1) void attn_bwd_kv_kernel(bsa_attn_ar
   const int64_t b = krow / a.nk, kb = krow % a.nk;
 
   int64_t pk[NH], pv[NHV];
-  bool any = a.dbias != nullptr;
+  bool any = DK && a.dbias != nullptr;
 #pragma unroll
   for (int h = 0; h < NH; ++h) {
     pk[h] = a.pidx_k[krow * NH + h];
     if (pk[h] >= a.n_k_blocks) pk[h] = -1;
-    any = any || pk[h] >= 0;
+    any = any || (DK && pk[h] >= 0);
   }
 #pragma unroll
   for (int h = 0; h < NHV; ++h) {
     pv[h] = a.pidx_v[krow * NHV + h];
     if (pv[h] >= a.n_v_blocks) pv[h] = -1;
-    any = any || pv[h] >= 0;
+    any = any || (DV && pv[h] >= 0);
   }
   if (!any) return;
 
@@ -168,19 +174,25 @@ __global__ __launch_bounds__(kBwdThreads, 1) void attn_bwd_kv_kernel(bsa_attn_ar
   u32x4 kfr[NH][4], vfr[NHV][4];
 #pragma unroll
   for (int h = 0; h < NH; ++h) load_resident(kfr[h], a.k, pk[h], a.n_k_blocks, 32 * wj + li, kg);
+  if constexpr (DK) {
 #pragma unroll
-  for (int h = 0; h < NHV; ++h) load_resident(vfr[h], a.v, pv[h], a.n_v_blocks, 32 * wj + li, kg);
+    for (int h = 0; h < NHV; ++h) load_resident(vfr[h], a.v, pv[h], a.n_v_blocks, 32 * wj + li, kg);
+  }
 
   // accumulators [slice][column half db]: D[m = d][n = j]
-  f32x16 dkacc[NH * 2], dvacc[NHV * 2];
+  f32x16 dkacc[DK ? NH * 2 : 1], dvacc[DV ? NHV * 2 : 1];
+  if constexpr (DK) {
 #pragma unroll
-  for (int n = 0; n < NH * 2; ++n)
+    for (int n = 0; n < NH * 2; ++n)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) dkacc[n][r] = 0.f;
+      for (int r = 0; r < 16; ++r) dkacc[n][r] = 0.f;
+  }
+  if constexpr (DV) {
 #pragma unroll
-  for (int n = 0; n < NHV * 2; ++n)
+    for (int n = 0; n < NHV * 2; ++n)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) dvacc[n][r] = 0.f;
+      for (int r = 0; r < 16; ++r) dvacc[n][r] = 0.f;
+  }
 
   const float qk_scale = a.scale * kLog2e;
   const bool causal = a.causal_lengths != nullptr;
@@ -221,8 +233,6 @@ __global__ __launch_bounds__(kBwdThreads, 1) void attn_bwd_kv_kernel(bsa_attn_ar
 
     // registers of the tile in flight (the blocks themselves go straight to LDS)
     float stat = 0.f;           // thread t < 64: lse of query t; 64 <= t < 128: delta of query t - 64
-    uint32_t mask_b[16];        // mask bytes of this lane's 16 score elements
-    uint32_t bias_b[16];        // bias elements likewise
     int qb_nxt, pm_nxt, pb_nxt;
 
     auto fetch = [&](int rec, int qb, int buf) {
@@ -249,19 +259,10 @@ __global__ __launch_bounds__(kBwdThreads, 1) void attn_bwd_kv_kernel(bsa_attn_ar
       if (pm_nxt >= a.n_mask_blocks) pm_nxt = -1;
       pb_nxt = __builtin_amdgcn_readlane(rec, kLaneBias);
       if (pb_nxt >= a.n_bias_blocks) pb_nxt = -1;
-      // element r of this lane: query 32 wi + 8 (r / 4) + 4 kg + r % 4, key 32 wj + li
-      if (pm_nxt >= 0) {
-        const uint8_t *mp = static_cast<const uint8_t *>(a.mask) + (int64_t)pm_nxt * (kSbs * kSbs) +
-                            (32 * wi + 4 * kg) * kSbs + 32 * wj + li;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) mask_b[r] = mp[(8 * (r >> 2) + (r & 3)) * kSbs];
-      }
-      if (pb_nxt >= 0) {
-        const uint16_t *bp = static_cast<const uint16_t *>(a.bias) + (int64_t)pb_nxt * (kSbs * kSbs) +
-                             (32 * wi + 4 * kg) * kSbs + 32 * wj + li;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) bias_b[r] = bp[(8 * (r >> 2) + (r & 3)) * kSbs];
-      }
+      // the mask block goes to LDS as it is: wave w copies its rows 16 w .. + 15 (1 KiB)
+      if (pm_nxt >= 0)
+        copy_1k_to_lds(static_cast<const char *>(a.mask) + (int64_t)pm_nxt * (kSbs * kSbs) + wave * 1024, lane * 16,
+                       base + kMask + wave * 1024);
     };
     // the statistics of the tile go to LDS through a register; then every copy of this wave has to have landed
     auto stage = [&](int buf) {
@@ -289,16 +290,13 @@ __global__ __launch_bounds__(kBwdThreads, 1) void attn_bwd_kv_kernel(bsa_attn_ar
       // facts and per-element inputs of tile e, before the fetch of tile e+1 replaces them
       const int qb = qb_nxt;
       const int64_t pm = pm_nxt, pb = pb_nxt;
-      // mask bytes (0 or 1) of the 16 elements -> one bit each, which frees their registers for the next tile
+      // mask bytes (0 or 1) of this lane's 16 elements -> one bit each; element r: query
+      // 32 wi + 8 (r / 4) + 4 kg + r % 4, key 32 wj + li
       uint32_t mbits = 0;
       if (pm >= 0) {
+        const uint8_t *mp = reinterpret_cast<const uint8_t *>(base + kMask) + (32 * wi + 4 * kg) * kSbs + 32 * wj + li;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) mbits |= mask_b[r] << r;
-      }
-      uint32_t bias_c[16];
-      if (pb >= 0) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) bias_c[r] = bias_b[r];
+        for (int r = 0; r < 16; ++r) mbits |= (uint32_t)mp[(8 * (r >> 2) + (r & 3)) * kSbs] << r;
       }
       const bool more = e + 1 < q_end;
       if (more) fetch(rec, qb_rec, buf ^ 1);
@@ -322,14 +320,24 @@ __global__ __launch_bounds__(kBwdThreads, 1) void attn_bwd_kv_kernel(bsa_attn_ar
   #pragma unroll
           for (int s = 0; s < 4; ++s)
             sacc = Tr::mfma(frag_rows(base + kQRows + h * kBlockBytes, 32 * wi + li, 2 * s + kg), kfr[h][s], sacc);
+        if constexpr (DK) {
   #pragma unroll
-        for (int h = 0; h < NHV; ++h)
+          for (int h = 0; h < NHV; ++h)
   #pragma unroll
-          for (int s = 0; s < 4; ++s)
-            dpacc = Tr::mfma(frag_rows(base + kDoRows + h * kBlockBytes, 32 * wi + li, 2 * s + kg), vfr[h][s], dpacc);
+            for (int s = 0; s < 4; ++s)
+              dpacc = Tr::mfma(frag_rows(base + kDoRows + h * kBlockBytes, 32 * wi + li, 2 * s + kg), vfr[h][s], dpacc);
+        }
 
         // ---- P and dS; element r: query 32 wi + 8 (r / 4) + 4 kg + r % 4 ----
         const float *stats = reinterpret_cast<const float *>(base + kStats);
+        // the bias elements are read where they are used: a bias is rare, its registers are not
+        uint32_t bias_c[16];
+        if (pb >= 0) {
+          const uint16_t *bp = static_cast<const uint16_t *>(a.bias) + pb * (kSbs * kSbs) +
+                               (32 * wi + 4 * kg) * kSbs + 32 * wj + li;
+  #pragma unroll
+          for (int r = 0; r < 16; ++r) bias_c[r] = bp[(8 * (r >> 2) + (r & 3)) * kSbs];
+        }
         float p[16], ds[16];
   #pragma unroll
         for (int q = 0; q < 4; ++q) {
@@ -351,7 +359,7 @@ __global__ __launch_bounds__(kBwdThreads, 1) void attn_bwd_kv_kernel(bsa_attn_ar
             ds[r] = p[r] * (dpacc[r] - del4[t]);
           }
         }
-        if (a.dbias != nullptr && pb >= 0) {
+        if (DK && a.dbias != nullptr && pb >= 0) {
           // every (query block, key block) pair is visited once, so this is a plain store
           float *dbp = a.dbias + pb * (kSbs * kSbs) + (32 * wi + 4 * kg) * kSbs + 32 * wj + li;
   #pragma unroll
@@ -367,6 +375,7 @@ __global__ __launch_bounds__(kBwdThreads, 1) void attn_bwd_kv_kernel(bsa_attn_ar
           }
 
         // ---- dV^T += dO^T P, dK^T += Q^T dS over this wave's 32 queries ----
+        if constexpr (DV) {
   #pragma unroll
         for (int h = 0; h < NHV; ++h)
   #pragma unroll
@@ -376,6 +385,8 @@ __global__ __launch_bounds__(kBwdThreads, 1) void attn_bwd_kv_kernel(bsa_attn_ar
               dvacc[2 * h + db] = Tr::mfma(frag_cols_t(base + kDoRows + h * kBlockBytes, 32 * wi + 16 * u + 4 * kg,
                                                        32 * db + 16 * ((lane >> 4) & 1), lane),
                                            pf[u], dvacc[2 * h + db]);
+        }
+        if constexpr (DK) {
   #pragma unroll
         for (int h = 0; h < NH; ++h)
   #pragma unroll
@@ -385,7 +396,7 @@ __global__ __launch_bounds__(kBwdThreads, 1) void attn_bwd_kv_kernel(bsa_attn_ar
               dkacc[2 * h + db] = Tr::mfma(frag_cols_t(base + kQRows + h * kBlockBytes, 32 * wi + 16 * u + 4 * kg,
                                                        32 * db + 16 * ((lane >> 4) & 1), lane),
                                            dsf[u], dkacc[2 * h + db]);
-
+        }
       }  // live
 
       // ---- tile e+1 into the other buffer; the barrier also ends the reads of tile e ----
@@ -395,12 +406,12 @@ __global__ __launch_bounds__(kBwdThreads, 1) void attn_bwd_kv_kernel(bsa_attn_ar
   }
 
   // ---- add the two query halves, scale, store ----
-  reduce_partner(dkacc, reinterpret_cast<float *>(smem), wi == 1, wj, lane);
-  reduce_partner(dvacc, reinterpret_cast<float *>(smem), wi == 1, wj, lane);
+  if constexpr (DK) reduce_partner(dkacc, reinterpret_cast<float *>(smem), wi == 1, wj, lane);
+  if constexpr (DV) reduce_partner(dvacc, reinterpret_cast<float *>(smem), wi == 1, wj, lane);
   if (wi == 1) return;
   // lane: key 32 wj + li; register 4 q + t of half db: column 32 db + 8 q + 4 kg + t
 #pragma unroll
-  for (int h = 0; h < NH; ++h) {
+  for (int h = 0; h < (DK ? NH : 0); ++h) {
     if (pk[h] < 0) continue;
     char *op = static_cast<char *>(a.dk) + pk[h] * kBlockBytes + (32 * wj + li) * 128 + kg * 8;
 #pragma unroll
@@ -415,7 +426,7 @@ __global__ __launch_bounds__(kBwdThreads, 1) void attn_bwd_kv_kernel(bsa_attn_ar
       }
   }
 #pragma unroll
-  for (int h = 0; h < NHV; ++h) {
+  for (int h = 0; h < (DV ? NHV : 0); ++h) {
     if (pv[h] < 0) continue;
     char *op = static_cast<char *>(a.dv) + pv[h] * kBlockBytes + (32 * wj + li) * 128 + kg * 8;
 #pragma unroll
@@ -684,11 +695,22 @@ int launch_bwd(const bsa_attn_args &a, hipStream_t s) {
     if (int rc = check_launch("attn_bwd_delta_kernel")) return rc;
   }
   if (krows > 0) {
-    constexpr int lds = 2 * ((NH + NHV) * kBlockBytes + kStatBytes);
-    BSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_bwd_kv_kernel<Tr, NH, NHV>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-    attn_bwd_kv_kernel<Tr, NH, NHV><<<(unsigned)(cdiv(krows, 8) * 8), kBwdThreads, lds, s>>>(a);
-    if (int rc = check_launch("attn_bwd_kv_kernel")) return rc;
+    constexpr int lds = 2 * ((NH + NHV) * kBlockBytes + kStatBytes + kSbs * kSbs);
+    if (kSplitKeyPass) {
+      BSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_bwd_kv_kernel<Tr, NH, NHV, true, false>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+      BSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_bwd_kv_kernel<Tr, NH, NHV, false, true>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+      attn_bwd_kv_kernel<Tr, NH, NHV, false, true><<<(unsigned)(cdiv(krows, 8) * 8), kBwdThreads, lds, s>>>(a);
+      if (int rc = check_launch("attn_bwd_kv_kernel (dV)")) return rc;
+      attn_bwd_kv_kernel<Tr, NH, NHV, true, false><<<(unsigned)(cdiv(krows, 8) * 8), kBwdThreads, lds, s>>>(a);
+      if (int rc = check_launch("attn_bwd_kv_kernel (dK)")) return rc;
+    } else {
+      BSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_bwd_kv_kernel<Tr, NH, NHV, true, true>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+      attn_bwd_kv_kernel<Tr, NH, NHV, true, true><<<(unsigned)(cdiv(krows, 8) * 8), kBwdThreads, lds, s>>>(a);
+      if (int rc = check_launch("attn_bwd_kv_kernel")) return rc;
+    }
   }
   if (qrows > 0) {
     constexpr int lds = 2 * (NH + NHV) * kBlockBytes;
