@@ -41,7 +41,7 @@ TRAFFIC_KIB = {  # config: (FETCH_SIZE, WRITE_SIZE)
     "c1": (616.2, 476.0),
     "c2": (592501.7, 514960.0),
     "c3": (148346.4, 296128.0),
-    "c4": (548540.2, 133281.6),
+    "c4": (374747.9, 133149.5),
     "c5": (127107.7, 143960.0),
 }
 
@@ -238,7 +238,7 @@ def make_workload(name, dev):
     if name == "c1":
         return matmul_workload("c1_matmul_fp32", 2, 8, 32, torch.float32, 0.5, True, 1.0, dev, 2)
     if name == "c2":
-        return matmul_workload("c2_matmul_bf16", 16, 64, 64, torch.bfloat16, 0.25, False, 1.0 / 64.0, dev, 2)
+        return matmul_workload("c2_matmul_bf16", 16, 64, 64, torch.bfloat16, 0.25, False, 1.0 / 64.0, dev, 16)
     if name == "c3":
         return softmax_workload(dev)
     if name == "c4":
