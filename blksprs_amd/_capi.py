@@ -59,8 +59,8 @@ SIGNATURES = {
     "bsa_softmax_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p]),
     "bsa_matmul": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int,
                            c_int, c_int, c_int, c_void_p]),
-    "bsa_matmul_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
-                                c_int64, c_int64, c_int64, c_int, c_int, c_void_p]),
+    "bsa_matmul_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_void_p]),
     "bsa_attn_fwd_records": (c_int, [ctypes.POINTER(AttnArgs), c_void_p, c_void_p, c_void_p]),
     "bsa_attn_fwd": (c_int, [ctypes.POINTER(AttnArgs), c_void_p]),
     "bsa_attn_bwd": (c_int, [ctypes.POINTER(AttnArgs), c_void_p]),

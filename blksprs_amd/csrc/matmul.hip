@@ -396,315 +396,6 @@ __global__ __launch_bounds__(256, 2) void matmul_mfma_kernel(const char *__restr
   }
 }
 
-// ---------------------------------------------------------------------------------------------------------
-// Row-panel kernel (16-bit operands, sbs == 64, untransposed operands): one workgroup of 8 waves owns one
-// output block row (b, i).  The x blocks of that row are consecutive in memory; up to 16 of them (128 KiB)
-// are copied once into LDS and stay there while the waves walk the row's output blocks, so x is read from
-// L2 once per row instead of once per use, and a wave never waits for x.  x blocks beyond the 16 resident
-// ones are read straight from global memory in fragment layout.
-//
-// Only y blocks stream.  A wave owns a contiguous run of the row's output blocks, hence one contiguous slice
-// of the pair list, and walks it as one flat sequence: the loads of the y block of pair t+1 are issued while
-// pair t is multiplied, across output-block boundaries, so the chain "offsets -> pair -> operands" is paid
-// once per wave rather than once per output block.  The inner loop over the pairs of one output block
-// contains no other memory instruction whose result is consumed later (the pair list and the block
-// boundaries sit in registers, 64 entries each, and are picked with v_readlane; the windows are refilled
-// between output blocks), which keeps the compiler's s_waitcnt placement exact inside it.
-//
-// Per pair: wait for the y block, interleave its (k, k+1) rows in registers (that frees the load registers:
-// the next block's loads are issued right away), then per k half write 4 KiB to the wave's LDS slice and run
-// 8 MFMAs with x fragments from the panel.
-
-constexpr int kPanelCap = 16;
-constexpr int kPanelWaves = 8;
-constexpr int kPanelLds = kPanelCap * 8192 + kPanelWaves * 4096;  // 160 KiB
-
-// loads one 64 x 64 y block (k rows, 128 bytes each): entry 2i / 2i+1 = rows 2kp / 2kp+1, 8 columns, of task
-// q = 64 i + lane (kp = q / 8, column octet q % 8)
-__device__ __forceinline__ void panel_load_y(u32x4 (&r)[8], const char *yb, int lane) {
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int q = i * 64 + lane;
-    const int ro = q & 7, kp = q >> 3;
-    r[2 * i] = *reinterpret_cast<const u32x4 *>(yb + (uint32_t)((2 * kp) * 128 + ro * 16));
-    r[2 * i + 1] = *reinterpret_cast<const u32x4 *>(yb + (uint32_t)((2 * kp + 1) * 128 + ro * 16));
-  }
-}
-
-// (k, k+1) interleave of the two rows of every task: pk[2i] = columns 0..3, pk[2i+1] = columns 4..7 of the octet
-__device__ __forceinline__ void panel_pack_y(u32x4 (&pk)[8], const u32x4 (&r)[8]) {
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const u32x4 e = r[2 * i], o = r[2 * i + 1];
-    pk[2 * i].x = __builtin_amdgcn_perm(o.x, e.x, 0x05040100u);
-    pk[2 * i].y = __builtin_amdgcn_perm(o.x, e.x, 0x07060302u);
-    pk[2 * i].z = __builtin_amdgcn_perm(o.y, e.y, 0x05040100u);
-    pk[2 * i].w = __builtin_amdgcn_perm(o.y, e.y, 0x07060302u);
-    pk[2 * i + 1].x = __builtin_amdgcn_perm(o.z, e.z, 0x05040100u);
-    pk[2 * i + 1].y = __builtin_amdgcn_perm(o.z, e.z, 0x07060302u);
-    pk[2 * i + 1].z = __builtin_amdgcn_perm(o.w, e.w, 0x05040100u);
-    pk[2 * i + 1].w = __builtin_amdgcn_perm(o.w, e.w, 0x07060302u);
-  }
-}
-
-// One (x block, y block) product into acc from the packed y block.  RESIDENT: xsrc is the x block's swizzled
-// copy in LDS; otherwise the x fragments come preloaded in xf.
-// x fragments of one non-resident block, all 4 k steps x 2 row blocks, straight from global memory
-__device__ __forceinline__ void panel_load_x_frags(u32x4 (&xf)[4][2], const char *xb, int lane) {
-  const int li = lane & 31, kg = lane >> 5;
-#pragma unroll
-  for (int s = 0; s < 4; ++s)
-#pragma unroll
-    for (int b = 0; b < 2; ++b)
-      xf[s][b] = *reinterpret_cast<const u32x4 *>(xb + (uint32_t)((32 * b + li) * 128 + (2 * s + kg) * 16));
-}
-
-template <typename Tr, bool RESIDENT>
-__device__ __forceinline__ void panel_pair(f32x16 (&acc)[2][2], const u32x4 (&pk)[8], const char *xsrc,
-                                           const u32x4 (&xf)[4][2], char *ystage, int lane) {
-  const int li = lane & 31, kg = lane >> 5;
-#pragma unroll
-  for (int half = 0; half < 2; ++half) {
-    // pair rows 16 half .. 16 half + 15 of y into the wave's LDS slice
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int q = i * 64 + lane;
-      const int ro = q & 7, kp = q >> 3;  // pair row inside the half: 0..15
-      uint32_t *dst = reinterpret_cast<uint32_t *>(ystage) + kp * 64;
-      *reinterpret_cast<u32x4 *>(dst + pair_col_offset<64>(kp, ro * 8)) = pk[4 * half + 2 * i];
-      *reinterpret_cast<u32x4 *>(dst + pair_col_offset<64>(kp, ro * 8 + 4)) = pk[4 * half + 2 * i + 1];
-    }
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-#pragma unroll
-    for (int sh = 0; sh < 2; ++sh) {
-      const int s = 2 * half + sh;
-      u32x4 fx[2], fy[2];
-#pragma unroll
-      for (int b = 0; b < 2; ++b) {
-        const int r = 32 * b + li;
-        if constexpr (RESIDENT)
-          fx[b] = *reinterpret_cast<const u32x4 *>(xsrc + r * 128 + (((2 * s + kg) ^ (r & 7)) * 16));
-        else
-          fx[b] = xf[s][b];
-        const uint32_t *p = reinterpret_cast<const uint32_t *>(ystage) + (8 * sh + 4 * kg) * 64 +
-                            pair_col_offset<64>(0, r);
-        fy[b][0] = p[0];
-        fy[b][1] = p[64];
-        fy[b][2] = p[128];
-        fy[b][3] = p[192];
-      }
-#pragma unroll
-      for (int bj = 0; bj < 2; ++bj)
-#pragma unroll
-        for (int bi = 0; bi < 2; ++bi) acc[bj][bi] = Tr::mfma(fy[bj], fx[bi], acc[bj][bi]);
-    }
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-  }
-}
-
-// Rounds the tile, passes it through the wave's LDS slice in two halves of 32 rows, writes it as one block
-// with 16-byte stores that cover whole rows, and clears the accumulators.
-template <typename Tr>
-__device__ __forceinline__ void panel_flush(f32x16 (&acc)[2][2], char *ob, char *ystage, int lane) {
-  const int li = lane & 31, kg = lane >> 5;
-#pragma unroll
-  for (int bi = 0; bi < 2; ++bi) {
-#pragma unroll
-    for (int bj = 0; bj < 2; ++bj)
-#pragma unroll
-      for (int rq = 0; rq < 4; ++rq) {
-        const int j = 32 * bj + 8 * rq + 4 * kg;
-        uint2 v;
-        v.x = (uint32_t)Tr::round(acc[bj][bi][4 * rq]) | ((uint32_t)Tr::round(acc[bj][bi][4 * rq + 1]) << 16);
-        v.y = (uint32_t)Tr::round(acc[bj][bi][4 * rq + 2]) | ((uint32_t)Tr::round(acc[bj][bi][4 * rq + 3]) << 16);
-        // rows li and li + 8 share a chunk position: their 8-byte pieces go to opposite halves of the chunk
-        *reinterpret_cast<uint2 *>(ystage + li * 128 + (((j >> 3) ^ (li & 7)) * 16) +
-                                   (((j & 7) * 2) ^ (((li >> 3) & 1) * 8))) = v;
-      }
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      const int q = t * 64 + lane;
-      const int r = q >> 3, ch = q & 7;
-      u32x4 v = *reinterpret_cast<const u32x4 *>(ystage + r * 128 + ((ch ^ (r & 7)) * 16));
-      if ((r >> 3) & 1) v = u32x4{v[2], v[3], v[0], v[1]};
-      // streaming store: the tile is not read again, keep it from displacing y blocks in L2
-      __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(ob + (uint32_t)((32 * bi + r) * 128 + ch * 16)));
-    }
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-  }
-#pragma unroll
-  for (int a = 0; a < 2; ++a)
-#pragma unroll
-    for (int b = 0; b < 2; ++b)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
-}
-
-template <typename Tr>
-__global__ __launch_bounds__(kPanelWaves * 64, 1) void matmul_panel_kernel(
-    const char *__restrict__ x, const char *__restrict__ y, char *__restrict__ out,
-    const int32_t *__restrict__ pair_offsets, const int32_t *__restrict__ pairs,
-    const int32_t *__restrict__ x_row_offsets, const int32_t *__restrict__ o_row_offsets, int n_rows, int64_t nnz_x,
-    int64_t nnz_y) {
-  extern __shared__ __attribute__((aligned(16))) char panel_smem[];
-  const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  // XCD c (workgroups c, c+8, ...) takes the c-th contiguous eighth of the rows: the rows in flight on one L2
-  // belong to one batch and stream through the same y blocks at about the same time
-  const int per_xcd = gridDim.x >> 3;
-  const int row = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  if (row >= n_rows) return;
-  const int n0 = o_row_offsets[row], n1 = o_row_offsets[row + 1];
-  if (n0 >= n1) return;
-  const int xs = x_row_offsets[row];
-  int nx = x_row_offsets[row + 1] - xs;
-  nx = nx < kPanelCap ? nx : kPanelCap;
-  if (xs < 0 || xs + nx > nnz_x) nx = 0;  // a corrupt table must not turn into a wild read
-  char *panel = panel_smem;
-  char *ystage = panel_smem + kPanelCap * 8192 + wave * 4096;
-
-  // this wave's run of output blocks and its slice of the pair list
-  const int per_wave = (n1 - n0 + kPanelWaves - 1) / kPanelWaves;
-  int wb0 = n0 + wave * per_wave;
-  wb0 = wb0 < n1 ? wb0 : n1;
-  int wb1 = wb0 + per_wave;
-  wb1 = wb1 < n1 ? wb1 : n1;
-  const int p_begin = __builtin_amdgcn_readfirstlane(pair_offsets[wb0]);
-  const int p_end = __builtin_amdgcn_readfirstlane(pair_offsets[wb1]);
-
-  // 64 entries of the pair list and 64 block boundaries at a time, one per lane
-  int win_base = p_begin, win_px = 0, win_py = 0;
-  int off_base = wb0, win_off = 0;
-  auto load_pair_window = [&](int base) {
-    win_base = base;
-    const int t = base + lane;
-    win_px = win_py = 0;
-    if (t < p_end) {
-      const int2 v = *reinterpret_cast<const int2 *>(pairs + 2 * (int64_t)t);
-      win_px = v.x;
-      win_py = v.y;
-    }
-  };
-  auto load_offset_window = [&](int base) {
-    off_base = base;
-    const int n = base + lane;
-    win_off = pair_offsets[n <= wb1 ? n : wb1];
-  };
-  load_pair_window(p_begin);
-  load_offset_window(wb0);
-
-  // pair t (inside the window) -> x block index, pointer to the y block
-  auto pair_at = [&](int t, int &px, const char *&yb) {
-    const int sel = __builtin_amdgcn_readfirstlane(t - win_base);
-    px = __builtin_amdgcn_readlane(win_px, sel);
-    int64_t py = __builtin_amdgcn_readlane(win_py, sel);
-    py = (py < 0 || py >= nnz_y) ? 0 : py;
-    yb = y + py * 8192;
-  };
-
-  u32x4 ry[8];
-  u32x4 xf[4][2];  // x fragments of a non-resident block (only the non-resident loop fills them)
-#pragma unroll
-  for (int s4 = 0; s4 < 4; ++s4)
-#pragma unroll
-    for (int b = 0; b < 2; ++b) xf[s4][b] = u32x4{0, 0, 0, 0};
-  int px_next = 0;
-  const bool has_pairs = p_begin < p_end;
-  if (has_pairs) {
-    const char *yb;
-    pair_at(p_begin, px_next, yb);
-    panel_load_y(ry, yb, lane);
-  }
-
-  // copy the row's x blocks into the panel (swizzled rows), all threads
-  {
-    const char *xsrc = x + (int64_t)xs * 8192;
-    const int n_chunks = nx * 512;
-    for (int c0 = 0; c0 < n_chunks; c0 += 4 * kPanelWaves * 64) {
-      u32x4 v[4];
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        int c = c0 + u * kPanelWaves * 64 + (int)threadIdx.x;
-        c = c < n_chunks ? c : n_chunks - 1;
-        v[u] = *reinterpret_cast<const u32x4 *>(xsrc + (uint32_t)c * 16);
-      }
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        int c = c0 + u * kPanelWaves * 64 + (int)threadIdx.x;
-        c = c < n_chunks ? c : n_chunks - 1;  // the surplus lanes rewrite the last chunk with its own value
-        const int r = (c >> 3) & 63, ch = c & 7;
-        *reinterpret_cast<u32x4 *>(panel + (c >> 9) * 8192 + r * 128 + ((ch ^ (r & 7)) * 16)) = v[u];
-      }
-    }
-  }
-  __syncthreads();
-
-  f32x16 acc[2][2];  // [block along j][block along i]
-#pragma unroll
-  for (int a = 0; a < 2; ++a)
-#pragma unroll
-    for (int b = 0; b < 2; ++b)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
-
-  int t = p_begin;
-  for (int cur = wb0; cur < wb1; ++cur) {
-    if (cur + 1 - off_base >= 64) load_offset_window(cur);
-    const int blk_end = __builtin_amdgcn_readlane(win_off, __builtin_amdgcn_readfirstlane(cur + 1 - off_base));
-    while (t < blk_end) {
-      // the window must hold pair t and the pair after it
-      if (t + 1 - win_base >= 64) load_pair_window(t);
-      int t_stop = win_base + 63;
-      t_stop = t_stop < blk_end ? t_stop : blk_end;
-      // The resident x blocks of a row are its first nx in k order and the pairs of an output block ascend
-      // in k, so a block's pairs split into a resident run followed by a non-resident run: two plain loops
-      // instead of a branch per pair (a branch would make the compiler copy the accumulators at the join).
-      while (t < t_stop && (unsigned)(px_next - xs) < (unsigned)nx) {
-        const int px = px_next;
-        u32x4 pk[8];
-        panel_pack_y(pk, ry);
-        // the load registers are free again: fetch the y block of the next pair of this wave (the last pair
-        // re-reads itself so that the loads stay unconditional)
-        const char *yb;
-        pair_at(t + 1 < p_end ? t + 1 : t, px_next, yb);
-        panel_load_y(ry, yb, lane);
-        panel_pair<Tr, true>(acc, pk, panel + (px - xs) * 8192, xf, ystage, lane);
-        ++t;
-      }
-      // non-resident run: the x fragments travel through registers, fetched one pair ahead like y
-      bool xf_ready = false;
-      while (t < t_stop && (unsigned)(px_next - xs) >= (unsigned)nx) {
-        if (!xf_ready) {
-          int64_t pxc = px_next;
-          pxc = (pxc < 0 || pxc >= nnz_x) ? 0 : pxc;
-          panel_load_x_frags(xf, x + pxc * 8192, lane);
-        }
-        u32x4 xcur[4][2];
-#pragma unroll
-        for (int s4 = 0; s4 < 4; ++s4)
-#pragma unroll
-          for (int b = 0; b < 2; ++b) xcur[s4][b] = xf[s4][b];
-        u32x4 pk[8];
-        panel_pack_y(pk, ry);
-        const char *yb;
-        pair_at(t + 1 < p_end ? t + 1 : t, px_next, yb);
-        panel_load_y(ry, yb, lane);
-        // fragments of the next pair's x block if that pair is non-resident too
-        xf_ready = (unsigned)(px_next - xs) >= (unsigned)nx;
-        if (xf_ready) {
-          int64_t pxc = px_next;
-          pxc = (pxc < 0 || pxc >= nnz_x) ? 0 : pxc;
-          panel_load_x_frags(xf, x + pxc * 8192, lane);
-        }
-        panel_pair<Tr, false>(acc, pk, nullptr, xcur, ystage, lane);
-        ++t;
-      }
-    }
-    panel_flush<Tr>(acc, out + (int64_t)cur * 8192, ystage, lane);
-  }
-}
-
 // sbs == 16: one wave per output block, fp32 FMAs; lane -> row lane/4, columns 4*(lane%4)..+3
 template <typename Tr>
 __global__ __launch_bounds__(256) void matmul_small_kernel(const typename Tr::store_t *__restrict__ x,
@@ -776,24 +467,6 @@ int launch_mfma(const void *x, const void *y, void *out, const int32_t *pair_off
 }
 
 template <typename Tr>
-int launch_panel(const void *x, const void *y, void *out, const int32_t *pair_offsets, const int32_t *pairs,
-                 const int32_t *x_row_offsets, const int32_t *o_row_offsets, int64_t n_rows, int64_t nnz_x,
-                 int64_t nnz_y, hipStream_t s) {
-  static bool configured = false;  // raising the dynamic LDS limit is per function, once per process
-  if (!configured) {
-    BSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&matmul_panel_kernel<Tr>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, kPanelLds));
-    configured = true;
-  }
-  const int64_t blocks = bsa::cdiv(n_rows, 8) * 8;
-  if (blocks > 0x7fffffffLL) return bsa::fail(BSA_ELIMIT, "bsa_matmul: too many block rows");
-  matmul_panel_kernel<Tr><<<(unsigned)blocks, kPanelWaves * 64, kPanelLds, s>>>(
-      static_cast<const char *>(x), static_cast<const char *>(y), static_cast<char *>(out), pair_offsets, pairs,
-      x_row_offsets, o_row_offsets, (int)n_rows, nnz_x, nnz_y);
-  return bsa::check_launch("matmul_panel_kernel");
-}
-
-template <typename Tr>
 int launch_any(const void *x, const void *y, void *out, const int32_t *pair_offsets, const int32_t *pairs,
                const int32_t *block_order, int64_t nnz_o, int64_t nnz_x, int64_t nnz_y, int sbs, int trans_x,
                int trans_y, hipStream_t s) {
@@ -814,25 +487,6 @@ int launch_any(const void *x, const void *y, void *out, const int32_t *pair_offs
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 }  // namespace
-
-extern "C" int bsa_matmul_rows(const void *x, const void *y, void *out, const int32_t *pair_offsets,
-                               const int32_t *pairs, const int32_t *x_row_offsets, const int32_t *o_row_offsets,
-                               int64_t n_rows, int64_t nnz_o, int64_t nnz_x, int64_t nnz_y, int sbs, int dtype,
-                               bsa_stream_t stream) {
-  BSA_REQUIRE(sbs == 64, "bsa_matmul_rows: sbs must be 64 (got %d)", sbs);
-  BSA_REQUIRE(dtype == BSA_F16 || dtype == BSA_BF16, "bsa_matmul_rows: dtype must be fp16 or bf16 (got %d)", dtype);
-  BSA_REQUIRE(nnz_o >= 0 && nnz_x >= 0 && nnz_y >= 0 && n_rows >= 0, "bsa_matmul_rows: negative size");
-  if (nnz_o == 0 || n_rows == 0) return BSA_OK;
-  BSA_REQUIRE(out && pair_offsets && x_row_offsets && o_row_offsets, "bsa_matmul_rows: NULL pointer");
-  BSA_REQUIRE(aligned16(x) && aligned16(y) && aligned16(out), "bsa_matmul_rows: buffers must be 16-byte aligned");
-  BSA_REQUIRE(n_rows < 0x7fffffffLL, "bsa_matmul_rows: too many block rows");
-  hipStream_t s = bsa::as_stream(stream);
-  if (dtype == BSA_BF16)
-    return launch_panel<Bf16Traits>(x, y, out, pair_offsets, pairs, x_row_offsets, o_row_offsets, n_rows, nnz_x,
-                                    nnz_y, s);
-  return launch_panel<F16Traits>(x, y, out, pair_offsets, pairs, x_row_offsets, o_row_offsets, n_rows, nnz_x, nnz_y,
-                                 s);
-}
 
 extern "C" int bsa_matmul(const void *x, const void *y, void *out, const int32_t *pair_offsets, const int32_t *pairs,
                           const int32_t *block_order, int64_t nnz_o, int64_t nnz_x, int64_t nnz_y, int sbs, int dtype, int trans_x, int trans_y,

@@ -1,0 +1,418 @@
+// Row kernel of the block-sparse GEMM (16-bit operands, sbs == 64, untransposed operands): one workgroup of
+// 8 waves owns one block row (b, i) of the output.
+//
+// x: the row's x blocks are consecutive in memory; up to 18 of them (144 KiB) are copied once into LDS by
+// asynchronous global -> LDS copies and stay there while the waves walk the row's output blocks, so x is
+// read from L2 once per row, and a wave never waits for x.  x blocks beyond the 18 resident ones are read
+// from global memory in fragment layout (slow path, rare).
+//
+// Work split: the row's output blocks are cut into 8 contiguous runs of about equal numbers of (x, y) pairs
+// (not of equal numbers of blocks), one run per wave; rows are handed to workgroups in the order the caller
+// gives (longest first keeps the tail of the launch short).
+//
+// y: only y blocks stream.  A wave walks its slice of the pair list as one flat sequence.  Each y block
+// travels global -> registers -> LDS -> matrix-core operand: two register slots of 8 KiB hold the y blocks of
+// the next two pairs, so a block is requested about one and a half pairs before it is used.  The loads are
+// issued from inline assembly and waited for with hand-placed s_waitcnt vmcnt(n): the compiler would join
+// the outstanding loads with vmcnt(0) at every branch.  vmcnt counts vector memory instructions in issue
+// order, so "all but the youngest n" is exact as long as n is not larger than the number of instructions
+// issued after the loads waited for; every n used below is such a lower bound (the other slot's 8 loads,
+// plus the 8 stores of an output block written since).
+//
+// Per pair, per quarter of the contraction (16 k): 2 KiB of the y block are written to the wave's LDS stage
+// as stored (k rows), and read back with the transposing LDS load, which delivers the matrix-core operand
+// whose contraction index runs over rows; the x operand is a 128-bit row read from the panel.  LDS executes
+// one wave's instructions in order, so stage writes and reads of consecutive quarters are queued back to
+// back without waits in between; only the fragment registers bound the depth.
+//
+// The product is formed transposed (y fragments as the A operand, x fragments as B), which leaves 4
+// consecutive output columns of one row in each lane; a finished block is rounded, passed through the stage
+// 16 rows at a time and written with 16-byte stores that cover whole rows.
+#include "attn_mfma_common.h"
+
+namespace {
+
+using namespace bsa::mfma;
+
+constexpr int kPanelCap = 18;
+constexpr int kWaves = 8;
+constexpr int kStageBytes = 2048;                                   // 16 rows of 128 bytes
+constexpr int kRowsLds = kPanelCap * 8192 + kWaves * kStageBytes;  // 160 KiB
+
+struct YSlot {
+  u32x4 v[8];  // v[i] = rows 8 i + lane / 8, chunk lane % 8 of one 64 x 64 block
+};
+
+// requests the 8 KiB block at yb into the slot; lane_lo = 16 * lane, lane_hi = lane_lo + 4096
+__device__ __forceinline__ void y_issue(YSlot &s, const char *yb, uint32_t lane_lo, uint32_t lane_hi) {
+  asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(s.v[0]) : "v"(lane_lo), "s"(yb) : "memory");
+  asm volatile("global_load_dwordx4 %0, %1, %2 offset:1024" : "=v"(s.v[1]) : "v"(lane_lo), "s"(yb) : "memory");
+  asm volatile("global_load_dwordx4 %0, %1, %2 offset:2048" : "=v"(s.v[2]) : "v"(lane_lo), "s"(yb) : "memory");
+  asm volatile("global_load_dwordx4 %0, %1, %2 offset:3072" : "=v"(s.v[3]) : "v"(lane_lo), "s"(yb) : "memory");
+  asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(s.v[4]) : "v"(lane_hi), "s"(yb) : "memory");
+  asm volatile("global_load_dwordx4 %0, %1, %2 offset:1024" : "=v"(s.v[5]) : "v"(lane_hi), "s"(yb) : "memory");
+  asm volatile("global_load_dwordx4 %0, %1, %2 offset:2048" : "=v"(s.v[6]) : "v"(lane_hi), "s"(yb) : "memory");
+  asm volatile("global_load_dwordx4 %0, %1, %2 offset:3072" : "=v"(s.v[7]) : "v"(lane_hi), "s"(yb) : "memory");
+}
+
+// waits until at most N vector memory instructions are outstanding; the slot's registers pass through the
+// statement so that no use of them can be moved in front of it
+#define BSA_Y_WAIT(slot_, n_)                                                                                  \
+  asm volatile("s_waitcnt vmcnt(" #n_ ")"                                                                      \
+               : "+v"((slot_).v[0]), "+v"((slot_).v[1]), "+v"((slot_).v[2]), "+v"((slot_).v[3]),               \
+                 "+v"((slot_).v[4]), "+v"((slot_).v[5]), "+v"((slot_).v[6]), "+v"((slot_).v[7])                \
+               :                                                                                               \
+               : "memory")
+
+// no instruction: the slot's registers pass through the statement, so that no use of them can be moved in
+// front of the wait that precedes it
+#define BSA_Y_TIE(slot_)                                                                                       \
+  asm volatile(""                                                                                              \
+               : "+v"((slot_).v[0]), "+v"((slot_).v[1]), "+v"((slot_).v[2]), "+v"((slot_).v[3]),               \
+                 "+v"((slot_).v[4]), "+v"((slot_).v[5]), "+v"((slot_).v[6]), "+v"((slot_).v[7])                \
+               :                                                                                               \
+               : "memory")
+
+__device__ __forceinline__ u32x2 read_tr(const char *p) {
+  const i16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4 *)p);
+  return __builtin_bit_cast(u32x2, v);
+}
+
+// per-lane LDS addresses that do not change during the kernel
+struct LaneAddr {
+  char *wr[2];      // stage write: rows lane / 8 and 8 + lane / 8 of a quarter, chunk lane % 8
+  const char *tr[2][2];  // transposing reads: [column block][rows k0 .. k0 + 3 | k0 + 4 .. k0 + 7]
+  uint32_t xoff[4];  // x fragment of k step s inside a panel block (row lane % 32; the second row block is + 4096)
+};
+
+// One (x block, y block) product.  xsrc is an x block's swizzled copy in LDS; if the x block is not resident,
+// its fragments are read from global memory at xglob instead (wave uniform).
+// `next` is the y block to request into the slot once its registers are free.
+template <typename Tr>
+__device__ __forceinline__ void rows_pair(f32x16 (&acc)[2][2], YSlot &ys, const char *xsrc, bool resident,
+                                          const char *xglob, const LaneAddr &la, const char *next, uint32_t lane_lo, uint32_t lane_hi,
+                                          int lane) {
+  const int li = lane & 31, kg = lane >> 5;
+  u32x4 fy[2][2], fx[2][2];  // [quarter parity][block]
+  auto stage_quarter = [&](int s) {
+    *reinterpret_cast<u32x4 *>(la.wr[0]) = ys.v[2 * s];
+    *reinterpret_cast<u32x4 *>(la.wr[1]) = ys.v[2 * s + 1];
+  };
+  auto read_quarter = [&](int s) {
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      const u32x2 lo = read_tr(la.tr[b][0]), hi = read_tr(la.tr[b][1]);
+      fy[s & 1][b] = u32x4{lo[0], lo[1], hi[0], hi[1]};
+      fx[s & 1][b] = *reinterpret_cast<const u32x4 *>(xsrc + la.xoff[s] + 4096 * b);
+    }
+    if (!resident) {
+      // rare: only the fragments pass through the branch (not the accumulators), and they are used inside it,
+      // which puts the wait for these loads here and not in front of the multiplications of every pair
+#pragma unroll
+      for (int b = 0; b < 2; ++b)
+        fx[s & 1][b] = *reinterpret_cast<const u32x4 *>(xglob + (uint32_t)((32 * b + li) * 128 + (2 * s + kg) * 16));
+      asm volatile("" : "+v"(fx[s & 1][0]), "+v"(fx[s & 1][1]));
+    }
+  };
+  auto multiply = [&](int s) {
+#pragma unroll
+    for (int bj = 0; bj < 2; ++bj)
+#pragma unroll
+      for (int bi = 0; bi < 2; ++bi) acc[bj][bi] = Tr::mfma(fy[s & 1][bj], fx[s & 1][bi], acc[bj][bi]);
+  };
+  stage_quarter(0);
+  read_quarter(0);
+  stage_quarter(1);
+  read_quarter(1);
+  __builtin_amdgcn_sched_barrier(0);
+  multiply(0);
+  stage_quarter(2);
+  read_quarter(2);
+  __builtin_amdgcn_sched_barrier(0);
+  multiply(1);
+  stage_quarter(3);
+  // the slot's registers have been handed to the LDS writes: request the block of the pair after next
+  y_issue(ys, next, lane_lo, lane_hi);
+  read_quarter(3);
+  __builtin_amdgcn_sched_barrier(0);
+  multiply(2);
+  multiply(3);
+}
+
+// Rounds the tile, passes it through the wave's stage 16 rows at a time, writes it as one block with 16-byte
+// stores that cover whole rows (8 stores per lane), and clears the accumulators.  A lane owns 4 columns of
+// one of 32 rows per accumulator; v_permlane16_swap regroups the packed values so that, for each half of 16
+// rows, all 64 lanes hold a piece (lanes 16 .. 31 and 48 .. 63 take over the right-hand column block of the
+// rows of the lanes 16 below them).  Every lane takes part in every step: the exchange between lanes through
+// LDS needs the wave to move as one.
+template <typename Tr>
+__device__ __forceinline__ void rows_flush(f32x16 (&acc)[2][2], char *ob, char *stage, int lane) {
+  const int rr = lane & 15, quad = lane >> 4;
+  // after the regrouping this lane holds row rr (or 16 + rr), column block quad % 2, column half quad / 2
+  char *wbase = stage + rr * 128 + 8 * (quad >> 1);
+  const int tw = t_swizzle(rr), cb = 4 * (quad & 1);
+#pragma unroll
+  for (int bi = 0; bi < 2; ++bi) {
+    uint32_t lo[8], hi[8];  // [2 rq + word]: rows 0 .. 15 / rows 16 .. 31 of this row block
+#pragma unroll
+    for (int rq = 0; rq < 4; ++rq)
+#pragma unroll
+      for (int w = 0; w < 2; ++w) {
+        const uint32_t left = Tr::pack2(acc[0][bi][4 * rq + 2 * w], acc[0][bi][4 * rq + 2 * w + 1]);
+        const uint32_t right = Tr::pack2(acc[1][bi][4 * rq + 2 * w], acc[1][bi][4 * rq + 2 * w + 1]);
+        // lanes 16 .. 31 / 48 .. 63 of `left` trade places with lanes 0 .. 15 / 32 .. 47 of `right`
+        const u32x2 sw = __builtin_bit_cast(u32x2, __builtin_amdgcn_permlane16_swap(left, right, false, false));
+        lo[2 * rq + w] = sw[0];
+        hi[2 * rq + w] = sw[1];
+      }
+#pragma unroll
+    for (int hr = 0; hr < 2; ++hr) {
+#pragma unroll
+      for (int rq = 0; rq < 4; ++rq) {
+        const u32x2 v = hr == 0 ? u32x2{lo[2 * rq], lo[2 * rq + 1]} : u32x2{hi[2 * rq], hi[2 * rq + 1]};
+        // columns 32 (quad % 2) + 8 rq + 4 (quad / 2) .. + 3: chunk 4 (quad % 2) + rq
+        *reinterpret_cast<u32x2 *>(wbase + (((cb + rq) ^ tw) << 4)) = v;
+      }
+      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const int q = t * 64 + lane;
+        const int r = q >> 3, ch = q & 7;
+        const u32x4 v = *reinterpret_cast<const u32x4 *>(stage + r * 128 + ((ch ^ t_swizzle(r)) << 4));
+        // streaming store: the tile is not read again
+        __builtin_nontemporal_store(
+            v, reinterpret_cast<u32x4 *>(ob + (uint32_t)((32 * bi + 16 * hr + r) * 128 + ch * 16)));
+      }
+      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    }
+  }
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+}
+
+template <typename Tr>
+__global__ __launch_bounds__(kWaves * 64, 1) void matmul_rows_kernel(
+    const char *__restrict__ x, const char *__restrict__ y, char *__restrict__ out,
+    const int32_t *__restrict__ pair_offsets, const int32_t *__restrict__ pairs,
+    const int32_t *__restrict__ x_row_offsets, const int32_t *__restrict__ o_row_offsets,
+    const int32_t *__restrict__ row_order, int n_rows, int64_t nnz_x, int64_t nnz_y) {
+  extern __shared__ __attribute__((aligned(16))) char rows_smem[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  if ((int)blockIdx.x >= n_rows) return;
+  int row = row_order ? row_order[blockIdx.x] : (int)blockIdx.x;
+  row = __builtin_amdgcn_readfirstlane(row);
+  if (row < 0 || row >= n_rows) return;  // a corrupt table must not turn into a wild read
+  const int n0 = o_row_offsets[row], n1 = o_row_offsets[row + 1];
+  if (n0 >= n1) return;
+  const int xs = x_row_offsets[row];
+  int nx = x_row_offsets[row + 1] - xs;
+  nx = nx < kPanelCap ? nx : kPanelCap;
+  if (xs < 0 || xs + nx > nnz_x) nx = 0;
+  char *panel = rows_smem;
+  char *stage = rows_smem + kPanelCap * 8192 + wave * kStageBytes;
+
+  // the row's x blocks into the panel: piece idx = 1 KiB = 8 rows; LDS slot (row, position) holds chunk
+  // position ^ t_swizzle(row) of the row, so the lanes read the source permuted and land in lane order
+  {
+    const char *xsrc = x + (int64_t)xs * 8192;
+    const int rl = lane >> 3;
+    const int tsw = (((lane >> 4) & 3) << 1) | (wave & 1);  // t_swizzle(8 * piece + rl), piece % 8 == wave
+    const uint32_t src_off = rl * 128 + (((lane & 7) ^ tsw) << 4);
+    for (int idx = wave; idx < nx * 8; idx += kWaves) copy_1k_to_lds(xsrc + idx * 1024, src_off, panel + idx * 1024);
+  }
+
+  // This wave's run of output blocks: block b belongs to wave w when the pairs in front of it number at least
+  // w / 8 and less than (w + 1) / 8 of the row's pairs.  pair_offsets ascends, so the blocks in front of a
+  // boundary are counted with one ballot per 64 blocks.
+  const int row_p0 = pair_offsets[n0], row_p1 = pair_offsets[n1];
+  int wb0 = n0, wb1 = n1;
+  {
+    const int64_t span = row_p1 - row_p0;
+    const int lo = row_p0 + (int)((span * wave + kWaves - 1) / kWaves);
+    const int hi = row_p0 + (int)((span * (wave + 1) + kWaves - 1) / kWaves);
+    int below_lo = 0, below_hi = 0;
+    for (int base = n0; base < n1; base += 64) {
+      const int b = base + lane;
+      const int off = b < n1 ? pair_offsets[b] : 0x7fffffff;
+      below_lo += __builtin_popcountll(__ballot(off < lo));
+      below_hi += __builtin_popcountll(__ballot(off < hi));
+    }
+    if (wave > 0) wb0 = n0 + below_lo;
+    if (wave < kWaves - 1) wb1 = n0 + below_hi;
+    wb0 = __builtin_amdgcn_readfirstlane(wb0);
+    wb1 = __builtin_amdgcn_readfirstlane(wb1);
+  }
+  const int p_begin = __builtin_amdgcn_readfirstlane(pair_offsets[wb0]);
+  const int p_end = __builtin_amdgcn_readfirstlane(pair_offsets[wb1]);
+
+  // 64 entries of the pair list and 64 block boundaries at a time, one per lane
+  int win_base = p_begin, win_px = 0, win_py = 0;
+  int off_base = wb0, win_off = 0;
+  auto load_pair_window = [&](int base) {
+    win_base = base;
+    const int t = base + lane;
+    win_px = win_py = 0;
+    if (t < p_end) {
+      const int2 v = *reinterpret_cast<const int2 *>(pairs + 2 * (int64_t)t);
+      win_px = v.x;
+      win_py = v.y;
+    }
+    // a use right here: the wait for the load lands inside this (rarely taken) branch, not at the join
+    asm volatile("" : "+v"(win_px), "+v"(win_py));
+  };
+  auto load_offset_window = [&](int base) {
+    off_base = base;
+    const int n = base + lane;
+    win_off = pair_offsets[n <= wb1 ? n : wb1];
+    asm volatile("" : "+v"(win_off));
+  };
+  // end of the pair list of block n (n < wb1)
+  auto block_end = [&](int n) {
+    if (n + 1 - off_base >= 64) load_offset_window(n);
+    return __builtin_amdgcn_readlane(win_off, __builtin_amdgcn_readfirstlane(n + 1 - off_base));
+  };
+  // y block of pair t, clamped to the wave's last pair (loads stay unconditional)
+  auto y_block_of = [&](int t) -> const char * {
+    t = t < p_end ? t : p_end - 1;
+    int64_t py = __builtin_amdgcn_readlane(win_py, __builtin_amdgcn_readfirstlane(t - win_base));
+    py = (py < 0 || py >= nnz_y) ? 0 : py;
+    return y + py * 8192;
+  };
+  load_pair_window(p_begin);
+  load_offset_window(wb0);
+
+  const uint32_t lane_lo = 16 * lane, lane_hi = 16 * lane + 4096;
+  YSlot slot_a, slot_b;
+  const bool has_pairs = p_begin < p_end;
+  if (has_pairs) {
+    y_issue(slot_a, y_block_of(p_begin), lane_lo, lane_hi);
+    y_issue(slot_b, y_block_of(p_begin + 1), lane_lo, lane_hi);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) slot_a.v[i] = slot_b.v[i] = u32x4{0, 0, 0, 0};
+  }
+
+  LaneAddr la;
+  {
+    const int li = lane & 31, kg = lane >> 5;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int rs = 8 * h + (lane >> 3);
+      la.wr[h] = stage + rs * 128 + (((lane & 7) ^ t_swizzle(rs)) << 4);
+    }
+    const int g = lane >> 4, ls = lane & 15;
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int rd = 0; rd < 2; ++rd) {
+        const int rs = 8 * (g >> 1) + 4 * rd + (ls >> 2);
+        const int col = 32 * b + 16 * (g & 1) + 4 * (ls & 3);
+        la.tr[b][rd] = stage + rs * 128 + (((col >> 3) ^ t_swizzle(rs)) << 4) + ((col & 4) << 1);
+      }
+#pragma unroll
+    for (int s = 0; s < 4; ++s) la.xoff[s] = li * 128 + (((2 * s + kg) ^ t_swizzle(li)) << 4);
+  }
+
+  f32x16 acc[2][2];  // [block along j][block along i]
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+
+  // everything requested so far has arrived: the panel pieces of this wave and both slots
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  BSA_Y_WAIT(slot_a, 0);
+  BSA_Y_WAIT(slot_b, 0);
+  __syncthreads();
+
+  int t = p_begin;
+  int cur = wb0;
+  int blk_end = cur < wb1 ? block_end(cur) : -1;
+  bool flushed = false;
+  // blocks without pairs in front of the first pair
+  while (cur < wb1 && blk_end == t) {
+    rows_flush<Tr>(acc, out + (int64_t)cur * 8192, stage, lane);
+    ++cur;
+    blk_end = cur < wb1 ? block_end(cur) : -1;
+  }
+
+  // one pair from the given slot; the slot is refilled with the block of pair t + 2
+  auto do_pair = [&](YSlot &slot) {
+    // the window must hold pairs t .. t + 2
+    if (t + 2 - win_base >= 64) load_pair_window(t);
+    const int px = __builtin_amdgcn_readlane(win_px, __builtin_amdgcn_readfirstlane(t - win_base));
+    const char *next = y_block_of(t + 2);
+    // younger than this slot's loads: the other slot's 8 loads, and the 8 stores of a block written since
+    if (flushed)
+      asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    BSA_Y_TIE(slot);
+    flushed = false;
+    const bool resident = (unsigned)(px - xs) < (unsigned)nx;
+    int64_t pxc = px;
+    pxc = (pxc < 0 || pxc >= nnz_x) ? 0 : pxc;  // a corrupt list must not turn into a wild read
+    rows_pair<Tr>(acc, slot, panel + (resident ? px - xs : 0) * 8192, resident, x + pxc * 8192, la, next, lane_lo,
+                  lane_hi, lane);
+    ++t;
+    while (cur < wb1 && blk_end == t) {
+      rows_flush<Tr>(acc, out + (int64_t)cur * 8192, stage, lane);
+      flushed = true;
+      ++cur;
+      blk_end = cur < wb1 ? block_end(cur) : -1;
+    }
+  };
+  while (t < p_end) {
+    do_pair(slot_a);
+    if (t >= p_end) break;
+    do_pair(slot_b);
+  }
+  // the loads of the clamped last requests are still in flight: let them land before the wave ends
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
+template <typename Tr>
+int launch_rows(const void *x, const void *y, void *out, const int32_t *pair_offsets, const int32_t *pairs,
+                const int32_t *x_row_offsets, const int32_t *o_row_offsets, const int32_t *row_order,
+                int64_t n_rows, int64_t nnz_x, int64_t nnz_y, hipStream_t s) {
+  static bool configured = false;  // raising the dynamic LDS limit is per function, once per process
+  if (!configured) {
+    BSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&matmul_rows_kernel<Tr>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kRowsLds));
+    configured = true;
+  }
+  matmul_rows_kernel<Tr><<<(unsigned)n_rows, kWaves * 64, kRowsLds, s>>>(
+      static_cast<const char *>(x), static_cast<const char *>(y), static_cast<char *>(out), pair_offsets, pairs,
+      x_row_offsets, o_row_offsets, row_order, (int)n_rows, nnz_x, nnz_y);
+  return bsa::check_launch("matmul_rows_kernel");
+}
+
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+}  // namespace
+
+extern "C" int bsa_matmul_rows(const void *x, const void *y, void *out, const int32_t *pair_offsets,
+                               const int32_t *pairs, const int32_t *x_row_offsets, const int32_t *o_row_offsets,
+                               const int32_t *row_order, int64_t n_rows, int64_t nnz_o, int64_t nnz_x,
+                               int64_t nnz_y, int sbs, int dtype, bsa_stream_t stream) {
+  BSA_REQUIRE(sbs == 64, "bsa_matmul_rows: sbs must be 64 (got %d)", sbs);
+  BSA_REQUIRE(dtype == BSA_F16 || dtype == BSA_BF16, "bsa_matmul_rows: dtype must be fp16 or bf16 (got %d)", dtype);
+  BSA_REQUIRE(nnz_o >= 0 && nnz_x >= 0 && nnz_y >= 0 && n_rows >= 0, "bsa_matmul_rows: negative size");
+  if (nnz_o == 0 || n_rows == 0) return BSA_OK;
+  BSA_REQUIRE(out && pair_offsets && x_row_offsets && o_row_offsets, "bsa_matmul_rows: NULL pointer");
+  BSA_REQUIRE(aligned16(x) && aligned16(y) && aligned16(out), "bsa_matmul_rows: buffers must be 16-byte aligned");
+  BSA_REQUIRE(n_rows < 0x7fffffffLL, "bsa_matmul_rows: too many block rows");
+  hipStream_t s = bsa::as_stream(stream);
+  if (dtype == BSA_BF16)
+    return launch_rows<MBf16>(x, y, out, pair_offsets, pairs, x_row_offsets, o_row_offsets, row_order, n_rows, nnz_x,
+                              nnz_y, s);
+  return launch_rows<MF16>(x, y, out, pair_offsets, pairs, x_row_offsets, o_row_offsets, row_order, n_rows, nnz_x,
+                           nnz_y, s);
+}

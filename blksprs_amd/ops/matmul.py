@@ -38,7 +38,8 @@ def _launch_rows(x: Tensor, y: Tensor, cache: dict, n_rows: int, sbs: int) -> Te
         with torch.cuda.device(x.device):
             _capi.call("bsa_matmul_rows", _capi.ptr(x), _capi.ptr(y), out.data_ptr(),
                        cache["contraction_offsets"].data_ptr(), _capi.ptr(cache["contraction_pairs"]),
-                       cache["row_offsets_x"].data_ptr(), cache["row_offsets_o"].data_ptr(), n_rows, n_out,
+                       cache["row_offsets_x"].data_ptr(), cache["row_offsets_o"].data_ptr(),
+                       _capi.ptr(cache.get("row_order")), n_rows, n_out,
                        x.size(0), y.size(0), sbs, _capi.DTYPE_CODES[x.dtype], _capi.stream(x.device))
     return out
 
@@ -55,6 +56,36 @@ def _block_order(layout_indices: Tensor) -> Tensor:
     n_j = int(j.max().item()) // t + 1 if j.numel() else 1
     key = ((b * n_i + i // t) * n_j + j // t) * (t * t) + (i % t) * t + (j % t)
     return torch.argsort(key, stable=True).to(torch.int32)
+
+
+_N_XCD = 8
+
+
+def _row_order(pair_offsets: Tensor, row_offsets_o: Tensor | None, rows_per_batch: int) -> Tensor | None:
+    """Order in which the row kernel hands output block rows to workgroups.
+
+    Workgroup ``g`` runs on XCD ``g % 8``.  Every XCD gets one contiguous eighth of the rows (so the rows in
+    flight on one L2 belong to the same batch entry and stream through the same y blocks), and walks it batch
+    entry by batch entry, rows with the most (x, y) pairs first, so that the last workgroups of a launch are
+    the short ones.
+    """
+    if row_offsets_o is None or row_offsets_o.numel() < 2:
+        return None
+    n_rows = row_offsets_o.numel() - 1
+    ends = pair_offsets[row_offsets_o.long()]
+    work = (ends[1:] - ends[:-1]).long()
+    rows = torch.arange(n_rows, device=work.device)
+    small, extra = divmod(n_rows, _N_XCD)
+    sizes = torch.tensor([small + (c < extra) for c in range(_N_XCD)], device=work.device)
+    starts = torch.cumsum(sizes, 0) - sizes
+    chunk = torch.repeat_interleave(torch.arange(_N_XCD, device=work.device), sizes)
+    key = (chunk * (n_rows // max(rows_per_batch, 1) + 1) + rows // max(rows_per_batch, 1)) * (int(work.max()) + 1) \
+        + (int(work.max()) - work)
+    by_chunk = torch.argsort(key, stable=True)           # chunk-major, batch entry ascending, work descending
+    place = (rows - starts[chunk]) * _N_XCD + chunk       # k-th row of chunk c goes to position 8 k + c
+    order = torch.empty(n_rows, dtype=torch.int32, device=work.device)
+    order[place] = by_chunk.to(torch.int32)
+    return order
 
 
 def _backward_lists(layout_cache: dict, shape_x, shape_y):
@@ -136,6 +167,7 @@ def matmul_build_layout_cache(layout_cache: dict | None, sparsity_layout_x: Tens
         layout_cache["block_order"] = _block_order(layout_cache["layout_indices_o"])
         layout_cache["row_offsets_x"] = info_x.row_offsets
         layout_cache["row_offsets_o"] = info_o.row_offsets
+        layout_cache["row_order"] = _row_order(lists.pair_offsets, info_o.row_offsets, R)
 
     validate_contiguous(sparsity_layout_x, layout_cache["packed_indices_x"],
                         sparsity_layout_y, layout_cache["packed_indices_y"],

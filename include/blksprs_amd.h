@@ -183,13 +183,16 @@ int bsa_matmul(const void *x, const void *y, void *out, const int32_t *pair_offs
  * The same product for fp16 / bf16 operands with sbs == 64, organised by output block row: the x
  * blocks of a row are kept in LDS while the row's output blocks are computed.  x_row_offsets and
  * o_row_offsets are the int32 CSR row offsets (n_rows + 1 entries, rows = B * R) of the x layout
- * and of the output layout as bsa_lut_packed(row_len = ...) writes them.  Bit-identical results to
- * bsa_matmul (same accumulation order).  Same reference counterpart as bsa_matmul.
+ * and of the output layout as bsa_lut_packed(row_len = ...) writes them.  row_order (n_rows int32,
+ * a permutation of the rows, or NULL for 0, 1, 2, ...) is the order in which rows are handed to
+ * workgroups; rows sorted by descending number of pairs keep the tail of the launch short.
+ * Bit-identical results to bsa_matmul (same accumulation order).  Same reference counterpart as
+ * bsa_matmul.
  */
 int bsa_matmul_rows(const void *x, const void *y, void *out, const int32_t *pair_offsets,
                     const int32_t *pairs, const int32_t *x_row_offsets, const int32_t *o_row_offsets,
-                    int64_t n_rows, int64_t nnz_o, int64_t nnz_x, int64_t nnz_y, int sbs, int dtype,
-                    bsa_stream_t stream);
+                    const int32_t *row_order, int64_t n_rows, int64_t nnz_o, int64_t nnz_x, int64_t nnz_y,
+                    int sbs, int dtype, bsa_stream_t stream);
 
 /* ------------------------------------------------------------- attention */
 
