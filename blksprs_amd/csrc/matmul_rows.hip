@@ -23,7 +23,8 @@
 // as stored (k rows), and read back with the transposing LDS load, which delivers the matrix-core operand
 // whose contraction index runs over rows; the x operand is a 128-bit row read from the panel.  LDS executes
 // one wave's instructions in order, so stage writes and reads of consecutive quarters are queued back to
-// back without waits in between; only the fragment registers bound the depth.
+// back without waits in between; only the fragment registers bound the depth.  The loop is software pipelined
+// across pairs (the first half of the next pair is staged while the second half of this one is multiplied).
 //
 // The product is formed transposed (y fragments as the A operand, x fragments as B), which leaves 4
 // consecutive output columns of one row in each lane; a finished block is rounded, passed through the stage
@@ -73,6 +74,11 @@ __device__ __forceinline__ void y_issue(YSlot &s, const char *yb, uint32_t lane_
                :                                                                                               \
                : "memory")
 
+// XOR applied to the 16-byte chunk index of row r of a y quarter in the stage.  A transposing read serves 32
+// lanes at a time: rows r .. r + 3 (r a multiple of 4), 64 consecutive bytes of each.  Two 128-byte rows span
+// the 64 banks once, so rows r and r + 2 must put their 64 bytes into different halves of the row.
+__device__ __forceinline__ int y_swizzle(int r) { return ((r >> 1) & 1) << 2; }
+
 __device__ __forceinline__ u32x2 read_tr(const char *p) {
   const i16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4 *)p);
   return __builtin_bit_cast(u32x2, v);
@@ -85,58 +91,49 @@ struct LaneAddr {
   uint32_t xoff[4];  // x fragment of k step s inside a panel block (row lane % 32; the second row block is + 4096)
 };
 
-// One (x block, y block) product.  xsrc is an x block's swizzled copy in LDS; if the x block is not resident,
-// its fragments are read from global memory at xglob instead (wave uniform).
-// `next` is the y block to request into the slot once its registers are free.
+// operand fragments of one quarter (16 k) of a pair: [column block] of y, [row block] of x
+struct Frags {
+  u32x4 fy[2], fx[2];
+};
+
+// where the x block of a pair is read from: its swizzled copy in the panel, or (not resident: rare) global
+// memory; all wave uniform
+struct XSource {
+  const char *lds;
+  const char *glob;
+  bool resident;
+};
+
+// Writes quarter S (k = 16 S .. 16 S + 15) of the y block in the slot to the stage and reads the quarter's
+// operand fragments: y with transposing reads from the stage, x with 128-bit row reads from the panel.
+template <int S>
+__device__ __forceinline__ void stage_and_read(Frags &f, const YSlot &ys, const XSource &xs, const LaneAddr &la,
+                                               int lane) {
+  *reinterpret_cast<u32x4 *>(la.wr[0]) = ys.v[2 * S];
+  *reinterpret_cast<u32x4 *>(la.wr[1]) = ys.v[2 * S + 1];
+#pragma unroll
+  for (int b = 0; b < 2; ++b) {
+    const u32x2 lo = read_tr(la.tr[b][0]), hi = read_tr(la.tr[b][1]);
+    f.fy[b] = u32x4{lo[0], lo[1], hi[0], hi[1]};
+    f.fx[b] = *reinterpret_cast<const u32x4 *>(xs.lds + la.xoff[S] + 4096 * b);
+  }
+  if (!xs.resident) {
+    // rare: only the fragments pass through the branch (not the accumulators), and they are used inside it,
+    // which puts the wait for these loads here and not in front of the multiplications of every pair
+    const int li = lane & 31, kg = lane >> 5;
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+      f.fx[b] = *reinterpret_cast<const u32x4 *>(xs.glob + (uint32_t)((32 * b + li) * 128 + (2 * S + kg) * 16));
+    asm volatile("" : "+v"(f.fx[0]), "+v"(f.fx[1]));
+  }
+}
+
 template <typename Tr>
-__device__ __forceinline__ void rows_pair(f32x16 (&acc)[2][2], YSlot &ys, const char *xsrc, bool resident,
-                                          const char *xglob, const LaneAddr &la, const char *next, uint32_t lane_lo, uint32_t lane_hi,
-                                          int lane) {
-  const int li = lane & 31, kg = lane >> 5;
-  u32x4 fy[2][2], fx[2][2];  // [quarter parity][block]
-  auto stage_quarter = [&](int s) {
-    *reinterpret_cast<u32x4 *>(la.wr[0]) = ys.v[2 * s];
-    *reinterpret_cast<u32x4 *>(la.wr[1]) = ys.v[2 * s + 1];
-  };
-  auto read_quarter = [&](int s) {
+__device__ __forceinline__ void multiply(f32x16 (&acc)[2][2], const Frags &f) {
 #pragma unroll
-    for (int b = 0; b < 2; ++b) {
-      const u32x2 lo = read_tr(la.tr[b][0]), hi = read_tr(la.tr[b][1]);
-      fy[s & 1][b] = u32x4{lo[0], lo[1], hi[0], hi[1]};
-      fx[s & 1][b] = *reinterpret_cast<const u32x4 *>(xsrc + la.xoff[s] + 4096 * b);
-    }
-    if (!resident) {
-      // rare: only the fragments pass through the branch (not the accumulators), and they are used inside it,
-      // which puts the wait for these loads here and not in front of the multiplications of every pair
+  for (int bj = 0; bj < 2; ++bj)
 #pragma unroll
-      for (int b = 0; b < 2; ++b)
-        fx[s & 1][b] = *reinterpret_cast<const u32x4 *>(xglob + (uint32_t)((32 * b + li) * 128 + (2 * s + kg) * 16));
-      asm volatile("" : "+v"(fx[s & 1][0]), "+v"(fx[s & 1][1]));
-    }
-  };
-  auto multiply = [&](int s) {
-#pragma unroll
-    for (int bj = 0; bj < 2; ++bj)
-#pragma unroll
-      for (int bi = 0; bi < 2; ++bi) acc[bj][bi] = Tr::mfma(fy[s & 1][bj], fx[s & 1][bi], acc[bj][bi]);
-  };
-  stage_quarter(0);
-  read_quarter(0);
-  stage_quarter(1);
-  read_quarter(1);
-  __builtin_amdgcn_sched_barrier(0);
-  multiply(0);
-  stage_quarter(2);
-  read_quarter(2);
-  __builtin_amdgcn_sched_barrier(0);
-  multiply(1);
-  stage_quarter(3);
-  // the slot's registers have been handed to the LDS writes: request the block of the pair after next
-  y_issue(ys, next, lane_lo, lane_hi);
-  read_quarter(3);
-  __builtin_amdgcn_sched_barrier(0);
-  multiply(2);
-  multiply(3);
+    for (int bi = 0; bi < 2; ++bi) acc[bj][bi] = Tr::mfma(f.fy[bj], f.fx[bi], acc[bj][bi]);
 }
 
 // Rounds the tile, passes it through the wave's stage 16 rows at a time, writes it as one block with 16-byte
@@ -151,6 +148,7 @@ __device__ __forceinline__ void rows_flush(f32x16 (&acc)[2][2], char *ob, char *
   // after the regrouping this lane holds row rr (or 16 + rr), column block quad % 2, column half quad / 2
   char *wbase = stage + rr * 128 + 8 * (quad >> 1);
   const int tw = t_swizzle(rr), cb = 4 * (quad & 1);
+  u32x4 back[2][2][2];  // [row block][half of 16 rows][store]
 #pragma unroll
   for (int bi = 0; bi < 2; ++bi) {
     uint32_t lo[8], hi[8];  // [2 rq + word]: rows 0 .. 15 / rows 16 .. 31 of this row block
@@ -165,6 +163,9 @@ __device__ __forceinline__ void rows_flush(f32x16 (&acc)[2][2], char *ob, char *
         lo[2 * rq + w] = sw[0];
         hi[2 * rq + w] = sw[1];
       }
+    // LDS executes this wave's instructions in order: the reads of one step see its writes and are done
+    // before the next step's writes land, so the four steps are queued without waiting in between (the wave
+    // barriers only keep the compiler from reordering them; they emit nothing)
 #pragma unroll
     for (int hr = 0; hr < 2; ++hr) {
 #pragma unroll
@@ -173,19 +174,28 @@ __device__ __forceinline__ void rows_flush(f32x16 (&acc)[2][2], char *ob, char *
         // columns 32 (quad % 2) + 8 rq + 4 (quad / 2) .. + 3: chunk 4 (quad % 2) + rq
         *reinterpret_cast<u32x2 *>(wbase + (((cb + rq) ^ tw) << 4)) = v;
       }
-      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+      __builtin_amdgcn_wave_barrier();
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
         const int q = t * 64 + lane;
         const int r = q >> 3, ch = q & 7;
-        const u32x4 v = *reinterpret_cast<const u32x4 *>(stage + r * 128 + ((ch ^ t_swizzle(r)) << 4));
-        // streaming store: the tile is not read again
-        __builtin_nontemporal_store(
-            v, reinterpret_cast<u32x4 *>(ob + (uint32_t)((32 * bi + 16 * hr + r) * 128 + ch * 16)));
+        back[bi][hr][t] = *reinterpret_cast<const u32x4 *>(stage + r * 128 + ((ch ^ t_swizzle(r)) << 4));
       }
-      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+      __builtin_amdgcn_wave_barrier();
     }
   }
+#pragma unroll
+  for (int bi = 0; bi < 2; ++bi)
+#pragma unroll
+    for (int hr = 0; hr < 2; ++hr)
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const int q = t * 64 + lane;
+        const int r = q >> 3, ch = q & 7;
+        // streaming store: the tile is not read again
+        __builtin_nontemporal_store(
+            back[bi][hr][t], reinterpret_cast<u32x4 *>(ob + (uint32_t)((32 * bi + 16 * hr + r) * 128 + ch * 16)));
+      }
 #pragma unroll
   for (int a = 0; a < 2; ++a)
 #pragma unroll
@@ -276,7 +286,7 @@ __global__ __launch_bounds__(kWaves * 64, 1) void matmul_rows_kernel(
     if (n + 1 - off_base >= 64) load_offset_window(n);
     return __builtin_amdgcn_readlane(win_off, __builtin_amdgcn_readfirstlane(n + 1 - off_base));
   };
-  // y block of pair t, clamped to the wave's last pair (loads stay unconditional)
+  // y block of pair t (clamped to the wave's last pair: the lookup stays in the window)
   auto y_block_of = [&](int t) -> const char * {
     t = t < p_end ? t : p_end - 1;
     int64_t py = __builtin_amdgcn_readlane(win_py, __builtin_amdgcn_readfirstlane(t - win_base));
@@ -289,13 +299,12 @@ __global__ __launch_bounds__(kWaves * 64, 1) void matmul_rows_kernel(
   const uint32_t lane_lo = 16 * lane, lane_hi = 16 * lane + 4096;
   YSlot slot_a, slot_b;
   const bool has_pairs = p_begin < p_end;
-  if (has_pairs) {
-    y_issue(slot_a, y_block_of(p_begin), lane_lo, lane_hi);
-    y_issue(slot_b, y_block_of(p_begin + 1), lane_lo, lane_hi);
-  } else {
+  // A block is only requested if its pair exists: registers whose contents are never used are free for the
+  // compiler to reuse, also while a load into them is still in flight.
 #pragma unroll
-    for (int i = 0; i < 8; ++i) slot_a.v[i] = slot_b.v[i] = u32x4{0, 0, 0, 0};
-  }
+  for (int i = 0; i < 8; ++i) slot_a.v[i] = slot_b.v[i] = u32x4{0, 0, 0, 0};
+  if (has_pairs) y_issue(slot_a, y_block_of(p_begin), lane_lo, lane_hi);
+  if (p_begin + 1 < p_end) y_issue(slot_b, y_block_of(p_begin + 1), lane_lo, lane_hi);
 
   LaneAddr la;
   {
@@ -303,7 +312,7 @@ __global__ __launch_bounds__(kWaves * 64, 1) void matmul_rows_kernel(
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       const int rs = 8 * h + (lane >> 3);
-      la.wr[h] = stage + rs * 128 + (((lane & 7) ^ t_swizzle(rs)) << 4);
+      la.wr[h] = stage + rs * 128 + (((lane & 7) ^ y_swizzle(rs)) << 4);
     }
     const int g = lane >> 4, ls = lane & 15;
 #pragma unroll
@@ -312,7 +321,7 @@ __global__ __launch_bounds__(kWaves * 64, 1) void matmul_rows_kernel(
       for (int rd = 0; rd < 2; ++rd) {
         const int rs = 8 * (g >> 1) + 4 * rd + (ls >> 2);
         const int col = 32 * b + 16 * (g & 1) + 4 * (ls & 3);
-        la.tr[b][rd] = stage + rs * 128 + (((col >> 3) ^ t_swizzle(rs)) << 4) + ((col & 4) << 1);
+        la.tr[b][rd] = stage + rs * 128 + (((col >> 3) ^ y_swizzle(rs)) << 4) + ((col & 4) << 1);
       }
 #pragma unroll
     for (int s = 0; s < 4; ++s) la.xoff[s] = li * 128 + (((2 * s + kg) ^ t_swizzle(li)) << 4);
@@ -335,7 +344,7 @@ __global__ __launch_bounds__(kWaves * 64, 1) void matmul_rows_kernel(
   int t = p_begin;
   int cur = wb0;
   int blk_end = cur < wb1 ? block_end(cur) : -1;
-  bool flushed = false;
+  int flushed = 0;  // a block was written after the last pair
   // blocks without pairs in front of the first pair
   while (cur < wb1 && blk_end == t) {
     rows_flush<Tr>(acc, out + (int64_t)cur * 8192, stage, lane);
@@ -343,38 +352,79 @@ __global__ __launch_bounds__(kWaves * 64, 1) void matmul_rows_kernel(
     blk_end = cur < wb1 ? block_end(cur) : -1;
   }
 
-  // one pair from the given slot; the slot is refilled with the block of pair t + 2
-  auto do_pair = [&](YSlot &slot) {
-    // the window must hold pairs t .. t + 2
-    if (t + 2 - win_base >= 64) load_pair_window(t);
+  // x block of pair t (the window must hold it)
+  auto x_source_of = [&](int t) {
     const int px = __builtin_amdgcn_readlane(win_px, __builtin_amdgcn_readfirstlane(t - win_base));
-    const char *next = y_block_of(t + 2);
-    // younger than this slot's loads: the other slot's 8 loads, and the 8 stores of a block written since
-    if (flushed)
-      asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
-    else
-      asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-    BSA_Y_TIE(slot);
-    flushed = false;
-    const bool resident = (unsigned)(px - xs) < (unsigned)nx;
+    XSource src;
+    src.resident = (unsigned)(px - xs) < (unsigned)nx;
     int64_t pxc = px;
     pxc = (pxc < 0 || pxc >= nnz_x) ? 0 : pxc;  // a corrupt list must not turn into a wild read
-    rows_pair<Tr>(acc, slot, panel + (resident ? px - xs : 0) * 8192, resident, x + pxc * 8192, la, next, lane_lo,
-                  lane_hi, lane);
+    src.lds = panel + (src.resident ? px - xs : 0) * 8192;
+    src.glob = x + pxc * 8192;
+    return src;
+  };
+
+  // The loop is software pipelined across pairs: while the last two quarters of pair t are multiplied, the
+  // first two quarters of pair t + 1 are staged and their fragments read, so the matrix core does not wait
+  // for LDS at the start of a pair.  f0 / f1 hold the fragments of the quarter multiplied next / after it.
+  Frags f0, f1;
+  XSource x_cur{panel, x, true};
+  if (has_pairs) {
+    x_cur = x_source_of(t);
+    stage_and_read<0>(f0, slot_a, x_cur, la, lane);
+    stage_and_read<1>(f1, slot_a, x_cur, la, lane);
+  } else {
+#pragma unroll
+    for (int b = 0; b < 2; ++b) f0.fy[b] = f0.fx[b] = f1.fy[b] = f1.fx[b] = u32x4{0, 0, 0, 0};
+  }
+
+  // pair t from slot `cur_slot` (its first two quarters are in f0 / f1 already); `next_slot` holds pair t + 1
+  auto do_pair = [&](YSlot &cur_slot, YSlot &next_slot) {
+    // the window must hold pairs t .. t + 2
+    if (t + 2 - win_base >= 64) load_pair_window(t);
+    const char *next = y_block_of(t + 2);
+    const bool more = t + 1 < p_end, request = t + 2 < p_end;
+    const XSource x_next = x_source_of(more ? t + 1 : t);
+    __builtin_amdgcn_sched_barrier(0);
+    multiply<Tr>(acc, f0);
+    stage_and_read<2>(f0, cur_slot, x_cur, la, lane);
+    __builtin_amdgcn_sched_barrier(0);
+    multiply<Tr>(acc, f1);
+    stage_and_read<3>(f1, cur_slot, x_cur, la, lane);
+    // the slot's registers have been handed to the LDS writes: request the block of the pair after next
+    if (request) y_issue(cur_slot, next, lane_lo, lane_hi);
+    __builtin_amdgcn_sched_barrier(0);
+    multiply<Tr>(acc, f0);
+    if (more) {
+      // younger than the next slot's loads (issued during the pair before this one): the 8 loads just issued
+      // (unless this is the last but one pair), and the 8 stores of a block written after that pair
+      if (!request)
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      else if (flushed)
+        asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+      else
+        asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+      BSA_Y_TIE(next_slot);
+      stage_and_read<0>(f0, next_slot, x_next, la, lane);
+    }
+    flushed = 0;
+    __builtin_amdgcn_sched_barrier(0);
+    multiply<Tr>(acc, f1);
+    if (more) stage_and_read<1>(f1, next_slot, x_next, la, lane);
+    x_cur = x_next;
     ++t;
     while (cur < wb1 && blk_end == t) {
       rows_flush<Tr>(acc, out + (int64_t)cur * 8192, stage, lane);
-      flushed = true;
+      flushed = 1;
       ++cur;
       blk_end = cur < wb1 ? block_end(cur) : -1;
     }
   };
   while (t < p_end) {
-    do_pair(slot_a);
+    do_pair(slot_a, slot_b);
     if (t >= p_end) break;
-    do_pair(slot_b);
+    do_pair(slot_b, slot_a);
   }
-  // the loads of the clamped last requests are still in flight: let them land before the wave ends
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
