@@ -44,9 +44,12 @@ struct YSlot {
   u32x4 v[8];  // v[i] = rows 8 i + lane / 8, chunk lane % 8 of one 64 x 64 block
 };
 
-// requests the 8 KiB block at yb into the slot; lane_lo = 16 * lane, lane_hi = lane_lo + 4096
+// requests the 8 KiB block at yb into the slot; lane_lo = 16 * lane, lane_hi = lane_lo + 4096.  The address
+// arrives in scalar registers that a vector instruction (v_readlane) may have written just before: a vector
+// memory instruction must not read such a register within the next 5 wait states, and the compiler does not
+// look into inline assembly, so the wait states are spelled out here.
 __device__ __forceinline__ void y_issue(YSlot &s, const char *yb, uint32_t lane_lo, uint32_t lane_hi) {
-  asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(s.v[0]) : "v"(lane_lo), "s"(yb) : "memory");
+  asm volatile("s_nop 4\n\tglobal_load_dwordx4 %0, %1, %2" : "=v"(s.v[0]) : "v"(lane_lo), "s"(yb) : "memory");
   asm volatile("global_load_dwordx4 %0, %1, %2 offset:1024" : "=v"(s.v[1]) : "v"(lane_lo), "s"(yb) : "memory");
   asm volatile("global_load_dwordx4 %0, %1, %2 offset:2048" : "=v"(s.v[2]) : "v"(lane_lo), "s"(yb) : "memory");
   asm volatile("global_load_dwordx4 %0, %1, %2 offset:3072" : "=v"(s.v[3]) : "v"(lane_lo), "s"(yb) : "memory");
@@ -100,7 +103,7 @@ struct Frags {
 // memory; all wave uniform
 struct XSource {
   const char *lds;
-  const char *glob;
+  int px;  // packed index of the x block (range checked), for the read from global memory
   bool resident;
 };
 
@@ -108,7 +111,7 @@ struct XSource {
 // operand fragments: y with transposing reads from the stage, x with 128-bit row reads from the panel.
 template <int S>
 __device__ __forceinline__ void stage_and_read(Frags &f, const YSlot &ys, const XSource &xs, const LaneAddr &la,
-                                               int lane) {
+                                               const char *x, int lane) {
   *reinterpret_cast<u32x4 *>(la.wr[0]) = ys.v[2 * S];
   *reinterpret_cast<u32x4 *>(la.wr[1]) = ys.v[2 * S + 1];
 #pragma unroll
@@ -121,9 +124,10 @@ __device__ __forceinline__ void stage_and_read(Frags &f, const YSlot &ys, const 
     // rare: only the fragments pass through the branch (not the accumulators), and they are used inside it,
     // which puts the wait for these loads here and not in front of the multiplications of every pair
     const int li = lane & 31, kg = lane >> 5;
+    const char *xglob = x + (int64_t)xs.px * 8192;
 #pragma unroll
     for (int b = 0; b < 2; ++b)
-      f.fx[b] = *reinterpret_cast<const u32x4 *>(xs.glob + (uint32_t)((32 * b + li) * 128 + (2 * S + kg) * 16));
+      f.fx[b] = *reinterpret_cast<const u32x4 *>(xglob + (uint32_t)((32 * b + li) * 128 + (2 * S + kg) * 16));
     asm volatile("" : "+v"(f.fx[0]), "+v"(f.fx[1]));
   }
 }
@@ -260,20 +264,29 @@ __global__ __launch_bounds__(kWaves * 64, 1) void matmul_rows_kernel(
   const int p_begin = __builtin_amdgcn_readfirstlane(pair_offsets[wb0]);
   const int p_end = __builtin_amdgcn_readfirstlane(pair_offsets[wb1]);
 
-  // 64 entries of the pair list and 64 block boundaries at a time, one per lane
-  int win_base = p_begin, win_px = 0, win_py = 0;
+  // 64 entries of the pair list and 64 block boundaries at a time, one per lane.  A lane turns its entry into
+  // what the loop needs per pair (the address of the y block; the panel offset of the x block, or -1 if it is
+  // not resident), so that a pair costs a few v_readlane and no address arithmetic.
+  int win_base = p_begin, win_px = 0, win_xoff = 0;
+  uint32_t win_ylo = 0, win_yhi = 0;
   int off_base = wb0, win_off = 0;
   auto load_pair_window = [&](int base) {
     win_base = base;
     const int t = base + lane;
-    win_px = win_py = 0;
+    int px = 0, py = 0;
     if (t < p_end) {
       const int2 v = *reinterpret_cast<const int2 *>(pairs + 2 * (int64_t)t);
-      win_px = v.x;
-      win_py = v.y;
+      px = v.x;
+      py = v.y;
     }
+    // a corrupt list must not turn into a wild read
+    const uint64_t ya = reinterpret_cast<uint64_t>(y) + (uint64_t)((py < 0 || py >= nnz_y) ? 0 : py) * 8192;
+    win_ylo = (uint32_t)ya;
+    win_yhi = (uint32_t)(ya >> 32);
+    win_px = (px < 0 || px >= nnz_x) ? 0 : px;
+    win_xoff = (unsigned)(px - xs) < (unsigned)nx ? (px - xs) * 8192 : -1;
     // a use right here: the wait for the load lands inside this (rarely taken) branch, not at the join
-    asm volatile("" : "+v"(win_px), "+v"(win_py));
+    asm volatile("" : "+v"(win_px), "+v"(win_xoff), "+v"(win_ylo), "+v"(win_yhi));
   };
   auto load_offset_window = [&](int base) {
     off_base = base;
@@ -289,22 +302,15 @@ __global__ __launch_bounds__(kWaves * 64, 1) void matmul_rows_kernel(
   // y block of pair t (clamped to the wave's last pair: the lookup stays in the window)
   auto y_block_of = [&](int t) -> const char * {
     t = t < p_end ? t : p_end - 1;
-    int64_t py = __builtin_amdgcn_readlane(win_py, __builtin_amdgcn_readfirstlane(t - win_base));
-    py = (py < 0 || py >= nnz_y) ? 0 : py;
-    return y + py * 8192;
+    const int sel = __builtin_amdgcn_readfirstlane(t - win_base);
+    const uint32_t lo = __builtin_amdgcn_readlane(win_ylo, sel), hi = __builtin_amdgcn_readlane(win_yhi, sel);
+    return reinterpret_cast<const char *>(((uint64_t)hi << 32) | lo);
   };
   load_pair_window(p_begin);
   load_offset_window(wb0);
 
   const uint32_t lane_lo = 16 * lane, lane_hi = 16 * lane + 4096;
-  YSlot slot_a, slot_b;
   const bool has_pairs = p_begin < p_end;
-  // A block is only requested if its pair exists: registers whose contents are never used are free for the
-  // compiler to reuse, also while a load into them is still in flight.
-#pragma unroll
-  for (int i = 0; i < 8; ++i) slot_a.v[i] = slot_b.v[i] = u32x4{0, 0, 0, 0};
-  if (has_pairs) y_issue(slot_a, y_block_of(p_begin), lane_lo, lane_hi);
-  if (p_begin + 1 < p_end) y_issue(slot_b, y_block_of(p_begin + 1), lane_lo, lane_hi);
 
   LaneAddr la;
   {
@@ -335,32 +341,53 @@ __global__ __launch_bounds__(kWaves * 64, 1) void matmul_rows_kernel(
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
 
+  int cur = wb0;
+  int blk_end = cur < wb1 ? block_end(cur) : -1;
+  // writes the blocks that end at pair t (the first holds the sums, the others have no pairs: zeros)
+  auto flush_until = [&](int t) {
+    bool any = false;
+    while (cur < wb1 && blk_end == t) {
+      rows_flush<Tr>(acc, out + (int64_t)cur * 8192, stage, lane);
+      any = true;
+      ++cur;
+      blk_end = cur < wb1 ? block_end(cur) : -1;
+    }
+    return any;
+  };
+
+  if (!has_pairs) {
+    // only blocks without pairs (or none at all): wait for this wave's panel pieces, then write zeros
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    flush_until(p_begin);
+    return;
+  }
+
+  // The registers of a slot are written by loads the compiler does not know of.  Two rules keep it from ever
+  // touching them while a load is in flight: (1) no load sits in a branch of its own (a join could make the
+  // compiler copy the registers), so blocks are requested unconditionally, the last two requests of a wave
+  // repeat its last block; (2) every request is consumed, the last ones by the statement after the loop that
+  // passes both slots through (registers whose contents are never used may be reused at once).
+  YSlot slot_a, slot_b;
+  y_issue(slot_a, y_block_of(p_begin), lane_lo, lane_hi);
+  y_issue(slot_b, y_block_of(p_begin + 1), lane_lo, lane_hi);
   // everything requested so far has arrived: the panel pieces of this wave and both slots
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   BSA_Y_WAIT(slot_a, 0);
-  BSA_Y_WAIT(slot_b, 0);
+  BSA_Y_TIE(slot_b);
   __syncthreads();
 
   int t = p_begin;
-  int cur = wb0;
-  int blk_end = cur < wb1 ? block_end(cur) : -1;
   int flushed = 0;  // a block was written after the last pair
-  // blocks without pairs in front of the first pair
-  while (cur < wb1 && blk_end == t) {
-    rows_flush<Tr>(acc, out + (int64_t)cur * 8192, stage, lane);
-    ++cur;
-    blk_end = cur < wb1 ? block_end(cur) : -1;
-  }
+  flush_until(t);   // blocks without pairs in front of the first pair
 
   // x block of pair t (the window must hold it)
   auto x_source_of = [&](int t) {
-    const int px = __builtin_amdgcn_readlane(win_px, __builtin_amdgcn_readfirstlane(t - win_base));
+    const int sel = __builtin_amdgcn_readfirstlane(t - win_base);
+    const int xoff = __builtin_amdgcn_readlane(win_xoff, sel);
     XSource src;
-    src.resident = (unsigned)(px - xs) < (unsigned)nx;
-    int64_t pxc = px;
-    pxc = (pxc < 0 || pxc >= nnz_x) ? 0 : pxc;  // a corrupt list must not turn into a wild read
-    src.lds = panel + (src.resident ? px - xs : 0) * 8192;
-    src.glob = x + pxc * 8192;
+    src.resident = xoff >= 0;
+    src.lds = panel + (xoff >= 0 ? xoff : 0);
+    src.px = __builtin_amdgcn_readlane(win_px, sel);
     return src;
   };
 
@@ -368,64 +395,51 @@ __global__ __launch_bounds__(kWaves * 64, 1) void matmul_rows_kernel(
   // first two quarters of pair t + 1 are staged and their fragments read, so the matrix core does not wait
   // for LDS at the start of a pair.  f0 / f1 hold the fragments of the quarter multiplied next / after it.
   Frags f0, f1;
-  XSource x_cur{panel, x, true};
-  if (has_pairs) {
-    x_cur = x_source_of(t);
-    stage_and_read<0>(f0, slot_a, x_cur, la, lane);
-    stage_and_read<1>(f1, slot_a, x_cur, la, lane);
-  } else {
-#pragma unroll
-    for (int b = 0; b < 2; ++b) f0.fy[b] = f0.fx[b] = f1.fy[b] = f1.fx[b] = u32x4{0, 0, 0, 0};
-  }
+  XSource x_cur = x_source_of(t);
+  stage_and_read<0>(f0, slot_a, x_cur, la, x, lane);
+  stage_and_read<1>(f1, slot_a, x_cur, la, x, lane);
 
   // pair t from slot `cur_slot` (its first two quarters are in f0 / f1 already); `next_slot` holds pair t + 1
   auto do_pair = [&](YSlot &cur_slot, YSlot &next_slot) {
     // the window must hold pairs t .. t + 2
     if (t + 2 - win_base >= 64) load_pair_window(t);
     const char *next = y_block_of(t + 2);
-    const bool more = t + 1 < p_end, request = t + 2 < p_end;
+    const bool more = t + 1 < p_end;
     const XSource x_next = x_source_of(more ? t + 1 : t);
     __builtin_amdgcn_sched_barrier(0);
     multiply<Tr>(acc, f0);
-    stage_and_read<2>(f0, cur_slot, x_cur, la, lane);
+    stage_and_read<2>(f0, cur_slot, x_cur, la, x, lane);
     __builtin_amdgcn_sched_barrier(0);
     multiply<Tr>(acc, f1);
-    stage_and_read<3>(f1, cur_slot, x_cur, la, lane);
+    stage_and_read<3>(f1, cur_slot, x_cur, la, x, lane);
     // the slot's registers have been handed to the LDS writes: request the block of the pair after next
-    if (request) y_issue(cur_slot, next, lane_lo, lane_hi);
+    y_issue(cur_slot, next, lane_lo, lane_hi);
     __builtin_amdgcn_sched_barrier(0);
     multiply<Tr>(acc, f0);
-    if (more) {
-      // younger than the next slot's loads (issued during the pair before this one): the 8 loads just issued
-      // (unless this is the last but one pair), and the 8 stores of a block written after that pair
-      if (!request)
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      else if (flushed)
-        asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
-      else
-        asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-      BSA_Y_TIE(next_slot);
-      stage_and_read<0>(f0, next_slot, x_next, la, lane);
-    }
+    // younger than the next slot's loads (issued during the pair before this one): the 8 loads just issued,
+    // and the 8 stores of a block written after that pair
+    if (flushed)
+      asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    BSA_Y_TIE(next_slot);
     flushed = 0;
+    if (more) stage_and_read<0>(f0, next_slot, x_next, la, x, lane);
     __builtin_amdgcn_sched_barrier(0);
     multiply<Tr>(acc, f1);
-    if (more) stage_and_read<1>(f1, next_slot, x_next, la, lane);
+    if (more) stage_and_read<1>(f1, next_slot, x_next, la, x, lane);
     x_cur = x_next;
     ++t;
-    while (cur < wb1 && blk_end == t) {
-      rows_flush<Tr>(acc, out + (int64_t)cur * 8192, stage, lane);
-      flushed = 1;
-      ++cur;
-      blk_end = cur < wb1 ? block_end(cur) : -1;
-    }
+    if (flush_until(t)) flushed = 1;
   };
   while (t < p_end) {
     do_pair(slot_a, slot_b);
     if (t >= p_end) break;
     do_pair(slot_b, slot_a);
   }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  // the last requests land here
+  BSA_Y_WAIT(slot_a, 0);
+  BSA_Y_TIE(slot_b);
 }
 
 template <typename Tr>
