@@ -47,11 +47,12 @@ constexpr int kBlockBytes = kSbs * kSbs * 2;  // one 16-bit block
 // rows of equal parity get eight different values.
 __device__ static inline int k_swizzle(int r) { return (r >> 1) & 7; }
 
-// XOR applied to the 16-byte chunk index of row r of a tile that is read both ways: by rows (128-bit reads,
-// 16 lanes = 16 consecutive rows, one chunk each: rows of equal parity need eight different values) and with
-// the transposing LDS load (16 lanes = four rows r .. r + 3, two neighbouring chunks of each: rows two apart
-// must land in different chunk pairs).
-__device__ static inline int t_swizzle(int r) { return (((r >> 1) & 3) << 1) | ((r >> 3) & 1); }
+// XOR applied to the 16-byte chunk index of row r of a tile that is read both ways: by rows (128-bit reads
+// serve 8 lanes = 8 consecutive rows at a time, one chunk each: they need eight different values) and with
+// the transposing LDS load (it serves 32 lanes at a time = four rows r .. r + 3, r a multiple of 4, 64
+// consecutive bytes of each; two 128-byte rows span the 64 banks once, so rows r and r + 2 must put their 64
+// bytes into different halves of the row: bit 2 of the value is bit 1 of the row).  Depends on r % 8 only.
+__device__ static inline int t_swizzle(int r) { return (((r >> 1) & 1) << 2) | (((r >> 2) & 1) << 1) | (r & 1); }
 
 typedef short i16x4 __attribute__((ext_vector_type(4)));
 

@@ -235,7 +235,7 @@ __global__ __launch_bounds__(kWaves * 64, 1) void matmul_rows_kernel(
   {
     const char *xsrc = x + (int64_t)xs * 8192;
     const int rl = lane >> 3;
-    const int tsw = (((lane >> 4) & 3) << 1) | (wave & 1);  // t_swizzle(8 * piece + rl), piece % 8 == wave
+    const int tsw = t_swizzle(rl);  // the swizzle of row 8 * piece + rl depends on rl only
     const uint32_t src_off = rl * 128 + (((lane & 7) ^ tsw) << 4);
     for (int idx = wave; idx < nx * 8; idx += kWaves) copy_1k_to_lds(xsrc + idx * 1024, src_off, panel + idx * 1024);
   }
