@@ -143,29 +143,25 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
     };
     __shared__ int dead_votes[2][4];
 
-    // K tile: copied global -> LDS without passing through registers.  One instruction moves 1 KiB
-    // (eight 128-byte rows); lane l supplies the 16-byte chunk that belongs at position l of that KiB,
-    // which is where the XOR swizzle of the chunk index is applied.  Wave w copies rows 16 w .. 16 w + 15.
+    // K and V tiles: copied global -> LDS without passing through registers.  One instruction moves 1 KiB
+    // (eight 128-byte rows); lane l supplies the 16-byte chunk that belongs at position l of that KiB, which
+    // is where the XOR swizzle of the chunk index is applied (it depends on row % 8 only, so both KiB of a
+    // wave's 16 rows use the same lane offsets).  Wave w copies rows 16 w .. 16 w + 15 of every slice.
+    const uint32_t copy_off = (uint32_t)(16 * wave + (lane >> 3)) * 128u + (uint32_t)(((lane & 7) ^ t_swizzle(lane >> 3)) << 4);
+    const uint32_t n_k32 = (uint32_t)(a.n_k_blocks < 0x7fffffffLL ? a.n_k_blocks : 0x7fffffffLL);
+    const uint32_t n_v32 = (uint32_t)(a.n_v_blocks < 0x7fffffffLL ? a.n_v_blocks : 0x7fffffffLL);
+    auto copy_slice = [&](const void *tensor, int32_t idx, uint32_t n_blocks, char *dst) {
+      if ((uint32_t)idx < n_blocks) {  // also false for -1 (no such block)
+        copy_2k_to_lds(static_cast<const char *>(tensor) + ((uint64_t)(uint32_t)idx << 13), copy_off, dst + wave * 2048);
+      } else {
+        // inactive slice: zeros
+#pragma unroll
+        for (int i = 0; i < 2; ++i) *reinterpret_cast<u32x4 *>(dst + (i * kThreads + tid) * 16) = u32x4{0u, 0u, 0u, 0u};
+      }
+    };
     auto copy_k = [&](const AttnFwdRecord &r, int buf) {
 #pragma unroll
-      for (int h = 0; h < NH; ++h) {
-        const int64_t pk = r.pk[h];
-        char *dst = lds_k + buf * kKBytes + h * kBlockBytes;
-        if (pk >= 0 && pk < a.n_k_blocks) {
-#pragma unroll
-          for (int i = 0; i < 2; ++i) {
-            // row r0 + lane / 8 of the block, chunk (lane % 8) ^ k_swizzle(row); r0 is a multiple of 8
-            const int r0 = 16 * wave + 8 * i;
-            const uint32_t lane_off = (lane >> 3) * 128 + (((lane & 7) ^ k_swizzle(8 * i + (lane >> 3))) << 4);
-            const char *kp = static_cast<const char *>(a.k) + pk * kBlockBytes + r0 * 128;
-            copy_1k_to_lds(kp, lane_off, dst + r0 * 128);
-          }
-        } else {
-          // inactive slice: zeros
-#pragma unroll
-          for (int i = 0; i < 2; ++i) *reinterpret_cast<u32x4 *>(dst + (i * kThreads + tid) * 16) = u32x4{0u, 0u, 0u, 0u};
-        }
-      }
+      for (int h = 0; h < NH; ++h) copy_slice(a.k, r.pk[h], n_k32, lds_k + buf * kKBytes + h * kBlockBytes);
     };
 
     // facts of one key block (without the mask, which arrives later)
@@ -181,26 +177,10 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
       return f;
     };
 
-    // V tile: copied like the K tile, row-major, with the chunk swizzle of the transposing LDS load that
-    // turns its rows into matrix-core operands later
+    // V tile: copied like the K tile; its rows become matrix-core operands through the transposing LDS load
     auto copy_v = [&](const AttnFwdRecord &r, int buf) {
 #pragma unroll
-      for (int h = 0; h < NHV; ++h) {
-        const int64_t pv = r.pv[h];
-        char *dst = lds_v + buf * kVBytes + h * kBlockBytes;
-        if (pv >= 0 && pv < a.n_v_blocks) {
-#pragma unroll
-          for (int i = 0; i < 2; ++i) {
-            const int r0 = 16 * wave + 8 * i;
-            const uint32_t lane_off = (lane >> 3) * 128 + (((lane & 7) ^ t_swizzle(8 * i + (lane >> 3))) << 4);
-            const char *vp = static_cast<const char *>(a.v) + pv * kBlockBytes + r0 * 128;
-            copy_1k_to_lds(vp, lane_off, dst + r0 * 128);
-          }
-        } else {
-#pragma unroll
-          for (int i = 0; i < 2; ++i) *reinterpret_cast<u32x4 *>(dst + (i * kThreads + tid) * 16) = u32x4{0u, 0u, 0u, 0u};
-        }
-      }
+      for (int h = 0; h < NHV; ++h) copy_slice(a.v, r.pv[h], n_v32, lds_v + buf * kVBytes + h * kBlockBytes);
     };
 
     // Mask words of the tile: lane (li, kg) needs bytes j = 32 jb + 8 q + 4 kg .. + 3 of mask row qi, that is
@@ -348,7 +328,7 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
               const int h = g >> 1, st = 2 * (g & 1) + (t >> 1), jb = t & 1;
               const int rj = 32 * jb + li;
               dst[t] = *reinterpret_cast<const u32x4 *>(kbuf + h * kBlockBytes + rj * 128 +
-                                                        (((2 * st + kg) ^ k_swizzle(rj)) << 4));
+                                                        (((2 * st + kg) ^ t_swizzle(rj)) << 4));
             }
           };
           read_batch(kf[0], 0);

@@ -98,6 +98,16 @@ __device__ static inline void copy_1k_to_lds(const char *base, uint32_t off, cha
                : "memory");
 }
 
+// Two such copies with one address setup: the KiB at base + off and the KiB 1024 bytes further on, to dst and
+// dst + 1024 (the instruction's offset field moves both the global and the LDS address).
+__device__ static inline void copy_2k_to_lds(const char *base, uint32_t off, char *dst) {
+  const uint32_t lds_addr = (uint32_t)(uintptr_t)(lds_ptr_t)dst;
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1\n\tglobal_load_lds_dwordx4 %0, %1 offset:1024"
+               :
+               : "v"(off), "s"(base), "s"(lds_addr)
+               : "memory");
+}
+
 // 16 bytes at base (wave uniform) + off (per lane): scalar base, 32-bit vector offset addressing
 __device__ static inline u32x4 load16(const char *base, uint32_t off) {
   return *reinterpret_cast<const u32x4 *>(base + off);
