@@ -39,9 +39,9 @@ PEAK_MFMA_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}
 # what leaves an L2, so reads served by the memory-side cache are included.  Not re-measured by this script.
 TRAFFIC_KIB = {  # config: (FETCH_SIZE, WRITE_SIZE)
     "c1": (616.2, 476.0),
-    "c2": (592501.7, 514960.0),
+    "c2": (484866.8, 514960.3),
     "c3": (148346.4, 296128.0),
-    "c4": (374747.9, 133149.5),
+    "c4": (373413.6, 133150.6),
     "c5": (127107.7, 143960.0),
 }
 
@@ -147,7 +147,7 @@ def matmul_workload(name, B, n, sbs, dtype, density, ensure_rows, value_scale, d
 
     dt_name = {torch.bfloat16: "bf16", torch.float16: "f16", torch.float32: "f32"}[dtype]
     return dict(step=step, flops=flops, alg_bytes=alg_bytes, dtype=dt_name, bound="hbm", cpu_baseline=cpu_baseline,
-                kernel=("matmul_panel_kernel" if sbs == 64 and dtype != torch.float32 else "matmul_mfma_kernel") if sbs > 16 else "matmul_small_kernel",
+                kernel=("matmul_rows_kernel" if sbs == 64 and dtype != torch.float32 else "matmul_mfma_kernel") if sbs > 16 else "matmul_small_kernel",
                 config={"workload": name, "B": B, "M": n * sbs, "K": n * sbs, "N": n * sbs,
                         "sparsity_block_size": sbs, "density": density, "nnz_x": nnz_x, "nnz_y": nnz_y,
                         "nnz_o": nnz_o, "block_pairs": pairs, "lut_build_ms": round(lut_ms, 3)})
