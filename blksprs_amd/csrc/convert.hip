@@ -52,6 +52,40 @@ __global__ __launch_bounds__(256) void to_dense_kernel(const uint4 *__restrict__
   }
 }
 
+// layout[b][r][c] = 1 if the sbs x sbs block (r, c) of dense[b] holds an element != 0.  One workgroup owns
+// one block row (sbs dense rows) and a chunk of kLayoutVecs 16-byte vectors of every row: thread t owns the
+// vectors t, t + 256, ... of the chunk in all sbs rows (every row read is one contiguous run), ORs the masked
+// words of its column positions over the rows, and reports to the blocks its positions belong to.  `mask`
+// clears the sign bits of floating-point elements: -0.0 equals 0, NaN does not.  Several threads (and, for
+// very wide blocks, several workgroups) may report the same block: they all store the same 1.
+constexpr int kLayoutPerThread = 4;
+constexpr int kLayoutVecs = 256 * kLayoutPerThread;
+
+__global__ __launch_bounds__(256) void layout_from_dense_kernel(const uint4 *__restrict__ dense,
+                                                                uint8_t *__restrict__ layout, int64_t row_vecs,
+                                                                int sbs, int vec_per_row_log2, int64_t C, uint4 mask) {
+  const int64_t block_row = blockIdx.x;  // b * R + r
+  const int64_t chunk0 = (int64_t)blockIdx.y * kLayoutVecs;
+  const uint4 *base = dense + block_row * sbs * row_vecs;
+  uint32_t any[kLayoutPerThread] = {0u, 0u, 0u, 0u};
+  for (int e = 0; e < sbs; ++e) {
+    const uint4 *row = base + (int64_t)e * row_vecs;
+#pragma unroll
+    for (int i = 0; i < kLayoutPerThread; ++i) {
+      const int64_t v = chunk0 + threadIdx.x + 256 * i;
+      if (v < row_vecs) {
+        const uint4 w = row[v];
+        any[i] |= (w.x & mask.x) | (w.y & mask.y) | (w.z & mask.z) | (w.w & mask.w);
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < kLayoutPerThread; ++i) {
+    const int64_t v = chunk0 + threadIdx.x + 256 * i;
+    if (v < row_vecs && any[i]) layout[block_row * C + (v >> vec_per_row_log2)] = 1;
+  }
+}
+
 int ilog2(int64_t v) {
   int l = 0;
   while (((int64_t)1 << l) < v) ++l;
@@ -113,4 +147,28 @@ extern "C" int bsa_to_dense(const void *blocks, const int64_t *packed, void *den
       static_cast<const uint4 *>(blocks), packed, static_cast<uint4 *>(dense), n_vec, nnz, R, C,
       ilog2(vec_per_row), ilog2(sbs), fill);
   return bsa::check_launch("to_dense_kernel");
+}
+
+extern "C" int bsa_layout_from_dense(const void *dense, uint8_t *layout, int64_t B, int64_t R, int64_t C, int sbs,
+                                     int elem_size, int is_float, bsa_stream_t stream) {
+  if (int rc = check_block_shape("bsa_layout_from_dense", sbs, elem_size)) return rc;
+  BSA_REQUIRE(B >= 0 && R >= 0 && C >= 0, "bsa_layout_from_dense: negative size");
+  BSA_REQUIRE(!is_float || elem_size >= 2, "bsa_layout_from_dense: no floating-point type of 1 byte");
+  if (B * R * C == 0) return BSA_OK;
+  BSA_REQUIRE(dense && layout, "bsa_layout_from_dense: NULL pointer");
+  BSA_REQUIRE(aligned16(dense), "bsa_layout_from_dense: buffer must be 16-byte aligned");
+  BSA_REQUIRE(B * R < 0x7fffffffLL, "bsa_layout_from_dense: too many block rows");
+  const int vec_per_row = sbs * elem_size / 16;
+  const int64_t row_vecs = C * vec_per_row;
+  const int64_t chunks = bsa::cdiv(row_vecs, kLayoutVecs);
+  BSA_REQUIRE(chunks <= 65535, "bsa_layout_from_dense: rows too long");
+  uint4 mask{0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
+  if (is_float) {
+    const uint32_t m = elem_size == 2 ? 0x7fff7fffu : 0x7fffffffu;
+    mask = uint4{m, m, m, m};
+    if (elem_size == 8) mask = uint4{0xffffffffu, 0x7fffffffu, 0xffffffffu, 0x7fffffffu};  // sign in the high word
+  }
+  layout_from_dense_kernel<<<dim3((unsigned)(B * R), (unsigned)chunks), 256, 0, bsa::as_stream(stream)>>>(
+      static_cast<const uint4 *>(dense), layout, row_vecs, sbs, ilog2(vec_per_row), C, mask);
+  return bsa::check_launch("layout_from_dense_kernel");
 }

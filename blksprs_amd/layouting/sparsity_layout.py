@@ -1,9 +1,9 @@
-"""Structural layout builders.
+"""Layout builders.
 
-Only the exact block product is built here, on the device, because the product
-layout is the default output layout of both ``matmul`` callers and
-``flash_attention`` (reference: blksprs/layouting/sparsity_layout.py:244-258,
-including the argument checks of ``_validate_sparsity_layout_matmul_inputs``).
+``build_sparsity_layout`` (the layout of a dense tensor: reference blksprs/layouting/sparsity_layout.py:17-109),
+``build_sparsity_layout_full`` (:322-337) and the exact block product ``build_sparsity_layout_matmul``, the
+default output layout of both ``matmul`` callers and ``flash_attention`` (:244-258, including the argument
+checks of ``_validate_sparsity_layout_matmul_inputs``).  The two that look at data run on the device.
 """
 
 import torch
@@ -11,8 +11,54 @@ from torch import Tensor
 
 from .. import _capi
 from ..utils.tools import _layout_bytes, as_base_tensor
-from ..utils.validation import (validate_contiguous, validate_device, validate_dimensions,
-                                validate_sparsity_layout, _validation_enabled, ensure_contiguous)
+from ..utils.validation import (validate_contiguous, validate_device, validate_dimensions, validate_dtype_supported,
+                                validate_sparsity_block_size, validate_sparsity_layout, _validation_enabled,
+                                ensure_contiguous)
+
+
+@torch.amp.custom_fwd(device_type="cuda")
+def build_sparsity_layout(x: Tensor, sparsity_block_size: int) -> Tensor:
+    """Builds the sparsity layout of a three-dimensional dense tensor.
+
+    Args:
+        x (Tensor): The dense tensor whose active blocks are represented by the layout.
+        sparsity_block_size (int): The size of the sparsity blocks.
+
+    Returns:
+        Tensor: A Boolean sparsity layout marking every block containing a non-zero or NaN value.
+
+    """
+    x = ensure_contiguous(x)
+    validate_dimensions(x)
+    validate_contiguous(x)
+    validate_device(x)
+    validate_dtype_supported(x)
+    validate_sparsity_block_size(sparsity_block_size, x)
+    B, R, C = x.size(0), x.size(1) // sparsity_block_size, x.size(2) // sparsity_block_size
+    out = torch.zeros((B, R, C), dtype=torch.bool, device=x.device)
+    if out.numel():
+        with torch.no_grad(), torch.cuda.device(x.device):
+            _capi.call("bsa_layout_from_dense", _capi.ptr(x.detach()), out.view(torch.uint8).data_ptr(), B, R, C,
+                       sparsity_block_size, x.element_size(), int(x.dtype.is_floating_point), _capi.stream(x.device))
+    return as_base_tensor(out)
+
+
+def build_sparsity_layout_full(x: Tensor, sparsity_block_size: int) -> Tensor:
+    """Builds a fully populated sparsity layout for a dense tensor.
+
+    Args:
+        x (Tensor): A three-dimensional dense tensor.
+        sparsity_block_size (int): The size of the sparsity blocks.
+
+    Returns:
+        Tensor: A boolean sparsity layout in which every block is active.
+
+    """
+    validate_dimensions(x)
+    validate_device(x)
+    validate_sparsity_block_size(sparsity_block_size, x)
+    return torch.ones(size=(x.size(0), x.size(1) // sparsity_block_size, x.size(2) // sparsity_block_size),
+                      dtype=torch.bool, device=x.device)
 
 
 def _check_product_inputs(sparsity_layout_x: Tensor, sparsity_layout_y: Tensor) -> None:

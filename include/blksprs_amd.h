@@ -194,6 +194,16 @@ int bsa_matmul_rows(const void *x, const void *y, void *out, const int32_t *pair
                     const int32_t *row_order, int64_t n_rows, int64_t nnz_o, int64_t nnz_x, int64_t nnz_y,
                     int sbs, int dtype, bsa_stream_t stream);
 
+/*
+ * Sparsity layout of a dense (B, R * sbs, C * sbs) array: layout[b][r][c] = 1 where the block holds an
+ * element != 0 (NaN counts, -0.0 does not).  `layout` (B * R * C bytes) must be zero on entry: the kernel
+ * only stores ones.  elem_size in {1, 2, 4, 8}; is_float says whether the elements are IEEE floating
+ * point (fp16 / bf16 / fp32 / fp64), whose sign bit does not make a value non-zero.
+ * Replaces build_sparsity_layout_kernel, blksprs/layouting/sparsity_layout.py:41-109.
+ */
+int bsa_layout_from_dense(const void *dense, uint8_t *layout, int64_t B, int64_t R, int64_t C, int sbs,
+                          int elem_size, int is_float, bsa_stream_t stream);
+
 /* ------------------------------------------------------------- attention */
 
 /*

@@ -78,6 +78,15 @@ def layout_matmul(layout_x, layout_y) -> np.ndarray:
     return np.einsum("bik,bkj->bij", lx, ly) > 0
 
 
+def build_sparsity_layout(x, sparsity_block_size: int) -> np.ndarray:
+    """blksprs/layouting/sparsity_layout.py:17-109: block (r, c) of batch entry b is active where any of its
+    elements compares unequal to zero (``blk_x != 0``, :100), so NaN activates a block and -0.0 does not."""
+    x = torch.as_tensor(x).detach().cpu()
+    s = sparsity_block_size
+    B, R, C = x.size(0), x.size(1) // s, x.size(2) // s
+    return (x.reshape(B, R, s, C, s) != 0).any(dim=4).any(dim=2).numpy()
+
+
 def contraction_lists(layout_x, layout_y, layout_o):
     """The work list implied by the reference kernel's scan (blksprs/ops/matmul.py:191-226): for every
     active output block, in row-major order, the ``(packed x index, packed y index)`` of every k where both

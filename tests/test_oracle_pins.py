@@ -99,6 +99,38 @@ def test_layout_matmul_bruteforce_and_float_bmm():
     assert not orc.layout_matmul(np.ones((1, 2, 0)), np.ones((1, 0, 3))).any()
 
 
+def test_build_sparsity_layout_bruteforce_and_known_answers():
+    """Loops over blocks and elements on tiny inputs; the reference's own facts (NaN activates a block:
+    test/cases/test_regressions.py:1943-1980; a to_dense round trip gives back the layout:
+    test/cases/test_blocksparse.py:990-1009); -0.0 equals 0 in IEEE comparison."""
+    g = torch.Generator().manual_seed(5)
+    s = 4
+    x = torch.randn((2, 3 * s, 5 * s), generator=g)
+    keep = torch.rand((2, 3, 5), generator=g) < 0.4
+    x = x * keep.repeat_interleave(s, 1).repeat_interleave(s, 2)
+    x[0, 0, 0] = -0.0 if not keep[0, 0, 0] else x[0, 0, 0]
+    brute = np.zeros((2, 3, 5), dtype=bool)
+    for b in range(2):
+        for r in range(3):
+            for c in range(5):
+                for i in range(s):
+                    for j in range(s):
+                        if x[b, r * s + i, c * s + j].item() != 0:
+                            brute[b, r, c] = True
+    got = orc.build_sparsity_layout(x, s)
+    assert np.array_equal(got, brute)
+    assert np.array_equal(got, keep.numpy())  # random normal values are never exactly zero
+    for dtype in (torch.float16, torch.bfloat16, torch.float32, torch.float64):
+        d = torch.zeros((1, s, 2 * s), dtype=dtype)
+        d[0, 0, s] = float("nan")
+        assert np.array_equal(orc.build_sparsity_layout(d, s), np.array([[[False, True]]]))
+        d[0, 0, s] = -0.0
+        assert not orc.build_sparsity_layout(d, s).any()
+    ints = torch.zeros((1, s, s), dtype=torch.int32)
+    ints[0, 3, 3] = -1
+    assert orc.build_sparsity_layout(ints, s).all()
+
+
 def test_contraction_lists_reproduce_the_dense_product():
     """The lists are a regrouping of a block matmul: summing x[px] @ y[py] per output block must equal the
     dense masked product; and within a block k ascends."""
