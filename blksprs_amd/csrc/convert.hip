@@ -86,6 +86,37 @@ __global__ __launch_bounds__(256) void layout_from_dense_kernel(const uint4 *__r
   }
 }
 
+// out[o] = transpose of blocks[packed[flat index of coords[o] in the (B, R, C) output layout]] (zeros where that
+// entry is negative or out of range): the gather of flow_pull fused with the element transposition.  One
+// workgroup moves one 64 x 64 (or sbs x sbs for smaller blocks) tile of elements through LDS: rows in, columns
+// out, both sides touching consecutive elements of a row.
+template <typename E>
+__global__ __launch_bounds__(256) void transpose_blocks_kernel(const E *__restrict__ blocks,
+                                                               const int64_t *__restrict__ coords,
+                                                               const int64_t *__restrict__ packed,
+                                                               E *__restrict__ out, int64_t n_src, int64_t R,
+                                                               int64_t C, int sbs, int tiles_per_side) {
+  __shared__ E tile[64][65];
+  const int T = sbs < 64 ? sbs : 64;
+  const int64_t o = blockIdx.x / (tiles_per_side * tiles_per_side);
+  const int t_id = blockIdx.x % (tiles_per_side * tiles_per_side);
+  const int tr = t_id / tiles_per_side, tc = t_id % tiles_per_side;  // tile of the OUTPUT block
+  const int64_t b = coords[o * 3 + 0], r = coords[o * 3 + 1], c = coords[o * 3 + 2];
+  const int64_t flat = (b * R + r) * C + c;
+  int64_t src = -1;
+  if (r >= 0 && r < R && c >= 0 && c < C && b >= 0) src = packed[flat];
+  const bool valid = src >= 0 && src < n_src;
+  const int col = threadIdx.x % T, row0 = threadIdx.x / T, rows_per_pass = 256 / T;
+  if (valid) {
+    // input tile (tc, tr) of the source block: rows 64 tc .., columns 64 tr ..
+    const E *in = blocks + src * sbs * sbs + ((int64_t)tc * T) * sbs + (int64_t)tr * T;
+    for (int row = row0; row < T; row += rows_per_pass) tile[row][col] = in[(int64_t)row * sbs + col];
+  }
+  __syncthreads();
+  E *dst = out + o * sbs * sbs + ((int64_t)tr * T) * sbs + (int64_t)tc * T;
+  for (int row = row0; row < T; row += rows_per_pass) dst[(int64_t)row * sbs + col] = valid ? tile[col][row] : E(0);
+}
+
 int ilog2(int64_t v) {
   int l = 0;
   while (((int64_t)1 << l) < v) ++l;
@@ -171,4 +202,28 @@ extern "C" int bsa_layout_from_dense(const void *dense, uint8_t *layout, int64_t
   layout_from_dense_kernel<<<dim3((unsigned)(B * R), (unsigned)chunks), 256, 0, bsa::as_stream(stream)>>>(
       static_cast<const uint4 *>(dense), layout, row_vecs, sbs, ilog2(vec_per_row), C, mask);
   return bsa::check_launch("layout_from_dense_kernel");
+}
+
+extern "C" int bsa_transpose_blocks(const void *blocks, const int64_t *coords, const int64_t *packed, void *out,
+                                    int64_t nnz_out, int64_t nnz_in, int64_t B, int64_t R, int64_t C, int sbs,
+                                    int elem_size, bsa_stream_t stream) {
+  if (int rc = check_block_shape("bsa_transpose_blocks", sbs, elem_size)) return rc;
+  BSA_REQUIRE(nnz_out >= 0 && nnz_in >= 0 && B >= 0 && R >= 0 && C >= 0, "bsa_transpose_blocks: negative size");
+  if (nnz_out == 0) return BSA_OK;
+  BSA_REQUIRE(coords && packed && out && (nnz_in == 0 || blocks), "bsa_transpose_blocks: NULL pointer");
+  const int tiles = sbs <= 64 ? 1 : sbs / 64;
+  const int64_t grid = nnz_out * tiles * tiles;
+  BSA_REQUIRE(grid < 0x7fffffffLL, "bsa_transpose_blocks: too many tiles");
+  hipStream_t s = bsa::as_stream(stream);
+#define BSA_TR_LAUNCH(E)                                                                                          \
+  transpose_blocks_kernel<E><<<(unsigned)grid, 256, 0, s>>>(static_cast<const E *>(blocks), coords, packed,       \
+                                                            static_cast<E *>(out), nnz_in, R, C, sbs, tiles)
+  switch (elem_size) {
+    case 1: BSA_TR_LAUNCH(uint8_t); break;
+    case 2: BSA_TR_LAUNCH(uint16_t); break;
+    case 4: BSA_TR_LAUNCH(uint32_t); break;
+    default: BSA_TR_LAUNCH(uint64_t); break;
+  }
+#undef BSA_TR_LAUNCH
+  return bsa::check_launch("transpose_blocks_kernel");
 }

@@ -4,6 +4,7 @@ from .conversion import from_blksprs, to_blksprs, to_dense, to_dense_shaped, to_
 from .flash_attention import flash_attention, flash_attention_build_layout_cache
 from .matmul import matmul
 from .softmax import softmax, softmax_fused, softmax_regular
+from .transpose import transpose
 
 __all__ = [
     "flash_attention",
@@ -18,4 +19,5 @@ __all__ = [
     "to_dense_shaped",
     "to_sparse",
     "to_sparse_shaped",
+    "transpose",
 ]

@@ -195,6 +195,18 @@ int bsa_matmul_rows(const void *x, const void *y, void *out, const int32_t *pair
                     int sbs, int dtype, bsa_stream_t stream);
 
 /*
+ * Block gather with element transposition: out[o] = transpose(blocks[packed[(b * R + r) * C + c]]) with
+ * (b, r, c) = coords[o] (int64 [nnz_out, 3], the non-zero coordinates of the OUTPUT layout, shape (B, R, C));
+ * `packed` is an int64 table over the output layout that names the source block of every position (-1 or
+ * out of [0, nnz_in): the output block becomes zeros).  With the packed indices of a layout arranged in
+ * transposed order this is the reference's transpose: x.transpose(-1, -2) followed by flow_pull_kernel,
+ * blksprs/ops/transpose.py:44-52, blksprs/ops/flow.py:11-111.  elem_size in {1, 2, 4, 8}.
+ */
+int bsa_transpose_blocks(const void *blocks, const int64_t *coords, const int64_t *packed, void *out,
+                         int64_t nnz_out, int64_t nnz_in, int64_t B, int64_t R, int64_t C, int sbs, int elem_size,
+                         bsa_stream_t stream);
+
+/*
  * Sparsity layout of a dense (B, R * sbs, C * sbs) array: layout[b][r][c] = 1 where the block holds an
  * element != 0 (NaN counts, -0.0 does not).  `layout` (B * R * C bytes) must be zero on entry: the kernel
  * only stores ones.  elem_size in {1, 2, 4, 8}; is_float says whether the elements are IEEE floating

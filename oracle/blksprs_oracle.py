@@ -106,6 +106,20 @@ def contraction_lists(layout_x, layout_y, layout_o):
 
 # --------------------------------------------------------------------------- conversion (bit exact)
 
+def transpose(x, layout, sparsity_block_size: int):
+    """blksprs/ops/transpose.py:13-52 (element transposition of every block, then flow_pull,
+    blksprs/ops/flow.py:11-111): the compressed form of the transposed dense tensor under the transposed
+    layout.  Returns ``(blocks in nonzero order of layout^T, layout^T)``."""
+    lay = np.asarray(layout) != 0
+    lay_t = np.ascontiguousarray(np.swapaxes(lay, -1, -2))
+    px = packed_indices(lay).reshape(lay.shape)
+    x = torch.as_tensor(x)
+    out = [x[px[b, c, r]].transpose(-1, -2) for b, r, c in np.argwhere(lay_t)]
+    s = sparsity_block_size
+    res = torch.stack(out) if out else torch.empty((0, s, s), dtype=x.dtype)
+    return res.contiguous(), lay_t
+
+
 
 def to_sparse(x: torch.Tensor, layout, sbs: int) -> torch.Tensor:
     """blksprs/ops/conversion.py:230-276: the active ``sbs x sbs`` tiles of dense ``(B, R*sbs, C*sbs)`` in

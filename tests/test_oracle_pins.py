@@ -178,6 +178,23 @@ def test_conversion_against_slice_loops():
     assert n == blocks.size(0)
 
 
+def test_transpose_is_the_conversion_of_the_transposed_dense_tensor():
+    """transpose(to_sparse(d, l), l) == to_sparse(d^T, l^T) for every dense d (the defining property, checked
+    through the independently pinned conversion), twice is the identity, and the layout returned is l^T."""
+    g = torch.Generator().manual_seed(11)
+    s = 4
+    layout = (torch.rand((3, 2, 5), generator=g) < 0.5).numpy()
+    dense = torch.randn((3, 2 * s, 5 * s), generator=g)
+    blocks = orc.to_sparse(dense, layout, s)
+    got, layout_t = orc.transpose(blocks, layout, s)
+    assert np.array_equal(layout_t, np.swapaxes(layout, 1, 2))
+    assert torch.equal(got, orc.to_sparse(dense.transpose(1, 2).contiguous(), layout_t, s))
+    back, layout_tt = orc.transpose(got, layout_t, s)
+    assert np.array_equal(layout_tt, layout) and torch.equal(back, blocks)
+    empty, _ = orc.transpose(torch.empty((0, s, s)), np.zeros((1, 2, 3), bool), s)
+    assert empty.shape == (0, s, s)
+
+
 def test_matmul_full_layout_is_bmm_and_inactive_blocks_do_not_contribute():
     g = torch.Generator().manual_seed(2)
     sbs = 4
