@@ -87,6 +87,60 @@ def build_sparsity_layout(x, sparsity_block_size: int) -> np.ndarray:
     return (x.reshape(B, R, s, C, s) != 0).any(dim=4).any(dim=2).numpy()
 
 
+def causal_token_mask(valid_length: int, padded_length: int, window_size=None) -> np.ndarray:
+    """Token-level statement of blksprs/layouting/causal.py:158-172: score (q, k) is ignored when the key lies
+    in the future, when either position is padding, or (windowed) when the key is ``window_size`` or more
+    tokens back.  bool ``(padded_length, padded_length)``, True = ignored.  Plain loops."""
+    m = np.zeros((padded_length, padded_length), dtype=bool)
+    for q in range(padded_length):
+        for k in range(padded_length):
+            ignored = k > q or q >= valid_length or k >= valid_length
+            if window_size is not None and q - k > window_size - 1:
+                ignored = True
+            m[q, k] = ignored
+    return m
+
+
+def causal_layout(valid_lengths, sparsity_block_size: int, window_size=None) -> np.ndarray:
+    """blksprs/layouting/causal.py:16-51 and :181-203 from the token-level mask: a block is active when
+    k_block <= q_block, both block rows reach into the valid prefix and (windowed) the block offset does not
+    exceed ceil((window_size - 1) / block size)."""
+    s = sparsity_block_size
+    lengths = [int(v) for v in valid_lengths]
+    n = (max(lengths, default=0) + s - 1) // s
+    out = np.zeros((len(lengths), n, n), dtype=bool)
+    for b, length in enumerate(lengths):
+        used = (length + s - 1) // s
+        for q in range(n):
+            for k in range(n):
+                ok = k <= q and q < used and k < used
+                if window_size is not None and q - k > (window_size - 1 + s - 1) // s:
+                    ok = False
+                out[b, q, k] = ok
+    return out
+
+
+def causal_mask_layout(valid_lengths, attention_layout, sparsity_block_size: int, window_size=None) -> np.ndarray:
+    """blksprs/layouting/causal.py:124-142: the blocks of the compact mask are the active blocks that lie on
+    the diagonal, at block offset ceil((window_size - 1) / block size) (windowed only), or in the block row
+    of a partial last query block.  (The reference keeps no other block, also not the block one offset
+    nearer that a window with (window_size - 1) % block size != 0 cuts as well.)  Plain loops."""
+    s = sparsity_block_size
+    lay = np.asarray(attention_layout) != 0
+    out = np.zeros_like(lay)
+    for b, length in enumerate(int(v) for v in valid_lengths):
+        last = (length + s - 1) // s - 1
+        for q in range(lay.shape[1]):
+            for k in range(lay.shape[2]):
+                keep = q == k
+                if window_size is not None and q - k == (window_size - 1 + s - 1) // s:
+                    keep = True
+                if length % s != 0 and q == last and k <= last:
+                    keep = True
+                out[b, q, k] = keep and lay[b, q, k]
+    return out
+
+
 def contraction_lists(layout_x, layout_y, layout_o):
     """The work list implied by the reference kernel's scan (blksprs/ops/matmul.py:191-226): for every
     active output block, in row-major order, the ``(packed x index, packed y index)`` of every k where both
