@@ -188,6 +188,60 @@ def softmax_workload(dev):
                         "sparsity_block_size": sbs, "nnz": nnz})
 
 
+def movement_workload(dev, which):
+    """The two data-movement rows next to the hot path, at the size of configuration 2's x operand:
+    ``transpose`` of the compressed x (bf16, 25 % of 16 x 64 x 64 blocks of 64) and ``build_sparsity_layout``
+    of its dense form (16 x 4096 x 4096 bf16)."""
+    import blksprs_amd as bs
+    from oracle import blksprs_oracle as orc
+
+    B, n, sbs = 16, 64, 64
+    g = torch.Generator().manual_seed(0)
+    layout = orc.random_layout((B, n, n), 0.25, g)
+    ld = layout.to(dev)
+    nnz = int(layout.sum())
+    gd = torch.Generator(device=dev).manual_seed(1)
+    x = torch.randn((nnz, sbs, sbs), device=dev, dtype=torch.bfloat16, generator=gd)
+    bs.utils.disable_validation()
+    if which == "transpose":
+        cache = {}
+        bs.ops.transpose(x, ld, sbs, layout_cache=cache)
+        alg_bytes = 2 * nnz * sbs * sbs * 2
+
+        def step():
+            return bs.ops.transpose(x, ld, sbs, layout_cache=cache)
+
+        def cpu_baseline():
+            nb = 2
+            cnt = int(layout[:nb].sum())
+            xs = x[:cnt].cpu()
+            reps, dt = _repeat_for(CPU_SAMPLE_SECONDS, lambda: orc.transpose(xs, layout[:nb].numpy(), sbs))
+            return {"value": 2 * cnt * sbs * sbs * 2 / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(),
+                    "kind": "port", "sample": f"{nb} of {B} batches x {reps} passes, per-block torch transpose, {dt * reps:.1f} s"}
+
+        return dict(step=step, flops=0.0, alg_bytes=alg_bytes, dtype="bf16", bound="hbm", cpu_baseline=cpu_baseline,
+                    kernel="transpose_blocks_kernel",
+                    config={"workload": "t1_transpose_bf16", "B": B, "rows": n * sbs, "cols": n * sbs,
+                            "sparsity_block_size": sbs, "nnz": nnz})
+    dense = bs.ops.to_dense(x, ld, sbs)
+    alg_bytes = dense.numel() * 2 + B * n * n
+
+    def step():
+        return bs.layouting.build_sparsity_layout(dense, sbs)
+
+    def cpu_baseline():
+        nb = 2
+        ds = dense[:nb].cpu()
+        reps, dt = _repeat_for(CPU_SAMPLE_SECONDS, lambda: orc.build_sparsity_layout(ds, sbs))
+        return {"value": ds.numel() * 2 / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+                "sample": f"{nb} of {B} batches x {reps} passes, torch != 0 and any over blocks, {dt * reps:.1f} s"}
+
+    return dict(step=step, flops=0.0, alg_bytes=alg_bytes, dtype="bf16", bound="hbm", cpu_baseline=cpu_baseline,
+                kernel="layout_from_dense_kernel",
+                config={"workload": "l1_build_sparsity_layout_bf16", "B": B, "rows": n * sbs, "cols": n * sbs,
+                        "sparsity_block_size": sbs, "active_blocks": nnz})
+
+
 def attention_workload(dev, backward):
     import blksprs_amd as bs
     from oracle import blksprs_oracle as orc
@@ -261,6 +315,10 @@ def make_workload(name, dev):
         return attention_workload(dev, backward=True)
     if name == "c5":
         return matmul_workload("c5_matmul_fp16", 64, 128, 16, torch.float16, 0.05, True, 1.0, dev, 8)
+    if name == "t1":
+        return movement_workload(dev, "transpose")
+    if name == "l1":
+        return movement_workload(dev, "layout")
     raise SystemExit(f"unknown config {name}")
 
 
@@ -271,7 +329,7 @@ def main():
     # with 10 warm-up steps the first timed steps of configuration 2 still run 10 % slower
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=100)
-    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c4bwd", "c5"])
+    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c4bwd", "c5", "t1", "l1"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
