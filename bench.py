@@ -220,7 +220,7 @@ def movement_workload(dev, which):
                     "kind": "port", "sample": f"{nb} of {B} batches x {reps} passes, per-block torch transpose, {dt * reps:.1f} s"}
 
         return dict(step=step, flops=0.0, alg_bytes=alg_bytes, dtype="bf16", bound="hbm", cpu_baseline=cpu_baseline,
-                    kernel="transpose_blocks_kernel",
+                    kernel="transpose_blocks16_kernel",
                     config={"workload": "t1_transpose_bf16", "B": B, "rows": n * sbs, "cols": n * sbs,
                             "sparsity_block_size": sbs, "nnz": nnz})
     dense = bs.ops.to_dense(x, ld, sbs)

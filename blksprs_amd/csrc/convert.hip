@@ -117,6 +117,79 @@ __global__ __launch_bounds__(256) void transpose_blocks_kernel(const E *__restri
   for (int row = row0; row < T; row += rows_per_pass) dst[(int64_t)row * sbs + col] = valid ? tile[col][row] : E(0);
 }
 
+// The same operation for 2-byte elements and sbs >= 64, moving 16-byte vectors on both sides.  A workgroup of
+// four waves stages one 64 x 64 tile of the source block (8 KiB) in LDS, turns it with the transposing LDS read
+// (sixteen lanes that point at a 4 x 16 patch of elements each get one column of it), parks the turned vectors
+// in a second tile and stores that row by row, so every global access is a full 128-byte row.
+using i16x4_t = short __attribute__((ext_vector_type(4)));
+using u32x2_t = uint32_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ u32x2_t read_turned(const char *p) {
+  const i16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4_t *)p);
+  return __builtin_bit_cast(u32x2_t, v);
+}
+
+// XOR on the 16-byte chunk index of row r of the staged tile: a transposing read serves 32 lanes at a time, rows
+// r .. r + 3 (r a multiple of 4) with 64 consecutive bytes of each, and two 128-byte rows span the 64 banks
+// once, so rows r and r + 2 keep their 64 bytes in different halves of the row.
+__device__ __forceinline__ int turn_swizzle(int r) { return ((r >> 1) & 1) << 2; }
+
+__global__ __launch_bounds__(256) void transpose_blocks16_kernel(const uint16_t *__restrict__ blocks,
+                                                                 const int64_t *__restrict__ coords,
+                                                                 const int64_t *__restrict__ packed,
+                                                                 uint16_t *__restrict__ out, int64_t n_src,
+                                                                 int64_t R, int64_t C, int sbs, int tiles_per_side) {
+  __shared__ __attribute__((aligned(16))) char in_tile[64 * 128];
+  __shared__ __attribute__((aligned(16))) char out_tile[64 * 128];
+  const int64_t o = blockIdx.x / (tiles_per_side * tiles_per_side);
+  const int t_id = blockIdx.x % (tiles_per_side * tiles_per_side);
+  const int tr = t_id / tiles_per_side, tc = t_id % tiles_per_side;  // tile of the OUTPUT block
+  const int64_t b = coords[o * 3 + 0], r = coords[o * 3 + 1], c = coords[o * 3 + 2];
+  int64_t src = -1;
+  if (r >= 0 && r < R && c >= 0 && c < C && b >= 0) src = packed[(b * R + r) * C + c];
+  const bool valid = src >= 0 && src < n_src;  // uniform over the workgroup
+  const int t = threadIdx.x;
+  const int64_t row_bytes = (int64_t)sbs * 2;
+  char *dst = reinterpret_cast<char *>(out) + o * sbs * row_bytes + ((int64_t)tr * 64) * row_bytes + tc * 128;
+  if (!valid) {
+    for (int v = t; v < 512; v += 256) *reinterpret_cast<uint4 *>(dst + (v >> 3) * row_bytes + (v & 7) * 16) = uint4{0, 0, 0, 0};
+    return;
+  }
+  // source tile (tc, tr): rows 64 tc .., columns 64 tr ..
+  const char *in = reinterpret_cast<const char *>(blocks) + src * sbs * row_bytes + ((int64_t)tc * 64) * row_bytes + tr * 128;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int v = t + 256 * i, row = v >> 3, chunk = v & 7;
+    const uint4 w = *reinterpret_cast<const uint4 *>(in + row * row_bytes + chunk * 16);
+    *reinterpret_cast<uint4 *>(in_tile + row * 128 + ((chunk ^ turn_swizzle(row)) << 4)) = w;
+  }
+  __syncthreads();
+  // wave w turns source rows 16 w .. 16 w + 15; lane group g: rows + 8 (g / 2), columns + 16 (g % 2)
+  const int wave = t >> 6, lane = t & 63, g = lane >> 4, ls = lane & 15;
+#pragma unroll
+  for (int cb = 0; cb < 2; ++cb) {
+    const int r0 = 16 * wave + 8 * (g >> 1);
+    const int col0 = 32 * cb + 16 * (g & 1);
+    u32x2_t half[2];
+#pragma unroll
+    for (int rd = 0; rd < 2; ++rd) {
+      const int rs = r0 + 4 * rd + (ls >> 2);
+      const int col = col0 + 4 * (ls & 3);
+      half[rd] = read_turned(in_tile + rs * 128 + (((col >> 3) ^ turn_swizzle(rs)) << 4) + ((col & 4) << 1));
+    }
+    // this lane now holds source[r0 .. r0 + 7][col0 + ls] = output row col0 + ls, columns r0 .. r0 + 7
+    *reinterpret_cast<uint4 *>(out_tile + (col0 + ls) * 128 + (r0 >> 3) * 16) =
+        uint4{half[0][0], half[0][1], half[1][0], half[1][1]};
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int v = t + 256 * i, row = v >> 3, chunk = v & 7;
+    *reinterpret_cast<uint4 *>(dst + row * row_bytes + chunk * 16) =
+        *reinterpret_cast<const uint4 *>(out_tile + row * 128 + chunk * 16);
+  }
+}
+
 int ilog2(int64_t v) {
   int l = 0;
   while (((int64_t)1 << l) < v) ++l;
@@ -215,6 +288,11 @@ extern "C" int bsa_transpose_blocks(const void *blocks, const int64_t *coords, c
   const int64_t grid = nnz_out * tiles * tiles;
   BSA_REQUIRE(grid < 0x7fffffffLL, "bsa_transpose_blocks: too many tiles");
   hipStream_t s = bsa::as_stream(stream);
+  if (elem_size == 2 && sbs >= 64 && aligned16(blocks) && aligned16(out)) {
+    transpose_blocks16_kernel<<<(unsigned)grid, 256, 0, s>>>(static_cast<const uint16_t *>(blocks), coords, packed,
+                                                             static_cast<uint16_t *>(out), nnz_in, R, C, sbs, tiles);
+    return bsa::check_launch("transpose_blocks16_kernel");
+  }
 #define BSA_TR_LAUNCH(E)                                                                                          \
   transpose_blocks_kernel<E><<<(unsigned)grid, 256, 0, s>>>(static_cast<const E *>(blocks), coords, packed,       \
                                                             static_cast<E *>(out), nnz_in, R, C, sbs, tiles)
