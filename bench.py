@@ -43,6 +43,10 @@ TRAFFIC_KIB = {  # config: (FETCH_SIZE, WRITE_SIZE)
     "c3": (148346.4, 296128.0),
     "c4": (373413.6, 133150.6),
     "c5": (127107.7, 143960.0),
+    "t1": (67086.4, 129576.0),
+    "l1": (262162.2, 64.0),
+    "r1": (64865.6, 8192.0),
+    "r2": (66875.5, 129576.0),
 }
 
 
@@ -189,9 +193,9 @@ def softmax_workload(dev):
 
 
 def movement_workload(dev, which):
-    """The two data-movement rows next to the hot path, at the size of configuration 2's x operand:
-    ``transpose`` of the compressed x (bf16, 25 % of 16 x 64 x 64 blocks of 64) and ``build_sparsity_layout``
-    of its dense form (16 x 4096 x 4096 bf16)."""
+    """The HBM-bound rows next to the hot path, at the size of configuration 2's x operand (bf16, 25 % of
+    16 x 64 x 64 blocks of 64): ``transpose``, ``row_wise_sum`` and ``row_wise_add`` of the compressed x, and
+    ``build_sparsity_layout`` of its dense form (16 x 4096 x 4096 bf16)."""
     import blksprs_amd as bs
     from oracle import blksprs_oracle as orc
 
@@ -222,6 +226,45 @@ def movement_workload(dev, which):
         return dict(step=step, flops=0.0, alg_bytes=alg_bytes, dtype="bf16", bound="hbm", cpu_baseline=cpu_baseline,
                     kernel="transpose_blocks16_kernel",
                     config={"workload": "t1_transpose_bf16", "B": B, "rows": n * sbs, "cols": n * sbs,
+                            "sparsity_block_size": sbs, "nnz": nnz})
+    if which in ("row_sum", "row_add"):
+        n_rows = int(layout.any(-1).sum())
+        lnp = layout.numpy()
+        nb = 2
+        cnt = int(layout[:nb].sum())
+        xs = x[:cnt].cpu()
+        if which == "row_sum":
+            alg_bytes = (nnz + n_rows) * sbs * sbs * 2
+
+            def step():
+                return bs.ops.misc.row_wise_sum(x, ld, sbs)
+
+            def cpu_baseline():
+                reps, dt = _repeat_for(CPU_SAMPLE_SECONDS, lambda: orc.row_wise_reduce(xs, lnp[:nb], sbs, "sum"))
+                return {"value": (cnt + nb * n) * sbs * sbs * 2 / dt / 1e9, "unit": "GB/s",
+                        "cores": torch.get_num_threads(), "kind": "port",
+                        "sample": f"{nb} of {B} batches x {reps} passes, per-block torch sums, {dt * reps:.1f} s"}
+
+            return dict(step=step, flops=0.0, alg_bytes=alg_bytes, dtype="bf16", bound="hbm",
+                        cpu_baseline=cpu_baseline, kernel="row_reduce_kernel",
+                        config={"workload": "r1_row_wise_sum_bf16", "B": B, "rows": n * sbs, "cols": n * sbs,
+                                "sparsity_block_size": sbs, "nnz": nnz})
+        y = torch.randn((n_rows, sbs, 1), device=dev, dtype=torch.bfloat16, generator=gd)
+        alg_bytes = 2 * nnz * sbs * sbs * 2 + n_rows * sbs * 2
+        ys = y[:nb * n].cpu()
+
+        def step():
+            return bs.ops.misc.row_wise_add(x, ld, y, sbs)
+
+        def cpu_baseline():
+            reps, dt = _repeat_for(CPU_SAMPLE_SECONDS, lambda: orc.row_wise_add(xs, lnp[:nb], ys, sbs))
+            return {"value": 2 * cnt * sbs * sbs * 2 / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(),
+                    "kind": "port",
+                    "sample": f"{nb} of {B} batches x {reps} passes, per-block torch adds, {dt * reps:.1f} s"}
+
+        return dict(step=step, flops=0.0, alg_bytes=alg_bytes, dtype="bf16", bound="hbm", cpu_baseline=cpu_baseline,
+                    kernel="row_add_kernel",
+                    config={"workload": "r2_row_wise_add_bf16", "B": B, "rows": n * sbs, "cols": n * sbs,
                             "sparsity_block_size": sbs, "nnz": nnz})
     dense = bs.ops.to_dense(x, ld, sbs)
     alg_bytes = dense.numel() * 2 + B * n * n
@@ -319,6 +362,10 @@ def make_workload(name, dev):
         return movement_workload(dev, "transpose")
     if name == "l1":
         return movement_workload(dev, "layout")
+    if name == "r1":
+        return movement_workload(dev, "row_sum")
+    if name == "r2":
+        return movement_workload(dev, "row_add")
     raise SystemExit(f"unknown config {name}")
 
 
@@ -329,7 +376,7 @@ def main():
     # with 10 warm-up steps the first timed steps of configuration 2 still run 10 % slower
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=100)
-    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c4bwd", "c5", "t1", "l1"])
+    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c4bwd", "c5", "t1", "l1", "r1", "r2"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:

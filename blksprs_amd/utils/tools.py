@@ -189,7 +189,19 @@ def prepare_layout_cache(layout_cache: LayoutCache | None, operation: str, *valu
     """
     if layout_cache is None:
         layout_cache = {}
+    key, refs = layout_cache_key(operation, *values)
+    recorded = layout_cache.get(_STATE)
+    stale = (layout_cache.get(_KEY) != key or recorded is None or _snapshot(layout_cache) != recorded)
+    if stale:
+        layout_cache.clear()
+        layout_cache[_KEY] = key
+        # holding the sources keeps their ids from being reused by other tensors
+        layout_cache[_REFS] = refs
+    return layout_cache
 
+
+def layout_cache_key(operation: str, *values: object) -> tuple[tuple, tuple]:
+    """The key ``prepare_layout_cache`` files a cache under, and the tensors it depends on."""
     refs: list[Tensor] = []
     never_equal = object()
 
@@ -203,15 +215,7 @@ def prepare_layout_cache(layout_cache: LayoutCache | None, operation: str, *valu
             return tuple(sorted((k, signature(v)) for k, v in value.items()))
         return value
 
-    key = (operation, tuple(signature(v) for v in values))
-    recorded = layout_cache.get(_STATE)
-    stale = (layout_cache.get(_KEY) != key or recorded is None or _snapshot(layout_cache) != recorded)
-    if stale:
-        layout_cache.clear()
-        layout_cache[_KEY] = key
-        # holding the sources keeps their ids from being reused by other tensors
-        layout_cache[_REFS] = tuple(refs)
-    return layout_cache
+    return (operation, tuple(signature(v) for v in values)), tuple(refs)
 
 
 def finalize_layout_cache(layout_cache: LayoutCache) -> LayoutCache:

@@ -144,6 +144,35 @@ int bsa_to_dense(const void *blocks, const int64_t *packed, void *dense, int64_t
                  int64_t C, int64_t nnz, int sbs, int elem_size, uint64_t fill_bits,
                  bsa_stream_t stream);
 
+/* ------------------------------------------------------------- row-wise */
+
+/*
+ * Row-wise sum (op 0) or maximum (op 1) over the active blocks of each block
+ * row; fp32 accumulation, rounded once to `dtype`.  row_offsets: int32
+ * [n_rows + 1] CSR offsets of the layout flattened to (B*R, C); packed_out:
+ * int64 [n_rows] reverse index of the (B, R, 1) output layout (-1 for block
+ * rows without blocks).  out is [n_out, sbs, sbs] (column 0 holds the result,
+ * the other columns 0 for the sum and -inf for the maximum) or, with
+ * slice_only, [n_out, sbs, 1].  A maximum over a row that holds a NaN is NaN.
+ * Replaces row_wise_sum_forward / row_wise_sum_kernel and row_wise_max_forward
+ * / row_wise_max_kernel (blksprs/ops/misc/row_wise.py:103-205, :283-419), which
+ * accumulate with atomics into an fp32 buffer and convert afterwards.
+ */
+int bsa_row_reduce(const void *x, const int32_t *row_offsets, const int64_t *packed_out, void *out,
+                   int64_t n_rows, int64_t n_out, int64_t nnz, int sbs, int dtype, int op, int slice_only,
+                   bsa_stream_t stream);
+
+/*
+ * out[n][e][:] = x[n][e][:] + y[packed_rows[b * R + r]][e][0] for block
+ * n = coords[n] = (b, r, c); y is [n_y, sbs, y_cols] with y_cols 1 or sbs.
+ * Blocks whose row has no entry in y are written as zeros.  Replaces
+ * row_wise_add_forward / row_wise_add_kernel
+ * (blksprs/ops/misc/row_wise.py:488-603).
+ */
+int bsa_row_add(const void *x, const int64_t *coords, const int64_t *packed_rows, const void *y, void *out,
+                int64_t nnz, int64_t n_y, int64_t B, int64_t R, int y_cols, int sbs, int dtype,
+                bsa_stream_t stream);
+
 /* --------------------------------------------------------------- softmax */
 
 /*

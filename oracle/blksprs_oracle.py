@@ -204,6 +204,44 @@ def matmul(x, layout_x, y, layout_y, layout_o, sbs: int, acc_dtype=torch.float32
     return to_sparse(torch.matmul(xd, yd), layout_o, sbs).to(x.dtype)
 
 
+def row_wise_reduce(x, layout, sbs: int, op: str, slice_only: bool = False):
+    """blksprs/ops/misc/row_wise.py:103-205 (``op="sum"``) and :283-419 (``op="max"``): every block folds the
+    reduction of each of its element rows into column 0 of the output block of its block row; the other
+    columns keep the initial value (0 for the sum, ``-inf`` for the maximum); a row that holds a NaN gives NaN
+    (:349-350); accumulation is wider than the storage type and the result is rounded once (:108-114, :146).
+    Returns ``(values, (B, R, 1) layout)`` with values ``(rows, sbs, sbs)`` or ``(rows, sbs, 1)``."""
+    lay = np.asarray(layout) != 0
+    B, R, _ = lay.shape
+    row_lay = lay.any(axis=-1, keepdims=True)
+    row_index = packed_indices(row_lay)
+    n_out = int(row_lay.sum())
+    x = torch.as_tensor(x)
+    start = 0.0 if op == "sum" else float("-inf")
+    acc = torch.full((n_out, sbs, 1 if slice_only else sbs), start, dtype=torch.float64)
+    for n, (b, r, _c) in enumerate(layout_indices(lay)):
+        k = int(row_index[b * R + r])
+        blk = x[n].to(torch.float64)
+        if op == "sum":
+            acc[k, :, 0] += blk.sum(dim=-1)
+        else:
+            acc[k, :, 0] = torch.maximum(acc[k, :, 0], blk.max(dim=-1).values)  # both propagate NaN
+    return acc.to(x.dtype), row_lay
+
+
+def row_wise_add(x, layout, y, sbs: int) -> torch.Tensor:
+    """blksprs/ops/misc/row_wise.py:488-603: block ``(b, r, c)`` of x plus column 0 of the block of y that
+    belongs to block row ``(b, r)``, broadcast over the columns; y holds ``sbs`` or 1 columns."""
+    lay = np.asarray(layout) != 0
+    B, R, _ = lay.shape
+    row_index = packed_indices(lay.any(axis=-1, keepdims=True))
+    x, y = torch.as_tensor(x), torch.as_tensor(y)
+    out = torch.zeros_like(x)
+    for n, (b, r, _c) in enumerate(layout_indices(lay)):
+        k = int(row_index[b * R + r])
+        out[n] = (x[n].to(torch.float64) + y[k, :, :1].to(torch.float64)).to(x.dtype)
+    return out
+
+
 def softmax(x, layout, sbs: int) -> torch.Tensor:
     """blksprs/ops/softmax.py:524-570: per element row, softmax over the concatenation of the row's active
     blocks; inactive blocks act as ``-inf`` and rows without blocks do not exist in the output."""

@@ -195,6 +195,78 @@ def test_transpose_is_the_conversion_of_the_transposed_dense_tensor():
     assert empty.shape == (0, s, s)
 
 
+def test_row_wise_reductions_against_dense_torch_and_loops():
+    """sum / max of the dense tensor (inactive blocks filled with the neutral element) for every row that holds
+    a block; element-by-element loops on the same input; columns other than 0 keep the neutral element; the
+    reference's own facts: NaN wins over everything in the maximum, also from a second block
+    (test/cases/test_regressions.py:1981-2004), a row of -inf stays -inf (:1173-1183)."""
+    g = torch.Generator().manual_seed(21)
+    s = 4
+    layout = (torch.rand((2, 3, 5), generator=g) < 0.5).numpy()
+    layout[1, 2, :] = False  # a block row without blocks
+    dense = torch.randn((2, 3 * s, 5 * s), generator=g, dtype=torch.float64)
+    blocks = orc.to_sparse(dense, layout, s)
+    rows = layout.any(-1)
+    for op, neutral, ref in (("sum", 0.0, lambda d: d.sum(-1)), ("max", float("-inf"), lambda d: d.max(-1).values)):
+        filled = orc.to_dense(blocks, layout, s, fill_value=neutral)
+        out, row_layout = orc.row_wise_reduce(blocks, layout, s, op)
+        assert row_layout.shape == (2, 3, 1) and np.array_equal(row_layout[..., 0], rows)
+        assert out.shape == (int(rows.sum()), s, s)
+        got = orc.to_dense(out, row_layout, s, fill_value=neutral)  # (B, R*s, s)
+        expected = ref(filled)
+        row_mask = torch.as_tensor(rows).repeat_interleave(s, 1)
+        assert torch.allclose(got[..., 0][row_mask], expected[row_mask], atol=1e-12)
+        assert torch.all(out[..., 1:] == neutral)
+        sliced, _ = orc.row_wise_reduce(blocks, layout, s, op, slice_only=True)
+        assert sliced.shape == (int(rows.sum()), s, 1) and torch.equal(sliced[..., 0], out[..., 0])
+        # loops
+        k = 0
+        for b in range(2):
+            for r in range(3):
+                if not rows[b, r]:
+                    continue
+                for e in range(s):
+                    vals = [dense[b, r * s + e, c * s + j].item() for c in range(5) if layout[b, r, c] for j in range(s)]
+                    want = sum(vals) if op == "sum" else max(vals)
+                    assert abs(out[k, e, 0].item() - want) < 1e-12
+                k += 1
+    two = np.ones((1, 1, 2), dtype=bool)
+    d = torch.arange(2.0 * s * s).reshape(1, s, 2 * s)
+    d[0, 0, 0] = float("nan")
+    d[0, 1, s] = float("nan")
+    d[0, 2, :] = float("-inf")
+    out, _ = orc.row_wise_reduce(orc.to_sparse(d, two, s), two, s, "max", slice_only=True)
+    assert torch.isnan(out[0, 0, 0]) and torch.isnan(out[0, 1, 0]) and torch.isneginf(out[0, 2, 0])
+    assert out[0, 3, 0] == d[0, 3].max()
+
+
+def test_row_wise_add_is_a_broadcast_add_on_the_dense_tensor():
+    """to_dense(row_wise_add(x, y)) == (dense + row values) on active blocks and 0 elsewhere, for slices and for
+    square blocks of y (only column 0 counts); adding the negated row sum of a one-block row centres it."""
+    g = torch.Generator().manual_seed(22)
+    s = 4
+    layout = (torch.rand((2, 3, 4), generator=g) < 0.6).numpy()
+    layout[0, 1, :] = False
+    dense = torch.randn((2, 3 * s, 4 * s), generator=g, dtype=torch.float64)
+    blocks = orc.to_sparse(dense, layout, s)
+    rows = layout.any(-1)
+    n_rows = int(rows.sum())
+    y = torch.randn((n_rows, s, 1), generator=g, dtype=torch.float64)
+    y_dense = torch.zeros((2, 3, s), dtype=torch.float64)
+    y_dense[torch.as_tensor(rows)] = y[..., 0]
+    expected = orc.to_dense(orc.to_sparse(dense + y_dense.reshape(2, 3 * s, 1), layout, s), layout, s)
+    got = orc.row_wise_add(blocks, layout, y, s)
+    assert torch.allclose(orc.to_dense(got, layout, s), expected, atol=1e-12)
+    y_square = torch.randn((n_rows, s, s), generator=g, dtype=torch.float64)
+    y_square[..., 0] = y[..., 0]
+    assert torch.equal(orc.row_wise_add(blocks, layout, y_square, s), got)
+    one = np.ones((1, 1, 1), dtype=bool)
+    blk = torch.randn((1, s, s), generator=g, dtype=torch.float64)
+    total, _ = orc.row_wise_reduce(blk, one, s, "sum", slice_only=True)
+    centred = orc.row_wise_add(blk, one, -total / s, s)
+    assert torch.allclose(centred.sum(-1), torch.zeros((1, s), dtype=torch.float64), atol=1e-12)
+
+
 def test_matmul_full_layout_is_bmm_and_inactive_blocks_do_not_contribute():
     g = torch.Generator().manual_seed(2)
     sbs = 4
