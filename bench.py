@@ -157,6 +157,50 @@ def matmul_workload(name, B, n, sbs, dtype, density, ensure_rows, value_scale, d
                         "nnz_o": nnz_o, "block_pairs": pairs, "lut_build_ms": round(lut_ms, 3)})
 
 
+def linear_workload(dev):
+    """``apply_torch_linear_cached`` on configuration 2's x operand: a 4096 -> 4096 linear layer with bias over a
+    bf16 input of 16 x 4096 x 4096 at 25 % block density (dense output, one un-replicated copy of the weight)."""
+    import blksprs_amd as bs
+    from oracle import blksprs_oracle as orc
+
+    B, n, sbs = 16, 64, 64
+    g = torch.Generator().manual_seed(0)
+    layout = orc.random_layout((B, n, n), 0.25, g)
+    ld = layout.to(dev)
+    nnz = int(layout.sum())
+    gd = torch.Generator(device=dev).manual_seed(1)
+    x = (torch.randn((nnz, sbs, sbs), generator=gd, device=dev) * 0.25).to(torch.bfloat16)
+    torch.manual_seed(2)
+    linear = torch.nn.Linear(n * sbs, n * sbs, bias=True, device=dev, dtype=torch.bfloat16)
+    cache = {}
+    with torch.no_grad():
+        bs.utils.apply_torch_linear_cached(x, ld, sbs, linear, layout_cache=cache)
+    nnz_o = B * n * n
+    flops = nnz * n * 2.0 * sbs ** 3
+    alg_bytes = (nnz + n * n + nnz_o) * sbs * sbs * 2
+    bs.utils.disable_validation()
+
+    def step():
+        with torch.no_grad():
+            return bs.utils.apply_torch_linear_cached(x, ld, sbs, linear, layout_cache=cache)
+
+    def cpu_baseline():
+        nb = 1
+        cnt = int(layout[:nb].sum())
+        xs = x[:cnt].float().cpu()
+        w, b = linear.weight.detach().float().cpu(), linear.bias.detach().float().cpu()
+        reps, dt = _repeat_for(CPU_SAMPLE_SECONDS, lambda: orc.linear(xs, layout[:nb].numpy(), w, b, sbs))
+        return {"value": cnt * n * 2.0 * sbs ** 3 / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+                "kind": "port", "sample": f"{nb} of {B} batches x {reps} passes, dense fp64 torch linear + to_sparse, "
+                                          f"{dt * reps:.1f} s (flops counted over non-zero input blocks)"}
+
+    return dict(step=step, flops=flops, alg_bytes=alg_bytes, dtype="bf16", bound="mfma", cpu_baseline=cpu_baseline,
+                kernel="matmul_rows_kernel",
+                config={"workload": "p1_apply_torch_linear_bf16", "B": B, "rows": n * sbs, "in_features": n * sbs,
+                        "out_features": n * sbs, "sparsity_block_size": sbs, "density": 0.25, "nnz_x": nnz,
+                        "nnz_o": nnz_o})
+
+
 def softmax_workload(dev):
     import blksprs_amd as bs
     from oracle import blksprs_oracle as orc
@@ -362,6 +406,8 @@ def make_workload(name, dev):
         return movement_workload(dev, "transpose")
     if name == "l1":
         return movement_workload(dev, "layout")
+    if name == "p1":
+        return linear_workload(dev)
     if name == "r1":
         return movement_workload(dev, "row_sum")
     if name == "r2":
@@ -376,7 +422,7 @@ def main():
     # with 10 warm-up steps the first timed steps of configuration 2 still run 10 % slower
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=100)
-    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c4bwd", "c5", "t1", "l1", "r1", "r2"])
+    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c4bwd", "c5", "t1", "l1", "r1", "r2", "p1"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:

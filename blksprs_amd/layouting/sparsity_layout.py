@@ -98,3 +98,45 @@ def build_sparsity_layout_matmul(sparsity_layout_x: Tensor, sparsity_layout_y: T
             _capi.call("bsa_layout_matmul", _capi.ptr(lx), _capi.ptr(ly), B, R, K, C,
                        out.view(torch.uint8).data_ptr(), _capi.stream(dev))
     return as_base_tensor(out)
+
+
+def _row_and_column_activity(sparsity_layout_x: Tensor, sparsity_layout_y: Tensor) -> tuple[Tensor, Tensor]:
+    """``(B, R, 1)`` rows of x and ``(B, 1, C)`` columns of y that hold a block."""
+    _check_product_inputs(sparsity_layout_x, sparsity_layout_y)
+    rows = torch.any(as_base_tensor(sparsity_layout_x) != 0, dim=-1, keepdim=True)
+    columns = torch.any(as_base_tensor(sparsity_layout_y) != 0, dim=-2, keepdim=True)
+    return rows, columns
+
+
+@torch.amp.custom_fwd(device_type="cuda")
+def build_sparsity_layout_matmul_fast(sparsity_layout_x: Tensor, sparsity_layout_y: Tensor) -> Tensor:
+    """Conservative product layout: block ``(i, j)`` is active when row ``i`` of x AND column ``j`` of y hold a
+    block, whether or not they meet at one ``k`` (blksprs/layouting/sparsity_layout.py:262-283).  A superset
+    of :func:`build_sparsity_layout_matmul`.
+
+    Args:
+        sparsity_layout_x (Tensor): Layout of the left operand, ``(B, R, K)``.
+        sparsity_layout_y (Tensor): Layout of the right operand, ``(B, K, C)``.
+
+    Returns:
+        Tensor: bool ``(B, R, C)`` layout.
+    """
+    rows, columns = _row_and_column_activity(sparsity_layout_x, sparsity_layout_y)
+    return as_base_tensor(torch.logical_and(rows, columns))
+
+
+@torch.amp.custom_fwd(device_type="cuda")
+def build_sparsity_layout_matmul_outer(sparsity_layout_x: Tensor, sparsity_layout_y: Tensor) -> Tensor:
+    """Outer product layout: block ``(i, j)`` is active when row ``i`` of x OR column ``j`` of y holds a block
+    (blksprs/layouting/sparsity_layout.py:286-311); for products followed by something that fills more
+    blocks, such as a bias.
+
+    Args:
+        sparsity_layout_x (Tensor): Layout of the left operand, ``(B, R, K)``.
+        sparsity_layout_y (Tensor): Layout of the right operand, ``(B, K, C)``.
+
+    Returns:
+        Tensor: bool ``(B, R, C)`` layout.
+    """
+    rows, columns = _row_and_column_activity(sparsity_layout_x, sparsity_layout_y)
+    return as_base_tensor(torch.logical_or(rows, columns))

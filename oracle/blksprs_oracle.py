@@ -242,6 +242,22 @@ def row_wise_add(x, layout, y, sbs: int) -> torch.Tensor:
     return out
 
 
+def linear(x, layout, weight, bias, sbs: int):
+    """blksprs/utils/processing.py:27-86: ``x @ weight^T (+ bias)`` on the dense form of x.  With a bias every
+    output block is active (:57-62); without one, the block rows of x that hold a block, over all output columns
+    (:63-64 with an all-ones weight layout).  Returns ``(blocks, layout)``."""
+    lay = np.asarray(layout) != 0
+    B, R, _ = lay.shape
+    n_out = weight.shape[0] // sbs
+    dense = to_dense(torch.as_tensor(x).to(torch.float64), lay, sbs)
+    out = torch.nn.functional.linear(dense, weight.to(torch.float64), None if bias is None else bias.to(torch.float64))
+    if bias is not None:
+        lay_out = np.ones((B, R, n_out), dtype=bool)
+    else:
+        lay_out = np.broadcast_to(lay.any(axis=-1, keepdims=True), (B, R, n_out)).copy()
+    return to_sparse(out, lay_out, sbs), lay_out
+
+
 def softmax(x, layout, sbs: int) -> torch.Tensor:
     """blksprs/ops/softmax.py:524-570: per element row, softmax over the concatenation of the row's active
     blocks; inactive blocks act as ``-inf`` and rows without blocks do not exist in the output."""

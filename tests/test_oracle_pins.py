@@ -267,6 +267,38 @@ def test_row_wise_add_is_a_broadcast_add_on_the_dense_tensor():
     assert torch.allclose(centred.sum(-1), torch.zeros((1, s), dtype=torch.float64), atol=1e-12)
 
 
+def test_linear_is_the_block_matmul_with_the_replicated_weight_plus_bias():
+    """The reference's own construction (blksprs/utils/processing.py:48-83): a block matmul with the transposed
+    weight repeated over the batch under an all-ones layout, then the bias added to every row, through the
+    independently pinned matmul; and a loop over output elements on a tiny case."""
+    g = torch.Generator().manual_seed(31)
+    s = 4
+    layout = (torch.rand((2, 3, 2), generator=g) < 0.6).numpy()
+    layout[1, 0, :] = False
+    x = orc.to_sparse(torch.randn((2, 3 * s, 2 * s), generator=g, dtype=torch.float64), layout, s)
+    weight = torch.randn((3 * s, 2 * s), generator=g, dtype=torch.float64)
+    bias = torch.randn((3 * s,), generator=g, dtype=torch.float64)
+    layout_w = np.ones((2, 2, 3), dtype=bool)
+    w_blocks = orc.to_sparse(weight.t().unsqueeze(0).repeat(2, 1, 1).contiguous(), layout_w, s)
+    dense_x = orc.to_dense(x, layout, s)
+    for b in (None, bias):
+        got, lay_out = orc.linear(x, layout, weight, b, s)
+        product = orc.matmul(x, layout, w_blocks, layout_w, lay_out, s, acc_dtype=torch.float64)
+        want = orc.to_dense(product, lay_out, s)
+        if b is not None:
+            want = want + b
+            assert lay_out.all()
+        else:
+            assert np.array_equal(lay_out[..., 0], layout.any(-1)) and (lay_out == lay_out[..., :1]).all()
+        assert torch.allclose(orc.to_dense(got, lay_out, s), orc.to_dense(orc.to_sparse(want, lay_out, s), lay_out, s),
+                              atol=1e-12)
+    got, lay_out = orc.linear(x, layout, weight, bias, s)
+    dense_out = orc.to_dense(got, lay_out, s)
+    for bi, i, j in ((0, 0, 0), (1, 2, 5), (1, 11, 11), (0, 7, 3)):
+        want = sum(dense_x[bi, i, k].item() * weight[j, k].item() for k in range(2 * s)) + bias[j].item()
+        assert abs(dense_out[bi, i, j].item() - want) < 1e-12
+
+
 def test_matmul_full_layout_is_bmm_and_inactive_blocks_do_not_contribute():
     g = torch.Generator().manual_seed(2)
     sbs = 4
