@@ -293,3 +293,65 @@ def test_pair_lists_cover_the_layout_and_masked_tiles_change_nothing(device):
     ref = orc.flash_attention(q.double(), full.numpy(), k.double(), fullk.numpy(), v.double(), fullk.numpy(),
                               la.numpy(), sbs, mask=mask, layout_mask=lmask.numpy(), acc_dtype=torch.float64)
     assert_close(out, ref, 2e-2, "O pair lists")
+
+
+def test_config4_full_size_against_sampled_oracle_rows_and_invariants(device):
+    """Configuration 4 at full size (bf16, 64 heads, 8192 positions, head_dim 128, sbs 64, BigBird layout with
+    causal mask blocks), where the oracle cannot run whole.  A query block row depends only on its own row of
+    the layout, so the oracle is run on single rows (1 x 1 x 128 layouts against all keys of the head) and gives
+    the exact output and dQ of those rows.  Everything else is held to invariants of attention:
+    rows of P sum to 1, hence with V = 1 the output is 1 and sum_k dV[k, f] = sum_q dO[q, f];
+    rows of dS sum to 0, hence sum_k dK[k, f] = 0; and two runs give identical bits (no atomics)."""
+    BH, n, sbs, nh = 64, 128, 64, 2
+    g = torch.Generator().manual_seed(0)
+    la = orc.bigbird_layout(BH, n, g)
+    lmask = la & torch.ones((n, n), dtype=torch.bool).triu()
+    lad, lmd = la.to(device), lmask.to(device)
+    full = torch.ones((BH, n, nh), dtype=torch.bool, device=device)
+    midx = torch.nonzero(lmd)
+    r = torch.arange(sbs, device=device)
+    mask = (midx[:, 2].view(-1, 1, 1) * sbs + r.view(1, 1, -1)) > (midx[:, 1].view(-1, 1, 1) * sbs + r.view(1, -1, 1))
+    gd = torch.Generator(device=device).manual_seed(1)
+    q, k, v, go = (torch.randn((BH * n * nh, sbs, sbs), device=device, generator=gd).to(torch.bfloat16)
+                   for _ in range(4))
+    q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
+    cache = {}
+
+    def run(values):
+        return bs.ops.flash_attention(q, full, k, full, values, full, lad, sbs, attention_mask=mask,
+                                      sparsity_layout_mask=lmd, layout_cache=cache)
+
+    out = run(v)
+    out.backward(go)
+    dq, dk, dv = q.grad.clone(), k.grad.clone(), v.grad.clone()
+    q.grad = k.grad = v.grad = None
+    out2 = run(v)
+    out2.backward(go)
+    assert torch.equal(out, out2) and torch.equal(dq, q.grad) and torch.equal(dk, k.grad) and torch.equal(dv, v.grad)
+
+    # sampled rows against the oracle (output and dQ)
+    mask_offsets = torch.cumsum(lmask.flatten().long(), 0) - 1
+    for h, i in ((0, 0), (0, 127), (17, 64), (63, 1), (40, 101)):
+        rows = slice((h * n + i) * nh, (h * n + i + 1) * nh)
+        head = slice(h * n * nh, (h + 1) * n * nh)
+        cols = torch.nonzero(lmask[h, i]).flatten()
+        mk = mask[mask_offsets[(h * n + i) * n + cols]].cpu() if len(cols) else None
+        q64 = q[rows].detach().cpu().double().requires_grad_(True)
+        ones = lambda a, b: torch.ones((1, a, b), dtype=torch.bool).numpy()
+        ref = orc.flash_attention(q64, ones(1, nh), k[head].detach().cpu().double(), ones(n, nh),
+                                  v[head].detach().cpu().double(), ones(n, nh), la[h:h + 1, i:i + 1].numpy(), sbs,
+                                  mask=mk, layout_mask=lmask[h:h + 1, i:i + 1].numpy() if mk is not None else None,
+                                  acc_dtype=torch.float64)
+        assert_close(out[rows], ref, 2e-2, f"O head {h} row {i}")
+        ref.backward(go[rows].cpu().double())
+        assert_close(dq[rows], q64.grad, 4e-2, f"dQ head {h} row {i}")
+
+    # invariants over all heads
+    with torch.no_grad():
+        unit = run(torch.ones_like(v))
+        assert float((unit.float() - 1).abs().max()) <= 2e-2
+        per_head = lambda t: t.detach().float().reshape(BH, n, nh, sbs, sbs).permute(0, 1, 3, 2, 4).reshape(BH, n * sbs, nh * sbs)
+        dv_h, go_h, dk_h = per_head(dv), per_head(go), per_head(dk)
+        mass, want = dv_h.sum(1), go_h.sum(1)
+        assert float((mass - want).abs().max()) <= 2e-2 * float(go_h.abs().sum(1).max())
+        assert float(dk_h.sum(1).abs().max()) <= 2e-2 * float(dk_h.abs().sum(1).max())
