@@ -26,6 +26,8 @@
 //
 // The two waves that share a half of the stationary block hold partial sums over the two halves of the streamed
 // blocks; they are added through LDS once, at the end.  No atomics, fixed summation order.
+#include <type_traits>
+
 #include "attn_mfma_common.h"
 
 namespace bsa {
@@ -38,21 +40,26 @@ constexpr int kStatBytes = 2 * kSbs * 4;  // lse and delta of the 64 queries of 
 // dK and dV in one pass over the query blocks (one workgroup per CU) or in two passes (two workgroups per CU,
 // scores computed twice): measured equal within 3 % on the BigBird configuration; one pass reads less
 constexpr bool kSplitKeyPass = false;
+// dK and dV by two teams of four waves in one workgroup of eight (the default); the two switches above
+// choose among the four-wave kernels otherwise
+constexpr bool kEightWaves = true;
 
-// One 64 x 64 16-bit block, global -> LDS, by the four waves of a workgroup: wave w copies rows 16 w .. + 15
-// with two asynchronous 1 KiB copies; lane l supplies the chunk that belongs at position l of the KiB, which
-// is where the chunk swizzle is applied.  An inactive block becomes zeros.
+// One 64 x 64 16-bit block, global -> LDS, by the NW (4 or 8) waves of a workgroup: wave w copies rows
+// (64 / NW) w .. with asynchronous 1 KiB copies (eight rows each); lane l supplies the chunk that belongs at
+// position l of the KiB, which is where the chunk swizzle is applied.  An inactive block becomes zeros.
+template <int NW = 4>
 __device__ inline void copy_block(const char *blk, bool valid, char *dst, int wave, int lane, int tid) {
+  constexpr int kCopies = 8 / NW;  // KiB per wave
   if (valid) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int r0 = 16 * wave + 8 * i;
+    for (int i = 0; i < kCopies; ++i) {
+      const int r0 = 8 * kCopies * wave + 8 * i;
       const uint32_t lane_off = (lane >> 3) * 128 + (((lane & 7) ^ t_swizzle(8 * i + (lane >> 3))) << 4);
       copy_1k_to_lds(blk + r0 * 128, lane_off, dst + r0 * 128);
     }
   } else {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) *reinterpret_cast<u32x4 *>(dst + (i * kBwdThreads + tid) * 16) = u32x4{0u, 0u, 0u, 0u};
+    for (int i = 0; i < kCopies; ++i) *reinterpret_cast<u32x4 *>(dst + (i * NW * 64 + tid) * 16) = u32x4{0u, 0u, 0u, 0u};
   }
 }
 
@@ -107,6 +114,79 @@ __device__ inline void reduce_partner(f32x16 (&acc)[N], float *lds, bool writer,
 }
 
 // ---------------------------------------------------------------------------------------------------------
+// Lists of the pairs that can contribute.  A (query block, key block) pair whose mask block masks every score, or
+// that the causal predicate rules out as a whole, has P = dS = 0.  Which pairs those are depends on the mask's
+// contents, so it is found out at the start of every backward call: one pass over the mask blocks, then the
+// two lists of the attention layout (key blocks per query block, query blocks per key block) are copied without
+// the dead pairs, in the same order.  The two main kernels then walk the shortened lists.
+struct BwdLists {
+  int32_t *key_idx, *query_idx;  // [n_layout_blocks] each, rows at the offsets of key_offsets / query_offsets
+  int32_t *key_end, *query_end;  // [B * nq], [B * nk]: end of the live part of a row's list
+  uint8_t *mask_dead;            // [n_mask_blocks]
+};
+
+__host__ __device__ inline BwdLists bwd_lists(const bsa_attn_args &a) {
+  BwdLists L;
+  L.key_idx = static_cast<int32_t *>(a.bwd_scratch);
+  L.query_idx = L.key_idx + a.n_layout_blocks;
+  L.key_end = L.query_idx + a.n_layout_blocks;
+  L.query_end = L.key_end + a.B * a.nq;
+  L.mask_dead = reinterpret_cast<uint8_t *>(L.query_end + a.B * a.nk);
+  return L;
+}
+
+// one wave per mask block (4 KiB of bytes 0 / 1)
+__global__ __launch_bounds__(kBwdThreads) void attn_bwd_mask_dead_kernel(const u32x4 *mask, uint8_t *dead, int64_t n) {
+  const int64_t m = ((int64_t)blockIdx.x * kBwdThreads + threadIdx.x) >> 6;
+  if (m >= n) return;
+  const int lane = threadIdx.x & 63;
+  const u32x4 *p = mask + m * (kSbs * kSbs / 16);
+  uint32_t all = 0x01010101u;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const u32x4 v = p[i * 64 + lane];
+    all &= v[0] & v[1] & v[2] & v[3];
+  }
+  const unsigned long long votes = __ballot(all == 0x01010101u);
+  if (lane == 0) dead[m] = votes == ~0ull ? 1 : 0;
+}
+
+// one wave per query block row, then one per key block row
+__global__ __launch_bounds__(kBwdThreads) void attn_bwd_live_lists_kernel(bsa_attn_args a) {
+  const int64_t w = ((int64_t)blockIdx.x * kBwdThreads + threadIdx.x) >> 6;
+  const int64_t qrows = a.B * a.nq, krows = a.B * a.nk;
+  if (w >= qrows + krows) return;
+  const int lane = threadIdx.x & 63;
+  const BwdLists L = bwd_lists(a);
+  const bool by_key = w >= qrows;
+  const int64_t row = by_key ? w - qrows : w;
+  const int64_t per_batch = by_key ? a.nk : a.nq;
+  const int64_t b = row / per_batch, mine = row % per_batch;
+  const int32_t *offsets = by_key ? a.query_offsets : a.key_offsets;
+  const int32_t *indices = by_key ? a.query_indices : a.key_indices;
+  int32_t *out = by_key ? L.query_idx : L.key_idx;
+  const bool causal = a.causal_lengths != nullptr;
+  const int64_t seq_len = causal ? a.causal_lengths[b] : 0;
+  const int begin = offsets[row], end = offsets[row + 1];
+  int n = begin;
+  for (int e0 = begin; e0 < end; e0 += 64) {
+    const int e = e0 + lane;
+    bool live = e < end;
+    const int64_t other = live ? indices[e] : 0;
+    const int64_t qb = by_key ? other : mine, kb = by_key ? mine : other;
+    if (live && causal && (kb > qb || qb * kSbs >= seq_len || kb * kSbs >= seq_len)) live = false;
+    if (live && a.mask) {
+      const int64_t pm = a.pidx_mask[(b * a.nq + qb) * a.nk + kb];
+      if (pm >= 0 && pm < a.n_mask_blocks && L.mask_dead[pm]) live = false;
+    }
+    const unsigned long long votes = __ballot(live);
+    if (live) out[n + __popcll(votes & ((1ull << lane) - 1))] = (int32_t)other;
+    n += __popcll(votes);
+  }
+  if (lane == 0) (by_key ? L.query_end : L.key_end)[row] = n;
+}
+
+// ---------------------------------------------------------------------------------------------------------
 // delta[b, qb, i] = sum over active output slices of rowsum(o * dO); four lanes per query row
 template <typename Tr>
 __global__ __launch_bounds__(kBwdThreads) void attn_bwd_delta_kernel(bsa_attn_args a) {
@@ -139,34 +219,40 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_delta_kernel(bsa_attn_ar
 // dK and dBias (DK) and / or dV (DV) of one key block.  The two are launched as separate passes: each then fits
 // two workgroups per CU (the combined kernel needs more than 256 registers per lane), which more than pays
 // for computing the scores twice.
-template <typename Tr, int NH, int NHV, bool DK, bool DV>
-__global__ __launch_bounds__(kBwdThreads, (DK &&DV) ? 1 : 2) void attn_bwd_kv_kernel(bsa_attn_args a) {
-  extern __shared__ __attribute__((aligned(1024))) char smem[];
+//
+// The body serves two kernels.  With NW = 4 the four waves of a workgroup each own a quadrant and compute
+// whatever DK / DV ask for.  With NW = 8 the workgroup has two teams of four waves, one running the body for dV
+// and one for dK (and dBias): `wave` (0 .. 7) says which rows of a tile the wave copies, `quad` which quadrant it
+// computes; both teams walk the same list, copy every tile together and meet at the same barriers, so neither
+// may leave early on its own (JOINT: leave only if there is nothing to do for either).
+template <typename Tr, int NH, int NHV, bool DK, bool DV, int NW>
+__device__ __forceinline__ void attn_bwd_kv_body(const bsa_attn_args &a, char *smem, float *reduce_lds, int wave,
+                                                 int quad) {
+  constexpr bool JOINT = NW == 8;
   constexpr int kQRows = 0, kDoRows = NH * kBlockBytes, kStats = (NH + NHV) * kBlockBytes,
                 kMask = kStats + kStatBytes;  // the tile's mask block, row-major bytes
   constexpr int kBufBytes = kMask + kSbs * kSbs;
 
   const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = first_lane(tid >> 6);
   const int li = lane & 31, kg = lane >> 5;
-  const int wi = wave & 1, wj = wave >> 1;  // query half and key half of this wave's quadrant
+  const int wi = quad & 1, wj = quad >> 1;  // query half and key half of this wave's quadrant
   const int64_t krow = xcd_row();
   if (krow >= a.B * a.nk) return;
   const int64_t b = krow / a.nk, kb = krow % a.nk;
 
   int64_t pk[NH], pv[NHV];
-  bool any = DK && a.dbias != nullptr;
+  bool any = (DK || JOINT) && a.dbias != nullptr;
 #pragma unroll
   for (int h = 0; h < NH; ++h) {
     pk[h] = a.pidx_k[krow * NH + h];
     if (pk[h] >= a.n_k_blocks) pk[h] = -1;
-    any = any || (DK && pk[h] >= 0);
+    any = any || ((DK || JOINT) && pk[h] >= 0);
   }
 #pragma unroll
   for (int h = 0; h < NHV; ++h) {
     pv[h] = a.pidx_v[krow * NHV + h];
     if (pv[h] >= a.n_v_blocks) pv[h] = -1;
-    any = any || (DV && pv[h] >= 0);
+    any = any || ((DV || JOINT) && pv[h] >= 0);
   }
   if (!any) return;
 
@@ -203,14 +289,21 @@ __global__ __launch_bounds__(kBwdThreads, (DK &&DV) ? 1 : 2) void attn_bwd_kv_ke
   }
   const int kpos = (int)kb * kSbs + 32 * wj + li;
 
-  const int q_begin = a.query_offsets[krow], q_end = a.query_offsets[krow + 1];
+  const int q_begin = a.query_offsets[krow];
+  int q_end = a.query_offsets[krow + 1];
+  const int32_t *q_list = a.query_indices;
+  if (a.bwd_scratch != nullptr) {
+    const BwdLists L = bwd_lists(a);
+    q_list = L.query_idx;
+    q_end = L.query_end[krow];
+  }
   if (q_begin < q_end) {
     // lanes 0 .. NH-1: packed Q indices of a query block, next NHV lanes: packed O (= dO) indices, then its mask and
     // bias block for this key block; lane 7: the list entry at `pos`
     constexpr int kLaneMask = NH + NHV, kLaneBias = NH + NHV + 1, kLaneEntry = 7;
     auto gather = [&](int qb, int pos) -> int {
       const int64_t qrow = b * a.nq + qb;
-      const int32_t *p = a.query_indices + pos;
+      const int32_t *p = q_list + pos;
       bool on = lane == kLaneEntry;
       if (lane < NH) {
         p = low_half_ptr(a.pidx_q, qrow * NH + lane);
@@ -242,14 +335,14 @@ __global__ __launch_bounds__(kBwdThreads, (DK &&DV) ? 1 : 2) void attn_bwd_kv_ke
       for (int h = 0; h < NH; ++h) {
         const int64_t pq = __builtin_amdgcn_readlane(rec, h);
         const bool valid = pq >= 0 && pq < a.n_q_blocks;
-        copy_block(static_cast<const char *>(a.q) + (valid ? pq : 0) * kBlockBytes, valid,
+        copy_block<NW>(static_cast<const char *>(a.q) + (valid ? pq : 0) * kBlockBytes, valid,
                    base + kQRows + h * kBlockBytes, wave, lane, tid);
       }
 #pragma unroll
       for (int h = 0; h < NHV; ++h) {
         const int64_t po = __builtin_amdgcn_readlane(rec, NH + h);
         const bool valid = po >= 0 && po < a.n_o_blocks;
-        copy_block(static_cast<const char *>(a.d_o) + (valid ? po : 0) * kBlockBytes, valid,
+        copy_block<NW>(static_cast<const char *>(a.d_o) + (valid ? po : 0) * kBlockBytes, valid,
                    base + kDoRows + h * kBlockBytes, wave, lane, tid);
       }
       const int64_t qrow = b * a.nq + qb;
@@ -260,14 +353,16 @@ __global__ __launch_bounds__(kBwdThreads, (DK &&DV) ? 1 : 2) void attn_bwd_kv_ke
       pb_nxt = __builtin_amdgcn_readlane(rec, kLaneBias);
       if (pb_nxt >= a.n_bias_blocks) pb_nxt = -1;
       // the mask block goes to LDS as it is: wave w copies its rows 16 w .. + 15 (1 KiB)
-      if (pm_nxt >= 0)
+      if (pm_nxt >= 0 && wave < 4)
         copy_1k_to_lds(static_cast<const char *>(a.mask) + (int64_t)pm_nxt * (kSbs * kSbs) + wave * 1024, lane * 16,
                        base + kMask + wave * 1024);
     };
     // the statistics of the tile go to LDS through a register; then every copy of this wave has to have landed
     auto stage = [&](int buf) {
       char *base = smem + buf * kBufBytes;
-      if (tid < 128) reinterpret_cast<float *>(base + kStats)[tid] = stat;
+      // a query without any visible key has lse = -inf and P = 0 everywhere: +inf gives exp2(s - lse) = 0 for it
+      // without a test per score
+      if (tid < 128) reinterpret_cast<float *>(base + kStats)[tid] = (tid < 64 && stat == -INFINITY) ? INFINITY : stat;
       __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     };
 
@@ -275,7 +370,7 @@ __global__ __launch_bounds__(kBwdThreads, (DK &&DV) ? 1 : 2) void attn_bwd_kv_ke
     // lane 7, the entry after that
     int rec, qb_rec;
     {
-      const int qb0 = first_lane(a.query_indices[as_vector(q_begin)]);
+      const int qb0 = first_lane(q_list[as_vector(q_begin)]);
       const int rec0 = gather(qb0, clamp_e(q_begin + 1));
       qb_rec = __builtin_amdgcn_readlane(rec0, kLaneEntry);
       rec = gather(qb_rec, clamp_e(q_begin + 2));
@@ -339,26 +434,40 @@ __global__ __launch_bounds__(kBwdThreads, (DK &&DV) ? 1 : 2) void attn_bwd_kv_ke
           for (int r = 0; r < 16; ++r) bias_c[r] = bp[(8 * (r >> 2) + (r & 3)) * kSbs];
         }
         float p[16], ds[16];
+        // Most tiles have no bias, no mask block and lie where the causal predicate holds for every score: they
+        // take the plain path.  The conditions are the same for the whole wave.
+        auto probabilities = [&](auto plain_tag) {
+          constexpr bool kPlain = decltype(plain_tag)::value;
   #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int i0 = 32 * wi + 8 * q + 4 * kg;
-          const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(stats + i0);
-          const f32x4 del4 = *reinterpret_cast<const f32x4 *>(stats + kSbs + i0);
+          for (int q = 0; q < 4; ++q) {
+            const int i0 = 32 * wi + 8 * q + 4 * kg;
+            const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(stats + i0);
+            const f32x4 del4 = *reinterpret_cast<const f32x4 *>(stats + kSbs + i0);
   #pragma unroll
-          for (int t = 0; t < 4; ++t) {
-            const int r = 4 * q + t;
-            float s = sacc[r] * qk_scale;
-            if (pb >= 0) s = s + Tr::widen((uint16_t)bias_c[r]) * kLog2e;
-            if (causal) {
-              const int qpos = qb * kSbs + i0 + t;
-              s = (kpos > qpos || qpos >= seq_len || kpos >= seq_len) ? -INFINITY : s;
+            for (int t = 0; t < 4; ++t) {
+              const int r = 4 * q + t;
+              float s = sacc[r] * qk_scale;
+              if constexpr (!kPlain) {
+                if (pb >= 0) s = s + Tr::widen((uint16_t)bias_c[r]) * kLog2e;
+                if (causal) {
+                  const int qpos = qb * kSbs + i0 + t;
+                  s = (kpos > qpos || qpos >= seq_len || kpos >= seq_len) ? -INFINITY : s;
+                }
+                if (pm >= 0) s = ((mbits >> r) & 1u) ? -INFINITY : s;
+              }
+              p[r] = __builtin_amdgcn_exp2f(s - lse4[t]);
+              ds[r] = p[r] * (dpacc[r] - del4[t]);
             }
-            if (pm >= 0) s = ((mbits >> r) & 1u) ? -INFINITY : s;
-            const float lse = lse4[t];
-            p[r] = (lse == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(s - lse);
-            ds[r] = p[r] * (dpacc[r] - del4[t]);
           }
+        };
+        bool plain = pb < 0 && pm < 0;
+        if (causal) {
+          // every key of the quadrant at or before every query of it, and all of them inside the sequence
+          const int k_last = (int)kb * kSbs + 32 * wj + 31, q_first = qb * kSbs + 32 * wi;
+          plain = plain && k_last <= q_first && q_first + 31 < seq_len;
         }
+        if (plain) probabilities(std::true_type{});
+        else probabilities(std::false_type{});
         if (DK && a.dbias != nullptr && pb >= 0) {
           // every (query block, key block) pair is visited once, so this is a plain store
           float *dbp = a.dbias + pb * (kSbs * kSbs) + (32 * wi + 4 * kg) * kSbs + 32 * wj + li;
@@ -406,8 +515,8 @@ __global__ __launch_bounds__(kBwdThreads, (DK &&DV) ? 1 : 2) void attn_bwd_kv_ke
   }
 
   // ---- add the two query halves, scale, store ----
-  if constexpr (DK) reduce_partner(dkacc, reinterpret_cast<float *>(smem), wi == 1, wj, lane);
-  if constexpr (DV) reduce_partner(dvacc, reinterpret_cast<float *>(smem), wi == 1, wj, lane);
+  if constexpr (DK) reduce_partner(dkacc, reduce_lds, wi == 1, wj, lane);
+  if constexpr (DV) reduce_partner(dvacc, reduce_lds, wi == 1, wj, lane);
   if (wi == 1) return;
   // lane: key 32 wj + li; register 4 q + t of half db: column 32 db + 8 q + 4 kg + t
 #pragma unroll
@@ -440,6 +549,26 @@ __global__ __launch_bounds__(kBwdThreads, (DK &&DV) ? 1 : 2) void attn_bwd_kv_ke
         *reinterpret_cast<u32x2 *>(op + 64 * db + 16 * q) = w;
       }
   }
+}
+
+template <typename Tr, int NH, int NHV, bool DK, bool DV>
+__global__ __launch_bounds__(kBwdThreads, (DK &&DV) ? 1 : 2) void attn_bwd_kv_kernel(bsa_attn_args a) {
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  const int wave = first_lane((int)threadIdx.x >> 6);
+  attn_bwd_kv_body<Tr, NH, NHV, DK, DV, 4>(a, smem, reinterpret_cast<float *>(smem), wave, wave);
+}
+
+// Eight waves: waves 0 .. 3 accumulate dV, waves 4 .. 7 dK and dBias, two waves per SIMD.  Each team fits 256
+// registers per lane, which the two sets of accumulators in one wave do not; the tile is fetched once for both.
+constexpr int kKv8Threads = 512;
+template <typename Tr, int NH, int NHV>
+__global__ __launch_bounds__(kKv8Threads, 1) void attn_bwd_kv8_kernel(bsa_attn_args a) {
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  const int wave = first_lane((int)threadIdx.x >> 6);
+  // the partial sums of a team take 2 * (slices * 2) * 16 * 64 floats
+  float *reduce_lds = reinterpret_cast<float *>(smem) + (wave >> 2) * (2 * (NH > NHV ? NH : NHV) * 2 * 16 * 64);
+  if (wave < 4) attn_bwd_kv_body<Tr, NH, NHV, false, true, 8>(a, smem, reduce_lds, wave, wave & 3);
+  else attn_bwd_kv_body<Tr, NH, NHV, true, false, 8>(a, smem, reduce_lds, wave, wave & 3);
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -475,7 +604,9 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_q_kernel(bsa_attn_arg
   for (int h = 0; h < NH; ++h) load_resident(qfr[h], a.q, pq[h], a.n_q_blocks, qi, kg);
 #pragma unroll
   for (int h = 0; h < NHV; ++h) load_resident(dofr[h], a.d_o, a.pidx_o[qrow * NHV + h], a.n_o_blocks, qi, kg);
-  const float lse = a.lse[qrow * kSbs + qi];
+  // a query without any visible key has lse = -inf and P = 0 everywhere: +inf gives exp2(s - lse) = 0 for it
+  const float lse_raw = a.lse[qrow * kSbs + qi];
+  const float lse = lse_raw == -INFINITY ? INFINITY : lse_raw;
   const float delta = a.delta[qrow * kSbs + qi];
 
   f32x16 dqacc[NH * 2];
@@ -493,12 +624,19 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_q_kernel(bsa_attn_arg
   }
   const int qpos = (int)qb * kSbs + qi;
 
-  const int k_begin = a.key_offsets[qrow], k_end = a.key_offsets[qrow + 1];
+  const int k_begin = a.key_offsets[qrow];
+  int k_end = a.key_offsets[qrow + 1];
+  const int32_t *k_list = a.key_indices;
+  if (a.bwd_scratch != nullptr) {
+    const BwdLists L = bwd_lists(a);
+    k_list = L.key_idx;
+    k_end = L.key_end[qrow];
+  }
   if (k_begin < k_end) {
     constexpr int kLaneMask = NH + NHV, kLaneBias = NH + NHV + 1, kLaneEntry = 7;
     auto gather = [&](int kb, int pos) -> int {
       const int64_t krow = b * a.nk + kb;
-      const int32_t *p = a.key_indices + pos;
+      const int32_t *p = k_list + pos;
       bool on = lane == kLaneEntry;
       if (lane < NH) {
         p = low_half_ptr(a.pidx_k, krow * NH + lane);
@@ -562,7 +700,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_q_kernel(bsa_attn_arg
 
     int rec, kb_rec;
     {
-      const int kb0 = first_lane(a.key_indices[as_vector(k_begin)]);
+      const int kb0 = first_lane(k_list[as_vector(k_begin)]);
       const int rec0 = gather(kb0, clamp_e(k_begin + 1));
       kb_rec = __builtin_amdgcn_readlane(rec0, kLaneEntry);
       rec = gather(kb_rec, clamp_e(k_begin + 2));
@@ -612,24 +750,37 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_q_kernel(bsa_attn_arg
             dpacc = Tr::mfma(frag_rows(base + kVRows + h * kBlockBytes, 32 * wj + li, 2 * s + kg), dofr[h][s], dpacc);
 
         float ds[16];
+        // the plain path: no bias, no mask block, causal predicate true for every score of the quadrant
+        auto gradients = [&](auto plain_tag) {
+          constexpr bool kPlain = decltype(plain_tag)::value;
   #pragma unroll
-        for (int q = 0; q < 4; ++q)
+          for (int q = 0; q < 4; ++q)
   #pragma unroll
-          for (int t = 0; t < 4; ++t) {
-            const int r = 4 * q + t;
-            float s = sacc[r] * qk_scale;
-            if (pb >= 0) {
-              const uint32_t bw = bias_c[q][t >> 1];
-              s = s + Tr::widen((uint16_t)((t & 1) ? (bw >> 16) : (bw & 0xffffu))) * kLog2e;
+            for (int t = 0; t < 4; ++t) {
+              const int r = 4 * q + t;
+              float s = sacc[r] * qk_scale;
+              if constexpr (!kPlain) {
+                if (pb >= 0) {
+                  const uint32_t bw = bias_c[q][t >> 1];
+                  s = s + Tr::widen((uint16_t)((t & 1) ? (bw >> 16) : (bw & 0xffffu))) * kLog2e;
+                }
+                if (causal) {
+                  const int kpos = kb * kSbs + 32 * wj + 8 * q + 4 * kg + t;
+                  s = (kpos > qpos || qpos >= seq_len || kpos >= seq_len) ? -INFINITY : s;
+                }
+                if (pm >= 0) s = ((mask_c[q] >> (8 * t)) & 0xffu) ? -INFINITY : s;
+              }
+              const float p = __builtin_amdgcn_exp2f(s - lse);
+              ds[r] = p * (dpacc[r] - delta);
             }
-            if (causal) {
-              const int kpos = kb * kSbs + 32 * wj + 8 * q + 4 * kg + t;
-              s = (kpos > qpos || qpos >= seq_len || kpos >= seq_len) ? -INFINITY : s;
-            }
-            if (pm >= 0) s = ((mask_c[q] >> (8 * t)) & 0xffu) ? -INFINITY : s;
-            const float p = (lse == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(s - lse);
-            ds[r] = p * (dpacc[r] - delta);
-          }
+        };
+        bool plain = pb < 0 && pm < 0;
+        if (causal) {
+          const int k_last = kb * kSbs + 32 * wj + 31, q_first = (int)qb * kSbs + 32 * wi;
+          plain = plain && k_last <= q_first && q_first + 31 < seq_len;
+        }
+        if (plain) gradients(std::true_type{});
+        else gradients(std::false_type{});
         u32x4 dsf[2];
   #pragma unroll
         for (int u = 0; u < 2; ++u)
@@ -690,13 +841,29 @@ int launch_bwd(const bsa_attn_args &a, hipStream_t s) {
     fill_zero_f32_kernel<<<(unsigned)blocks, 256, 0, s>>>(a.dbias, n);
     if (int rc = check_launch("fill_zero_f32_kernel")) return rc;
   }
+  if (a.bwd_scratch != nullptr && qrows + krows > 0) {
+    const BwdLists L = bwd_lists(a);
+    if (a.mask != nullptr && a.n_mask_blocks > 0) {
+      attn_bwd_mask_dead_kernel<<<(unsigned)cdiv(a.n_mask_blocks, 4), kBwdThreads, 0, s>>>(
+          static_cast<const u32x4 *>(a.mask), L.mask_dead, a.n_mask_blocks);
+      if (int rc = check_launch("attn_bwd_mask_dead_kernel")) return rc;
+    }
+    attn_bwd_live_lists_kernel<<<(unsigned)cdiv(qrows + krows, 4), kBwdThreads, 0, s>>>(a);
+    if (int rc = check_launch("attn_bwd_live_lists_kernel")) return rc;
+  }
   if (qrows > 0) {
     attn_bwd_delta_kernel<Tr><<<(unsigned)qrows, kBwdThreads, 0, s>>>(a);
     if (int rc = check_launch("attn_bwd_delta_kernel")) return rc;
   }
   if (krows > 0) {
     constexpr int lds = 2 * ((NH + NHV) * kBlockBytes + kStatBytes + kSbs * kSbs);
-    if (kSplitKeyPass) {
+    if (kEightWaves) {
+      constexpr int lds8 = lds > 65536 ? lds : 65536;  // the tile buffers; at the end, the partial sums of both teams
+      BSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_bwd_kv8_kernel<Tr, NH, NHV>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds8));
+      attn_bwd_kv8_kernel<Tr, NH, NHV><<<(unsigned)(cdiv(krows, 8) * 8), kKv8Threads, lds8, s>>>(a);
+      if (int rc = check_launch("attn_bwd_kv8_kernel")) return rc;
+    } else if (kSplitKeyPass) {
       BSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_bwd_kv_kernel<Tr, NH, NHV, true, false>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds));
       BSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_bwd_kv_kernel<Tr, NH, NHV, false, true>),
@@ -732,6 +899,11 @@ int dispatch_bwd(const bsa_attn_args &a, hipStream_t s) {
 }
 
 }  // namespace
+
+size_t attn_bwd_scratch_bytes(int64_t B, int64_t nq, int64_t nk, int64_t n_layout_blocks, int64_t n_mask_blocks) {
+  const size_t bytes = 4 * (size_t)(2 * n_layout_blocks + B * nq + B * nk) + (size_t)n_mask_blocks;
+  return (bytes + 15) & ~(size_t)15;
+}
 
 int attn_bwd_mfma(const bsa_attn_args &a, hipStream_t s) {
   if (a.sbs != kSbs || (a.dtype != BSA_BF16 && a.dtype != BSA_F16)) return 1;

@@ -282,6 +282,14 @@ typedef struct bsa_attn_args {
    * of a pair.  No counterpart in the reference. */
   const int32_t *group_offsets, *group_records;
   int32_t group_size;
+  /* Optional, backward only (NULL: every pair of the attention layout is visited).  Scratch of
+   * bsa_attn_bwd_scratch_bytes(...) bytes in which bsa_attn_bwd first lists, per query block and per key block,
+   * the pairs that some score survives (a pair whose mask block masks everything, or that the causal predicate
+   * rules out as a whole, adds nothing to any gradient and is then neither fetched nor computed).
+   * n_layout_blocks = number of active blocks of the attention layout (= key_offsets[B * nq]).
+   * No counterpart in the reference, which visits every pair (blksprs/ops/flash_attention.py:1322-1330). */
+  void *bwd_scratch;
+  int64_t n_layout_blocks;
 } bsa_attn_args;
 
 #define BSA_ATTN_RECORD_INTS 16
@@ -305,6 +313,9 @@ int bsa_attn_fwd_records(const bsa_attn_args *args, const int32_t *group_entries
  * Every block of `o` that is active in the output layout is written.
  */
 int bsa_attn_fwd(const bsa_attn_args *args, bsa_stream_t stream);
+
+/* Size in bytes of bsa_attn_args.bwd_scratch for these sizes (16-byte aligned buffer). */
+size_t bsa_attn_bwd_scratch_bytes(int64_t B, int64_t nq, int64_t nk, int64_t n_layout_blocks, int64_t n_mask_blocks);
 
 /*
  * dq, dk, dv (and dbias) from the saved lse.  Replaces
