@@ -79,15 +79,6 @@ __device__ inline void load_resident(u32x4 (&f)[4], const void *base, int64_t pi
   }
 }
 
-__device__ inline const int32_t *low_half_ptr(const int64_t *p, int64_t i) {
-  return reinterpret_cast<const int32_t *>(p) + 2 * i;
-}
-
-__device__ inline int as_vector(int v) {
-  asm volatile("" : "+v"(v));
-  return v;
-}
-
 // XCD-aware row of a workgroup: every XCD gets a contiguous range of rows, so that the blocks in flight on one
 // L2 belong to the same batch entries
 __device__ inline int64_t xcd_row() { return (int64_t)(blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3); }
@@ -114,22 +105,33 @@ __device__ inline void reduce_partner(f32x16 (&acc)[N], float *lds, bool writer,
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// Lists of the pairs that can contribute.  A (query block, key block) pair whose mask block masks every score, or
-// that the causal predicate rules out as a whole, has P = dS = 0.  Which pairs those are depends on the mask's
+// Records of the pairs that can contribute.  A (query block, key block) pair whose mask block masks every score,
+// or that the causal predicate rules out as a whole, has P = dS = 0.  Which pairs those are depends on the mask's
 // contents, so it is found out at the start of every backward call: one pass over the mask blocks, then the
-// two lists of the attention layout (key blocks per query block, query blocks per key block) are copied without
-// the dead pairs, in the same order.  The two main kernels then walk the shortened lists.
+// two lists of the attention layout (key blocks per query block, query blocks per key block) are written out
+// without the dead pairs, in the same order, each entry as a record that already holds every index its tile
+// needs.  The two main kernels walk those records: one 32-byte load per tile instead of a chain of gathers.
+struct BwdRecord {
+  int32_t other;   // the query block (lists per key block) or key block (lists per query block)
+  int32_t pa[2];   // packed indices of its Q (resp. K) slices, -1: none
+  int32_t pb[2];   // packed indices of its O / dO (resp. V) slices
+  int32_t mask;    // mask block of the pair, -1: none
+  int32_t bias;    // bias block of the pair
+  int32_t pad;
+};
+static_assert(sizeof(BwdRecord) == 32, "one record is eight int32");
+
 struct BwdLists {
-  int32_t *key_idx, *query_idx;  // [n_layout_blocks] each, rows at the offsets of key_offsets / query_offsets
-  int32_t *key_end, *query_end;  // [B * nq], [B * nk]: end of the live part of a row's list
-  uint8_t *mask_dead;            // [n_mask_blocks]
+  BwdRecord *key_rec, *query_rec;  // [n_layout_blocks] each, rows at the offsets of key_offsets / query_offsets
+  int32_t *key_end, *query_end;    // [B * nq], [B * nk]: end of the live part of a row's list
+  uint8_t *mask_dead;              // [n_mask_blocks]
 };
 
 __host__ __device__ inline BwdLists bwd_lists(const bsa_attn_args &a) {
   BwdLists L;
-  L.key_idx = static_cast<int32_t *>(a.bwd_scratch);
-  L.query_idx = L.key_idx + a.n_layout_blocks;
-  L.key_end = L.query_idx + a.n_layout_blocks;
+  L.key_rec = static_cast<BwdRecord *>(a.bwd_scratch);
+  L.query_rec = L.key_rec + a.n_layout_blocks;
+  L.key_end = reinterpret_cast<int32_t *>(L.query_rec + a.n_layout_blocks);
   L.query_end = L.key_end + a.B * a.nq;
   L.mask_dead = reinterpret_cast<uint8_t *>(L.query_end + a.B * a.nk);
   return L;
@@ -151,8 +153,13 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_mask_dead_kernel(const u
   if (lane == 0) dead[m] = votes == ~0ull ? 1 : 0;
 }
 
+__device__ inline int32_t checked_index(const int64_t *table, int64_t at, int64_t n) {
+  const int64_t v = table[at];
+  return (v >= 0 && v < n) ? (int32_t)v : -1;
+}
+
 // one wave per query block row, then one per key block row
-__global__ __launch_bounds__(kBwdThreads) void attn_bwd_live_lists_kernel(bsa_attn_args a) {
+__global__ __launch_bounds__(kBwdThreads) void attn_bwd_records_kernel(bsa_attn_args a) {
   const int64_t w = ((int64_t)blockIdx.x * kBwdThreads + threadIdx.x) >> 6;
   const int64_t qrows = a.B * a.nq, krows = a.B * a.nk;
   if (w >= qrows + krows) return;
@@ -164,7 +171,7 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_live_lists_kernel(bsa_at
   const int64_t b = row / per_batch, mine = row % per_batch;
   const int32_t *offsets = by_key ? a.query_offsets : a.key_offsets;
   const int32_t *indices = by_key ? a.query_indices : a.key_indices;
-  int32_t *out = by_key ? L.query_idx : L.key_idx;
+  BwdRecord *out = by_key ? L.query_rec : L.key_rec;
   const bool causal = a.causal_lengths != nullptr;
   const int64_t seq_len = causal ? a.causal_lengths[b] : 0;
   const int begin = offsets[row], end = offsets[row + 1];
@@ -174,13 +181,30 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_live_lists_kernel(bsa_at
     bool live = e < end;
     const int64_t other = live ? indices[e] : 0;
     const int64_t qb = by_key ? other : mine, kb = by_key ? mine : other;
+    const int64_t pair = (b * a.nq + qb) * a.nk + kb;
     if (live && causal && (kb > qb || qb * kSbs >= seq_len || kb * kSbs >= seq_len)) live = false;
+    int32_t pm = -1;
     if (live && a.mask) {
-      const int64_t pm = a.pidx_mask[(b * a.nq + qb) * a.nk + kb];
-      if (pm >= 0 && pm < a.n_mask_blocks && L.mask_dead[pm]) live = false;
+      pm = checked_index(a.pidx_mask, pair, a.n_mask_blocks);
+      if (pm >= 0 && L.mask_dead[pm]) live = false;
     }
     const unsigned long long votes = __ballot(live);
-    if (live) out[n + __popcll(votes & ((1ull << lane) - 1))] = (int32_t)other;
+    if (live) {
+      BwdRecord r;
+      r.other = (int32_t)other;
+      // what streams past the stationary block: Q and dO of the query block, or K and V of the key block
+      const int64_t orow = by_key ? b * a.nq + qb : b * a.nk + kb;
+      const int64_t *ta = by_key ? a.pidx_q : a.pidx_k, *tb = by_key ? a.pidx_o : a.pidx_v;
+      const int64_t na = by_key ? a.n_q_blocks : a.n_k_blocks, nb = by_key ? a.n_o_blocks : a.n_v_blocks;
+      for (int h = 0; h < 2; ++h) {
+        r.pa[h] = h < a.nh ? checked_index(ta, orow * a.nh + h, na) : -1;
+        r.pb[h] = h < a.nhv ? checked_index(tb, orow * a.nhv + h, nb) : -1;
+      }
+      r.mask = pm;
+      r.bias = a.bias ? checked_index(a.pidx_bias, pair, a.n_bias_blocks) : -1;
+      r.pad = 0;
+      out[n + __popcll(votes & ((1ull << lane) - 1))] = r;
+    }
     n += __popcll(votes);
   }
   if (lane == 0) (by_key ? L.query_end : L.key_end)[row] = n;
@@ -289,37 +313,14 @@ __device__ __forceinline__ void attn_bwd_kv_body(const bsa_attn_args &a, char *s
   }
   const int kpos = (int)kb * kSbs + 32 * wj + li;
 
-  const int q_begin = a.query_offsets[krow];
-  int q_end = a.query_offsets[krow + 1];
-  const int32_t *q_list = a.query_indices;
-  if (a.bwd_scratch != nullptr) {
-    const BwdLists L = bwd_lists(a);
-    q_list = L.query_idx;
-    q_end = L.query_end[krow];
-  }
+  const BwdLists lists = bwd_lists(a);
+  const int q_begin = a.query_offsets[krow], q_end = lists.query_end[krow];
   if (q_begin < q_end) {
-    // lanes 0 .. NH-1: packed Q indices of a query block, next NHV lanes: packed O (= dO) indices, then its mask and
-    // bias block for this key block; lane 7: the list entry at `pos`
-    constexpr int kLaneMask = NH + NHV, kLaneBias = NH + NHV + 1, kLaneEntry = 7;
-    auto gather = [&](int qb, int pos) -> int {
-      const int64_t qrow = b * a.nq + qb;
-      const int32_t *p = q_list + pos;
-      bool on = lane == kLaneEntry;
-      if (lane < NH) {
-        p = low_half_ptr(a.pidx_q, qrow * NH + lane);
-        on = true;
-      } else if (lane < NH + NHV) {
-        p = low_half_ptr(a.pidx_o, qrow * NHV + (lane - NH));
-        on = true;
-      } else if (lane == kLaneMask && a.mask) {
-        p = low_half_ptr(a.pidx_mask, qrow * a.nk + kb);
-        on = true;
-      } else if (lane == kLaneBias && a.bias) {
-        p = low_half_ptr(a.pidx_bias, qrow * a.nk + kb);
-        on = true;
-      }
+    // the record of a list entry, field i in lane i: one 32-byte load, two tiles before the tile is used
+    const int32_t *recs = reinterpret_cast<const int32_t *>(lists.query_rec);
+    auto load_record = [&](int pos) -> int {
       int v = -1;
-      if (on) v = *p;
+      if (lane < 8) v = recs[(int64_t)pos * 8 + lane];
       return v;
     };
     auto clamp_e = [&](int e) { return e < q_end ? e : q_end - 1; };
@@ -328,30 +329,27 @@ __device__ __forceinline__ void attn_bwd_kv_body(const bsa_attn_args &a, char *s
     float stat = 0.f;           // thread t < 64: lse of query t; 64 <= t < 128: delta of query t - 64
     int qb_nxt, pm_nxt, pb_nxt;
 
-    auto fetch = [&](int rec, int qb, int buf) {
+    auto fetch = [&](int rec, int buf) {
+      const int qb = __builtin_amdgcn_readlane(rec, 0);
       qb_nxt = qb;
       char *base = smem + buf * kBufBytes;
 #pragma unroll
       for (int h = 0; h < NH; ++h) {
-        const int64_t pq = __builtin_amdgcn_readlane(rec, h);
-        const bool valid = pq >= 0 && pq < a.n_q_blocks;
-        copy_block<NW>(static_cast<const char *>(a.q) + (valid ? pq : 0) * kBlockBytes, valid,
-                   base + kQRows + h * kBlockBytes, wave, lane, tid);
+        const int pq = __builtin_amdgcn_readlane(rec, 1 + h);
+        copy_block<NW>(static_cast<const char *>(a.q) + (int64_t)(pq >= 0 ? pq : 0) * kBlockBytes, pq >= 0,
+                       base + kQRows + h * kBlockBytes, wave, lane, tid);
       }
 #pragma unroll
       for (int h = 0; h < NHV; ++h) {
-        const int64_t po = __builtin_amdgcn_readlane(rec, NH + h);
-        const bool valid = po >= 0 && po < a.n_o_blocks;
-        copy_block<NW>(static_cast<const char *>(a.d_o) + (valid ? po : 0) * kBlockBytes, valid,
-                   base + kDoRows + h * kBlockBytes, wave, lane, tid);
+        const int po = __builtin_amdgcn_readlane(rec, 3 + h);
+        copy_block<NW>(static_cast<const char *>(a.d_o) + (int64_t)(po >= 0 ? po : 0) * kBlockBytes, po >= 0,
+                       base + kDoRows + h * kBlockBytes, wave, lane, tid);
       }
       const int64_t qrow = b * a.nq + qb;
       if (tid < 64) stat = a.lse[qrow * kSbs + tid];
       else if (tid < 128) stat = a.delta[qrow * kSbs + tid - 64];
-      pm_nxt = __builtin_amdgcn_readlane(rec, kLaneMask);
-      if (pm_nxt >= a.n_mask_blocks) pm_nxt = -1;
-      pb_nxt = __builtin_amdgcn_readlane(rec, kLaneBias);
-      if (pb_nxt >= a.n_bias_blocks) pb_nxt = -1;
+      pm_nxt = __builtin_amdgcn_readlane(rec, 5);
+      pb_nxt = __builtin_amdgcn_readlane(rec, 6);
       // the mask block goes to LDS as it is: wave w copies its rows 16 w .. + 15 (1 KiB)
       if (pm_nxt >= 0 && wave < 4)
         copy_1k_to_lds(static_cast<const char *>(a.mask) + (int64_t)pm_nxt * (kSbs * kSbs) + wave * 1024, lane * 16,
@@ -366,15 +364,12 @@ __device__ __forceinline__ void attn_bwd_kv_body(const bsa_attn_args &a, char *s
       __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     };
 
-    // index pipeline: `rec` holds the indices of query block qb_rec (the entry after the tile in flight) and, in
-    // lane 7, the entry after that
-    int rec, qb_rec;
+    // `rec` is the record of the tile after the one in flight
+    int rec;
     {
-      const int qb0 = first_lane(q_list[as_vector(q_begin)]);
-      const int rec0 = gather(qb0, clamp_e(q_begin + 1));
-      qb_rec = __builtin_amdgcn_readlane(rec0, kLaneEntry);
-      rec = gather(qb_rec, clamp_e(q_begin + 2));
-      fetch(rec0, qb0, 0);
+      const int rec0 = load_record(q_begin);
+      rec = load_record(clamp_e(q_begin + 1));
+      fetch(rec0, 0);
       stage(0);
       __syncthreads();
     }
@@ -394,9 +389,8 @@ __device__ __forceinline__ void attn_bwd_kv_body(const bsa_attn_args &a, char *s
         for (int r = 0; r < 16; ++r) mbits |= (uint32_t)mp[(8 * (r >> 2) + (r & 3)) * kSbs] << r;
       }
       const bool more = e + 1 < q_end;
-      if (more) fetch(rec, qb_rec, buf ^ 1);
-      qb_rec = __builtin_amdgcn_readlane(rec, kLaneEntry);
-      rec = gather(qb_rec, clamp_e(e + 3));
+      if (more) fetch(rec, buf ^ 1);
+      rec = load_record(clamp_e(e + 2));
 
       // A quadrant whose every score is masked has P = dS = 0: nothing to add, nothing to compute.
       bool live = true;
@@ -624,35 +618,14 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_q_kernel(bsa_attn_arg
   }
   const int qpos = (int)qb * kSbs + qi;
 
-  const int k_begin = a.key_offsets[qrow];
-  int k_end = a.key_offsets[qrow + 1];
-  const int32_t *k_list = a.key_indices;
-  if (a.bwd_scratch != nullptr) {
-    const BwdLists L = bwd_lists(a);
-    k_list = L.key_idx;
-    k_end = L.key_end[qrow];
-  }
+  const BwdLists lists = bwd_lists(a);
+  const int k_begin = a.key_offsets[qrow], k_end = lists.key_end[qrow];
   if (k_begin < k_end) {
-    constexpr int kLaneMask = NH + NHV, kLaneBias = NH + NHV + 1, kLaneEntry = 7;
-    auto gather = [&](int kb, int pos) -> int {
-      const int64_t krow = b * a.nk + kb;
-      const int32_t *p = k_list + pos;
-      bool on = lane == kLaneEntry;
-      if (lane < NH) {
-        p = low_half_ptr(a.pidx_k, krow * NH + lane);
-        on = true;
-      } else if (lane < NH + NHV) {
-        p = low_half_ptr(a.pidx_v, krow * NHV + (lane - NH));
-        on = true;
-      } else if (lane == kLaneMask && a.mask) {
-        p = low_half_ptr(a.pidx_mask, qrow * a.nk + kb);
-        on = true;
-      } else if (lane == kLaneBias && a.bias) {
-        p = low_half_ptr(a.pidx_bias, qrow * a.nk + kb);
-        on = true;
-      }
+    // the record of a list entry, field i in lane i: one 32-byte load, two tiles before the tile is used
+    const int32_t *recs = reinterpret_cast<const int32_t *>(lists.key_rec);
+    auto load_record = [&](int pos) -> int {
       int v = -1;
-      if (on) v = *p;
+      if (lane < 8) v = recs[(int64_t)pos * 8 + lane];
       return v;
     };
     auto clamp_e = [&](int e) { return e < k_end ? e : k_end - 1; };
@@ -661,27 +634,23 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_q_kernel(bsa_attn_arg
     u32x2 bias_w[4];     // bias elements likewise
     int kb_nxt, pm_nxt, pb_nxt;
 
-    auto fetch = [&](int rec, int kb, int buf) {
-      kb_nxt = kb;
+    auto fetch = [&](int rec, int buf) {
+      kb_nxt = __builtin_amdgcn_readlane(rec, 0);
       char *base = smem + buf * kBufBytes;
 #pragma unroll
       for (int h = 0; h < NH; ++h) {
-        const int64_t pk = __builtin_amdgcn_readlane(rec, h);
-        const bool valid = pk >= 0 && pk < a.n_k_blocks;
-        copy_block(static_cast<const char *>(a.k) + (valid ? pk : 0) * kBlockBytes, valid,
+        const int pk = __builtin_amdgcn_readlane(rec, 1 + h);
+        copy_block(static_cast<const char *>(a.k) + (int64_t)(pk >= 0 ? pk : 0) * kBlockBytes, pk >= 0,
                    base + kKRows + h * kBlockBytes, wave, lane, tid);
       }
 #pragma unroll
       for (int h = 0; h < NHV; ++h) {
-        const int64_t pv = __builtin_amdgcn_readlane(rec, NH + h);
-        const bool valid = pv >= 0 && pv < a.n_v_blocks;
-        copy_block(static_cast<const char *>(a.v) + (valid ? pv : 0) * kBlockBytes, valid,
+        const int pv = __builtin_amdgcn_readlane(rec, 3 + h);
+        copy_block(static_cast<const char *>(a.v) + (int64_t)(pv >= 0 ? pv : 0) * kBlockBytes, pv >= 0,
                    base + kVRows + h * kBlockBytes, wave, lane, tid);
       }
-      pm_nxt = __builtin_amdgcn_readlane(rec, kLaneMask);
-      if (pm_nxt >= a.n_mask_blocks) pm_nxt = -1;
-      pb_nxt = __builtin_amdgcn_readlane(rec, kLaneBias);
-      if (pb_nxt >= a.n_bias_blocks) pb_nxt = -1;
+      pm_nxt = __builtin_amdgcn_readlane(rec, 5);
+      pb_nxt = __builtin_amdgcn_readlane(rec, 6);
       if (pm_nxt >= 0) {
         const char *mp = static_cast<const char *>(a.mask) + (int64_t)pm_nxt * (kSbs * kSbs);
         const uint32_t off = (uint32_t)qi * 64u + 32u * wj + 4u * kg;
@@ -698,13 +667,11 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_q_kernel(bsa_attn_arg
     // every copy of this wave has to have landed before the barrier
     auto stage = [&](int) { __builtin_amdgcn_s_waitcnt(0x0F70); };
 
-    int rec, kb_rec;
+    int rec;
     {
-      const int kb0 = first_lane(k_list[as_vector(k_begin)]);
-      const int rec0 = gather(kb0, clamp_e(k_begin + 1));
-      kb_rec = __builtin_amdgcn_readlane(rec0, kLaneEntry);
-      rec = gather(kb_rec, clamp_e(k_begin + 2));
-      fetch(rec0, kb0, 0);
+      const int rec0 = load_record(k_begin);
+      rec = load_record(clamp_e(k_begin + 1));
+      fetch(rec0, 0);
       stage(0);
       __syncthreads();
     }
@@ -723,9 +690,8 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_q_kernel(bsa_attn_arg
         for (int q = 0; q < 4; ++q) bias_c[q] = bias_w[q];
       }
       const bool more = e + 1 < k_end;
-      if (more) fetch(rec, kb_rec, buf ^ 1);
-      kb_rec = __builtin_amdgcn_readlane(rec, kLaneEntry);
-      rec = gather(kb_rec, clamp_e(e + 3));
+      if (more) fetch(rec, buf ^ 1);
+      rec = load_record(clamp_e(e + 2));
 
       bool live = true;
       if (pm >= 0) live = !__all((mask_c[0] & mask_c[1] & mask_c[2] & mask_c[3]) == 0x01010101u);
@@ -841,15 +807,15 @@ int launch_bwd(const bsa_attn_args &a, hipStream_t s) {
     fill_zero_f32_kernel<<<(unsigned)blocks, 256, 0, s>>>(a.dbias, n);
     if (int rc = check_launch("fill_zero_f32_kernel")) return rc;
   }
-  if (a.bwd_scratch != nullptr && qrows + krows > 0) {
+  if (qrows + krows > 0) {
     const BwdLists L = bwd_lists(a);
     if (a.mask != nullptr && a.n_mask_blocks > 0) {
       attn_bwd_mask_dead_kernel<<<(unsigned)cdiv(a.n_mask_blocks, 4), kBwdThreads, 0, s>>>(
           static_cast<const u32x4 *>(a.mask), L.mask_dead, a.n_mask_blocks);
       if (int rc = check_launch("attn_bwd_mask_dead_kernel")) return rc;
     }
-    attn_bwd_live_lists_kernel<<<(unsigned)cdiv(qrows + krows, 4), kBwdThreads, 0, s>>>(a);
-    if (int rc = check_launch("attn_bwd_live_lists_kernel")) return rc;
+    attn_bwd_records_kernel<<<(unsigned)cdiv(qrows + krows, 4), kBwdThreads, 0, s>>>(a);
+    if (int rc = check_launch("attn_bwd_records_kernel")) return rc;
   }
   if (qrows > 0) {
     attn_bwd_delta_kernel<Tr><<<(unsigned)qrows, kBwdThreads, 0, s>>>(a);
@@ -901,13 +867,14 @@ int dispatch_bwd(const bsa_attn_args &a, hipStream_t s) {
 }  // namespace
 
 size_t attn_bwd_scratch_bytes(int64_t B, int64_t nq, int64_t nk, int64_t n_layout_blocks, int64_t n_mask_blocks) {
-  const size_t bytes = 4 * (size_t)(2 * n_layout_blocks + B * nq + B * nk) + (size_t)n_mask_blocks;
+  const size_t bytes = 2 * sizeof(BwdRecord) * (size_t)n_layout_blocks + 4 * (size_t)(B * nq + B * nk) + (size_t)n_mask_blocks;
   return (bytes + 15) & ~(size_t)15;
 }
 
 int attn_bwd_mfma(const bsa_attn_args &a, hipStream_t s) {
   if (a.sbs != kSbs || (a.dtype != BSA_BF16 && a.dtype != BSA_F16)) return 1;
   if ((a.B * a.nq > 0 && a.key_indices == nullptr) || (a.B * a.nk > 0 && a.query_indices == nullptr)) return 1;
+  if (a.bwd_scratch == nullptr) return 1;  // the matrix-core kernels walk the records built in the scratch
   return a.dtype == BSA_BF16 ? dispatch_bwd<MBf16>(a, s) : dispatch_bwd<MF16>(a, s);
 }
 

@@ -319,14 +319,12 @@ class _FlashAttention(torch.autograd.Function):
         args = _fill_args(meta, q, k, v, bias)
         args.o, args.d_o, args.lse, args.delta = _capi.ptr(out), _capi.ptr(grad_output), _capi.ptr(lse), _capi.ptr(delta)
         args.dq, args.dk, args.dv, args.dbias = _capi.ptr(dq), _capi.ptr(dk), _capi.ptr(dv), _capi.ptr(dbias)
-        scratch = None
-        if meta.mask is not None or meta.causal_lengths is not None:
-            # room for the lists of the pairs that some score survives (built and used inside bsa_attn_bwd)
-            n_layout_blocks = meta.cache["key_indices_i32"].numel()
-            n_mask_blocks = meta.mask.size(0) if meta.mask is not None else 0
-            size = _capi.load().bsa_attn_bwd_scratch_bytes(B, nq, nk, n_layout_blocks, n_mask_blocks)
-            scratch = torch.empty(max(size, 16), dtype=torch.uint8, device=q.device)
-            args.bwd_scratch, args.n_layout_blocks = scratch.data_ptr(), n_layout_blocks
+        # room for the records of the pairs that some score survives (built and used inside bsa_attn_bwd)
+        n_layout_blocks = meta.cache["key_indices_i32"].numel()
+        n_mask_blocks = meta.mask.size(0) if meta.mask is not None else 0
+        size = _capi.load().bsa_attn_bwd_scratch_bytes(B, nq, nk, n_layout_blocks, n_mask_blocks)
+        scratch = torch.empty(max(size, 16), dtype=torch.uint8, device=q.device)
+        args.bwd_scratch, args.n_layout_blocks = scratch.data_ptr(), n_layout_blocks
         with torch.cuda.device(q.device):
             _capi.call("bsa_attn_bwd", ctypes.byref(args), _capi.stream(q.device))
         grad_bias = dbias.to(bias.dtype) if meta.has_bias else None

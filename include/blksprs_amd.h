@@ -282,10 +282,10 @@ typedef struct bsa_attn_args {
    * of a pair.  No counterpart in the reference. */
   const int32_t *group_offsets, *group_records;
   int32_t group_size;
-  /* Optional, backward only (NULL: every pair of the attention layout is visited).  Scratch of
-   * bsa_attn_bwd_scratch_bytes(...) bytes in which bsa_attn_bwd first lists, per query block and per key block,
-   * the pairs that some score survives (a pair whose mask block masks everything, or that the causal predicate
-   * rules out as a whole, adds nothing to any gradient and is then neither fetched nor computed).
+  /* Backward only.  Scratch of bsa_attn_bwd_scratch_bytes(...) bytes in which bsa_attn_bwd first writes, per query
+   * block and per key block, one record for every pair that some score survives (a pair whose mask block masks
+   * everything, or that the causal predicate rules out as a whole, adds nothing to any gradient and is then
+   * neither fetched nor computed); the matrix-core kernels walk those records.  NULL: the generic kernels run.
    * n_layout_blocks = number of active blocks of the attention layout (= key_offsets[B * nq]).
    * No counterpart in the reference, which visits every pair (blksprs/ops/flash_attention.py:1322-1330). */
   void *bwd_scratch;
