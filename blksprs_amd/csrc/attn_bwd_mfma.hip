@@ -79,6 +79,24 @@ __device__ inline void load_resident(u32x4 (&f)[4], const void *base, int64_t pi
   }
 }
 
+// A run of matrix-core products whose A operands come from LDS, four fragments to a stage: the reads of stage
+// k + 1 are issued before the products of stage k, so that a read's latency is paid behind four products and not
+// in front of each one.  `load(k, f)` fills the four fragments of stage k, `multiply(k, f)` consumes them.  The
+// empty statement that names a fragment keeps its read from sinking to its use.
+template <int K, typename Load, typename Multiply>
+__device__ __forceinline__ void staged_products(Load load, Multiply multiply) {
+  u32x4 f[2][4];
+  load(0, f[0]);
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    if (k + 1 < K) load(k + 1, f[(k + 1) & 1]);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(f[k & 1][i]));
+    multiply(k, f[k & 1]);
+  }
+}
+
 // XCD-aware row of a workgroup: every XCD gets a contiguous range of rows, so that the blocks in flight on one
 // L2 belong to the same batch entries
 __device__ inline int64_t xcd_row() { return (int64_t)(blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3); }
@@ -404,18 +422,19 @@ __device__ __forceinline__ void attn_bwd_kv_body(const bsa_attn_args &a, char *s
         f32x16 sacc, dpacc;
   #pragma unroll
         for (int r = 0; r < 16; ++r) sacc[r] = dpacc[r] = 0.f;
+        staged_products<NH + (DK ? NHV : 0)>(
+            [&](int k, u32x4(&f)[4]) {
+              const char *src = base + (k < NH ? kQRows + k * kBlockBytes : kDoRows + (k - NH) * kBlockBytes);
   #pragma unroll
-        for (int h = 0; h < NH; ++h)
+              for (int s = 0; s < 4; ++s) f[s] = frag_rows(src, 32 * wi + li, 2 * s + kg);
+            },
+            [&](int k, u32x4(&f)[4]) {
   #pragma unroll
-          for (int s = 0; s < 4; ++s)
-            sacc = Tr::mfma(frag_rows(base + kQRows + h * kBlockBytes, 32 * wi + li, 2 * s + kg), kfr[h][s], sacc);
-        if constexpr (DK) {
-  #pragma unroll
-          for (int h = 0; h < NHV; ++h)
-  #pragma unroll
-            for (int s = 0; s < 4; ++s)
-              dpacc = Tr::mfma(frag_rows(base + kDoRows + h * kBlockBytes, 32 * wi + li, 2 * s + kg), vfr[h][s], dpacc);
-        }
+              for (int s = 0; s < 4; ++s) {
+                if (k < NH) sacc = Tr::mfma(f[s], kfr[k < NH ? k : 0][s], sacc);
+                else dpacc = Tr::mfma(f[s], vfr[k < NH ? 0 : k - NH][s], dpacc);
+              }
+            });
 
         // ---- P and dS; element r: query 32 wi + 8 (r / 4) + 4 kg + r % 4 ----
         const float *stats = reinterpret_cast<const float *>(base + kStats);
@@ -478,27 +497,30 @@ __device__ __forceinline__ void attn_bwd_kv_body(const bsa_attn_args &a, char *s
           }
 
         // ---- dV^T += dO^T P, dK^T += Q^T dS over this wave's 32 queries ----
+        const int col_t = 16 * ((lane >> 4) & 1);
         if constexpr (DV) {
+          staged_products<NHV>(
+              [&](int h, u32x4(&f)[4]) {
   #pragma unroll
-        for (int h = 0; h < NHV; ++h)
+                for (int i = 0; i < 4; ++i)
+                  f[i] = frag_cols_t(base + kDoRows + h * kBlockBytes, 32 * wi + 16 * (i & 1) + 4 * kg, 32 * (i >> 1) + col_t, lane);
+              },
+              [&](int h, u32x4(&f)[4]) {
   #pragma unroll
-          for (int db = 0; db < 2; ++db)
-  #pragma unroll
-            for (int u = 0; u < 2; ++u)
-              dvacc[2 * h + db] = Tr::mfma(frag_cols_t(base + kDoRows + h * kBlockBytes, 32 * wi + 16 * u + 4 * kg,
-                                                       32 * db + 16 * ((lane >> 4) & 1), lane),
-                                           pf[u], dvacc[2 * h + db]);
+                for (int i = 0; i < 4; ++i) dvacc[2 * h + (i >> 1)] = Tr::mfma(f[i], pf[i & 1], dvacc[2 * h + (i >> 1)]);
+              });
         }
         if constexpr (DK) {
+          staged_products<NH>(
+              [&](int h, u32x4(&f)[4]) {
   #pragma unroll
-        for (int h = 0; h < NH; ++h)
+                for (int i = 0; i < 4; ++i)
+                  f[i] = frag_cols_t(base + kQRows + h * kBlockBytes, 32 * wi + 16 * (i & 1) + 4 * kg, 32 * (i >> 1) + col_t, lane);
+              },
+              [&](int h, u32x4(&f)[4]) {
   #pragma unroll
-          for (int db = 0; db < 2; ++db)
-  #pragma unroll
-            for (int u = 0; u < 2; ++u)
-              dkacc[2 * h + db] = Tr::mfma(frag_cols_t(base + kQRows + h * kBlockBytes, 32 * wi + 16 * u + 4 * kg,
-                                                       32 * db + 16 * ((lane >> 4) & 1), lane),
-                                           dsf[u], dkacc[2 * h + db]);
+                for (int i = 0; i < 4; ++i) dkacc[2 * h + (i >> 1)] = Tr::mfma(f[i], dsf[i & 1], dkacc[2 * h + (i >> 1)]);
+              });
         }
       }  // live
 
@@ -704,16 +726,19 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_q_kernel(bsa_attn_arg
         f32x16 sacc, dpacc;
   #pragma unroll
         for (int r = 0; r < 16; ++r) sacc[r] = dpacc[r] = 0.f;
+        staged_products<NH + NHV>(
+            [&](int k, u32x4(&f)[4]) {
+              const char *src = base + (k < NH ? kKRows + k * kBlockBytes : kVRows + (k - NH) * kBlockBytes);
   #pragma unroll
-        for (int h = 0; h < NH; ++h)
+              for (int s = 0; s < 4; ++s) f[s] = frag_rows(src, 32 * wj + li, 2 * s + kg);
+            },
+            [&](int k, u32x4(&f)[4]) {
   #pragma unroll
-          for (int s = 0; s < 4; ++s)
-            sacc = Tr::mfma(frag_rows(base + kKRows + h * kBlockBytes, 32 * wj + li, 2 * s + kg), qfr[h][s], sacc);
-  #pragma unroll
-        for (int h = 0; h < NHV; ++h)
-  #pragma unroll
-          for (int s = 0; s < 4; ++s)
-            dpacc = Tr::mfma(frag_rows(base + kVRows + h * kBlockBytes, 32 * wj + li, 2 * s + kg), dofr[h][s], dpacc);
+              for (int s = 0; s < 4; ++s) {
+                if (k < NH) sacc = Tr::mfma(f[s], qfr[k < NH ? k : 0][s], sacc);
+                else dpacc = Tr::mfma(f[s], dofr[k < NH ? 0 : k - NH][s], dpacc);
+              }
+            });
 
         float ds[16];
         // the plain path: no bias, no mask block, causal predicate true for every score of the quadrant
@@ -754,15 +779,17 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_q_kernel(bsa_attn_arg
           for (int t = 0; t < 4; ++t) dsf[u][t] = Tr::pack2(ds[8 * u + 2 * t], ds[8 * u + 2 * t + 1]);
 
         // ---- dQ^T += K^T dS^T over this wave's 32 keys ----
+        const int col_t = 16 * ((lane >> 4) & 1);
+        staged_products<NH>(
+            [&](int h, u32x4(&f)[4]) {
   #pragma unroll
-        for (int h = 0; h < NH; ++h)
+              for (int i = 0; i < 4; ++i)
+                f[i] = frag_cols_t(base + kKRows + h * kBlockBytes, 32 * wj + 16 * (i & 1) + 4 * kg, 32 * (i >> 1) + col_t, lane);
+            },
+            [&](int h, u32x4(&f)[4]) {
   #pragma unroll
-          for (int db = 0; db < 2; ++db)
-  #pragma unroll
-            for (int u = 0; u < 2; ++u)
-              dqacc[2 * h + db] = Tr::mfma(frag_cols_t(base + kKRows + h * kBlockBytes, 32 * wj + 16 * u + 4 * kg,
-                                                       32 * db + 16 * ((lane >> 4) & 1), lane),
-                                           dsf[u], dqacc[2 * h + db]);
+              for (int i = 0; i < 4; ++i) dqacc[2 * h + (i >> 1)] = Tr::mfma(f[i], dsf[i & 1], dqacc[2 * h + (i >> 1)]);
+            });
 
       }  // live
 
