@@ -142,6 +142,7 @@ static_assert(sizeof(BwdRecord) == 32, "one record is eight int32");
 struct BwdLists {
   BwdRecord *key_rec, *query_rec;  // [n_layout_blocks] each, rows at the offsets of key_offsets / query_offsets
   int32_t *key_end, *query_end;    // [B * nq], [B * nk]: end of the live part of a row's list
+  int32_t *q_order, *k_order;      // [B * nq], [B * nk]: the order in which rows are handed to workgroups
   uint8_t *mask_dead;              // [n_mask_blocks]
 };
 
@@ -151,7 +152,9 @@ __host__ __device__ inline BwdLists bwd_lists(const bsa_attn_args &a) {
   L.query_rec = L.key_rec + a.n_layout_blocks;
   L.key_end = reinterpret_cast<int32_t *>(L.query_rec + a.n_layout_blocks);
   L.query_end = L.key_end + a.B * a.nq;
-  L.mask_dead = reinterpret_cast<uint8_t *>(L.query_end + a.B * a.nk);
+  L.q_order = L.query_end + a.B * a.nk;
+  L.k_order = L.q_order + a.B * a.nq;
+  L.mask_dead = reinterpret_cast<uint8_t *>(L.k_order + a.B * a.nk);
   return L;
 }
 
@@ -228,6 +231,58 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_records_kernel(bsa_attn_
   if (lane == 0) (by_key ? L.query_end : L.key_end)[row] = n;
 }
 
+// Workgroup g of a main kernel runs on XCD g % 8, and every XCD is given a contiguous eighth of the rows, so that
+// the blocks in flight on one L2 belong to the same batch entries.  Inside its eighth an XCD takes the rows with
+// the most live pairs first when its longest row has more than four times the mean (a row that every query
+// attends to can be a hundred times longer than the others and must not be the last to start).  Workgroups 0 .. 7 order the query rows, 8 .. 15 the key rows, by a
+// counting sort on min(pairs, 255); rows of equal count come in no fixed order, which changes no result.
+__global__ __launch_bounds__(kBwdThreads) void attn_bwd_order_kernel(bsa_attn_args a) {
+  __shared__ int bins[256];
+  const BwdLists L = bwd_lists(a);
+  const bool by_key = blockIdx.x >= 8;
+  const int64_t rows = by_key ? a.B * a.nk : a.B * a.nq;
+  const int32_t *offsets = by_key ? a.query_offsets : a.key_offsets;
+  const int32_t *ends = by_key ? L.query_end : L.key_end;
+  int32_t *order = by_key ? L.k_order : L.q_order;
+  const int64_t chunk = (rows + 7) / 8;  // = gridDim.x / 8 of the main kernels
+  const int64_t r0 = (int64_t)(blockIdx.x & 7) * chunk, r1 = r0 + chunk < rows ? r0 + chunk : rows;
+  const int tid = threadIdx.x;
+  __shared__ int longest;
+  __shared__ unsigned long long total;
+  bins[tid] = 0;
+  if (tid == 0) {
+    longest = 0;
+    total = 0;
+  }
+  __syncthreads();
+  auto bin_of = [&](int64_t r) {
+    const int n = ends[r] - offsets[r];
+    return 255 - (n < 255 ? n : 255);
+  };
+  for (int64_t r = r0 + tid; r < r1; r += kBwdThreads) {
+    const int n = ends[r] - offsets[r];
+    atomicAdd(&bins[bin_of(r)], 1);
+    atomicMax(&longest, n);
+    atomicAdd(&total, (unsigned long long)n);
+  }
+  __syncthreads();
+  // rows of similar length stay in their natural order, which keeps neighbours (who share blocks) together
+  if ((unsigned long long)longest * (unsigned long long)(r1 - r0) <= 4ull * total) {
+    for (int64_t r = r0 + tid; r < r1; r += kBwdThreads) order[r] = (int32_t)r;
+    return;
+  }
+  if (tid == 0) {
+    int at = 0;
+    for (int i = 0; i < 256; ++i) {
+      const int n = bins[i];
+      bins[i] = at;
+      at += n;
+    }
+  }
+  __syncthreads();
+  for (int64_t r = r0 + tid; r < r1; r += kBwdThreads) order[r0 + atomicAdd(&bins[bin_of(r)], 1)] = (int32_t)r;
+}
+
 // ---------------------------------------------------------------------------------------------------------
 // delta[b, qb, i] = sum over active output slices of rowsum(o * dO); four lanes per query row
 template <typename Tr>
@@ -278,8 +333,9 @@ __device__ __forceinline__ void attn_bwd_kv_body(const bsa_attn_args &a, char *s
   const int tid = threadIdx.x, lane = tid & 63;
   const int li = lane & 31, kg = lane >> 5;
   const int wi = quad & 1, wj = quad >> 1;  // query half and key half of this wave's quadrant
-  const int64_t krow = xcd_row();
-  if (krow >= a.B * a.nk) return;
+  const int64_t kpos_in_order = xcd_row();
+  if (kpos_in_order >= a.B * a.nk) return;
+  const int64_t krow = bwd_lists(a).k_order[kpos_in_order];
   const int64_t b = krow / a.nk, kb = krow % a.nk;
 
   int64_t pk[NH], pv[NHV];
@@ -599,8 +655,9 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_q_kernel(bsa_attn_arg
   const int wave = first_lane(tid >> 6);
   const int li = lane & 31, kg = lane >> 5;
   const int wi = wave & 1, wj = wave >> 1;
-  const int64_t qrow = xcd_row();
-  if (qrow >= a.B * a.nq) return;
+  const int64_t qpos_in_order = xcd_row();
+  if (qpos_in_order >= a.B * a.nq) return;
+  const int64_t qrow = bwd_lists(a).q_order[qpos_in_order];
   const int64_t b = qrow / a.nq, qb = qrow % a.nq;
 
   int64_t pq[NH];
@@ -843,6 +900,8 @@ int launch_bwd(const bsa_attn_args &a, hipStream_t s) {
     }
     attn_bwd_records_kernel<<<(unsigned)cdiv(qrows + krows, 4), kBwdThreads, 0, s>>>(a);
     if (int rc = check_launch("attn_bwd_records_kernel")) return rc;
+    attn_bwd_order_kernel<<<16, kBwdThreads, 0, s>>>(a);
+    if (int rc = check_launch("attn_bwd_order_kernel")) return rc;
   }
   if (qrows > 0) {
     attn_bwd_delta_kernel<Tr><<<(unsigned)qrows, kBwdThreads, 0, s>>>(a);
@@ -894,7 +953,7 @@ int dispatch_bwd(const bsa_attn_args &a, hipStream_t s) {
 }  // namespace
 
 size_t attn_bwd_scratch_bytes(int64_t B, int64_t nq, int64_t nk, int64_t n_layout_blocks, int64_t n_mask_blocks) {
-  const size_t bytes = 2 * sizeof(BwdRecord) * (size_t)n_layout_blocks + 4 * (size_t)(B * nq + B * nk) + (size_t)n_mask_blocks;
+  const size_t bytes = 2 * sizeof(BwdRecord) * (size_t)n_layout_blocks + 8 * (size_t)(B * nq + B * nk) + (size_t)n_mask_blocks;
   return (bytes + 15) & ~(size_t)15;
 }
 
