@@ -142,7 +142,12 @@ static_assert(sizeof(BwdRecord) == 32, "one record is eight int32");
 struct BwdLists {
   BwdRecord *key_rec, *query_rec;  // [n_layout_blocks] each, rows at the offsets of key_offsets / query_offsets
   int32_t *key_end, *query_end;    // [B * nq], [B * nk]: end of the live part of a row's list
-  int32_t *q_order, *k_order;      // [B * nq], [B * nk]: the order in which rows are handed to workgroups
+  // [B * nq][16], [B * nk][16]: one 64-byte header per workgroup of the dQ resp. dK / dV kernel, in the order in
+  // which rows are handed out: ints 0 .. 7 the first record of the row's list, 8 the row, 9 and 10 the bounds of
+  // its live list, 11 .. 12 and 13 .. 14 the packed indices of the stationary block's slices (Q and O for a
+  // query row, K and V for a key row; -1: none).  Everything a workgroup has to know before its first tile
+  // comes with one load.
+  int32_t *q_head, *k_head;
   uint8_t *mask_dead;              // [n_mask_blocks]
 };
 
@@ -152,9 +157,9 @@ __host__ __device__ inline BwdLists bwd_lists(const bsa_attn_args &a) {
   L.query_rec = L.key_rec + a.n_layout_blocks;
   L.key_end = reinterpret_cast<int32_t *>(L.query_rec + a.n_layout_blocks);
   L.query_end = L.key_end + a.B * a.nq;
-  L.q_order = L.query_end + a.B * a.nk;
-  L.k_order = L.q_order + a.B * a.nq;
-  L.mask_dead = reinterpret_cast<uint8_t *>(L.k_order + a.B * a.nk);
+  L.q_head = L.query_end + a.B * a.nk;
+  L.k_head = L.q_head + 16 * a.B * a.nq;
+  L.mask_dead = reinterpret_cast<uint8_t *>(L.k_head + 16 * a.B * a.nk);
   return L;
 }
 
@@ -235,21 +240,40 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_records_kernel(bsa_attn_
 // the blocks in flight on one L2 belong to the same batch entries.  Inside its eighth an XCD takes the rows with
 // the most live pairs first when its longest row has more than four times the mean (a row that every query
 // attends to can be a hundred times longer than the others and must not be the last to start).  Workgroups 0 .. 7 order the query rows, 8 .. 15 the key rows, by a
-// counting sort on min(pairs, 255); rows of equal count come in no fixed order, which changes no result.
-__global__ __launch_bounds__(kBwdThreads) void attn_bwd_order_kernel(bsa_attn_args a) {
+// counting sort on min(pairs, 255); rows of equal count come in no fixed order, which changes no result.  What
+// is written per position is the 64-byte header of the workgroup that takes it.
+constexpr int kOrderThreads = 1024;
+__global__ __launch_bounds__(kOrderThreads) void attn_bwd_order_kernel(bsa_attn_args a) {
   __shared__ int bins[256];
   const BwdLists L = bwd_lists(a);
   const bool by_key = blockIdx.x >= 8;
   const int64_t rows = by_key ? a.B * a.nk : a.B * a.nq;
   const int32_t *offsets = by_key ? a.query_offsets : a.key_offsets;
   const int32_t *ends = by_key ? L.query_end : L.key_end;
-  int32_t *order = by_key ? L.k_order : L.q_order;
+  int32_t *heads = by_key ? L.k_head : L.q_head;
+  const BwdRecord *recs = by_key ? L.query_rec : L.key_rec;
+  const int64_t *ta = by_key ? a.pidx_k : a.pidx_q, *tb = by_key ? a.pidx_v : a.pidx_o;
+  const int64_t na = by_key ? a.n_k_blocks : a.n_q_blocks, nb = by_key ? a.n_v_blocks : a.n_o_blocks;
+  auto emit = [&](int64_t pos, int64_t r) {
+    int32_t *h = heads + pos * 16;
+    const int begin = offsets[r], end = ends[r];
+    const int32_t *first = reinterpret_cast<const int32_t *>(recs + begin);
+    for (int i = 0; i < 8; ++i) h[i] = begin < end ? first[i] : -1;
+    h[8] = (int32_t)r;
+    h[9] = begin;
+    h[10] = end;
+    for (int s = 0; s < 2; ++s) {
+      h[11 + s] = s < a.nh ? checked_index(ta, r * a.nh + s, na) : -1;
+      h[13 + s] = s < a.nhv ? checked_index(tb, r * a.nhv + s, nb) : -1;
+    }
+    h[15] = 0;
+  };
   const int64_t chunk = (rows + 7) / 8;  // = gridDim.x / 8 of the main kernels
   const int64_t r0 = (int64_t)(blockIdx.x & 7) * chunk, r1 = r0 + chunk < rows ? r0 + chunk : rows;
   const int tid = threadIdx.x;
   __shared__ int longest;
   __shared__ unsigned long long total;
-  bins[tid] = 0;
+  if (tid < 256) bins[tid] = 0;
   if (tid == 0) {
     longest = 0;
     total = 0;
@@ -259,7 +283,7 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_order_kernel(bsa_attn_ar
     const int n = ends[r] - offsets[r];
     return 255 - (n < 255 ? n : 255);
   };
-  for (int64_t r = r0 + tid; r < r1; r += kBwdThreads) {
+  for (int64_t r = r0 + tid; r < r1; r += kOrderThreads) {
     const int n = ends[r] - offsets[r];
     atomicAdd(&bins[bin_of(r)], 1);
     atomicMax(&longest, n);
@@ -268,19 +292,17 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_order_kernel(bsa_attn_ar
   __syncthreads();
   // rows of similar length stay in their natural order, which keeps neighbours (who share blocks) together
   if ((unsigned long long)longest * (unsigned long long)(r1 - r0) <= 4ull * total) {
-    for (int64_t r = r0 + tid; r < r1; r += kBwdThreads) order[r] = (int32_t)r;
+    for (int64_t r = r0 + tid; r < r1; r += kOrderThreads) emit(r, r);
     return;
   }
-  if (tid == 0) {
-    int at = 0;
-    for (int i = 0; i < 256; ++i) {
-      const int n = bins[i];
-      bins[i] = at;
-      at += n;
-    }
-  }
+  // exclusive prefix sum of the 256 bins: thread t adds up the bins before its own
+  int before = 0;
+  if (tid < 256)
+    for (int i = 0; i < tid; ++i) before += bins[i];
   __syncthreads();
-  for (int64_t r = r0 + tid; r < r1; r += kBwdThreads) order[r0 + atomicAdd(&bins[bin_of(r)], 1)] = (int32_t)r;
+  if (tid < 256) bins[tid] = before;
+  __syncthreads();
+  for (int64_t r = r0 + tid; r < r1; r += kOrderThreads) emit(r0 + atomicAdd(&bins[bin_of(r)], 1), r);
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -335,21 +357,23 @@ __device__ __forceinline__ void attn_bwd_kv_body(const bsa_attn_args &a, char *s
   const int wi = quad & 1, wj = quad >> 1;  // query half and key half of this wave's quadrant
   const int64_t kpos_in_order = xcd_row();
   if (kpos_in_order >= a.B * a.nk) return;
-  const int64_t krow = bwd_lists(a).k_order[kpos_in_order];
+  const BwdLists lists = bwd_lists(a);
+  // the workgroup's header, int i in lane i (lanes 0 .. 7 double as the record of the first tile)
+  int head = -1;
+  if (lane < 16) head = lists.k_head[kpos_in_order * 16 + lane];
+  const int64_t krow = __builtin_amdgcn_readlane(head, 8);
   const int64_t b = krow / a.nk, kb = krow % a.nk;
 
   int64_t pk[NH], pv[NHV];
   bool any = (DK || JOINT) && a.dbias != nullptr;
 #pragma unroll
   for (int h = 0; h < NH; ++h) {
-    pk[h] = a.pidx_k[krow * NH + h];
-    if (pk[h] >= a.n_k_blocks) pk[h] = -1;
+    pk[h] = __builtin_amdgcn_readlane(head, 11 + h);
     any = any || ((DK || JOINT) && pk[h] >= 0);
   }
 #pragma unroll
   for (int h = 0; h < NHV; ++h) {
-    pv[h] = a.pidx_v[krow * NHV + h];
-    if (pv[h] >= a.n_v_blocks) pv[h] = -1;
+    pv[h] = __builtin_amdgcn_readlane(head, 13 + h);
     any = any || ((DV || JOINT) && pv[h] >= 0);
   }
   if (!any) return;
@@ -387,8 +411,7 @@ __device__ __forceinline__ void attn_bwd_kv_body(const bsa_attn_args &a, char *s
   }
   const int kpos = (int)kb * kSbs + 32 * wj + li;
 
-  const BwdLists lists = bwd_lists(a);
-  const int q_begin = a.query_offsets[krow], q_end = lists.query_end[krow];
+  const int q_begin = __builtin_amdgcn_readlane(head, 9), q_end = __builtin_amdgcn_readlane(head, 10);
   if (q_begin < q_end) {
     // the record of a list entry, field i in lane i: one 32-byte load, two tiles before the tile is used
     const int32_t *recs = reinterpret_cast<const int32_t *>(lists.query_rec);
@@ -441,9 +464,8 @@ __device__ __forceinline__ void attn_bwd_kv_body(const bsa_attn_args &a, char *s
     // `rec` is the record of the tile after the one in flight
     int rec;
     {
-      const int rec0 = load_record(q_begin);
       rec = load_record(clamp_e(q_begin + 1));
-      fetch(rec0, 0);
+      fetch(head, 0);
       stage(0);
       __syncthreads();
     }
@@ -657,15 +679,18 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_q_kernel(bsa_attn_arg
   const int wi = wave & 1, wj = wave >> 1;
   const int64_t qpos_in_order = xcd_row();
   if (qpos_in_order >= a.B * a.nq) return;
-  const int64_t qrow = bwd_lists(a).q_order[qpos_in_order];
+  const BwdLists lists = bwd_lists(a);
+  // the workgroup's header, int i in lane i (lanes 0 .. 7 double as the record of the first tile)
+  int head = -1;
+  if (lane < 16) head = lists.q_head[qpos_in_order * 16 + lane];
+  const int64_t qrow = __builtin_amdgcn_readlane(head, 8);
   const int64_t b = qrow / a.nq, qb = qrow % a.nq;
 
   int64_t pq[NH];
   bool any = false;
 #pragma unroll
   for (int h = 0; h < NH; ++h) {
-    pq[h] = a.pidx_q[qrow * NH + h];
-    if (pq[h] >= a.n_q_blocks) pq[h] = -1;
+    pq[h] = __builtin_amdgcn_readlane(head, 11 + h);
     any = any || pq[h] >= 0;
   }
   if (!any) return;
@@ -676,7 +701,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_q_kernel(bsa_attn_arg
 #pragma unroll
   for (int h = 0; h < NH; ++h) load_resident(qfr[h], a.q, pq[h], a.n_q_blocks, qi, kg);
 #pragma unroll
-  for (int h = 0; h < NHV; ++h) load_resident(dofr[h], a.d_o, a.pidx_o[qrow * NHV + h], a.n_o_blocks, qi, kg);
+  for (int h = 0; h < NHV; ++h) load_resident(dofr[h], a.d_o, __builtin_amdgcn_readlane(head, 13 + h), a.n_o_blocks, qi, kg);
   // a query without any visible key has lse = -inf and P = 0 everywhere: +inf gives exp2(s - lse) = 0 for it
   const float lse_raw = a.lse[qrow * kSbs + qi];
   const float lse = lse_raw == -INFINITY ? INFINITY : lse_raw;
@@ -697,8 +722,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_q_kernel(bsa_attn_arg
   }
   const int qpos = (int)qb * kSbs + qi;
 
-  const BwdLists lists = bwd_lists(a);
-  const int k_begin = a.key_offsets[qrow], k_end = lists.key_end[qrow];
+  const int k_begin = __builtin_amdgcn_readlane(head, 9), k_end = __builtin_amdgcn_readlane(head, 10);
   if (k_begin < k_end) {
     // the record of a list entry, field i in lane i: one 32-byte load, two tiles before the tile is used
     const int32_t *recs = reinterpret_cast<const int32_t *>(lists.key_rec);
@@ -748,9 +772,8 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_q_kernel(bsa_attn_arg
 
     int rec;
     {
-      const int rec0 = load_record(k_begin);
       rec = load_record(clamp_e(k_begin + 1));
-      fetch(rec0, 0);
+      fetch(head, 0);
       stage(0);
       __syncthreads();
     }
@@ -900,7 +923,7 @@ int launch_bwd(const bsa_attn_args &a, hipStream_t s) {
     }
     attn_bwd_records_kernel<<<(unsigned)cdiv(qrows + krows, 4), kBwdThreads, 0, s>>>(a);
     if (int rc = check_launch("attn_bwd_records_kernel")) return rc;
-    attn_bwd_order_kernel<<<16, kBwdThreads, 0, s>>>(a);
+    attn_bwd_order_kernel<<<16, kOrderThreads, 0, s>>>(a);
     if (int rc = check_launch("attn_bwd_order_kernel")) return rc;
   }
   if (qrows > 0) {
@@ -953,7 +976,7 @@ int dispatch_bwd(const bsa_attn_args &a, hipStream_t s) {
 }  // namespace
 
 size_t attn_bwd_scratch_bytes(int64_t B, int64_t nq, int64_t nk, int64_t n_layout_blocks, int64_t n_mask_blocks) {
-  const size_t bytes = 2 * sizeof(BwdRecord) * (size_t)n_layout_blocks + 8 * (size_t)(B * nq + B * nk) + (size_t)n_mask_blocks;
+  const size_t bytes = 2 * sizeof(BwdRecord) * (size_t)n_layout_blocks + (4 + 64) * (size_t)(B * nq + B * nk) + (size_t)n_mask_blocks;
   return (bytes + 15) & ~(size_t)15;
 }
 
