@@ -42,7 +42,7 @@ TRAFFIC_KIB = {  # config: (FETCH_SIZE, WRITE_SIZE)
     "c2": (484866.8, 514960.3),
     "c3": (148346.4, 296128.0),
     "c4": (373413.6, 133150.6),
-    "c5": (127107.7, 143960.0),
+    "c5": (30070.4, 143960.0),
     "t1": (67086.4, 129576.0),
     "l1": (262162.2, 64.0),
     "r1": (64865.6, 8192.0),
@@ -151,7 +151,7 @@ def matmul_workload(name, B, n, sbs, dtype, density, ensure_rows, value_scale, d
 
     dt_name = {torch.bfloat16: "bf16", torch.float16: "f16", torch.float32: "f32"}[dtype]
     return dict(step=step, flops=flops, alg_bytes=alg_bytes, dtype=dt_name, bound="hbm", cpu_baseline=cpu_baseline,
-                kernel=("matmul_rows_kernel" if sbs == 64 and dtype != torch.float32 else "matmul_mfma_kernel") if sbs > 16 else "matmul_small_kernel",
+                kernel=("matmul_rows_kernel" if sbs == 64 and dtype != torch.float32 else "matmul_mfma_kernel") if sbs > 16 else ("matmul_small16_kernel" if dtype != torch.float32 else "matmul_small_kernel"),
                 config={"workload": name, "B": B, "M": n * sbs, "K": n * sbs, "N": n * sbs,
                         "sparsity_block_size": sbs, "density": density, "nnz_x": nnz_x, "nnz_y": nnz_y,
                         "nnz_o": nnz_o, "block_pairs": pairs, "lut_build_ms": round(lut_ms, 3)})

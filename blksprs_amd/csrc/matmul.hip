@@ -24,10 +24,12 @@
 // is rounded to the output type, staged through LDS and written with 16-byte
 // stores that cover whole rows.
 //
-// sbs == 16 uses a small FMA kernel instead (one wave per block): at 13 flop/byte
-// the matrix core has nothing to add.
+// sbs == 16 has kernels of its own (16 x 16 x 16 products for 16-bit elements, FMAs
+// for fp32): at 13 flop/byte it is a gather problem, not a matrix-core problem.
 #include <hip/hip_bf16.h>
 #include <hip/hip_fp16.h>
+
+#include <type_traits>
 
 #include "common.h"
 
@@ -441,6 +443,129 @@ __global__ __launch_bounds__(256) void matmul_small_kernel(const typename Tr::st
   for (int e = 0; e < 4; ++e) ob[e] = Tr::round(acc[e]);
 }
 
+// sbs == 16, 16-bit elements: one 16 x 16 x 16 matrix-core product per pair.  A block is 512 bytes and an output
+// block has one or two pairs, so a wave that handled a single block would be a chain of dependent loads
+// (offsets -> pairs -> operands -> store) and nothing else.  Here a wave owns a run of consecutive output blocks,
+// whose pairs are one contiguous range of the pair list: it reads that range and the run's offsets once (one
+// entry per lane), then walks the pairs with the operand loads of the next two pairs in flight.
+// The product is formed transposed (A = y fragment, B = x fragment), which leaves four consecutive output columns
+// of one row in each lane: the wave's 8-byte stores cover the whole output block.  An operand whose contraction
+// index is contiguous in memory (x, or y when it is used transposed) is loaded straight into its fragment; the
+// other one passes through 512 bytes of LDS and comes back through the transposing read.
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+
+struct Bf16Small {
+  __device__ static f32x4 mfma(u32x2 a, u32x2 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(i16x4, a), __builtin_bit_cast(i16x4, b), c, 0, 0, 0);
+  }
+  __device__ static uint32_t pack2(float lo, float hi) {
+    return (uint32_t)Bf16Traits::round(lo) | ((uint32_t)Bf16Traits::round(hi) << 16);
+  }
+};
+struct F16Small {
+  __device__ static f32x4 mfma(u32x2 a, u32x2 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4, a), __builtin_bit_cast(f16x4, b), c, 0, 0, 0);
+  }
+  __device__ static uint32_t pack2(float lo, float hi) {
+    return (uint32_t)F16Traits::round(lo) | ((uint32_t)F16Traits::round(hi) << 16);
+  }
+};
+
+constexpr int kSmallRunMax = 63;  // output blocks per wave: their offsets (one more) fit one entry per lane
+
+template <typename Ts, bool XT, bool YT>
+__global__ __launch_bounds__(256) void matmul_small16_kernel(const char *__restrict__ x, const char *__restrict__ y,
+                                                             char *__restrict__ out,
+                                                             const int32_t *__restrict__ pair_offsets,
+                                                             const int32_t *__restrict__ pairs, int64_t nnz_o,
+                                                             int64_t nnz_x, int64_t nnz_y, int run) {
+  __shared__ __attribute__((aligned(16))) char stage[4][512];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  // workgroup g runs on XCD g % 8: every XCD takes a contiguous eighth of the runs, so that the operand blocks in
+  // flight on one L2 belong to few batch entries
+  const int64_t group = (int64_t)(blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+  const int64_t n0 = (group * 4 + wave) * run;
+  if (n0 >= nnz_o) return;
+  const int count = (int)(nnz_o - n0 < run ? nnz_o - n0 : run);
+  // fragment of a k-contiguous operand: row lane % 16, values 4 (lane / 16) .. + 3
+  const int direct_off = (lane & 15) * 32 + (lane >> 4) * 8;
+  // the other operand is copied as it lies (lane l moves bytes 8 l .. 8 l + 7) and read back transposed: inside
+  // a group of 16 lanes, lane s points at row 4 (lane / 16) + s / 4, values 4 (s % 4) .. + 3
+  const int turned_off = (4 * (lane >> 4) + ((lane & 15) >> 2)) * 32 + (lane & 3) * 8;
+  char *slot = stage[wave];
+
+  // offsets of the run (count + 1 of them) and the first 64 pairs
+  const int off_win = pair_offsets[n0 + (lane <= count ? lane : count)];
+  const int p_first = __builtin_amdgcn_readlane(off_win, 0);
+  const int p_last = __builtin_amdgcn_readlane(off_win, count);
+  int win_base = p_first;
+  u32x2 win{0u, 0u};
+  auto load_window = [&]() {
+    if (win_base + lane < p_last) win = *reinterpret_cast<const u32x2 *>(pairs + 2 * (int64_t)(win_base + lane));
+  };
+  load_window();
+
+  auto issue = [&](int p, u32x2 &xr, u32x2 &yr) {
+    // p is inside the window (the caller moves the window first)
+    int64_t px = __builtin_amdgcn_readlane((int)win[0], p - win_base);
+    int64_t py = __builtin_amdgcn_readlane((int)win[1], p - win_base);
+    if (px < 0 || px >= nnz_x) px = 0;
+    if (py < 0 || py >= nnz_y) py = 0;
+    xr = *reinterpret_cast<const u32x2 *>(x + px * 512 + (XT ? lane * 8 : direct_off));
+    yr = *reinterpret_cast<const u32x2 *>(y + py * 512 + (YT ? direct_off : lane * 8));
+  };
+  auto turned = [&](u32x2 v) {
+    *reinterpret_cast<u32x2 *>(slot + lane * 8) = v;
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    const i16x4 t = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4 *)(slot + turned_off));
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    return __builtin_bit_cast(u32x2, t);
+  };
+
+  f32x4 acc{0.f, 0.f, 0.f, 0.f};
+  int done = 0;                                           // output blocks of the run already stored
+  int block_end = __builtin_amdgcn_readlane(off_win, 1);  // end of the pairs of block `done`
+  auto flush_until = [&](int p) {
+    // store every block whose pairs end at or before p (blocks without pairs become zeros)
+    while (done < count && block_end <= p) {
+      u32x2 w;
+      w[0] = Ts::pack2(acc[0], acc[1]);
+      w[1] = Ts::pack2(acc[2], acc[3]);
+      *reinterpret_cast<u32x2 *>(out + (n0 + done) * 512 + direct_off) = w;
+      acc = f32x4{0.f, 0.f, 0.f, 0.f};
+      ++done;
+      block_end = __builtin_amdgcn_readlane(off_win, done + 1 <= count ? done + 1 : count);
+    }
+  };
+
+  int p = p_first;
+  u32x2 xa{0u, 0u}, ya{0u, 0u}, xb{0u, 0u}, yb{0u, 0u};
+  if (p < p_last) issue(p, xa, ya);
+  if (p + 1 < p_last) issue(p + 1, xb, yb);
+  auto step = [&](u32x2 &xr, u32x2 &yr) {
+    flush_until(p);
+    const u32x2 fx = XT ? turned(xr) : xr;
+    const u32x2 fy = YT ? yr : turned(yr);
+    acc = Ts::mfma(fy, fx, acc);
+    if (p + 2 < p_last) {
+      if (p + 2 - win_base >= 64) {
+        win_base = p + 2;
+        load_window();
+      }
+      issue(p + 2, xr, yr);
+    }
+    ++p;
+  };
+  while (p < p_last) {
+    step(xa, ya);
+    if (p >= p_last) break;
+    step(xb, yb);
+  }
+  flush_until(p_last);
+}
+
 template <typename Tr, int TILE>
 int launch_mfma(const void *x, const void *y, void *out, const int32_t *pair_offsets, const int32_t *pairs,
                 const int32_t *block_order, int64_t nnz_o, int64_t nnz_x, int64_t nnz_y, int sbs, int trans_x,
@@ -470,6 +595,26 @@ template <typename Tr>
 int launch_any(const void *x, const void *y, void *out, const int32_t *pair_offsets, const int32_t *pairs,
                const int32_t *block_order, int64_t nnz_o, int64_t nnz_x, int64_t nnz_y, int sbs, int trans_x,
                int trans_y, hipStream_t s) {
+  if (sbs == 16 && Tr::kElem == 2) {
+    using Ts = std::conditional_t<std::is_same_v<Tr, Bf16Traits>, Bf16Small, F16Small>;
+    // enough waves to fill the chip, each with a run long enough to overlap its loads
+    int64_t run = bsa::cdiv(nnz_o, 256 * 32 * 4);
+    run = run < 8 ? 8 : (run > kSmallRunMax ? kSmallRunMax : run);
+    const int64_t blocks = bsa::cdiv(bsa::cdiv(bsa::cdiv(nnz_o, run), 4), 8) * 8;
+    if (blocks > 0x7fffffffLL) return bsa::fail(BSA_ELIMIT, "bsa_matmul: too many output blocks");
+    const char *xc = static_cast<const char *>(x);
+    const char *yc = static_cast<const char *>(y);
+    char *oc = static_cast<char *>(out);
+#define BSA_MM_SMALL(XT, YT)                                                                                        \
+  matmul_small16_kernel<Ts, XT, YT><<<(unsigned)blocks, 256, 0, s>>>(xc, yc, oc, pair_offsets, pairs, nnz_o, nnz_x, \
+                                                                     nnz_y, (int)run)
+    if (!trans_x && !trans_y) BSA_MM_SMALL(false, false);
+    else if (!trans_x && trans_y) BSA_MM_SMALL(false, true);
+    else if (trans_x && !trans_y) BSA_MM_SMALL(true, false);
+    else BSA_MM_SMALL(true, true);
+#undef BSA_MM_SMALL
+    return bsa::check_launch("matmul_small16_kernel");
+  }
   if (sbs == 16) {
     using E = typename Tr::store_t;
     const int64_t blocks = bsa::cdiv(nnz_o, 4);
