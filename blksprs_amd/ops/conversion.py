@@ -47,15 +47,18 @@ def _launch_to_dense(x: Tensor, shape, packed_indices: Tensor, sbs: int, fill_va
 
 
 class _ToSparse(torch.autograd.Function):
+    # The layout is metadata, not a differentiable input: it is kept as a plain attribute, so that a compressed
+    # tensor held in a cache (the packed weight of apply_torch_linear_cached) can be differentiated through in
+    # every training iteration, not only in the first.
     @staticmethod
     def forward(ctx, x, sparsity_layout, layout_indices, sparsity_block_size, n_sparse_blocks):
-        ctx.save_for_backward(sparsity_layout)
+        ctx.sparsity_layout = sparsity_layout
         ctx.sparsity_block_size = sparsity_block_size
         return _launch_to_sparse(x, layout_indices, sparsity_block_size, n_sparse_blocks)
 
     @staticmethod
     def backward(ctx, grad_output):
-        (sparsity_layout,) = ctx.saved_tensors
+        sparsity_layout = ctx.sparsity_layout
         grad = to_dense(grad_output.contiguous(), sparsity_layout, ctx.sparsity_block_size)
         return grad, None, None, None, None
 
@@ -63,13 +66,13 @@ class _ToSparse(torch.autograd.Function):
 class _ToDense(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, sparsity_layout, packed_indices, sparsity_block_size, fill_value):
-        ctx.save_for_backward(sparsity_layout)
+        ctx.sparsity_layout = sparsity_layout
         ctx.sparsity_block_size = sparsity_block_size
         return _launch_to_dense(x, sparsity_layout.shape, packed_indices, sparsity_block_size, fill_value)
 
     @staticmethod
     def backward(ctx, grad_output):
-        (sparsity_layout,) = ctx.saved_tensors
+        sparsity_layout = ctx.sparsity_layout
         grad = to_sparse(grad_output.contiguous(), sparsity_layout, ctx.sparsity_block_size)
         return grad, None, None, None, None
 

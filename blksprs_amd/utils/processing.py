@@ -19,7 +19,7 @@ import torch
 from torch import Tensor, nn
 
 from .blksprs_tensor import BlksprsTensor
-from .tools import as_base_tensor, finalize_layout_cache, prepare_layout_cache
+from .tools import CacheHolder, as_base_tensor, finalize_layout_cache, prepare_layout_cache
 from .validation import (ensure_contiguous, validate_contiguous, validate_device, validate_dimensions,
                          validate_dtype_float, validate_dtype_supported, validate_shape, validate_sparsity,
                          validate_sparsity_block_size)
@@ -157,7 +157,7 @@ def apply_torch_linear_cached(x: BlksprsTensor, sparsity_layout: Tensor, sparsit
 
     out = _project(x, stacked_layout, layout_cache["w_t_bs"], layout_w_t, stacked_layout_output,
                    layout_cache.get("bias_slice_bs"), sparsity_block_size,
-                   layout_cache.setdefault("matmul_layout_cache", dict()))
+                   layout_cache.setdefault("matmul_layout_cache", CacheHolder()).cache)
     layout_output = layout_cache["sparsity_layout_output"]
     finalize_layout_cache(layout_cache)
     return out, layout_output

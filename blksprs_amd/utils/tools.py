@@ -21,7 +21,8 @@ LayoutCache = dict[str, Any]
 _KEY = "_blksprs_cache_key"
 _REFS = "_blksprs_cache_refs"
 _STATE = "_blksprs_cache_state"
-_PRIVATE = frozenset((_KEY, _REFS, _STATE))
+_CHECKED = "_blksprs_cache_checked"  # number of entries when the recorded state was last found valid
+_PRIVATE = frozenset((_KEY, _REFS, _STATE, _CHECKED))
 
 
 def as_base_tensor(value: Tensor) -> Tensor:
@@ -174,7 +175,8 @@ def build_contraction_lists(pidx_x: Tensor, pidx_y: Tensor, pidx_o: Tensor, B: i
 # --------------------------------------------------------------------------- layout cache
 
 def _tensor_signature(value: Tensor, version):
-    return ("tensor", id(value), version, tuple(value.shape), tuple(value.stride()), value.dtype, value.device,
+    # torch.Size and the stride tuple compare and hash like plain tuples
+    return ("tensor", id(value), version, value.shape, value.stride(), value.dtype, value.device,
             value.requires_grad)
 
 
@@ -197,6 +199,9 @@ def prepare_layout_cache(layout_cache: LayoutCache | None, operation: str, *valu
         layout_cache[_KEY] = key
         # holding the sources keeps their ids from being reused by other tensors
         layout_cache[_REFS] = refs
+    else:
+        layout_cache.setdefault(_CHECKED, None)  # counted by len() below
+        layout_cache[_CHECKED] = len(layout_cache)
     return layout_cache
 
 
@@ -218,9 +223,25 @@ def layout_cache_key(operation: str, *values: object) -> tuple[tuple, tuple]:
     return (operation, tuple(signature(v) for v in values)), tuple(refs)
 
 
+class CacheHolder:
+    """A cache of a nested operation, kept inside a caller's cache as one opaque entry: the nested operation
+    validates it itself, and what it adds later (the lists of a backward pass, say) does not make the outer cache
+    look modified."""
+
+    __slots__ = ("cache",)
+
+    def __init__(self):
+        self.cache: LayoutCache = {}
+
+
 def finalize_layout_cache(layout_cache: LayoutCache) -> LayoutCache:
     """Records what the cache holds now; a later change of any entry invalidates it."""
+    # a cache that prepare_layout_cache has just found equal to its recorded state, and that has gained no entry
+    # since, is in that state still (builders add entries, they replace none)
+    if layout_cache.get(_CHECKED) == len(layout_cache) and _STATE in layout_cache:
+        return layout_cache
     layout_cache[_STATE] = _snapshot(layout_cache)
+    layout_cache[_CHECKED] = None
     return layout_cache
 
 

@@ -195,6 +195,25 @@ def test_linear_cache_follows_layout_and_parameter_state(device):
     assert linear.weight.grad is None
 
 
+def test_linear_cache_survives_training_iterations(device):
+    """Forward and backward, three times over: the compressed parameters and the product's lookup tables are
+    built once (the lists the backward pass adds to the product's cache do not invalidate the linear cache)."""
+    layout = rand_layout((2, 3, 2), 0.7, seed=3).to(device)
+    linear = _linear(2 * SBS, 3 * SBS, True, device)
+    dense = torch.randn((2, 3 * SBS, 2 * SBS), device=device)
+    sparse = bs.ops.to_sparse(dense, layout, SBS)
+    cache = {}
+    seen = []
+    for _ in range(3):
+        out, _ = bs.utils.apply_torch_linear_cached(sparse, layout, SBS, linear, layout_cache=cache)
+        out.square().sum().backward()
+        product_cache = cache["matmul_layout_cache"].cache
+        seen.append((cache["w_t_bs"], product_cache["contraction_pairs"], product_cache["grad_x_pairs"]))
+        linear.zero_grad(set_to_none=False)  # in place: the parameters stay the same objects and versions...
+    # ... except that zeroing bumps the version of .grad only, not of the parameters
+    assert all(a is b for a, b in zip(seen[0], seen[1])) and all(a is b for a, b in zip(seen[1], seen[2]))
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_normalisation_and_dropout_through_packed_rows(device, dtype):
     """test/cases/test_blocksparse.py:1197-1265: layer norm over the feature dimension of a tensor whose inactive
