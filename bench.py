@@ -40,9 +40,11 @@ PEAK_MFMA_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}
 TRAFFIC_KIB = {  # config: (FETCH_SIZE, WRITE_SIZE)
     "c1": (616.2, 476.0),
     "c2": (484866.8, 514960.3),
-    "c3": (148346.4, 296128.0),
+    "c3": (148176.3, 296129.7),
     "c4": (373413.6, 133150.6),
     "c5": (30070.4, 143960.0),
+    "v1": (66312.1, 129576.0),
+    "v2": (66851.5, 524499.4),
     "t1": (67086.4, 129576.0),
     "l1": (262162.2, 64.0),
     "r1": (64865.6, 8192.0),
@@ -311,6 +313,47 @@ def movement_workload(dev, which):
                     config={"workload": "r2_row_wise_add_bf16", "B": B, "rows": n * sbs, "cols": n * sbs,
                             "sparsity_block_size": sbs, "nnz": nnz})
     dense = bs.ops.to_dense(x, ld, sbs)
+    if which in ("to_sparse", "to_dense"):
+        nb = 2
+        cnt = int(layout[:nb].sum())
+        lnp = layout.numpy()
+        cache = {}
+        if which == "to_sparse":
+            bs.ops.to_sparse(dense, ld, sbs, layout_cache=cache)
+            alg_bytes = 2 * nnz * sbs * sbs * 2
+
+            def step():
+                return bs.ops.to_sparse(dense, ld, sbs, layout_cache=cache)
+
+            ds = dense[:nb].cpu()
+
+            def cpu_baseline():
+                reps, dt = _repeat_for(CPU_SAMPLE_SECONDS, lambda: orc.to_sparse(ds, lnp[:nb], sbs))
+                return {"value": 2 * cnt * sbs * sbs * 2 / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(),
+                        "kind": "port", "sample": f"{nb} of {B} batches x {reps} passes, torch reshape / permute / "
+                                                  f"boolean index, {dt * reps:.1f} s"}
+
+            kernel, workload = "to_sparse_kernel", "v1_to_sparse_bf16"
+        else:
+            bs.ops.to_dense(x, ld, sbs, layout_cache=cache)
+            alg_bytes = dense.numel() * 2 + nnz * sbs * sbs * 2
+
+            def step():
+                return bs.ops.to_dense(x, ld, sbs, layout_cache=cache)
+
+            xs = x[:cnt].cpu()
+
+            def cpu_baseline():
+                reps, dt = _repeat_for(CPU_SAMPLE_SECONDS, lambda: orc.to_dense(xs, lnp[:nb], sbs))
+                return {"value": (nb * n * n + cnt) * sbs * sbs * 2 / dt / 1e9, "unit": "GB/s",
+                        "cores": torch.get_num_threads(), "kind": "port",
+                        "sample": f"{nb} of {B} batches x {reps} passes, torch fill / boolean index / permute, "
+                                  f"{dt * reps:.1f} s"}
+
+            kernel, workload = "to_dense_kernel", "v2_to_dense_bf16"
+        return dict(step=step, flops=0.0, alg_bytes=alg_bytes, dtype="bf16", bound="hbm", cpu_baseline=cpu_baseline,
+                    kernel=kernel, config={"workload": workload, "B": B, "rows": n * sbs, "cols": n * sbs,
+                                           "sparsity_block_size": sbs, "nnz": nnz})
     alg_bytes = dense.numel() * 2 + B * n * n
 
     def step():
@@ -406,6 +449,10 @@ def make_workload(name, dev):
         return movement_workload(dev, "transpose")
     if name == "l1":
         return movement_workload(dev, "layout")
+    if name == "v1":
+        return movement_workload(dev, "to_sparse")
+    if name == "v2":
+        return movement_workload(dev, "to_dense")
     if name == "p1":
         return linear_workload(dev)
     if name == "r1":
@@ -422,7 +469,7 @@ def main():
     # with 10 warm-up steps the first timed steps of configuration 2 still run 10 % slower
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=100)
-    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c4bwd", "c5", "t1", "l1", "r1", "r2", "p1"])
+    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c4bwd", "c5", "t1", "l1", "r1", "r2", "p1", "v1", "v2"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:

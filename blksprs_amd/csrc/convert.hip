@@ -30,26 +30,36 @@ __global__ __launch_bounds__(256) void to_sparse_kernel(const uint4 *__restrict_
   }
 }
 
-// dense[b][row][:] <- blocks[packed[b, row/sbs, col/sbs]] or the fill pattern
-__global__ __launch_bounds__(256) void to_dense_kernel(const uint4 *__restrict__ blocks,
+// dense[b][row][:] <- blocks[packed[b, row/sbs, col/sbs]] or the fill pattern.  A thread owns one 16-byte
+// column position in kDenseRows consecutive rows of the dense array (they lie in one block row, so one look-up
+// serves them all); a wave writes 1 KiB of a row at a time.  The dense array is written once and not read
+// back by this kernel: the stores bypass the caches.
+constexpr int kDenseRows = 4;  // divides every sbs
+
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(256) void to_dense_kernel(const u32x4_t *__restrict__ blocks,
                                                        const int64_t *__restrict__ packed,
-                                                       uint4 *__restrict__ dense, int64_t n_vec, int64_t nnz,
-                                                       int64_t R, int64_t C, int vec_per_row_log2, int sbs_log2,
-                                                       uint4 fill) {
-  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  const int64_t dense_row_vecs = C << vec_per_row_log2;
-  for (int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; g < n_vec; g += stride) {
-    const int64_t col_vec = g % dense_row_vecs;
-    const int64_t row_all = g / dense_row_vecs;  // b * R*sbs + row
-    const int64_t c = col_vec >> vec_per_row_log2;
-    const int64_t q = col_vec & (((int64_t)1 << vec_per_row_log2) - 1);
-    const int64_t e = row_all & (((int64_t)1 << sbs_log2) - 1);
-    const int64_t br = row_all >> sbs_log2;  // b * R + r
-    const int64_t idx = packed[br * C + c];
-    uint4 v = fill;
-    if (idx >= 0 && idx < nnz) v = blocks[(((idx << sbs_log2) + e) << vec_per_row_log2) + q];
-    dense[g] = v;
+                                                       u32x4_t *__restrict__ dense, int64_t nnz, int64_t C,
+                                                       int64_t dense_row_vecs, int vec_per_row_log2, int sbs_log2,
+                                                       u32x4_t fill) {
+  const int64_t col_vec = (int64_t)blockIdx.y * 256 + threadIdx.x;
+  if (col_vec >= dense_row_vecs) return;
+  const int64_t row0 = (int64_t)blockIdx.x * kDenseRows;  // b * R * sbs + row
+  const int64_t c = col_vec >> vec_per_row_log2;
+  const int64_t q = col_vec & (((int64_t)1 << vec_per_row_log2) - 1);
+  const int64_t e0 = row0 & (((int64_t)1 << sbs_log2) - 1);
+  const int64_t br = row0 >> sbs_log2;  // b * R + r
+  const int64_t idx = packed[br * C + c];
+  const bool active = idx >= 0 && idx < nnz;
+  u32x4_t v[kDenseRows];
+#pragma unroll
+  for (int i = 0; i < kDenseRows; ++i) {
+    v[i] = fill;
+    if (active) v[i] = blocks[(((idx << sbs_log2) + e0 + i) << vec_per_row_log2) + q];
   }
+#pragma unroll
+  for (int i = 0; i < kDenseRows; ++i) __builtin_nontemporal_store(v[i], dense + (row0 + i) * dense_row_vecs + col_vec);
 }
 
 // layout[b][r][c] = 1 if the sbs x sbs block (r, c) of dense[b] holds an element != 0.  One workgroup owns
@@ -244,11 +254,14 @@ extern "C" int bsa_to_dense(const void *blocks, const int64_t *packed, void *den
   uint64_t pat = fill_bits;
   if (elem_size < 8) pat &= ((uint64_t)1 << (8 * elem_size)) - 1;
   for (int w = elem_size; w < 8; w *= 2) pat |= pat << (8 * w);
-  uint4 fill;
-  fill.x = fill.z = (uint32_t)(pat & 0xffffffffu);
-  fill.y = fill.w = (uint32_t)(pat >> 32);
-  to_dense_kernel<<<copy_grid(n_vec), 256, 0, bsa::as_stream(stream)>>>(
-      static_cast<const uint4 *>(blocks), packed, static_cast<uint4 *>(dense), n_vec, nnz, R, C,
+  const u32x4_t fill{(uint32_t)(pat & 0xffffffffu), (uint32_t)(pat >> 32), (uint32_t)(pat & 0xffffffffu),
+                     (uint32_t)(pat >> 32)};
+  const int64_t dense_row_vecs = C * vec_per_row;
+  const int64_t row_groups = B * R * sbs / kDenseRows;
+  const int64_t col_groups = bsa::cdiv(dense_row_vecs, 256);
+  BSA_REQUIRE(row_groups < 0x7fffffffLL && col_groups <= 65535, "bsa_to_dense: dense array too large for one launch");
+  to_dense_kernel<<<dim3((unsigned)row_groups, (unsigned)col_groups), 256, 0, bsa::as_stream(stream)>>>(
+      static_cast<const u32x4_t *>(blocks), packed, static_cast<u32x4_t *>(dense), nnz, C, dense_row_vecs,
       ilog2(vec_per_row), ilog2(sbs), fill);
   return bsa::check_launch("to_dense_kernel");
 }
