@@ -9,6 +9,13 @@
 
 namespace {
 
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+
+// results that are written once and not read back by the kernel bypass the caches
+__device__ inline void store_streaming(uint4 *p, uint4 v) {
+  __builtin_nontemporal_store(u32x4_t{v.x, v.y, v.z, v.w}, reinterpret_cast<u32x4_t *>(p));
+}
+
 // blocks[n][e][:] <- dense[b][r*sbs + e][c*sbs : (c+1)*sbs]
 __global__ __launch_bounds__(256) void to_sparse_kernel(const uint4 *__restrict__ dense,
                                                         const int64_t *__restrict__ coords,
@@ -26,7 +33,7 @@ __global__ __launch_bounds__(256) void to_sparse_kernel(const uint4 *__restrict_
     const int64_t r = coords[n * 3 + 1];
     const int64_t c = coords[n * 3 + 2];
     const int64_t src = b * dense_batch_vecs + ((r << sbs_log2) + e) * dense_row_vecs + (c << vec_per_row_log2) + q;
-    blocks[g] = dense[src];
+    store_streaming(blocks + g, dense[src]);
   }
 }
 
@@ -35,8 +42,6 @@ __global__ __launch_bounds__(256) void to_sparse_kernel(const uint4 *__restrict_
 // serves them all); a wave writes 1 KiB of a row at a time.  The dense array is written once and not read
 // back by this kernel: the stores bypass the caches.
 constexpr int kDenseRows = 4;  // divides every sbs
-
-typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
 
 __global__ __launch_bounds__(256) void to_dense_kernel(const u32x4_t *__restrict__ blocks,
                                                        const int64_t *__restrict__ packed,
@@ -195,8 +200,8 @@ __global__ __launch_bounds__(256) void transpose_blocks16_kernel(const uint16_t 
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int v = t + 256 * i, row = v >> 3, chunk = v & 7;
-    *reinterpret_cast<uint4 *>(dst + row * row_bytes + chunk * 16) =
-        *reinterpret_cast<const uint4 *>(out_tile + row * 128 + chunk * 16);
+    store_streaming(reinterpret_cast<uint4 *>(dst + row * row_bytes + chunk * 16),
+                    *reinterpret_cast<const uint4 *>(out_tile + row * 128 + chunk * 16));
   }
 }
 

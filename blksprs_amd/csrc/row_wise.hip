@@ -15,6 +15,8 @@
 
 namespace {
 
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+
 struct RowGeom {
   int sbs_log2;
   int vec_log2;   // elements per 16-byte vector, as log2
@@ -183,7 +185,8 @@ __global__ __launch_bounds__(256) void row_add_kernel(const uint4 *__restrict__ 
 #pragma unroll
       for (int i = 0; i < E::kPerVec; ++i) E::store(v, i, E::load(xv, i) + add);
     }
-    out[gi] = v;
+    // written once, not read back here: bypass the caches
+    __builtin_nontemporal_store(u32x4_t{v.x, v.y, v.z, v.w}, reinterpret_cast<u32x4_t *>(out + gi));
   }
 }
 
