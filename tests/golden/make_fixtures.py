@@ -61,7 +61,35 @@ def compute_fixture():
              mask=mask.numpy(), attention=at.numpy())
 
 
+def neighbours_fixture():
+    """The operations next to the hot path: transpose, layout of a dense tensor, row-wise sum / max / add, a
+    linear layer with bias, causal layouts and compact masks."""
+    g = torch.Generator().manual_seed(13)
+    sbs = 16
+    layout = orc.random_layout((2, 3, 4), 0.6, g, ensure_rows=True).numpy()
+    layout[1, 2, :] = False
+    x = torch.randn((int(layout.sum()), sbs, sbs), generator=g, dtype=torch.float64)
+    xt, layout_t = orc.transpose(x, layout, sbs)
+    dense = orc.to_dense(x, layout, sbs)
+    row_sum, row_layout = orc.row_wise_reduce(x, layout, sbs, "sum")
+    row_max, _ = orc.row_wise_reduce(x, layout, sbs, "max", slice_only=True)
+    centred = orc.row_wise_add(x, layout, -row_max, sbs)
+    weight = torch.randn((2 * sbs, 4 * sbs), generator=g, dtype=torch.float64) / 8
+    bias = torch.randn((2 * sbs,), generator=g, dtype=torch.float64)
+    lin, lin_layout = orc.linear(x, layout, weight, bias, sbs)
+    lengths = np.array([37, 64, 1], dtype=np.int64)
+    causal = orc.causal_layout(lengths, sbs)
+    window = orc.causal_layout(lengths, sbs, window_size=23)
+    np.savez(HERE / "neighbours.npz", sbs=np.int64(sbs), layout=layout, x=x.numpy(), transposed=xt.numpy(),
+             layout_t=layout_t, dense_layout=orc.build_sparsity_layout(dense, sbs), row_layout=row_layout,
+             row_sum=row_sum.numpy(), row_max=row_max.numpy(), centred=centred.numpy(), weight=weight.numpy(),
+             bias=bias.numpy(), linear=lin.numpy(), linear_layout=lin_layout, lengths=lengths, causal_layout=causal,
+             window_layout=window, causal_mask_layout=orc.causal_mask_layout(lengths, causal, sbs),
+             window_mask_layout=orc.causal_mask_layout(lengths, window, sbs, window_size=23))
+
+
 if __name__ == "__main__":
     lut_fixture()
     compute_fixture()
+    neighbours_fixture()
     print("wrote", sorted(p.name for p in HERE.glob("*.npz")))

@@ -87,3 +87,66 @@ def test_device_results_match_the_compute_fixture(device):
     out = bs.ops.flash_attention(f32("q"), ones(nq), f32("k"), ones(nk), f32("v"), ones(nk), lay("attention_layout"),
                                  sbs, attention_mask=lay("mask"), sparsity_layout_mask=lay("layout_mask"))
     assert_close(out, torch.from_numpy(d["attention"]), 2e-5, "attention fp32")
+
+
+def test_oracle_reproduces_the_neighbours_fixture():
+    d = _load("neighbours.npz")
+    sbs = int(d["sbs"])
+    t = lambda k: torch.from_numpy(d[k])
+    layout = d["layout"]
+    xt, layout_t = orc.transpose(t("x"), layout, sbs)
+    assert torch.equal(xt, t("transposed")) and np.array_equal(layout_t, d["layout_t"])
+    assert np.array_equal(orc.build_sparsity_layout(orc.to_dense(t("x"), layout, sbs), sbs), d["dense_layout"])
+    row_sum, row_layout = orc.row_wise_reduce(t("x"), layout, sbs, "sum")
+    assert np.array_equal(row_layout, d["row_layout"])
+    assert_close(row_sum, t("row_sum"), 1e-12, "row sum")
+    row_max, _ = orc.row_wise_reduce(t("x"), layout, sbs, "max", slice_only=True)
+    assert torch.equal(row_max, t("row_max"))
+    assert torch.equal(orc.row_wise_add(t("x"), layout, -row_max, sbs), t("centred"))
+    lin, lin_layout = orc.linear(t("x"), layout, t("weight"), t("bias"), sbs)
+    assert np.array_equal(lin_layout, d["linear_layout"])
+    assert_close(lin, t("linear"), 1e-12, "linear")
+    lengths = d["lengths"]
+    assert np.array_equal(orc.causal_layout(lengths, sbs), d["causal_layout"])
+    assert np.array_equal(orc.causal_layout(lengths, sbs, window_size=23), d["window_layout"])
+    assert np.array_equal(orc.causal_mask_layout(lengths, d["causal_layout"], sbs), d["causal_mask_layout"])
+    assert np.array_equal(orc.causal_mask_layout(lengths, d["window_layout"], sbs, window_size=23),
+                          d["window_mask_layout"])
+
+
+@pytest.mark.gpu
+def test_device_results_match_the_neighbours_fixture(device):
+    import blksprs_amd as bs
+    d = _load("neighbours.npz")
+    sbs = int(d["sbs"])
+    f32 = lambda k: torch.from_numpy(d[k]).float().to(device)
+    lay = lambda k: torch.from_numpy(d[k]).to(device)
+    x, layout = bs.BlksprsTensor.wrap(f32("x")), lay("layout")
+    xt, layout_t = bs.ops.transpose(x, layout, sbs)
+    assert torch.equal(xt.cpu(), torch.from_numpy(d["transposed"]).float())
+    assert np.array_equal(layout_t.cpu().numpy() != 0, d["layout_t"])
+    dense = bs.ops.to_dense(x, layout, sbs)
+    assert np.array_equal(bs.layouting.build_sparsity_layout(dense, sbs).cpu().numpy() != 0, d["dense_layout"])
+    row_sum, row_layout = bs.ops.misc.row_wise_sum(x, layout, sbs)
+    assert np.array_equal(row_layout.cpu().numpy() != 0, d["row_layout"])
+    assert_close(row_sum, torch.from_numpy(d["row_sum"]), 1e-5, "row sum fp32")
+    row_max, _ = bs.ops.misc.row_wise_max(x, layout, sbs, flag_slice_only=True)
+    assert torch.equal(row_max.cpu(), torch.from_numpy(d["row_max"]).float())
+    centred = bs.ops.misc.row_wise_sub(x, layout, row_max, sbs)
+    assert_close(centred, torch.from_numpy(d["centred"]), 1e-6, "x - row max")
+    linear = torch.nn.Linear(d["weight"].shape[1], d["weight"].shape[0], device=device)
+    with torch.no_grad():
+        linear.weight.copy_(f32("weight"))
+        linear.bias.copy_(f32("bias"))
+    lin, lin_layout = bs.utils.apply_torch_linear(x, layout, sbs, linear)
+    assert np.array_equal(lin_layout.cpu().numpy() != 0, d["linear_layout"])
+    assert_close(lin, torch.from_numpy(d["linear"]), 1e-5, "linear fp32")
+    lengths = lay("lengths")
+    causal = bs.layouting.build_causal_self_attention_layout(lengths, sbs)
+    window = bs.layouting.build_causal_window_self_attention_layout(lengths, sbs, 23)
+    assert np.array_equal(causal.cpu().numpy() != 0, d["causal_layout"])
+    assert np.array_equal(window.cpu().numpy() != 0, d["window_layout"])
+    _, mask_layout = bs.layouting.build_causal_self_attention_mask(lengths, causal, sbs)
+    assert np.array_equal(mask_layout.cpu().numpy() != 0, d["causal_mask_layout"])
+    _, mask_layout = bs.layouting.build_causal_window_self_attention_mask(lengths, window, sbs, 23)
+    assert np.array_equal(mask_layout.cpu().numpy() != 0, d["window_mask_layout"])
