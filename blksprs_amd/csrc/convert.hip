@@ -83,16 +83,24 @@ __global__ __launch_bounds__(256) void layout_from_dense_kernel(const uint4 *__r
   const int64_t chunk0 = (int64_t)blockIdx.y * kLayoutVecs;
   const uint4 *base = dense + block_row * sbs * row_vecs;
   uint32_t any[kLayoutPerThread] = {0u, 0u, 0u, 0u};
-  for (int e = 0; e < sbs; ++e) {
-    const uint4 *row = base + (int64_t)e * row_vecs;
+  // sbs is a multiple of 4: four rows (16 loads) are in flight at a time
+  for (int e0 = 0; e0 < sbs; e0 += 4) {
+    uint4 w[4][kLayoutPerThread];
 #pragma unroll
-    for (int i = 0; i < kLayoutPerThread; ++i) {
-      const int64_t v = chunk0 + threadIdx.x + 256 * i;
-      if (v < row_vecs) {
-        const uint4 w = row[v];
-        any[i] |= (w.x & mask.x) | (w.y & mask.y) | (w.z & mask.z) | (w.w & mask.w);
+    for (int de = 0; de < 4; ++de) {
+      const uint4 *row = base + (int64_t)(e0 + de) * row_vecs;
+#pragma unroll
+      for (int i = 0; i < kLayoutPerThread; ++i) {
+        const int64_t v = chunk0 + threadIdx.x + 256 * i;
+        w[de][i] = uint4{0u, 0u, 0u, 0u};
+        if (v < row_vecs) w[de][i] = row[v];
       }
     }
+#pragma unroll
+    for (int de = 0; de < 4; ++de)
+#pragma unroll
+      for (int i = 0; i < kLayoutPerThread; ++i)
+        any[i] |= (w[de][i].x & mask.x) | (w[de][i].y & mask.y) | (w[de][i].z & mask.z) | (w[de][i].w & mask.w);
   }
 #pragma unroll
   for (int i = 0; i < kLayoutPerThread; ++i) {
