@@ -44,3 +44,24 @@ def test_bad_arguments_are_rejected_on_the_host():
     # empty problems are accepted without touching the device
     assert lib.bsa_matmul(0, 0, 0, 0, 0, 0, 0, 0, 0, 64, 2, 0, 0, 0) == 0
     assert lib.bsa_softmax_fwd(0, 0, 0, 0, 0, 32, 0) == 0
+
+
+def test_bad_arguments_of_the_neighbouring_entry_points_are_rejected_on_the_host():
+    lib = _capi.load()
+    F32, BF16 = _capi.F32, _capi.BF16
+    # row-wise reduction: unknown operation, unknown dtype, block size not a power of two
+    assert lib.bsa_row_reduce(0, 0, 0, 0, 1, 1, 1, 64, F32, 2, 0, 0) == -1 and b"op must be" in lib.bsa_last_error()
+    assert lib.bsa_row_reduce(0, 0, 0, 0, 1, 1, 1, 64, 99, 0, 0, 0) == -1 and b"dtype" in lib.bsa_last_error()
+    assert lib.bsa_row_reduce(0, 0, 0, 0, 1, 1, 1, 48, F32, 0, 0, 0) == -1 and b"power of two" in lib.bsa_last_error()
+    assert lib.bsa_row_reduce(0, 0, 0, 0, 0, 0, 0, 64, BF16, 1, 1, 0) == 0  # nothing to do
+    # row-wise add: y has 1 or sbs columns
+    assert lib.bsa_row_add(0, 0, 0, 0, 0, 1, 1, 1, 1, 2, 64, F32, 0) == -1 and b"1 or sbs columns" in lib.bsa_last_error()
+    assert lib.bsa_row_add(0, 0, 0, 0, 0, 0, 0, 1, 1, 1, 64, F32, 0) == 0
+    # transpose and layout of a dense tensor: element size, and a 1-byte floating-point type does not exist
+    assert lib.bsa_transpose_blocks(0, 0, 0, 0, 1, 1, 1, 1, 1, 64, 3, 0) == -1 and b"element size" in lib.bsa_last_error()
+    assert lib.bsa_transpose_blocks(0, 0, 0, 0, 0, 0, 1, 1, 1, 64, 2, 0) == 0
+    assert lib.bsa_layout_from_dense(0, 0, 1, 1, 1, 64, 1, 1, 0) == -1 and b"1 byte" in lib.bsa_last_error()
+    assert lib.bsa_layout_from_dense(0, 0, 0, 1, 1, 64, 2, 1, 0) == 0
+    # scratch of the attention backward: 2 x 32 bytes per layout block, (4 + 64) per row, one per mask block
+    assert lib.bsa_attn_bwd_scratch_bytes(2, 3, 5, 7, 11) == (2 * 32 * 7 + 68 * (2 * 3 + 2 * 5) + 11 + 15) // 16 * 16
+    assert lib.bsa_attn_bwd_scratch_bytes(-1, 3, 5, 7, 11) == 0
