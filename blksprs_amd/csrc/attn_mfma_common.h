@@ -42,11 +42,6 @@ struct MF16 {
 constexpr int kSbs = 64;
 constexpr int kBlockBytes = kSbs * kSbs * 2;  // one 16-bit block
 
-// XOR applied to the 16-byte chunk index of K tile row r in LDS.  Two 128-byte rows span the 64 banks once, so
-// the 16 lanes a 128-bit read serves together (16 consecutive rows, one chunk each) are conflict free when
-// rows of equal parity get eight different values.
-__device__ static inline int k_swizzle(int r) { return (r >> 1) & 7; }
-
 // XOR applied to the 16-byte chunk index of row r of a tile that is read both ways: by rows (128-bit reads
 // serve 8 lanes = 8 consecutive rows at a time, one chunk each: they need eight different values) and with
 // the transposing LDS load (it serves 32 lanes at a time = four rows r .. r + 3, r a multiple of 4, 64
@@ -70,14 +65,6 @@ __device__ static inline u32x4 frag_cols_t(const char *lds, int row0, int col0, 
   const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4 *)p1);
   const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
   return u32x4{l2[0], l2[1], h2[0], h2[1]};
-}
-
-// dword offset of column c in a pair row of the (j, j+1)-packed V tile; the placement of the column
-// quads keeps both the 128-bit writes of the staging step and the 32-bit fragment reads conflict free
-__device__ static inline int pair_col_offset(int c) {
-  const int q = c >> 2, a = q >> 1, h = q & 1;
-  const int pos = ((a + 4 * h) & 7) + 8 * h;
-  return 4 * pos + (c & 3);
 }
 
 __device__ static inline int first_lane(int v) { return __builtin_amdgcn_readfirstlane(v); }
