@@ -67,6 +67,17 @@ extern "C" int bsa_attn_fwd_records(const bsa_attn_args *a, const int32_t *group
   return bsa::attn_fwd_records(*a, group_entries, records, bsa::as_stream(stream));
 }
 
+extern "C" int bsa_attn_mask_dead(const void *mask, int64_t n_mask_blocks, int32_t sbs, uint8_t *dead,
+                                  bsa_stream_t stream) {
+  const char *who = "bsa_attn_mask_dead";
+  BSA_REQUIRE(sbs == 64, "%s: only 64 x 64 blocks (got %d)", who, sbs);
+  BSA_REQUIRE(n_mask_blocks >= 0 && n_mask_blocks < 0x7fffffffLL, "%s: bad number of mask blocks", who);
+  if (n_mask_blocks == 0) return BSA_OK;
+  BSA_REQUIRE(mask != nullptr && dead != nullptr, "%s: NULL argument", who);
+  BSA_REQUIRE((reinterpret_cast<uintptr_t>(mask) & 15) == 0, "%s: mask must be 16-byte aligned", who);
+  return bsa::attn_mask_dead(mask, n_mask_blocks, dead, bsa::as_stream(stream));
+}
+
 extern "C" size_t bsa_attn_bwd_scratch_bytes(int64_t B, int64_t nq, int64_t nk, int64_t n_layout_blocks,
                                              int64_t n_mask_blocks) {
   if (B < 0 || nq < 0 || nk < 0 || n_layout_blocks < 0 || n_mask_blocks < 0) return 0;

@@ -914,7 +914,7 @@ int launch_bwd(const bsa_attn_args &a, hipStream_t s) {
     fill_zero_f32_kernel<<<(unsigned)blocks, 256, 0, s>>>(a.dbias, n);
     if (int rc = check_launch("fill_zero_f32_kernel")) return rc;
   }
-  if (qrows + krows > 0) {
+  if (qrows + krows > 0 && !a.bwd_scratch_ready) {
     const BwdLists L = bwd_lists(a);
     if (a.mask != nullptr && a.n_mask_blocks > 0) {
       attn_bwd_mask_dead_kernel<<<(unsigned)cdiv(a.n_mask_blocks, 4), kBwdThreads, 0, s>>>(
@@ -974,6 +974,12 @@ int dispatch_bwd(const bsa_attn_args &a, hipStream_t s) {
 }
 
 }  // namespace
+
+int attn_mask_dead(const void *mask, int64_t n_mask_blocks, uint8_t *dead, hipStream_t s) {
+  attn_bwd_mask_dead_kernel<<<(unsigned)cdiv(n_mask_blocks, 4), kBwdThreads, 0, s>>>(static_cast<const u32x4 *>(mask),
+                                                                                     dead, n_mask_blocks);
+  return check_launch("attn_bwd_mask_dead_kernel");
+}
 
 size_t attn_bwd_scratch_bytes(int64_t B, int64_t nq, int64_t nk, int64_t n_layout_blocks, int64_t n_mask_blocks) {
   const size_t bytes = 2 * sizeof(BwdRecord) * (size_t)n_layout_blocks + (4 + 64) * (size_t)(B * nq + B * nk) + (size_t)n_mask_blocks;

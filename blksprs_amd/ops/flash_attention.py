@@ -18,7 +18,7 @@ from torch import Tensor
 from .. import _capi
 from ..layouting.sparsity_layout import build_sparsity_layout_matmul
 from ..utils.blksprs_tensor import BlksprsTensor
-from ..utils.tools import (INT32_INDEX_MAX, as_base_tensor, cast_for_autocast, csr_indices_from_packed,
+from ..utils.tools import (INT32_INDEX_MAX, CacheHolder, as_base_tensor, cast_for_autocast, csr_indices_from_packed,
                            finalize_layout_cache, pack_layout, prepare_layout_cache)
 from ..utils.validation import (ensure_contiguous, validate_binary, validate_contiguous, validate_device,
                                 validate_dimensions, validate_dtype_float, validate_shape, validate_sparsity,
@@ -232,9 +232,9 @@ def _as_index(t: Tensor | None, dtype: torch.dtype) -> Tensor | None:
 
 
 def _build_forward_records(layout_cache: dict, attention_layout: Tensor, n_batches: int, nq: int, nk: int,
-                           nh: int, nhv: int) -> None:
-    """Adds ``group_offsets`` / ``group_records`` / ``group_size`` (the lists the matrix-core forward kernel
-    walks) to a layout cache that already holds the packed indices."""
+                           nh: int, nhv: int) -> tuple[Tensor, Tensor, int]:
+    """``(group_offsets, group_records, group_size)``: the lists the matrix-core forward kernel walks, for an
+    attention layout and a layout cache that already holds the packed indices."""
     offsets, entries, group_size = _build_group_lists(attention_layout, n_batches, nq, nk)
     records = torch.zeros(entries.numel() * _capi.ATTN_RECORD_INTS, dtype=torch.int32, device=entries.device)
     a = _capi.AttnArgs()
@@ -248,14 +248,70 @@ def _build_forward_records(layout_cache: dict, attention_layout: Tensor, n_batch
     with torch.cuda.device(entries.device):
         _capi.check(_capi.load().bsa_attn_fwd_records(ctypes.byref(a), _capi.ptr(entries), _capi.ptr(records),
                                                       _capi.stream(entries.device)), "bsa_attn_fwd_records")
-    layout_cache["group_offsets"], layout_cache["group_records"] = offsets, as_base_tensor(records)
-    layout_cache["group_size"] = group_size
+    return offsets, as_base_tensor(records), group_size
+
+
+class _MaskFacts:
+    """What one mask tensor (and one tensor of causal lengths) adds to the layout metadata.
+
+    A pair of blocks whose mask block masks every position adds nothing to the output or to any gradient.  The
+    forward lists without those pairs and the records the backward kernels walk depend on the values of the
+    mask, so they are kept per mask: ``key`` names its memory, version counter, shape and dtype (an in-place
+    change of the mask bumps the version), ``refs`` keeps that memory from being handed out again while the
+    facts live.  A mask that changes through ``.data`` is not noticed, like a layout in the layout cache.
+    No counterpart in the reference, which visits every pair (blksprs/ops/flash_attention.py:1058-1175).
+    """
+
+    __slots__ = ("key", "refs", "sightings", "group_offsets", "group_records", "bwd_scratch", "bwd_stream")
+
+    def __init__(self, key, refs):
+        self.key, self.refs, self.sightings = key, refs, 0
+        self.group_offsets = self.group_records = self.bwd_scratch = self.bwd_stream = None
+
+
+def _tensor_identity(t: Tensor | None):
+    if t is None:
+        return None
+    # inference tensors have no version counter: never equal to anything seen before
+    version = object() if torch.is_inference(t) else t._version
+    return t.data_ptr(), version, tuple(t.shape), t.dtype
+
+
+def _mask_facts(layout_cache: dict, attention_layout: Tensor, mask: Tensor | None, mask_bytes: Tensor | None,
+                lengths: Tensor | None, dims: tuple[int, int, int, int, int]) -> _MaskFacts:
+    """The facts for this mask in ``layout_cache``, renewed when another mask (or another version) arrives.
+
+    The forward lists without dead pairs are built when a mask is seen for the second time in a row: a caller
+    that brings a new mask with every call never pays for lists it would use once.
+    """
+    holder = layout_cache.get("mask_facts")
+    if holder is None:
+        holder = layout_cache["mask_facts"] = CacheHolder()
+        finalize_layout_cache(layout_cache)
+    key = (_tensor_identity(mask), _tensor_identity(lengths))
+    facts = holder.cache.get("facts")
+    if facts is None or facts.key != key:
+        facts = holder.cache["facts"] = _MaskFacts(key, (mask, lengths))
+    facts.sightings += 1
+    if (facts.sightings == 2 and facts.group_offsets is None and mask_bytes is not None and mask_bytes.size(0) > 0
+            and "group_offsets" in layout_cache and not torch.cuda.is_current_stream_capturing()):
+        B, nq, nk, nh, nhv = dims
+        dead = torch.empty(mask_bytes.size(0), dtype=torch.uint8, device=mask_bytes.device)
+        with torch.cuda.device(dead.device):
+            _capi.call("bsa_attn_mask_dead", _capi.ptr(mask_bytes), mask_bytes.size(0), mask_bytes.size(-1),
+                       _capi.ptr(dead), _capi.stream(dead.device))
+        block_of_pair = layout_cache["packed_indices_mask"].reshape(B, nq, nk)
+        dead_pairs = (block_of_pair >= 0) & (dead != 0)[block_of_pair.clamp(min=0)]
+        live_layout = (attention_layout.reshape(B, nq, nk) != 0) & ~dead_pairs
+        facts.group_offsets, facts.group_records, _ = _build_forward_records(layout_cache, live_layout, B, nq, nk,
+                                                                             nh, nhv)
+    return facts
 
 
 class _Meta:
     """Everything the kernels need besides the differentiable tensors."""
 
-    __slots__ = ("cache", "dims", "sbs", "scale", "mask", "causal_lengths", "has_bias")
+    __slots__ = ("cache", "dims", "sbs", "scale", "mask", "causal_lengths", "has_bias", "facts")
 
 
 def _fill_args(meta: "_Meta", q, k, v, bias) -> _capi.AttnArgs:
@@ -277,6 +333,9 @@ def _fill_args(meta: "_Meta", q, k, v, bias) -> _capi.AttnArgs:
         a.group_offsets = c["group_offsets"].data_ptr()
         a.group_records = _capi.ptr(c["group_records"])
         a.group_size = c["group_size"]
+        if meta.facts is not None and meta.facts.group_offsets is not None:
+            a.group_offsets = meta.facts.group_offsets.data_ptr()
+            a.group_records = _capi.ptr(meta.facts.group_records)
     if meta.mask is not None:
         a.mask, a.pidx_mask = _capi.ptr(meta.mask), _capi.ptr(c["packed_indices_mask"])
         a.n_mask_blocks = meta.mask.size(0)
@@ -322,11 +381,20 @@ class _FlashAttention(torch.autograd.Function):
         # room for the records of the pairs that some score survives (built and used inside bsa_attn_bwd)
         n_layout_blocks = meta.cache["key_indices_i32"].numel()
         n_mask_blocks = meta.mask.size(0) if meta.mask is not None else 0
-        size = _capi.load().bsa_attn_bwd_scratch_bytes(B, nq, nk, n_layout_blocks, n_mask_blocks)
-        scratch = torch.empty(max(size, 16), dtype=torch.uint8, device=q.device)
+        size = max(_capi.load().bsa_attn_bwd_scratch_bytes(B, nq, nk, n_layout_blocks, n_mask_blocks), 16)
+        stream = _capi.stream(q.device)
+        facts = meta.facts
+        # the records depend on the layouts and on the values of the mask and of the causal lengths only: a
+        # later call on the same stream with the same ones reads what this call wrote
+        scratch = facts.bwd_scratch if facts is not None and facts.bwd_stream == stream else None
+        args.bwd_scratch_ready = 1 if scratch is not None and scratch.numel() == size else 0
+        if not args.bwd_scratch_ready:
+            scratch = torch.empty(size, dtype=torch.uint8, device=q.device)
         args.bwd_scratch, args.n_layout_blocks = scratch.data_ptr(), n_layout_blocks
         with torch.cuda.device(q.device):
-            _capi.call("bsa_attn_bwd", ctypes.byref(args), _capi.stream(q.device))
+            _capi.call("bsa_attn_bwd", ctypes.byref(args), stream)
+        if facts is not None and not args.bwd_scratch_ready and not torch.cuda.is_current_stream_capturing():
+            facts.bwd_scratch, facts.bwd_stream = scratch, stream
         grad_bias = dbias.to(bias.dtype) if meta.has_bias else None
         return dq, dk, dv, grad_bias, None
 
@@ -471,8 +539,11 @@ def flash_attention(q: BlksprsTensor, sparsity_layout_q: Tensor,
             layout_cache[name + "_i32"] = _as_index(layout_cache[name], torch.int32)
         if (n_seq_blocks_k < (1 << 28) and layout_cache["key_indices"].numel() < INT32_INDEX_MAX
                 and n_head_blocks_qk <= 2 and n_head_blocks_v <= 2 and sparsity_block_size == 64):
-            _build_forward_records(layout_cache, attention_layout, int(n_batches), int(n_seq_blocks_q),
-                                   int(n_seq_blocks_k), int(n_head_blocks_qk), int(n_head_blocks_v))
+            offsets, records, group_size = _build_forward_records(
+                layout_cache, attention_layout, int(n_batches), int(n_seq_blocks_q), int(n_seq_blocks_k),
+                int(n_head_blocks_qk), int(n_head_blocks_v))
+            layout_cache["group_offsets"], layout_cache["group_records"] = offsets, records
+            layout_cache["group_size"] = group_size
         finalize_layout_cache(layout_cache)
 
     meta = _Meta()
@@ -484,5 +555,6 @@ def flash_attention(q: BlksprsTensor, sparsity_layout_q: Tensor,
     meta.mask = mask_bytes
     meta.causal_lengths = lengths
     meta.has_bias = has_bias
+    meta.facts = _mask_facts(layout_cache, attention_layout, attention_mask, mask_bytes, lengths, meta.dims)
 
     return BlksprsTensor.wrap(_FlashAttention.apply(q, k, v, attention_bias, meta))

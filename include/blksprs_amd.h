@@ -290,6 +290,10 @@ typedef struct bsa_attn_args {
    * No counterpart in the reference, which visits every pair (blksprs/ops/flash_attention.py:1322-1330). */
   void *bwd_scratch;
   int64_t n_layout_blocks;
+  /* Non-zero: bwd_scratch still holds what an earlier bsa_attn_bwd call wrote for the same layouts, packed
+   * indices, head counts, mask values and causal lengths (the records depend on nothing else), and the call
+   * reads it without writing it again. */
+  int64_t bwd_scratch_ready;
 } bsa_attn_args;
 
 #define BSA_ATTN_RECORD_INTS 16
@@ -313,6 +317,14 @@ int bsa_attn_fwd_records(const bsa_attn_args *args, const int32_t *group_entries
  * Every block of `o` that is active in the output layout is written.
  */
 int bsa_attn_fwd(const bsa_attn_args *args, bsa_stream_t stream);
+
+/*
+ * dead[m] = 1 where block m of a compressed mask (one byte per element, 0 or 1; 64 x 64 blocks only) masks every
+ * position, else 0.  A pair whose mask block is dead adds nothing to the output or to any gradient, so a caller
+ * may drop it from the lists it hands to bsa_attn_fwd.  No counterpart in the reference, which visits every pair
+ * (blksprs/ops/flash_attention.py:1058-1175).
+ */
+int bsa_attn_mask_dead(const void *mask, int64_t n_mask_blocks, int32_t sbs, uint8_t *dead, bsa_stream_t stream);
 
 /* Size in bytes of bsa_attn_args.bwd_scratch for these sizes (16-byte aligned buffer). */
 size_t bsa_attn_bwd_scratch_bytes(int64_t B, int64_t nq, int64_t nk, int64_t n_layout_blocks, int64_t n_mask_blocks);

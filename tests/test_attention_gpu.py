@@ -355,3 +355,83 @@ def test_config4_full_size_against_sampled_oracle_rows_and_invariants(device):
         mass, want = dv_h.sum(1), go_h.sum(1)
         assert float((mass - want).abs().max()) <= 2e-2 * float(go_h.abs().sum(1).max())
         assert float(dk_h.sum(1).abs().max()) <= 2e-2 * float(dk_h.abs().sum(1).max())
+
+
+@pytest.mark.parametrize("use_causal", [False, True])
+def test_lists_kept_per_mask_follow_the_mask(device, use_causal):
+    """From the second call with one mask tensor on, the forward walks lists without the pairs whose mask block
+    masks everything and the backward reads the records of the call before.  Every call gives the bits of the
+    first one; a mask changed in place, another mask tensor and other causal lengths give what a fresh cache
+    gives."""
+    g = torch.Generator().manual_seed(21)
+    B, n, nh, sbs = 2, 8, 2, 64
+    la = orc.random_layout((B, n, n), 0.7, g, ensure_rows=True).to(device)
+    full = torch.ones((B, n, nh), dtype=torch.bool, device=device)
+    q, k, v = (rand_blocks(B * n * nh, sbs, torch.bfloat16, s).to(device) for s in (1, 2, 3))
+    lmask = la.clone()
+    lmask[0, 3] = False
+    n_mask = int(lmask.sum())
+
+    def new_mask(seed):
+        gm = torch.Generator().manual_seed(seed)
+        m = torch.rand((n_mask, sbs, sbs), generator=gm) < 0.4
+        m[torch.rand(n_mask, generator=gm) < 0.4] = True  # dead pairs
+        rows = torch.cumsum(lmask.reshape(-1).long().cpu(), 0).view(B, n, n)
+        m[rows[1, 1, -1]:rows[1, 2, -1]] = True  # a query block with nothing left (its blocks are contiguous)
+        return m.to(device)
+
+    def run(mask, lengths, cache):
+        qq, kk, vv = (t.clone().requires_grad_(True) for t in (q, k, v))
+        out = bs.ops.flash_attention(qq, full, kk, full, vv, full, la, sbs, attention_mask=mask,
+                                     sparsity_layout_mask=lmask, layout_cache=cache, causal_lengths=lengths)
+        out.backward(go)
+        return out.detach(), qq.grad, kk.grad, vv.grad
+
+    go = rand_blocks(B * n * nh, sbs, torch.bfloat16, 4).to(device)
+
+    def same(a, b):
+        for x, y in zip(a, b):
+            assert torch.equal(x, y)
+
+    lengths = torch.tensor([n * sbs, 5 * sbs - 7], device=device) if use_causal else None
+    cache = {}
+    mask = new_mask(1)
+    first = run(mask, lengths, cache)
+    facts = cache["mask_facts"].cache["facts"]
+    assert facts.group_offsets is None and facts.bwd_scratch is not None
+    same(run(mask, lengths, cache), first)
+    assert cache["mask_facts"].cache["facts"] is facts and facts.group_offsets is not None
+    assert int(facts.group_offsets[-1]) < int(cache["group_offsets"][-1])
+    same(run(mask, lengths, cache), first)
+    same(run(mask, lengths, {}), first)
+
+    mask[::2] = False  # in place: the version counter moves
+    changed = run(mask, lengths, cache)
+    assert cache["mask_facts"].cache["facts"] is not facts
+    fresh = run(mask, lengths, {})
+    assert not torch.equal(changed[0], first[0])
+    same(changed, fresh)
+    same(run(mask, lengths, cache), fresh)
+    same(run(mask, lengths, cache), fresh)
+
+    other = new_mask(2)
+    same(run(other, lengths, cache), run(other, lengths, {}))
+    same(run(other, lengths, cache), run(other, lengths, {}))
+    if use_causal:
+        shorter = torch.tensor([3 * sbs + 1, n * sbs], device=device)
+        same(run(other, shorter, cache), run(other, shorter, {}))
+        same(run(other, shorter, cache), run(other, shorter, {}))
+        shorter[0] = 2 * sbs  # in place
+        same(run(other, shorter, cache), run(other, shorter, {}))
+
+    # against the oracle, with the lists of the second sighting
+    ref_q, ref_k, ref_v = (t.cpu().double().requires_grad_(True) for t in (q, k, v))
+    ref = orc.flash_attention(ref_q, full.cpu().numpy(), ref_k, full.cpu().numpy(), ref_v, full.cpu().numpy(),
+                              la.cpu().numpy(), sbs, mask=other.cpu(), layout_mask=lmask.cpu().numpy(),
+                              causal_lengths=None if lengths is None else lengths.cpu(), acc_dtype=torch.float64)
+    ref.backward(go.cpu().double())
+    run(other, lengths, cache)
+    got = run(other, lengths, cache)
+    assert_close(got[0], ref, 2e-2, "O")
+    for name, a, b in (("dQ", got[1], ref_q.grad), ("dK", got[2], ref_k.grad), ("dV", got[3], ref_v.grad)):
+        assert_close(a, b, 4e-2, name)

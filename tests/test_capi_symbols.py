@@ -27,9 +27,10 @@ def test_library_exports_every_declared_symbol():
 
 def test_argument_block_matches_the_header_layout():
     # 24 pointers, 11 int64, 3 int32 and one float, then 2 pointers and one int32 (padded to 8 bytes), a pointer
-    # and an int64
-    assert ctypes.sizeof(_capi.AttnArgs) == 24 * 8 + 11 * 8 + 4 * 4 + 2 * 8 + 8 + 2 * 8
+    # and two int64
+    assert ctypes.sizeof(_capi.AttnArgs) == 24 * 8 + 11 * 8 + 4 * 4 + 2 * 8 + 8 + 3 * 8
     assert _capi.AttnArgs.bwd_scratch.offset == 40 * 8 and _capi.AttnArgs.n_layout_blocks.offset == 41 * 8
+    assert _capi.AttnArgs.bwd_scratch_ready.offset == 42 * 8
     assert _capi.AttnArgs.group_offsets.offset == 37 * 8 and _capi.AttnArgs.group_size.offset == 39 * 8
     assert _capi.AttnArgs.sbs.offset == 35 * 8
 
