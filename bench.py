@@ -40,7 +40,7 @@ PEAK_MFMA_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}
 TRAFFIC_KIB = {  # config: (FETCH_SIZE, WRITE_SIZE)
     "c1": (616.2, 476.0),
     "c2": (484866.8, 514960.3),
-    "c3": (148176.3, 296129.7),
+    "c3": (148153.3, 296259.0),
     "c4": (238469.4, 133139.0),
     "c5": (30070.4, 143960.0),
     "v1": (66312.1, 129576.0),

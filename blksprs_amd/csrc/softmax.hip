@@ -13,12 +13,13 @@
 namespace {
 
 constexpr int kMaxUnits = 32;
+constexpr int kWaves = 4;  // waves (tasks) per workgroup
 
 struct RowGeom {
   int sbs_log2;
   int lpr;       // lanes per element row = min(64, sbs/4)
   int nq_log2;   // float4 units per lane per block = max(1, sbs/256), as log2
-  int groups;    // wave tasks per block row = sbs * lpr / 64
+  int groups_log2;  // wave tasks per block row = sbs * lpr / 64, as log2
 };
 
 __device__ inline float lanes_max(float v, int lpr) {
@@ -30,20 +31,28 @@ __device__ inline float lanes_sum(float v, int lpr) {
   return v;
 }
 
-// float offset of unit u of this lane, relative to the first block of the row
-__device__ inline int64_t unit_offset(int u, const RowGeom &g, int64_t lane_base) {
+// float offset of unit u, relative to the first block of the row and to the lane's own offset (the same for every
+// lane: the compiler keeps it in scalar registers)
+__device__ inline int64_t unit_offset(int u, const RowGeom &g) {
   const int t = u >> g.nq_log2;
   const int q = u & ((1 << g.nq_log2) - 1);
-  return ((int64_t)t << (2 * g.sbs_log2)) + lane_base + q * 256;
+  return ((int64_t)t << (2 * g.sbs_log2)) + q * 256;
 }
 
+// What this wave works on: `first` (float offset of the row's first block), `units` (float4 units per lane) and the
+// task index are the same for all lanes and are computed from values the compiler knows to be wave-uniform, so
+// the loops over units branch on scalar registers instead of masking lanes.
 __device__ inline bool wave_task(const RowGeom &g, const int32_t *row_offsets, int64_t n_tasks, int64_t &first,
-                                 int &units, int64_t &lane_base) {
-  const int64_t wave = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
-  if (wave >= n_tasks) return false;
+                                 int &units, int &lane_base) {
+  // Workgroup b runs on XCD b % 8: each XCD takes a contiguous eighth of the tasks, so the waves that read
+  // neighbouring KiB of the same blocks (the tasks of one block row) share one L2.
+  const int64_t n_groups = (n_tasks + kWaves - 1) / kWaves, per_xcd = (n_groups + 7) >> 3;
+  const int64_t group = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  const int64_t wave = group * kWaves + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  if (group >= n_groups || wave >= n_tasks) return false;
   const int lane = threadIdx.x & 63;
-  const int64_t r = wave / g.groups;
-  const int grp = (int)(wave % g.groups);
+  const int64_t r = wave >> g.groups_log2;
+  const int grp = (int)(wave & ((1 << g.groups_log2) - 1));
   const int start = row_offsets[r];
   const int count = row_offsets[r + 1] - start;
   if (count <= 0) return false;
@@ -51,7 +60,7 @@ __device__ inline bool wave_task(const RowGeom &g, const int32_t *row_offsets, i
   units = count << g.nq_log2;
   const int rows_per_wave = 64 / g.lpr;
   const int row_in_block = grp * rows_per_wave + lane / g.lpr;
-  lane_base = ((int64_t)row_in_block << g.sbs_log2) + (lane % g.lpr) * 4;
+  lane_base = (row_in_block << g.sbs_log2) + (lane % g.lpr) * 4;
   return true;
 }
 
@@ -62,41 +71,72 @@ __device__ inline void store_streaming(float *p, float4 o) {
   __builtin_nontemporal_store(f32x4_t{o.x, o.y, o.z, o.w}, reinterpret_cast<f32x4_t *>(p));
 }
 
-// e^d for d <= 0 through the hardware's 2^x: one multiplication and one transcendental instruction.  The rounded
-// argument d * log2(e) limits the relative accuracy to about |d| * 1e-7, far inside the 1e-5 the operation is
-// held to; the library routine costs five times the instructions, which made the kernel compute-bound.
-__device__ inline float exp_of(float d) { return __builtin_amdgcn_exp2f(d * 1.44269504088896341f); }
+// e^(v - m) through the hardware's 2^x as 2^(v * log2(e) - m2) with m2 = m * log2(e): one fused multiply-add and
+// one transcendental instruction per element.  The rounding of m2 is a factor common to every element of the
+// row and cancels against the row sum; what is left is the rounding of the exponent's argument, a relative
+// error of about |v - m| * 1e-7, far inside the 1e-5 the operation is held to.  (The library's expf costs ten
+// times the instructions, which made the kernel compute-bound.)
+constexpr float kLog2e = 1.44269504088896341f;
+__device__ inline float exp_rel(float v, float m2) { return __builtin_amdgcn_exp2f(__builtin_fmaf(v, kLog2e, -m2)); }
+__device__ inline float exp2_of(float d) { return __builtin_amdgcn_exp2f(d); }
 
 __device__ inline float max4(float4 v) { return fmaxf(fmaxf(v.x, v.y), fmaxf(v.z, v.w)); }
 
-__global__ __launch_bounds__(256) void softmax_fwd_kernel(const float *__restrict__ x, float *__restrict__ out,
+// max(m, v.x, v.y, v.z, v.w) in two instructions.  fmaxf first quiets signalling NaNs (one more instruction per
+// operand); here a NaN may come out either way: it reaches every output of the row through the exponentials.
+__device__ inline float max_with(float m, float4 v) {
+  float t;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(t) : "v"(v.x), "v"(v.y), "v"(v.z));
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(t) : "v"(t), "v"(v.w), "v"(m));
+  return t;
+}
+
+// Loads units [0, units) of a row into v, four at a time: within a group of four the index is clamped to the last
+// unit (a repeated load of a line just fetched) so that the group has no branch, and no load is followed by its
+// use: all loads of the row are in flight together.  Entries at and beyond `units` hold copies of the last unit.
+template <int N>
+__device__ inline void load_row(float4 (&v)[N], const float *row, int units, const RowGeom &g) {
+#pragma unroll
+  for (int c = 0; c < N; c += 4) {
+    if (c < units) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int u = c + j < units ? c + j : units - 1;
+        v[c + j] = *reinterpret_cast<const float4 *>(row + unit_offset(u, g));
+      }
+    }
+  }
+}
+
+__global__ __launch_bounds__(64 * kWaves) void softmax_fwd_kernel(const float *__restrict__ x, float *__restrict__ out,
                                                           const int32_t *__restrict__ row_offsets, int64_t n_tasks,
                                                           RowGeom g) {
-  int64_t first, lane_base;
-  int units;
+  int64_t first;
+  int units, lane_base;
   if (!wave_task(g, row_offsets, n_tasks, first, units, lane_base)) return;
-  const float *xr = x + first;
-  float *orow = out + first;
+  const float *xr = x + first + lane_base;
+  float *orow = out + first + lane_base;
 
   if (units <= kMaxUnits) {
     float4 v[kMaxUnits];
+    load_row(v, xr, units, g);
     float m = -INFINITY;
 #pragma unroll
-    for (int u = 0; u < kMaxUnits; ++u) {
-      if (u < units) {
-        v[u] = *reinterpret_cast<const float4 *>(xr + unit_offset(u, g, lane_base));
-        m = fmaxf(m, max4(v[u]));
+    for (int c = 0; c < kMaxUnits; c += 4) {
+      if (c < units) {  // the copies of the last unit change no maximum
+#pragma unroll
+        for (int j = 0; j < 4; ++j) m = max_with(m, v[c + j]);
       }
     }
-    m = lanes_max(m, g.lpr);
+    const float m2 = lanes_max(m, g.lpr) * kLog2e;
     float s = 0.f;
 #pragma unroll
     for (int u = 0; u < kMaxUnits; ++u) {
       if (u < units) {
-        v[u].x = exp_of(v[u].x - m);
-        v[u].y = exp_of(v[u].y - m);
-        v[u].z = exp_of(v[u].z - m);
-        v[u].w = exp_of(v[u].w - m);
+        v[u].x = exp_rel(v[u].x, m2);
+        v[u].y = exp_rel(v[u].y, m2);
+        v[u].z = exp_rel(v[u].z, m2);
+        v[u].w = exp_rel(v[u].w, m2);
         s += (v[u].x + v[u].y) + (v[u].z + v[u].w);
       }
     }
@@ -110,7 +150,7 @@ __global__ __launch_bounds__(256) void softmax_fwd_kernel(const float *__restric
         o.y = v[u].y * inv;
         o.z = v[u].z * inv;
         o.w = v[u].w * inv;
-        store_streaming(orow + unit_offset(u, g, lane_base), o);
+        store_streaming(orow + unit_offset(u, g), o);
       }
     }
     return;
@@ -119,54 +159,54 @@ __global__ __launch_bounds__(256) void softmax_fwd_kernel(const float *__restric
   // long rows: max pass, sum pass folded into one online pass, then the write pass
   float m = -INFINITY, s = 0.f;
   for (int u = 0; u < units; ++u) {
-    const float4 v = *reinterpret_cast<const float4 *>(xr + unit_offset(u, g, lane_base));
+    const float4 v = *reinterpret_cast<const float4 *>(xr + unit_offset(u, g));
     const float mn = fmaxf(m, max4(v));
     if (mn != -INFINITY) {
-      s = s * exp_of(m - mn) + (exp_of(v.x - mn) + exp_of(v.y - mn)) + (exp_of(v.z - mn) + exp_of(v.w - mn));
+      const float mn2 = mn * kLog2e;
+      s = s * exp2_of(m * kLog2e - mn2) + (exp_rel(v.x, mn2) + exp_rel(v.y, mn2)) +
+          (exp_rel(v.z, mn2) + exp_rel(v.w, mn2));
     } else if (v.x != v.x || v.y != v.y || v.z != v.z || v.w != v.w) {
       s = NAN;  // fmaxf drops NaN; keep it visible in the sum
     }
     m = mn;
   }
   const float mall = lanes_max(m, g.lpr);
-  float part = (m == -INFINITY) ? ((s != s) ? s : 0.f) : s * exp_of(m - mall);
+  const float mall2 = mall * kLog2e;
+  float part = (m == -INFINITY) ? ((s != s) ? s : 0.f) : s * exp2_of(m * kLog2e - mall2);
   const float sall = lanes_sum(part, g.lpr);
   const float inv_all = 1.f / sall;
   for (int u = 0; u < units; ++u) {
-    const int64_t off = unit_offset(u, g, lane_base);
+    const int64_t off = unit_offset(u, g);
     const float4 v = *reinterpret_cast<const float4 *>(xr + off);
     float4 o;
-    o.x = exp_of(v.x - mall) * inv_all;
-    o.y = exp_of(v.y - mall) * inv_all;
-    o.z = exp_of(v.z - mall) * inv_all;
-    o.w = exp_of(v.w - mall) * inv_all;
+    o.x = exp_rel(v.x, mall2) * inv_all;
+    o.y = exp_rel(v.y, mall2) * inv_all;
+    o.z = exp_rel(v.z, mall2) * inv_all;
+    o.w = exp_rel(v.w, mall2) * inv_all;
     store_streaming(orow + off, o);
   }
 }
 
-__global__ __launch_bounds__(256) void softmax_bwd_kernel(const float *__restrict__ grad_out,
+__global__ __launch_bounds__(64 * kWaves) void softmax_bwd_kernel(const float *__restrict__ grad_out,
                                                           const float *__restrict__ y, float *__restrict__ grad_in,
                                                           const int32_t *__restrict__ row_offsets, int64_t n_tasks,
                                                           RowGeom g) {
-  int64_t first, lane_base;
-  int units;
+  int64_t first;
+  int units, lane_base;
   if (!wave_task(g, row_offsets, n_tasks, first, units, lane_base)) return;
-  const float *gr = grad_out + first;
-  const float *yr = y + first;
-  float *dr = grad_in + first;
+  const float *gr = grad_out + first + lane_base;
+  const float *yr = y + first + lane_base;
+  float *dr = grad_in + first + lane_base;
 
   if (units <= kMaxUnits / 2) {
     constexpr int kU = kMaxUnits / 2;
     float4 yv[kU], gv[kU];
+    load_row(yv, yr, units, g);
+    load_row(gv, gr, units, g);
     float s = 0.f;
 #pragma unroll
     for (int u = 0; u < kU; ++u) {
-      if (u < units) {
-        const int64_t off = unit_offset(u, g, lane_base);
-        yv[u] = *reinterpret_cast<const float4 *>(yr + off);
-        gv[u] = *reinterpret_cast<const float4 *>(gr + off);
-        s += (yv[u].x * gv[u].x + yv[u].y * gv[u].y) + (yv[u].z * gv[u].z + yv[u].w * gv[u].w);
-      }
+      if (u < units) s += (yv[u].x * gv[u].x + yv[u].y * gv[u].y) + (yv[u].z * gv[u].z + yv[u].w * gv[u].w);
     }
     s = lanes_sum(s, g.lpr);
 #pragma unroll
@@ -177,7 +217,7 @@ __global__ __launch_bounds__(256) void softmax_bwd_kernel(const float *__restric
         o.y = yv[u].y * (gv[u].y - s);
         o.z = yv[u].z * (gv[u].z - s);
         o.w = yv[u].w * (gv[u].w - s);
-        store_streaming(dr + unit_offset(u, g, lane_base), o);
+        store_streaming(dr + unit_offset(u, g), o);
       }
     }
     return;
@@ -185,14 +225,14 @@ __global__ __launch_bounds__(256) void softmax_bwd_kernel(const float *__restric
 
   float s = 0.f;
   for (int u = 0; u < units; ++u) {
-    const int64_t off = unit_offset(u, g, lane_base);
+    const int64_t off = unit_offset(u, g);
     const float4 yv = *reinterpret_cast<const float4 *>(yr + off);
     const float4 gv = *reinterpret_cast<const float4 *>(gr + off);
     s += (yv.x * gv.x + yv.y * gv.y) + (yv.z * gv.z + yv.w * gv.w);
   }
   s = lanes_sum(s, g.lpr);
   for (int u = 0; u < units; ++u) {
-    const int64_t off = unit_offset(u, g, lane_base);
+    const int64_t off = unit_offset(u, g);
     const float4 yv = *reinterpret_cast<const float4 *>(yr + off);
     const float4 gv = *reinterpret_cast<const float4 *>(gr + off);
     float4 o;
@@ -213,7 +253,8 @@ int make_geom(const char *who, int sbs, RowGeom &g) {
   int nq = sbs / 256 > 1 ? sbs / 256 : 1;
   g.nq_log2 = 0;
   while ((1 << g.nq_log2) < nq) ++g.nq_log2;
-  g.groups = sbs * g.lpr / 64;
+  g.groups_log2 = 0;
+  while ((1 << g.groups_log2) < sbs * g.lpr / 64) ++g.groups_log2;
   return BSA_OK;
 }
 
@@ -230,10 +271,10 @@ extern "C" int bsa_softmax_fwd(const float *x, float *out, const int32_t *row_of
   BSA_REQUIRE(x && out && row_offsets, "bsa_softmax_fwd: NULL pointer");
   BSA_REQUIRE(aligned16(x) && aligned16(out), "bsa_softmax_fwd: buffers must be 16-byte aligned");
   if (nnz > 0x7fffffffLL) return bsa::fail(BSA_ELIMIT, "bsa_softmax_fwd: more than 2^31-1 blocks");
-  const int64_t n_tasks = n_rows * g.groups;
-  const int64_t blocks = bsa::cdiv(n_tasks, 4);
+  const int64_t n_tasks = n_rows << g.groups_log2;
+  const int64_t blocks = bsa::cdiv(bsa::cdiv(n_tasks, kWaves), 8) * 8;  // a whole number of workgroups per XCD
   if (blocks > 0x7fffffffLL) return bsa::fail(BSA_ELIMIT, "bsa_softmax_fwd: too many rows");
-  softmax_fwd_kernel<<<(unsigned)blocks, 256, 0, bsa::as_stream(stream)>>>(x, out, row_offsets, n_tasks, g);
+  softmax_fwd_kernel<<<(unsigned)blocks, 64 * kWaves, 0, bsa::as_stream(stream)>>>(x, out, row_offsets, n_tasks, g);
   return bsa::check_launch("softmax_fwd_kernel");
 }
 
@@ -247,10 +288,10 @@ extern "C" int bsa_softmax_bwd(const float *grad_out, const float *y, float *gra
   BSA_REQUIRE(aligned16(grad_out) && aligned16(y) && aligned16(grad_in),
               "bsa_softmax_bwd: buffers must be 16-byte aligned");
   if (nnz > 0x7fffffffLL) return bsa::fail(BSA_ELIMIT, "bsa_softmax_bwd: more than 2^31-1 blocks");
-  const int64_t n_tasks = n_rows * g.groups;
-  const int64_t blocks = bsa::cdiv(n_tasks, 4);
+  const int64_t n_tasks = n_rows << g.groups_log2;
+  const int64_t blocks = bsa::cdiv(bsa::cdiv(n_tasks, kWaves), 8) * 8;  // a whole number of workgroups per XCD
   if (blocks > 0x7fffffffLL) return bsa::fail(BSA_ELIMIT, "bsa_softmax_bwd: too many rows");
-  softmax_bwd_kernel<<<(unsigned)blocks, 256, 0, bsa::as_stream(stream)>>>(grad_out, y, grad_in, row_offsets,
+  softmax_bwd_kernel<<<(unsigned)blocks, 64 * kWaves, 0, bsa::as_stream(stream)>>>(grad_out, y, grad_in, row_offsets,
                                                                            n_tasks, g);
   return bsa::check_launch("softmax_bwd_kernel");
 }
