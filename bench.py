@@ -42,7 +42,7 @@ TRAFFIC_KIB = {  # config: (FETCH_SIZE, WRITE_SIZE)
     "c2": (484866.8, 514960.3),
     "c3": (148153.3, 296259.0),
     "c4": (238469.4, 133139.0),
-    "c5": (30070.4, 143960.0),
+    "c5": (28438.4, 143960.0),
     "v1": (66312.1, 129576.0),
     "v2": (66851.5, 524499.4),
     "t1": (67086.4, 129576.0),
@@ -82,24 +82,59 @@ def _events(n):
     return [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
 
 
+def _sleep_cycles_per_ms():
+    """How many cycles of torch.cuda._sleep make one millisecond on this card."""
+    probe = 2_000_000
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda._sleep(probe)
+    torch.cuda.synchronize()
+    a.record()
+    torch.cuda._sleep(probe)
+    b.record()
+    torch.cuda.synchronize()
+    return probe / max(a.elapsed_time(b), 1e-3)
+
+
 def time_steps(step, steps, warmup):
-    """Returns (wall ms per step over exactly `steps` steps, mean per-launch ms from stream events)."""
+    """Returns (wall ms per step over exactly `steps` steps, mean and median per-launch ms from stream events).
+
+    The per-launch figure must not contain the time the card waits for the host: a step whose kernels are
+    shorter than the host's work per call leaves the stream empty between launches, and an event recorded on an
+    empty stream fires at once, long before the kernel behind it is enqueued.  When the host is the slower side,
+    the timed launches are therefore enqueued in chunks behind a short delay kernel, so that every event pair
+    brackets kernels that are already waiting in the stream.  (Not otherwise: the card clocks down during the
+    delays, which slows a long kernel.)
+    """
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):
         step()
+    host_ms = (time.perf_counter() - t0) * 1e3 / steps  # what the host needs to enqueue a step
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
     ev = _events(steps)
-    for s, e in ev:
-        s.record()
-        step()
-        e.record()
-    torch.cuda.synchronize()
+    if host_ms < 0.7 * wall_ms:
+        # the card is the slower side: the stream never runs empty, events between the steps see the kernels only
+        for s, e in ev:
+            s.record()
+            step()
+            e.record()
+        torch.cuda.synchronize()
+    else:
+        per_ms = _sleep_cycles_per_ms()
+        chunk = 20
+        for c in range(0, steps, chunk):
+            # long enough for the host to enqueue the whole chunk (the wall time per step bounds its work per step)
+            torch.cuda._sleep(int(per_ms * (1.0 + 2.0 * wall_ms * chunk)))
+            for s, e in ev[c:c + chunk]:
+                s.record()
+                step()
+                e.record()
+            torch.cuda.synchronize()
     per = sorted(s.elapsed_time(e) for s, e in ev)
-    return wall_ms, sum(per) / len(per), per[len(per) // 2]
+    return wall_ms, sum(per) / len(per), per[len(per) // 2], host_ms
 
 
 # --------------------------------------------------------------------------- workloads
@@ -484,7 +519,7 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     w = make_workload(args.config, dev)
-    wall_ms, mean_ms, median_ms = time_steps(w["step"], args.steps, args.warmup)
+    wall_ms, mean_ms, median_ms, host_ms = time_steps(w["step"], args.steps, args.warmup)
     tflops = w["flops"] / (wall_ms * 1e-3) / 1e12
     gbs = w["alg_bytes"] / (mean_ms * 1e-3) / 1e9
     if w["bound"] == "hbm":
@@ -505,6 +540,7 @@ def main():
     roofline["kernel"] = w["kernel"]
     roofline["launch_ms_mean"] = round(mean_ms, 4)
     roofline["launch_ms_median"] = round(median_ms, 4)
+    roofline["host_ms_per_step"] = round(host_ms, 4)  # what the host needs to enqueue one step
     line = {
         "metric": "effective TFLOP/s on nonzero blocks" if w["flops"] else "achieved GB/s on nonzero blocks",
         "value": round(tflops, 3) if w["flops"] else round(gbs, 1),

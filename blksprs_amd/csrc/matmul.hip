@@ -449,9 +449,11 @@ __global__ __launch_bounds__(256) void matmul_small_kernel(const typename Tr::st
 // whose pairs are one contiguous range of the pair list: it reads that range and the run's offsets once (one
 // entry per lane), then walks the pairs with the operand loads of the next two pairs in flight.
 // The product is formed transposed (A = y fragment, B = x fragment), which leaves four consecutive output columns
-// of one row in each lane: the wave's 8-byte stores cover the whole output block.  An operand whose contraction
-// index is contiguous in memory (x, or y when it is used transposed) is loaded straight into its fragment; the
-// other one passes through 512 bytes of LDS and comes back through the transposing read.
+// of one row in each lane: the wave's 8-byte stores cover the whole output block.  One 16-byte load per lane
+// fetches both operand blocks of a pair (lanes 0-31 the x block, lanes 32-63 the y block: one memory instruction
+// per pair instead of two, which is what the kernel's time follows); both pass through 1 KiB of LDS, from which
+// an operand whose contraction index is contiguous in memory (x, or y when it is used transposed) is read as it
+// lies and the other one through the transposing read.
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 typedef short i16x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
@@ -473,7 +475,14 @@ struct F16Small {
   }
 };
 
+constexpr int kSmallDepth = 2;    // pairs whose operand loads are in flight
 constexpr int kSmallRunMax = 63;  // output blocks per wave: their offsets (one more) fit one entry per lane
+
+// The output of a run as a buffer resource: the block's byte offset travels in a scalar register (`soffset`) and
+// the lane's offset inside a block is a constant, so a store needs no per-lane address arithmetic.
+__device__ inline __amdgpu_buffer_rsrc_t small_resource(const char *base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(base), 0, (int)bytes, 0x00020000);
+}
 
 template <typename Ts, bool XT, bool YT>
 __global__ __launch_bounds__(256) void matmul_small16_kernel(const char *__restrict__ x, const char *__restrict__ y,
@@ -481,8 +490,10 @@ __global__ __launch_bounds__(256) void matmul_small16_kernel(const char *__restr
                                                              const int32_t *__restrict__ pair_offsets,
                                                              const int32_t *__restrict__ pairs, int64_t nnz_o,
                                                              int64_t nnz_x, int64_t nnz_y, int run) {
-  __shared__ __attribute__((aligned(16))) char stage[4][512];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  __shared__ __attribute__((aligned(16))) char stage[4][1024];  // per wave: the x block, then the y block
+  const int lane = threadIdx.x & 63;
+  // everything that steers the loops below is built from values the compiler knows to be the same in all lanes
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   // workgroup g runs on XCD g % 8: every XCD takes a contiguous eighth of the runs, so that the operand blocks in
   // flight on one L2 belong to few batch entries
   const int64_t group = (int64_t)(blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
@@ -491,38 +502,17 @@ __global__ __launch_bounds__(256) void matmul_small16_kernel(const char *__restr
   const int count = (int)(nnz_o - n0 < run ? nnz_o - n0 : run);
   // fragment of a k-contiguous operand: row lane % 16, values 4 (lane / 16) .. + 3
   const int direct_off = (lane & 15) * 32 + (lane >> 4) * 8;
-  // the other operand is copied as it lies (lane l moves bytes 8 l .. 8 l + 7) and read back transposed: inside
-  // a group of 16 lanes, lane s points at row 4 (lane / 16) + s / 4, values 4 (s % 4) .. + 3
+  // the other operand is read transposed: inside a group of 16 lanes, lane s points at row
+  // 4 (lane / 16) + s / 4, values 4 (s % 4) .. + 3
   const int turned_off = (4 * (lane >> 4) + ((lane & 15) >> 2)) * 32 + (lane & 3) * 8;
   char *slot = stage[wave];
+  const uint32_t nx = (uint32_t)nnz_x, ny = (uint32_t)nnz_y;  // the pair list holds 32-bit indices
+  const __amdgpu_buffer_rsrc_t ro = small_resource(out + n0 * 512, (uint32_t)count * 512u);
 
-  // offsets of the run (count + 1 of them) and the first 64 pairs
+  // offsets of the run (count + 1 of them), one per lane
   const int off_win = pair_offsets[n0 + (lane <= count ? lane : count)];
   const int p_first = __builtin_amdgcn_readlane(off_win, 0);
   const int p_last = __builtin_amdgcn_readlane(off_win, count);
-  int win_base = p_first;
-  u32x2 win{0u, 0u};
-  auto load_window = [&]() {
-    if (win_base + lane < p_last) win = *reinterpret_cast<const u32x2 *>(pairs + 2 * (int64_t)(win_base + lane));
-  };
-  load_window();
-
-  auto issue = [&](int p, u32x2 &xr, u32x2 &yr) {
-    // p is inside the window (the caller moves the window first)
-    int64_t px = __builtin_amdgcn_readlane((int)win[0], p - win_base);
-    int64_t py = __builtin_amdgcn_readlane((int)win[1], p - win_base);
-    if (px < 0 || px >= nnz_x) px = 0;
-    if (py < 0 || py >= nnz_y) py = 0;
-    xr = *reinterpret_cast<const u32x2 *>(x + px * 512 + (XT ? lane * 8 : direct_off));
-    yr = *reinterpret_cast<const u32x2 *>(y + py * 512 + (YT ? direct_off : lane * 8));
-  };
-  auto turned = [&](u32x2 v) {
-    *reinterpret_cast<u32x2 *>(slot + lane * 8) = v;
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    const i16x4 t = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4 *)(slot + turned_off));
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    return __builtin_bit_cast(u32x2, t);
-  };
 
   f32x4 acc{0.f, 0.f, 0.f, 0.f};
   int done = 0;                                           // output blocks of the run already stored
@@ -533,35 +523,52 @@ __global__ __launch_bounds__(256) void matmul_small16_kernel(const char *__restr
       u32x2 w;
       w[0] = Ts::pack2(acc[0], acc[1]);
       w[1] = Ts::pack2(acc[2], acc[3]);
-      *reinterpret_cast<u32x2 *>(out + (n0 + done) * 512 + direct_off) = w;
+      // written once, not read back by this kernel: past the caches
+      __builtin_amdgcn_raw_buffer_store_b64(w, ro, direct_off, done * 512, 2);
       acc = f32x4{0.f, 0.f, 0.f, 0.f};
       ++done;
       block_end = __builtin_amdgcn_readlane(off_win, done + 1 <= count ? done + 1 : count);
     }
   };
 
-  int p = p_first;
-  u32x2 xa{0u, 0u}, ya{0u, 0u}, xb{0u, 0u}, yb{0u, 0u};
-  if (p < p_last) issue(p, xa, ya);
-  if (p + 1 < p_last) issue(p + 1, xb, yb);
-  auto step = [&](u32x2 &xr, u32x2 &yr) {
-    flush_until(p);
-    const u32x2 fx = XT ? turned(xr) : xr;
-    const u32x2 fy = YT ? yr : turned(yr);
-    acc = Ts::mfma(fy, fx, acc);
-    if (p + 2 < p_last) {
-      if (p + 2 - win_base >= 64) {
-        win_base = p + 2;
-        load_window();
+  // the pairs of the run, 64 at a time: one entry per lane, handed out with readlane
+  for (int base = p_first; base < p_last; base += 64) {
+    const int n = p_last - base < 64 ? p_last - base : 64;
+    u32x2 win{0u, 0u};
+    if (lane < n) win = *reinterpret_cast<const u32x2 *>(pairs + 2 * (int64_t)(base + lane));
+    auto issue = [&](int i, u32x4 &xy) {
+      // past the end: the last pair again (a cache hit), so that every step issues the same loads and the
+      // compiler can count the loads in flight instead of waiting for all of them in front of every use
+      const int at = i < n ? i : n - 1;
+      const uint32_t px = (uint32_t)__builtin_amdgcn_readlane((int)win[0], at);
+      const uint32_t py = (uint32_t)__builtin_amdgcn_readlane((int)win[1], at);
+      // a corrupt list must not turn into a wild read: such a pair reads block 0
+      const char *xb = x + (int64_t)(px < nx ? px : 0) * 512;
+      const char *yb = y + (int64_t)(py < ny ? py : 0) * 512;
+      const char *mine = (lane < 32 ? xb : yb) + (lane & 31) * 16;
+      xy = *reinterpret_cast<const u32x4 *>(mine);
+    };
+    u32x4 xys[kSmallDepth];
+#pragma unroll
+    for (int d = 0; d < kSmallDepth; ++d) issue(d, xys[d]);
+    for (int i = 0; i < n; i += kSmallDepth) {
+#pragma unroll
+      for (int d = 0; d < kSmallDepth; ++d) {
+        if (i + d < n) {
+          flush_until(base + i + d);
+          *reinterpret_cast<u32x4 *>(slot + lane * 16) = xys[d];
+          __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+          u32x2 fx, fy;
+          if (XT) fx = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4 *)(slot + turned_off)));
+          else fx = *reinterpret_cast<const u32x2 *>(slot + direct_off);
+          if (YT) fy = *reinterpret_cast<const u32x2 *>(slot + 512 + direct_off);
+          else fy = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4 *)(slot + 512 + turned_off)));
+          __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+          acc = Ts::mfma(fy, fx, acc);
+        }
+        issue(i + d + kSmallDepth, xys[d]);
       }
-      issue(p + 2, xr, yr);
     }
-    ++p;
-  };
-  while (p < p_last) {
-    step(xa, ya);
-    if (p >= p_last) break;
-    step(xb, yb);
   }
   flush_until(p_last);
 }
