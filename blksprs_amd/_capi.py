@@ -119,7 +119,8 @@ def ptr(t) -> int:
 
 def stream(device) -> int:
     """The current torch stream of ``device`` as a raw hipStream_t."""
-    return torch.cuda.current_stream(device).cuda_stream
+    index = device.index
+    return torch._C._cuda_getCurrentRawStream(torch.cuda.current_device() if index is None else index)
 
 
 def call(name: str, *args) -> None:

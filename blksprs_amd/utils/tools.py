@@ -246,14 +246,20 @@ def finalize_layout_cache(layout_cache: LayoutCache) -> LayoutCache:
 
 
 def _snapshot(layout_cache: LayoutCache) -> tuple:
-    return tuple((k, _entry_state(v)) for k, v in sorted(layout_cache.items()) if k not in _PRIVATE)
+    # in insertion order: builders only add entries, so an unchanged cache lists them in the same order
+    return tuple((k, _entry_state(v)) for k, v in layout_cache.items() if k not in _PRIVATE)
 
 
 def _entry_state(value):
     if isinstance(value, Tensor):
-        return _tensor_signature(value, object() if torch.is_inference(value) else int(value._version))
+        # a derived tensor is the same while it is the same object with the same version counter (this runs for
+        # every entry on every call: no more than that)
+        try:
+            return id(value), value._version
+        except RuntimeError:  # an inference tensor has no version counter: never equal to an earlier state
+            return object()
     if isinstance(value, dict):
-        return tuple((k, _entry_state(v)) for k, v in sorted(value.items()) if k not in _PRIVATE)
+        return tuple((k, _entry_state(v)) for k, v in value.items() if k not in _PRIVATE)
     if isinstance(value, (tuple, list, Size)):
         return tuple(_entry_state(v) for v in value)
     if isinstance(value, (PackedLayout, ContractionLists)):
