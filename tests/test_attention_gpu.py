@@ -357,6 +357,21 @@ def test_config4_full_size_against_sampled_oracle_rows_and_invariants(device):
         assert float(dk_h.sum(1).abs().max()) <= 2e-2 * float(dk_h.abs().sum(1).max())
 
 
+def test_mask_blocks_that_mask_everything_are_found(device):
+    import ctypes
+
+    from blksprs_amd import _capi
+    g = torch.Generator().manual_seed(3)
+    mask = (torch.rand((37, 64, 64), generator=g) < 0.5).to(device)
+    mask[::5] = True
+    mask[7, 63, 63] = False  # one open position keeps a block alive
+    mask[12] = True
+    dead = torch.full((37,), 7, dtype=torch.uint8, device=device)
+    _capi.call("bsa_attn_mask_dead", _capi.ptr(mask.view(torch.uint8)), 37, 64, _capi.ptr(dead), _capi.stream(device))
+    assert torch.equal(dead.bool(), mask.view(37, -1).all(dim=1))
+    assert not bool(dead[7]) and bool(dead[12]) and bool(dead[35])
+
+
 @pytest.mark.parametrize("use_causal", [False, True])
 def test_lists_kept_per_mask_follow_the_mask(device, use_causal):
     """From the second call with one mask tensor on, the forward walks lists without the pairs whose mask block

@@ -66,3 +66,7 @@ def test_bad_arguments_of_the_neighbouring_entry_points_are_rejected_on_the_host
     # scratch of the attention backward: 2 x 32 bytes per layout block, (4 + 64) per row, one per mask block
     assert lib.bsa_attn_bwd_scratch_bytes(2, 3, 5, 7, 11) == (2 * 32 * 7 + 68 * (2 * 3 + 2 * 5) + 11 + 15) // 16 * 16
     assert lib.bsa_attn_bwd_scratch_bytes(-1, 3, 5, 7, 11) == 0
+    # mask blocks that mask everything: 64 x 64 blocks only, no mask blocks is nothing to do
+    assert lib.bsa_attn_mask_dead(0, 1, 32, 0, 0) == -1 and b"64 x 64" in lib.bsa_last_error()
+    assert lib.bsa_attn_mask_dead(0, 1, 64, 0, 0) == -1 and b"NULL" in lib.bsa_last_error()
+    assert lib.bsa_attn_mask_dead(0, 0, 64, 0, 0) == 0

@@ -199,3 +199,31 @@ def test_row_panel_kernel_is_bit_identical_to_the_tile_kernel(device, dtype, dim
                y.size(0), sbs, _capi.DTYPE_CODES[dtype], 0, 0, _capi.stream(device))
     assert torch.equal(out, ref)
     assert_close(out, _oracle(x.cpu(), lx.cpu(), y.cpu(), ly.cpu(), lo.cpu(), sbs), 2e-2, "row panel vs oracle")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("trans", ["nn", "grads"])
+@pytest.mark.parametrize("dims,density", [
+    ((1, 3, 40, 5), 1.0),    # 40 pairs per output block: a run of 8 blocks spans several 64-pair windows
+    ((2, 9, 70, 9), 0.95),   # a single output block with more pairs than one window holds
+    ((3, 20, 4, 30), 0.3),   # many output blocks without any pair inside a run, runs that end mid-row
+    ((1, 1, 1, 1), 1.0),     # one block, one pair: a run shorter than the pipeline is deep
+])
+def test_sbs16_runs_and_pair_windows(device, dtype, trans, dims, density):
+    """The 16-bit sbs-16 kernel hands every wave a run of consecutive output blocks and walks their pairs 64
+    at a time with two loads in flight: runs whose pairs cross window boundaries, blocks without pairs, a run
+    shorter than the pipeline, and the transposed reads of the backward pass."""
+    sbs = 16
+    B, R, K, C = dims
+    lx, ly, lo, x, y = _problem(B, R, K, C, sbs, dtype, density, seed=R + K, product_layout=density >= 0.9)
+    xd, yd = x.to(device).requires_grad_(trans == "grads"), y.to(device).requires_grad_(trans == "grads")
+    out = bs.ops.matmul(xd, lx.to(device), yd, ly.to(device), lo.to(device), sbs)
+    x64, y64 = x.double().requires_grad_(True), y.double().requires_grad_(True)
+    ref = orc.matmul(x64, lx.numpy(), y64, ly.numpy(), lo.numpy(), sbs, acc_dtype=torch.float64)
+    assert_close(out, ref, TOL[dtype], f"sbs16 {dtype} {dims}")
+    if trans == "grads":
+        go = rand_blocks(int(lo.sum()), sbs, dtype, 99, 1.0 / math.sqrt(C * sbs))
+        out.backward(go.to(device))
+        ref.backward(go.double())
+        assert_close(xd.grad, x64.grad, 2 * TOL[dtype], "dX")   # x^T-free: go @ y^T reads y transposed
+        assert_close(yd.grad, y64.grad, 2 * TOL[dtype], "dY")   # x^T @ go reads x transposed
