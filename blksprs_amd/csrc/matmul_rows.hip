@@ -213,15 +213,24 @@ __global__ __launch_bounds__(kWaves * 64, 1) void matmul_rows_kernel(
     const char *__restrict__ x, const char *__restrict__ y, char *__restrict__ out,
     const int32_t *__restrict__ pair_offsets, const int32_t *__restrict__ pairs,
     const int32_t *__restrict__ x_row_offsets, const int32_t *__restrict__ o_row_offsets,
-    const int32_t *__restrict__ row_order, int n_rows, int64_t nnz_x, int64_t nnz_y) {
+    const int32_t *__restrict__ work_table, int parts_log2, int n_rows, int64_t nnz_x, int64_t nnz_y) {
   extern __shared__ __attribute__((aligned(16))) char rows_smem[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  if ((int)blockIdx.x >= n_rows) return;
-  int row = row_order ? row_order[blockIdx.x] : (int)blockIdx.x;
-  row = __builtin_amdgcn_readfirstlane(row);
-  if (row < 0 || row >= n_rows) return;  // a corrupt table must not turn into a wild read
-  const int n0 = o_row_offsets[row], n1 = o_row_offsets[row + 1];
+  // the grid has one workgroup per table entry: row << parts_log2 | part, or -1 for nothing
+  int item = work_table ? work_table[blockIdx.x] : (int)blockIdx.x;
+  item = __builtin_amdgcn_readfirstlane(item);
+  if (item < 0) return;
+  const int part = item & ((1 << parts_log2) - 1);
+  const int row = item >> parts_log2;
+  if (row >= n_rows) return;  // a corrupt table must not turn into a wild read
+  int n0 = o_row_offsets[row], n1 = o_row_offsets[row + 1];
+  if (parts_log2) {  // this workgroup's run of the row's output blocks
+    const int64_t len = n1 - n0;
+    const int first = n0 + (int)((len * part) >> parts_log2), last = n0 + (int)((len * (part + 1)) >> parts_log2);
+    n0 = first;
+    n1 = last;
+  }
   if (n0 >= n1) return;
   const int xs = x_row_offsets[row];
   int nx = x_row_offsets[row + 1] - xs;
@@ -444,17 +453,17 @@ __global__ __launch_bounds__(kWaves * 64, 1) void matmul_rows_kernel(
 
 template <typename Tr>
 int launch_rows(const void *x, const void *y, void *out, const int32_t *pair_offsets, const int32_t *pairs,
-                const int32_t *x_row_offsets, const int32_t *o_row_offsets, const int32_t *row_order,
-                int64_t n_rows, int64_t nnz_x, int64_t nnz_y, hipStream_t s) {
+                const int32_t *x_row_offsets, const int32_t *o_row_offsets, const int32_t *work_table,
+                int64_t n_items, int parts_log2, int64_t n_rows, int64_t nnz_x, int64_t nnz_y, hipStream_t s) {
   static bool configured = false;  // raising the dynamic LDS limit is per function, once per process
   if (!configured) {
     BSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&matmul_rows_kernel<Tr>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kRowsLds));
     configured = true;
   }
-  matmul_rows_kernel<Tr><<<(unsigned)n_rows, kWaves * 64, kRowsLds, s>>>(
+  matmul_rows_kernel<Tr><<<(unsigned)n_items, kWaves * 64, kRowsLds, s>>>(
       static_cast<const char *>(x), static_cast<const char *>(y), static_cast<char *>(out), pair_offsets, pairs,
-      x_row_offsets, o_row_offsets, row_order, (int)n_rows, nnz_x, nnz_y);
+      x_row_offsets, o_row_offsets, work_table, parts_log2, (int)n_rows, nnz_x, nnz_y);
   return bsa::check_launch("matmul_rows_kernel");
 }
 
@@ -464,19 +473,25 @@ bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 
 
 extern "C" int bsa_matmul_rows(const void *x, const void *y, void *out, const int32_t *pair_offsets,
                                const int32_t *pairs, const int32_t *x_row_offsets, const int32_t *o_row_offsets,
-                               const int32_t *row_order, int64_t n_rows, int64_t nnz_o, int64_t nnz_x,
-                               int64_t nnz_y, int sbs, int dtype, bsa_stream_t stream) {
+                               const int32_t *work_table, int64_t n_items, int parts_log2, int64_t n_rows,
+                               int64_t nnz_o, int64_t nnz_x, int64_t nnz_y, int sbs, int dtype,
+                               bsa_stream_t stream) {
   BSA_REQUIRE(sbs == 64, "bsa_matmul_rows: sbs must be 64 (got %d)", sbs);
   BSA_REQUIRE(dtype == BSA_F16 || dtype == BSA_BF16, "bsa_matmul_rows: dtype must be fp16 or bf16 (got %d)", dtype);
   BSA_REQUIRE(nnz_o >= 0 && nnz_x >= 0 && nnz_y >= 0 && n_rows >= 0, "bsa_matmul_rows: negative size");
   if (nnz_o == 0 || n_rows == 0) return BSA_OK;
   BSA_REQUIRE(out && pair_offsets && x_row_offsets && o_row_offsets, "bsa_matmul_rows: NULL pointer");
   BSA_REQUIRE(aligned16(x) && aligned16(y) && aligned16(out), "bsa_matmul_rows: buffers must be 16-byte aligned");
-  BSA_REQUIRE(n_rows < 0x7fffffffLL, "bsa_matmul_rows: too many block rows");
+  BSA_REQUIRE(parts_log2 >= 0 && parts_log2 <= 3, "bsa_matmul_rows: parts_log2 must be 0..3 (got %d)", parts_log2);
+  BSA_REQUIRE((n_rows << parts_log2) < 0x7fffffffLL, "bsa_matmul_rows: too many block rows");
+  BSA_REQUIRE(n_items >= 0 && n_items < 0x7fffffffLL, "bsa_matmul_rows: bad number of table entries");
+  BSA_REQUIRE(work_table != nullptr || (parts_log2 == 0 && n_items == n_rows),
+              "bsa_matmul_rows: without a work table the rows are taken whole and in order");
+  if (n_items == 0) return BSA_OK;
   hipStream_t s = bsa::as_stream(stream);
   if (dtype == BSA_BF16)
-    return launch_rows<MBf16>(x, y, out, pair_offsets, pairs, x_row_offsets, o_row_offsets, row_order, n_rows, nnz_x,
-                              nnz_y, s);
-  return launch_rows<MF16>(x, y, out, pair_offsets, pairs, x_row_offsets, o_row_offsets, row_order, n_rows, nnz_x,
-                           nnz_y, s);
+    return launch_rows<MBf16>(x, y, out, pair_offsets, pairs, x_row_offsets, o_row_offsets, work_table, n_items,
+                              parts_log2, n_rows, nnz_x, nnz_y, s);
+  return launch_rows<MF16>(x, y, out, pair_offsets, pairs, x_row_offsets, o_row_offsets, work_table, n_items,
+                           parts_log2, n_rows, nnz_x, nnz_y, s);
 }

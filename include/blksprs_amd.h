@@ -212,16 +212,21 @@ int bsa_matmul(const void *x, const void *y, void *out, const int32_t *pair_offs
  * The same product for fp16 / bf16 operands with sbs == 64, organised by output block row: the x
  * blocks of a row are kept in LDS while the row's output blocks are computed.  x_row_offsets and
  * o_row_offsets are the int32 CSR row offsets (n_rows + 1 entries, rows = B * R) of the x layout
- * and of the output layout as bsa_lut_packed(row_len = ...) writes them.  row_order (n_rows int32,
- * a permutation of the rows, or NULL for 0, 1, 2, ...) is the order in which rows are handed to
- * workgroups; rows sorted by descending number of pairs keep the tail of the launch short.
+ * and of the output layout as bsa_lut_packed(row_len = ...) writes them.  A workgroup computes one
+ * part of a row: the row's output blocks are cut into 2^parts_log2 runs of equal length (parts_log2
+ * 0..3; more parts keep fewer y blocks in flight at the price of loading the x row once per part).
+ * work_table (n_items int32) is the order in which parts are handed to workgroups: entry
+ * row << parts_log2 | part, or -1 for nothing; every (row, part) once.  NULL (with parts_log2 == 0 and
+ * n_items == n_rows): rows 0, 1, 2, ...  Workgroup g runs on XCD g % 8, so a table that gives position
+ * 8 k + c to the k-th item of a contiguous eighth c of the rows, heaviest rows first, keeps the y
+ * blocks in flight on one L2 few and the tail of the launch short.
  * Bit-identical results to bsa_matmul (same accumulation order).  Same reference counterpart as
  * bsa_matmul.
  */
 int bsa_matmul_rows(const void *x, const void *y, void *out, const int32_t *pair_offsets,
                     const int32_t *pairs, const int32_t *x_row_offsets, const int32_t *o_row_offsets,
-                    const int32_t *row_order, int64_t n_rows, int64_t nnz_o, int64_t nnz_x, int64_t nnz_y,
-                    int sbs, int dtype, bsa_stream_t stream);
+                    const int32_t *work_table, int64_t n_items, int parts_log2, int64_t n_rows, int64_t nnz_o,
+                    int64_t nnz_x, int64_t nnz_y, int sbs, int dtype, bsa_stream_t stream);
 
 /*
  * Block gather with element transposition: out[o] = transpose(blocks[packed[(b * R + r) * C + c]]) with

@@ -168,3 +168,40 @@ def test_unknown_autotune_mode_is_rejected():
     proc = subprocess.run([sys.executable, "-c", "import blksprs_amd"], env=env, capture_output=True, text=True,
                           cwd=str(__import__("pathlib").Path(__file__).resolve().parent.parent))
     assert proc.returncode != 0 and "Unknown autotune mode" in proc.stderr
+
+
+def test_row_work_table_holds_every_part_once_and_keeps_eighths_together():
+    """The table of the row kernel: entries row << parts_log2 | part, the k-th item of the c-th contiguous
+    eighth of the rows at position 8 k + c, -1 where an eighth has a row less; inside an eighth batch entries
+    ascend, parts ascend inside an entry, and inside a part the rows with the most pairs come first."""
+    import importlib
+    mm = importlib.import_module("blksprs_amd.ops.matmul")
+    g = torch.Generator().manual_seed(5)
+    for n_rows, rows_per_batch, parts_log2 in ((1024, 64, 0), (1024, 64, 1), (21, 7, 2), (5, 5, 1), (8, 1, 3)):
+        blocks_per_row = 9
+        row_offsets = torch.arange(n_rows + 1, dtype=torch.int32) * blocks_per_row
+        pair_offsets = torch.cumsum(torch.randint(0, 6, (n_rows * blocks_per_row + 1,), generator=g), 0).to(torch.int32)
+        work = (pair_offsets[row_offsets.long()][1:] - pair_offsets[row_offsets.long()][:-1]).tolist()
+        table = mm._row_work_table(pair_offsets, row_offsets, rows_per_batch, parts_log2)
+        parts = 1 << parts_log2
+        assert table.dtype == torch.int32 and table.numel() % 8 == 0
+        live = table[table >= 0].long()
+        assert torch.equal(torch.sort(live)[0], torch.arange(n_rows * parts))
+        assert table.numel() == -(-n_rows // 8) * parts * 8
+        small, extra = divmod(n_rows, 8)
+        start = 0
+        for c in range(8):
+            size = small + (c < extra)
+            items = [int(e) for e in table[c::8].tolist()]
+            assert all(e == -1 for e in items[size * parts:])
+            items = items[:size * parts]
+            rows = [e >> parts_log2 for e in items]
+            assert sorted(set(rows)) == list(range(start, start + size))
+            order = [(r // rows_per_batch, e & (parts - 1), -work[r]) for e, r in zip(items, rows)]
+            assert order == sorted(order)
+            start += size
+    assert mm._row_work_table(torch.zeros(1, dtype=torch.int32), torch.zeros(1, dtype=torch.int32), 1, 1).numel() == 0
+    # two parts only when an entry's y blocks overflow one L2 and the rows are long enough to feed the waves twice
+    assert mm._row_parts_log2(1024, 64, 16287, 64370, 8192) == 1      # configuration 2
+    assert mm._row_parts_log2(1024, 64, 4096, 64370, 8192) == 0       # y of an entry fits
+    assert mm._row_parts_log2(1024, 64, 16287, 16000, 8192) == 0      # short rows
