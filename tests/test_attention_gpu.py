@@ -450,3 +450,25 @@ def test_lists_kept_per_mask_follow_the_mask(device, use_causal):
     assert_close(got[0], ref, 2e-2, "O")
     for name, a, b in (("dQ", got[1], ref_q.grad), ("dK", got[2], ref_k.grad), ("dV", got[3], ref_v.grad)):
         assert_close(a, b, 4e-2, name)
+
+
+def test_a_mask_that_masks_everything_leaves_empty_lists(device):
+    """Every mask block masks everything: from the second call on the forward's lists are empty.  Output and
+    gradients are zeros, as on the first call."""
+    B, n, nh, sbs = 1, 4, 1, 64
+    la = torch.ones((B, n, n), dtype=torch.bool, device=device)
+    full = torch.ones((B, n, nh), dtype=torch.bool, device=device)
+    q, k, v = (rand_blocks(B * n * nh, sbs, torch.bfloat16, s).to(device) for s in (1, 2, 3))
+    mask = torch.ones((B * n * n, sbs, sbs), dtype=torch.bool, device=device)
+    cache = {}
+    results = []
+    for _ in range(3):
+        qq = q.clone().requires_grad_(True)
+        out = bs.ops.flash_attention(qq, full, k, full, v, full, la, sbs, attention_mask=mask,
+                                     sparsity_layout_mask=la, layout_cache=cache)
+        out.sum().backward()
+        results.append((out.detach(), qq.grad))
+    facts = cache["mask_facts"].cache["facts"]
+    assert facts.group_offsets is not None and int(facts.group_offsets[-1]) == 0
+    for out, grad in results:
+        assert torch.all(out == 0) and torch.all(grad == 0)
