@@ -205,3 +205,28 @@ def test_row_work_table_holds_every_part_once_and_keeps_eighths_together():
     assert mm._row_parts_log2(1024, 64, 16287, 64370, 8192) == 1      # configuration 2
     assert mm._row_parts_log2(1024, 64, 4096, 64370, 8192) == 0       # y of an entry fits
     assert mm._row_parts_log2(1024, 64, 16287, 16000, 8192) == 0      # short rows
+
+
+def test_library_operators_are_registered_with_shape_functions():
+    """The launchers are torch.library operators of the namespace blksprs_amd (the reference registers its own
+    as blksprs::..., blksprs/ops/matmul.py:70): their schemas mutate nothing and their shape functions run on
+    fake tensors, without a device."""
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    ops = torch.ops.blksprs_amd
+    for name in ("matmul_forward", "to_sparse_forward", "to_dense_forward", "softmax_fused_forward",
+                 "softmax_fused_backward"):
+        schema = getattr(ops, name).default._schema
+        assert not schema.is_mutable and len(schema.returns) == 1, name
+    with FakeTensorMode():
+        x = torch.empty((5, 32, 32), dtype=torch.float16, device="meta")
+        y = torch.empty((7, 32, 32), dtype=torch.float16, device="meta")
+        table = torch.empty((9, 2), dtype=torch.int32, device="meta")
+        layout = torch.empty((2, 3, 4), dtype=torch.bool, device="meta")
+        out = ops.matmul_forward(x, y, table, table, 3, 32, False, True)
+        assert out.shape == (3, 32, 32) and out.dtype == torch.float16
+        dense = torch.empty((2, 96, 128), dtype=torch.float16, device="meta")
+        assert ops.to_sparse_forward(dense, table, 32, 5).shape == (5, 32, 32)
+        assert ops.to_dense_forward(x, layout, table, 32, 0.0).shape == (2, 96, 128)
+        xf = torch.empty((5, 32, 32), device="meta")
+        assert ops.softmax_fused_forward(xf, table, 6, 32).shape == xf.shape
+        assert ops.softmax_fused_backward(xf, xf, table, 6, 32).dtype == torch.float32
