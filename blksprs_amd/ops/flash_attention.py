@@ -278,7 +278,7 @@ def _tensor_identity(t: Tensor | None):
 
 
 def _mask_facts(layout_cache: dict, attention_layout: Tensor, mask: Tensor | None, mask_bytes: Tensor | None,
-                lengths: Tensor | None, dims: tuple[int, int, int, int, int]) -> _MaskFacts:
+                lengths: Tensor | None, dims: tuple[int, int, int, int, int], sbs: int) -> _MaskFacts:
     """The facts for this mask in ``layout_cache``, renewed when another mask (or another version) arrives.
 
     The forward lists without dead pairs are built when a mask is seen for the second time in a row: a caller
@@ -293,16 +293,27 @@ def _mask_facts(layout_cache: dict, attention_layout: Tensor, mask: Tensor | Non
     if facts is None or facts.key != key:
         facts = holder.cache["facts"] = _MaskFacts(key, (mask, lengths))
     facts.sightings += 1
-    if (facts.sightings == 2 and facts.group_offsets is None and mask_bytes is not None and mask_bytes.size(0) > 0
+    has_mask = mask_bytes is not None and mask_bytes.size(0) > 0
+    if (facts.sightings == 2 and facts.group_offsets is None and (has_mask or lengths is not None)
             and "group_offsets" in layout_cache and not torch.cuda.is_current_stream_capturing()):
         B, nq, nk, nh, nhv = dims
-        dead = torch.empty(mask_bytes.size(0), dtype=torch.uint8, device=mask_bytes.device)
-        with torch.cuda.device(dead.device):
-            _capi.call("bsa_attn_mask_dead", _capi.ptr(mask_bytes), mask_bytes.size(0), mask_bytes.size(-1),
-                       _capi.ptr(dead), _capi.stream(dead.device))
-        block_of_pair = layout_cache["packed_indices_mask"].reshape(B, nq, nk)
-        dead_pairs = (block_of_pair >= 0) & (dead != 0)[block_of_pair.clamp(min=0)]
-        live_layout = (attention_layout.reshape(B, nq, nk) != 0) & ~dead_pairs
+        device = attention_layout.device
+        live_layout = attention_layout.reshape(B, nq, nk) != 0
+        if has_mask:
+            dead = torch.empty(mask_bytes.size(0), dtype=torch.uint8, device=device)
+            with torch.cuda.device(device):
+                _capi.call("bsa_attn_mask_dead", _capi.ptr(mask_bytes), mask_bytes.size(0), mask_bytes.size(-1),
+                           _capi.ptr(dead), _capi.stream(device))
+            block_of_pair = layout_cache["packed_indices_mask"].reshape(B, nq, nk)
+            live_layout = live_layout & ~((block_of_pair >= 0) & (dead != 0)[block_of_pair.clamp(min=0)])
+        if lengths is not None:
+            # pairs the causal predicate rules out as a whole (blksprs/ops/flash_attention.py:1133-1137):
+            # every key after every query, or all queries / all keys at or beyond the valid length
+            query_block = torch.arange(nq, device=device).view(1, nq, 1)
+            key_block = torch.arange(nk, device=device).view(1, 1, nk)
+            valid = lengths.to(device).view(B, 1, 1)
+            live_layout = live_layout & (key_block <= query_block) & (query_block * sbs < valid) \
+                & (key_block * sbs < valid)
         facts.group_offsets, facts.group_records, _ = _build_forward_records(layout_cache, live_layout, B, nq, nk,
                                                                              nh, nhv)
     return facts
@@ -555,6 +566,7 @@ def flash_attention(q: BlksprsTensor, sparsity_layout_q: Tensor,
     meta.mask = mask_bytes
     meta.causal_lengths = lengths
     meta.has_bias = has_bias
-    meta.facts = _mask_facts(layout_cache, attention_layout, attention_mask, mask_bytes, lengths, meta.dims)
+    meta.facts = _mask_facts(layout_cache, attention_layout, attention_mask, mask_bytes, lengths, meta.dims,
+                             sparsity_block_size)
 
     return BlksprsTensor.wrap(_FlashAttention.apply(q, k, v, attention_bias, meta))

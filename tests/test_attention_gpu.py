@@ -472,3 +472,46 @@ def test_a_mask_that_masks_everything_leaves_empty_lists(device):
     assert facts.group_offsets is not None and int(facts.group_offsets[-1]) == 0
     for out, grad in results:
         assert torch.all(out == 0) and torch.all(grad == 0)
+
+
+def test_lists_kept_per_causal_lengths(device):
+    """Native causal attention without a mask tensor: from the second call with one tensor of lengths on, the
+    forward walks lists without the pairs the causal predicate rules out as a whole.  Same bits as the first
+    call and as a fresh cache; lengths changed in place give what a fresh cache gives."""
+    g = torch.Generator().manual_seed(22)
+    B, n, nh, sbs = 2, 8, 2, 64
+    la = orc.random_layout((B, n, n), 0.8, g, ensure_rows=True).to(device)
+    full = torch.ones((B, n, nh), dtype=torch.bool, device=device)
+    q, k, v = (rand_blocks(B * n * nh, sbs, torch.bfloat16, s).to(device) for s in (1, 2, 3))
+    go = rand_blocks(B * n * nh, sbs, torch.bfloat16, 4).to(device)
+    lengths = torch.tensor([n * sbs, 5 * sbs - 9], device=device)
+
+    def run(cache):
+        qq, kk, vv = (t.clone().requires_grad_(True) for t in (q, k, v))
+        out = bs.ops.flash_attention(qq, full, kk, full, vv, full, la, sbs, layout_cache=cache,
+                                     causal_lengths=lengths)
+        out.backward(go)
+        return out.detach(), qq.grad, kk.grad, vv.grad
+
+    cache = {}
+    first = run(cache)
+    for _ in range(2):
+        for a, b in zip(run(cache), first):
+            assert torch.equal(a, b)
+    facts = cache["mask_facts"].cache["facts"]
+    assert int(facts.group_offsets[-1]) < int(cache["group_offsets"][-1])
+    lengths[1] = 2 * sbs + 1
+    changed, fresh = run(cache), run({})
+    assert not torch.equal(changed[0], first[0])
+    for a, b in zip(changed, fresh):
+        assert torch.equal(a, b)
+    for a, b in zip(run(cache), fresh):
+        assert torch.equal(a, b)
+    ref_q, ref_k, ref_v = (t.cpu().double().requires_grad_(True) for t in (q, k, v))
+    ref = orc.flash_attention(ref_q, full.cpu().numpy(), ref_k, full.cpu().numpy(), ref_v, full.cpu().numpy(),
+                              la.cpu().numpy(), sbs, causal_lengths=lengths.cpu(), acc_dtype=torch.float64)
+    ref.backward(go.cpu().double())
+    got = run(cache)
+    assert_close(got[0], ref, 2e-2, "O")
+    for name, a, b in (("dQ", got[1], ref_q.grad), ("dK", got[2], ref_k.grad), ("dV", got[3], ref_v.grad)):
+        assert_close(a, b, 4e-2, name)
