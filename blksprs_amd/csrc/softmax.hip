@@ -80,8 +80,6 @@ constexpr float kLog2e = 1.44269504088896341f;
 __device__ inline float exp_rel(float v, float m2) { return __builtin_amdgcn_exp2f(__builtin_fmaf(v, kLog2e, -m2)); }
 __device__ inline float exp2_of(float d) { return __builtin_amdgcn_exp2f(d); }
 
-__device__ inline float max4(float4 v) { return fmaxf(fmaxf(v.x, v.y), fmaxf(v.z, v.w)); }
-
 // max(m, v.x, v.y, v.z, v.w) in two instructions.  fmaxf first quiets signalling NaNs (one more instruction per
 // operand); here a NaN may come out either way: it reaches every output of the row through the exponentials.
 __device__ inline float max_with(float m, float4 v) {
@@ -105,6 +103,18 @@ __device__ inline void load_row(float4 (&v)[N], const float *row, int units, con
         v[c + j] = *reinterpret_cast<const float4 *>(row + unit_offset(u, g));
       }
     }
+  }
+}
+
+// Units [u0, u0 + count) of a row, count <= N: the index is clamped to the last of them, so the loads have no
+// branch between them; entries at and beyond `count` hold copies of the last unit.
+constexpr int kChunk = 8;
+template <int N>
+__device__ inline void load_chunk(float4 (&v)[N], const float *row, int u0, int count, const RowGeom &g) {
+#pragma unroll
+  for (int j = 0; j < N; ++j) {
+    const int u = u0 + (j < count ? j : count - 1);
+    v[j] = *reinterpret_cast<const float4 *>(row + unit_offset(u, g));
   }
 }
 
@@ -156,17 +166,30 @@ __global__ __launch_bounds__(64 * kWaves) void softmax_fwd_kernel(const float *_
     return;
   }
 
-  // long rows: max pass, sum pass folded into one online pass, then the write pass
+  // long rows: max pass and sum pass folded into one online pass, then the write pass; both in chunks of
+  // kChunk units whose loads are all issued before the first one is used
   float m = -INFINITY, s = 0.f;
-  for (int u = 0; u < units; ++u) {
-    const float4 v = *reinterpret_cast<const float4 *>(xr + unit_offset(u, g));
-    const float mn = fmaxf(m, max4(v));
+  for (int u0 = 0; u0 < units; u0 += kChunk) {
+    const int count = units - u0 < kChunk ? units - u0 : kChunk;
+    float4 v[kChunk];
+    load_chunk(v, xr, u0, count, g);
+    float mn = m;
+#pragma unroll
+    for (int j = 0; j < kChunk; ++j) mn = max_with(mn, v[j]);  // the copies of the last unit change no maximum
     if (mn != -INFINITY) {
       const float mn2 = mn * kLog2e;
-      s = s * exp2_of(m * kLog2e - mn2) + (exp_rel(v.x, mn2) + exp_rel(v.y, mn2)) +
-          (exp_rel(v.z, mn2) + exp_rel(v.w, mn2));
-    } else if (v.x != v.x || v.y != v.y || v.z != v.z || v.w != v.w) {
-      s = NAN;  // fmaxf drops NaN; keep it visible in the sum
+      float add = 0.f;
+#pragma unroll
+      for (int j = 0; j < kChunk; ++j)
+        if (j < count)
+          add += (exp_rel(v[j].x, mn2) + exp_rel(v[j].y, mn2)) + (exp_rel(v[j].z, mn2) + exp_rel(v[j].w, mn2));
+      s = s * exp2_of(m * kLog2e - mn2) + add;
+    } else {
+      bool any_nan = false;  // a maximum that dropped a NaN: keep it visible in the sum
+#pragma unroll
+      for (int j = 0; j < kChunk; ++j)
+        any_nan |= v[j].x != v[j].x || v[j].y != v[j].y || v[j].z != v[j].z || v[j].w != v[j].w;
+      if (any_nan) s = NAN;
     }
     m = mn;
   }
@@ -175,15 +198,21 @@ __global__ __launch_bounds__(64 * kWaves) void softmax_fwd_kernel(const float *_
   float part = (m == -INFINITY) ? ((s != s) ? s : 0.f) : s * exp2_of(m * kLog2e - mall2);
   const float sall = lanes_sum(part, g.lpr);
   const float inv_all = 1.f / sall;
-  for (int u = 0; u < units; ++u) {
-    const int64_t off = unit_offset(u, g);
-    const float4 v = *reinterpret_cast<const float4 *>(xr + off);
-    float4 o;
-    o.x = exp_rel(v.x, mall2) * inv_all;
-    o.y = exp_rel(v.y, mall2) * inv_all;
-    o.z = exp_rel(v.z, mall2) * inv_all;
-    o.w = exp_rel(v.w, mall2) * inv_all;
-    store_streaming(orow + off, o);
+  for (int u0 = 0; u0 < units; u0 += kChunk) {
+    const int count = units - u0 < kChunk ? units - u0 : kChunk;
+    float4 v[kChunk];
+    load_chunk(v, xr, u0, count, g);
+#pragma unroll
+    for (int j = 0; j < kChunk; ++j) {
+      if (j < count) {
+        float4 o;
+        o.x = exp_rel(v[j].x, mall2) * inv_all;
+        o.y = exp_rel(v[j].y, mall2) * inv_all;
+        o.z = exp_rel(v[j].z, mall2) * inv_all;
+        o.w = exp_rel(v[j].w, mall2) * inv_all;
+        store_streaming(orow + unit_offset(u0 + j, g), o);
+      }
+    }
   }
 }
 
@@ -223,24 +252,34 @@ __global__ __launch_bounds__(64 * kWaves) void softmax_bwd_kernel(const float *_
     return;
   }
 
+  // long rows: two passes in chunks whose loads are all issued before the first one is used
   float s = 0.f;
-  for (int u = 0; u < units; ++u) {
-    const int64_t off = unit_offset(u, g);
-    const float4 yv = *reinterpret_cast<const float4 *>(yr + off);
-    const float4 gv = *reinterpret_cast<const float4 *>(gr + off);
-    s += (yv.x * gv.x + yv.y * gv.y) + (yv.z * gv.z + yv.w * gv.w);
+  for (int u0 = 0; u0 < units; u0 += kChunk) {
+    const int count = units - u0 < kChunk ? units - u0 : kChunk;
+    float4 yv[kChunk], gv[kChunk];
+    load_chunk(yv, yr, u0, count, g);
+    load_chunk(gv, gr, u0, count, g);
+#pragma unroll
+    for (int j = 0; j < kChunk; ++j)
+      if (j < count) s += (yv[j].x * gv[j].x + yv[j].y * gv[j].y) + (yv[j].z * gv[j].z + yv[j].w * gv[j].w);
   }
   s = lanes_sum(s, g.lpr);
-  for (int u = 0; u < units; ++u) {
-    const int64_t off = unit_offset(u, g);
-    const float4 yv = *reinterpret_cast<const float4 *>(yr + off);
-    const float4 gv = *reinterpret_cast<const float4 *>(gr + off);
-    float4 o;
-    o.x = yv.x * (gv.x - s);
-    o.y = yv.y * (gv.y - s);
-    o.z = yv.z * (gv.z - s);
-    o.w = yv.w * (gv.w - s);
-    store_streaming(dr + off, o);
+  for (int u0 = 0; u0 < units; u0 += kChunk) {
+    const int count = units - u0 < kChunk ? units - u0 : kChunk;
+    float4 yv[kChunk], gv[kChunk];
+    load_chunk(yv, yr, u0, count, g);
+    load_chunk(gv, gr, u0, count, g);
+#pragma unroll
+    for (int j = 0; j < kChunk; ++j) {
+      if (j < count) {
+        float4 o;
+        o.x = yv[j].x * (gv[j].x - s);
+        o.y = yv[j].y * (gv[j].y - s);
+        o.z = yv[j].z * (gv[j].z - s);
+        o.w = yv[j].w * (gv[j].w - s);
+        store_streaming(dr + unit_offset(u0 + j, g), o);
+      }
+    }
   }
 }
 
