@@ -36,6 +36,7 @@ class AttnArgs(ctypes.Structure):
 
 
 ATTN_RECORD_INTS = 16  # BSA_ATTN_RECORD_INTS
+ROWS_RECORD_INTS = 32  # BSA_ROWS_RECORD_INTS
 
 # name -> (restype, argtypes); must list every symbol of include/blksprs_amd.h
 SIGNATURES = {
@@ -67,8 +68,10 @@ SIGNATURES = {
     "bsa_softmax_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p]),
     "bsa_matmul": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int,
                            c_int, c_int, c_int, c_void_p]),
-    "bsa_matmul_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                                c_int64, c_int, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_void_p]),
+    "bsa_matmul_rows_records": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
+                                        c_void_p, c_void_p]),
+    "bsa_matmul_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
+                                c_int64, c_int64, c_int, c_int, c_void_p]),
     "bsa_attn_fwd_records": (c_int, [ctypes.POINTER(AttnArgs), c_void_p, c_void_p, c_void_p]),
     "bsa_attn_mask_dead": (c_int, [c_void_p, c_int64, ctypes.c_int32, c_void_p, c_void_p]),
     "bsa_attn_bwd_scratch_bytes": (c_size_t, [c_int64, c_int64, c_int64, c_int64, c_int64]),

@@ -208,32 +208,95 @@ __device__ __forceinline__ void rows_flush(f32x16 (&acc)[2][2], char *ob, char *
       for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
 }
 
+// What a workgroup needs to know about its part of a row, in one 128-byte record (one load, where walking the
+// tables is a chain of five dependent loads and a loop of ballots): the row, the x blocks of the row, and for
+// each of the eight waves its run of output blocks and the pairs of that run.  Wave w takes the output blocks
+// in front of which at least w / 8 and less than (w + 1) / 8 of the part's pairs lie.
+struct RowsRecord {
+  int32_t row;                    // -1: nothing to do
+  int32_t x_first, x_count;       // the row's blocks in x
+  int32_t pad0;
+  int32_t block_begin[kWaves + 1];  // wave w: output blocks [block_begin[w], block_begin[w + 1])
+  int32_t pair_begin[kWaves + 1];   // pair_offsets at those blocks
+  int32_t pad1[32 - 4 - 2 * (kWaves + 1)];
+};
+static_assert(sizeof(RowsRecord) == BSA_ROWS_RECORD_INTS * 4, "record layout");
+
+// one wave per work table entry
+__global__ __launch_bounds__(256) void rows_records_kernel(const int32_t *__restrict__ work_table, int64_t n_items,
+                                                           int parts_log2, const int32_t *__restrict__ pair_offsets,
+                                                           const int32_t *__restrict__ x_row_offsets,
+                                                           const int32_t *__restrict__ o_row_offsets, int n_rows,
+                                                           int64_t nnz_x, RowsRecord *__restrict__ records) {
+  const int64_t at = (int64_t)blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  if (at >= n_items) return;
+  const int lane = threadIdx.x & 63;
+  int32_t *out = reinterpret_cast<int32_t *>(records + at);
+  int item = work_table ? work_table[at] : (int)at;
+  item = __builtin_amdgcn_readfirstlane(item);
+  const int part = item & ((1 << parts_log2) - 1);
+  const int row = item < 0 ? -1 : item >> parts_log2;
+  int value = 0;  // lane l writes int l of the record
+  if (row < 0 || row >= n_rows) {  // nothing, or a corrupt table (which must not turn into a wild read)
+    if (lane == 0) value = -1;
+  } else {
+    int n0 = o_row_offsets[row], n1 = o_row_offsets[row + 1];
+    if (parts_log2) {  // this part's run of the row's output blocks
+      const int64_t len = n1 - n0;
+      const int first = n0 + (int)((len * part) >> parts_log2), last = n0 + (int)((len * (part + 1)) >> parts_log2);
+      n0 = first;
+      n1 = last;
+    }
+    const int xs = x_row_offsets[row];
+    int nx = x_row_offsets[row + 1] - xs;
+    if (xs < 0 || nx < 0 || (int64_t)xs + nx > nnz_x) nx = 0;
+    const int row_p0 = pair_offsets[n0], row_p1 = pair_offsets[n1];
+    const int64_t span = row_p1 - row_p0;
+    // lane w < 8 counts the blocks in front of wave w's boundary: pair_offsets ascends, one ballot per 64 blocks
+    // for each boundary
+    int below[kWaves];
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) below[w] = 0;
+    for (int base = n0; base < n1; base += 64) {
+      const int b = base + lane;
+      const int off = b < n1 ? pair_offsets[b] : 0x7fffffff;
+#pragma unroll
+      for (int w = 1; w < kWaves; ++w) {
+        const int lo = row_p0 + (int)((span * w + kWaves - 1) / kWaves);
+        below[w] += __builtin_popcountll(__ballot(off < lo));
+      }
+    }
+    int begin = n0;  // boundary number lane (for lanes 0 .. 8)
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w)
+      if (lane == w) begin = n0 + below[w];
+    if (lane >= kWaves) begin = n1;
+    const int pair_at = pair_offsets[begin];
+    const int moved = __shfl(begin, lane - 4), moved_pair = __shfl(pair_at, lane - 4 - (kWaves + 1));
+    if (lane == 0) value = n0 >= n1 ? -1 : row;
+    else if (lane == 1) value = xs;
+    else if (lane == 2) value = nx;
+    else if (lane >= 4 && lane < 4 + kWaves + 1) value = moved;
+    else if (lane >= 4 + kWaves + 1 && lane < 4 + 2 * (kWaves + 1)) value = moved_pair;
+  }
+  if (lane < BSA_ROWS_RECORD_INTS) out[lane] = value;
+}
+
 template <typename Tr>
 __global__ __launch_bounds__(kWaves * 64, 1) void matmul_rows_kernel(
     const char *__restrict__ x, const char *__restrict__ y, char *__restrict__ out,
     const int32_t *__restrict__ pair_offsets, const int32_t *__restrict__ pairs,
-    const int32_t *__restrict__ x_row_offsets, const int32_t *__restrict__ o_row_offsets,
-    const int32_t *__restrict__ work_table, int parts_log2, int n_rows, int64_t nnz_x, int64_t nnz_y) {
+    const RowsRecord *__restrict__ records, int64_t nnz_x, int64_t nnz_y) {
   extern __shared__ __attribute__((aligned(16))) char rows_smem[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  // the grid has one workgroup per table entry: row << parts_log2 | part, or -1 for nothing
-  int item = work_table ? work_table[blockIdx.x] : (int)blockIdx.x;
-  item = __builtin_amdgcn_readfirstlane(item);
-  if (item < 0) return;
-  const int part = item & ((1 << parts_log2) - 1);
-  const int row = item >> parts_log2;
-  if (row >= n_rows) return;  // a corrupt table must not turn into a wild read
-  int n0 = o_row_offsets[row], n1 = o_row_offsets[row + 1];
-  if (parts_log2) {  // this workgroup's run of the row's output blocks
-    const int64_t len = n1 - n0;
-    const int first = n0 + (int)((len * part) >> parts_log2), last = n0 + (int)((len * (part + 1)) >> parts_log2);
-    n0 = first;
-    n1 = last;
-  }
-  if (n0 >= n1) return;
-  const int xs = x_row_offsets[row];
-  int nx = x_row_offsets[row + 1] - xs;
+  // the grid has one workgroup per record; lane l < 32 fetches int l of it
+  const int32_t *rec = reinterpret_cast<const int32_t *>(records + blockIdx.x);
+  const int mine = rec[lane & 31];
+  const int row = __builtin_amdgcn_readlane(mine, 0);
+  if (row < 0) return;
+  const int xs = __builtin_amdgcn_readlane(mine, 1);
+  int nx = __builtin_amdgcn_readlane(mine, 2);
   nx = nx < kPanelCap ? nx : kPanelCap;
   if (xs < 0 || xs + nx > nnz_x) nx = 0;
   char *panel = rows_smem;
@@ -249,29 +312,10 @@ __global__ __launch_bounds__(kWaves * 64, 1) void matmul_rows_kernel(
     for (int idx = wave; idx < nx * 8; idx += kWaves) copy_1k_to_lds(xsrc + idx * 1024, src_off, panel + idx * 1024);
   }
 
-  // This wave's run of output blocks: block b belongs to wave w when the pairs in front of it number at least
-  // w / 8 and less than (w + 1) / 8 of the row's pairs.  pair_offsets ascends, so the blocks in front of a
-  // boundary are counted with one ballot per 64 blocks.
-  const int row_p0 = pair_offsets[n0], row_p1 = pair_offsets[n1];
-  int wb0 = n0, wb1 = n1;
-  {
-    const int64_t span = row_p1 - row_p0;
-    const int lo = row_p0 + (int)((span * wave + kWaves - 1) / kWaves);
-    const int hi = row_p0 + (int)((span * (wave + 1) + kWaves - 1) / kWaves);
-    int below_lo = 0, below_hi = 0;
-    for (int base = n0; base < n1; base += 64) {
-      const int b = base + lane;
-      const int off = b < n1 ? pair_offsets[b] : 0x7fffffff;
-      below_lo += __builtin_popcountll(__ballot(off < lo));
-      below_hi += __builtin_popcountll(__ballot(off < hi));
-    }
-    if (wave > 0) wb0 = n0 + below_lo;
-    if (wave < kWaves - 1) wb1 = n0 + below_hi;
-    wb0 = __builtin_amdgcn_readfirstlane(wb0);
-    wb1 = __builtin_amdgcn_readfirstlane(wb1);
-  }
-  const int p_begin = __builtin_amdgcn_readfirstlane(pair_offsets[wb0]);
-  const int p_end = __builtin_amdgcn_readfirstlane(pair_offsets[wb1]);
+  // this wave's run of output blocks and its pairs
+  const int wb0 = __builtin_amdgcn_readlane(mine, 4 + wave), wb1 = __builtin_amdgcn_readlane(mine, 5 + wave);
+  const int p_begin = __builtin_amdgcn_readlane(mine, 4 + kWaves + 1 + wave);
+  const int p_end = __builtin_amdgcn_readlane(mine, 5 + kWaves + 1 + wave);
 
   // 64 entries of the pair list and 64 block boundaries at a time, one per lane.  A lane turns its entry into
   // what the loop needs per pair (the address of the y block; the panel offset of the x block, or -1 if it is
@@ -453,8 +497,7 @@ __global__ __launch_bounds__(kWaves * 64, 1) void matmul_rows_kernel(
 
 template <typename Tr>
 int launch_rows(const void *x, const void *y, void *out, const int32_t *pair_offsets, const int32_t *pairs,
-                const int32_t *x_row_offsets, const int32_t *o_row_offsets, const int32_t *work_table,
-                int64_t n_items, int parts_log2, int64_t n_rows, int64_t nnz_x, int64_t nnz_y, hipStream_t s) {
+                const int32_t *records, int64_t n_items, int64_t nnz_x, int64_t nnz_y, hipStream_t s) {
   static bool configured = false;  // raising the dynamic LDS limit is per function, once per process
   if (!configured) {
     BSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&matmul_rows_kernel<Tr>),
@@ -463,7 +506,7 @@ int launch_rows(const void *x, const void *y, void *out, const int32_t *pair_off
   }
   matmul_rows_kernel<Tr><<<(unsigned)n_items, kWaves * 64, kRowsLds, s>>>(
       static_cast<const char *>(x), static_cast<const char *>(y), static_cast<char *>(out), pair_offsets, pairs,
-      x_row_offsets, o_row_offsets, work_table, parts_log2, (int)n_rows, nnz_x, nnz_y);
+      reinterpret_cast<const RowsRecord *>(records), nnz_x, nnz_y);
   return bsa::check_launch("matmul_rows_kernel");
 }
 
@@ -471,27 +514,38 @@ bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 
 
 }  // namespace
 
+extern "C" int bsa_matmul_rows_records(const int32_t *work_table, int64_t n_items, int parts_log2,
+                                       const int32_t *pair_offsets, const int32_t *x_row_offsets,
+                                       const int32_t *o_row_offsets, int64_t n_rows, int64_t nnz_x,
+                                       int32_t *records, bsa_stream_t stream) {
+  const char *who = "bsa_matmul_rows_records";
+  BSA_REQUIRE(parts_log2 >= 0 && parts_log2 <= 3, "%s: parts_log2 must be 0..3 (got %d)", who, parts_log2);
+  BSA_REQUIRE(n_rows >= 0 && (n_rows << parts_log2) < 0x7fffffffLL, "%s: bad number of block rows", who);
+  BSA_REQUIRE(n_items >= 0 && n_items < 0x7fffffffLL, "%s: bad number of table entries", who);
+  BSA_REQUIRE(nnz_x >= 0, "%s: negative size", who);
+  BSA_REQUIRE(work_table != nullptr || (parts_log2 == 0 && n_items == n_rows),
+              "%s: without a work table the rows are taken whole and in order", who);
+  if (n_items == 0) return BSA_OK;
+  BSA_REQUIRE(pair_offsets && x_row_offsets && o_row_offsets && records, "%s: NULL pointer", who);
+  BSA_REQUIRE((reinterpret_cast<uintptr_t>(records) & 127) == 0, "%s: records must be 128-byte aligned", who);
+  rows_records_kernel<<<(unsigned)bsa::cdiv(n_items, 4), 256, 0, bsa::as_stream(stream)>>>(
+      work_table, n_items, parts_log2, pair_offsets, x_row_offsets, o_row_offsets, (int)n_rows, nnz_x,
+      reinterpret_cast<RowsRecord *>(records));
+  return bsa::check_launch("rows_records_kernel");
+}
+
 extern "C" int bsa_matmul_rows(const void *x, const void *y, void *out, const int32_t *pair_offsets,
-                               const int32_t *pairs, const int32_t *x_row_offsets, const int32_t *o_row_offsets,
-                               const int32_t *work_table, int64_t n_items, int parts_log2, int64_t n_rows,
-                               int64_t nnz_o, int64_t nnz_x, int64_t nnz_y, int sbs, int dtype,
-                               bsa_stream_t stream) {
+                               const int32_t *pairs, const int32_t *records, int64_t n_items, int64_t nnz_o,
+                               int64_t nnz_x, int64_t nnz_y, int sbs, int dtype, bsa_stream_t stream) {
   BSA_REQUIRE(sbs == 64, "bsa_matmul_rows: sbs must be 64 (got %d)", sbs);
   BSA_REQUIRE(dtype == BSA_F16 || dtype == BSA_BF16, "bsa_matmul_rows: dtype must be fp16 or bf16 (got %d)", dtype);
-  BSA_REQUIRE(nnz_o >= 0 && nnz_x >= 0 && nnz_y >= 0 && n_rows >= 0, "bsa_matmul_rows: negative size");
-  if (nnz_o == 0 || n_rows == 0) return BSA_OK;
-  BSA_REQUIRE(out && pair_offsets && x_row_offsets && o_row_offsets, "bsa_matmul_rows: NULL pointer");
+  BSA_REQUIRE(nnz_o >= 0 && nnz_x >= 0 && nnz_y >= 0, "bsa_matmul_rows: negative size");
+  BSA_REQUIRE(n_items >= 0 && n_items < 0x7fffffffLL, "bsa_matmul_rows: bad number of records");
+  if (nnz_o == 0 || n_items == 0) return BSA_OK;
+  BSA_REQUIRE(out && pair_offsets && records, "bsa_matmul_rows: NULL pointer");
   BSA_REQUIRE(aligned16(x) && aligned16(y) && aligned16(out), "bsa_matmul_rows: buffers must be 16-byte aligned");
-  BSA_REQUIRE(parts_log2 >= 0 && parts_log2 <= 3, "bsa_matmul_rows: parts_log2 must be 0..3 (got %d)", parts_log2);
-  BSA_REQUIRE((n_rows << parts_log2) < 0x7fffffffLL, "bsa_matmul_rows: too many block rows");
-  BSA_REQUIRE(n_items >= 0 && n_items < 0x7fffffffLL, "bsa_matmul_rows: bad number of table entries");
-  BSA_REQUIRE(work_table != nullptr || (parts_log2 == 0 && n_items == n_rows),
-              "bsa_matmul_rows: without a work table the rows are taken whole and in order");
-  if (n_items == 0) return BSA_OK;
+  BSA_REQUIRE((reinterpret_cast<uintptr_t>(records) & 127) == 0, "bsa_matmul_rows: records must be 128-byte aligned");
   hipStream_t s = bsa::as_stream(stream);
-  if (dtype == BSA_BF16)
-    return launch_rows<MBf16>(x, y, out, pair_offsets, pairs, x_row_offsets, o_row_offsets, work_table, n_items,
-                              parts_log2, n_rows, nnz_x, nnz_y, s);
-  return launch_rows<MF16>(x, y, out, pair_offsets, pairs, x_row_offsets, o_row_offsets, work_table, n_items,
-                           parts_log2, n_rows, nnz_x, nnz_y, s);
+  if (dtype == BSA_BF16) return launch_rows<MBf16>(x, y, out, pair_offsets, pairs, records, n_items, nnz_x, nnz_y, s);
+  return launch_rows<MF16>(x, y, out, pair_offsets, pairs, records, n_items, nnz_x, nnz_y, s);
 }

@@ -38,9 +38,7 @@ def _launch_rows(x: Tensor, y: Tensor, cache: dict, n_rows: int, sbs: int) -> Te
         with torch.cuda.device(x.device):
             _capi.call("bsa_matmul_rows", _capi.ptr(x), _capi.ptr(y), out.data_ptr(),
                        cache["contraction_offsets"].data_ptr(), _capi.ptr(cache["contraction_pairs"]),
-                       cache["row_offsets_x"].data_ptr(), cache["row_offsets_o"].data_ptr(),
-                       _capi.ptr(cache["row_work_table"]), cache["row_work_table"].numel(),
-                       cache["row_parts_log2"], n_rows, n_out,
+                       _capi.ptr(cache["row_records"]), cache["row_records"].size(0), n_out,
                        x.size(0), y.size(0), sbs, _capi.DTYPE_CODES[x.dtype], _capi.stream(x.device))
     return out
 
@@ -77,6 +75,20 @@ def _row_parts_log2(n_rows: int, rows_per_batch: int, n_blocks_y: int, n_blocks_
     y_bytes_per_entry = n_blocks_y * block_bytes // batches
     blocks_per_row = n_blocks_o // max(n_rows, 1)
     return 1 if y_bytes_per_entry > _L2_BYTES and blocks_per_row >= 32 else 0
+
+
+def _row_records(work_table: Tensor, parts_log2: int, pair_offsets: Tensor, row_offsets_x: Tensor,
+                 row_offsets_o: Tensor, n_rows: int, n_blocks_x: int) -> Tensor:
+    """One record per work table entry with what a workgroup of the row kernel needs to know about its part of
+    a row (``bsa_matmul_rows_records``): int32 ``[n_items, 32]``."""
+    records = torch.empty((work_table.numel(), _capi.ROWS_RECORD_INTS), dtype=torch.int32,
+                          device=work_table.device)
+    if work_table.numel():
+        with torch.cuda.device(work_table.device):
+            _capi.call("bsa_matmul_rows_records", _capi.ptr(work_table), work_table.numel(), parts_log2,
+                       pair_offsets.data_ptr(), row_offsets_x.data_ptr(), row_offsets_o.data_ptr(), n_rows,
+                       n_blocks_x, _capi.ptr(records), _capi.stream(work_table.device))
+    return records
 
 
 def _row_work_table(pair_offsets: Tensor, row_offsets_o: Tensor, rows_per_batch: int, parts_log2: int) -> Tensor:
@@ -143,7 +155,7 @@ class _Matmul(torch.autograd.Function):
         ctx.shapes = (shape_x, shape_y)
         ctx.sparsity_block_size = sparsity_block_size
         if (sparsity_block_size == 64 and x.dtype in (torch.float16, torch.bfloat16)
-                and layout_cache["row_offsets_x"] is not None and layout_cache["row_offsets_o"] is not None):
+                and layout_cache["row_records"] is not None):
             return _launch_rows(x, y, layout_cache, shape_x[0] * shape_x[1], sparsity_block_size)
         return _launch(x, y, layout_cache["contraction_offsets"], layout_cache["contraction_pairs"],
                        layout_cache["block_order"], layout_cache["n_sparse_blocks"], sparsity_block_size, False,
@@ -193,9 +205,13 @@ def matmul_build_layout_cache(layout_cache: dict | None, sparsity_layout_x: Tens
         layout_cache["block_order"] = _block_order(layout_cache["layout_indices_o"])
         layout_cache["row_offsets_x"] = info_x.row_offsets
         layout_cache["row_offsets_o"] = info_o.row_offsets
-        parts_log2 = _row_parts_log2(B * R, R, info_y.count, info_o.count, 64 * 64 * 2)
-        layout_cache["row_parts_log2"] = parts_log2
-        layout_cache["row_work_table"] = _row_work_table(lists.pair_offsets, info_o.row_offsets, R, parts_log2)
+        layout_cache["row_records"] = None
+        if info_x.row_offsets is not None and info_o.row_offsets is not None:
+            parts_log2 = _row_parts_log2(B * R, R, info_y.count, info_o.count, 64 * 64 * 2)
+            table = _row_work_table(lists.pair_offsets, info_o.row_offsets, R, parts_log2)
+            layout_cache["row_parts_log2"], layout_cache["row_work_table"] = parts_log2, table
+            layout_cache["row_records"] = _row_records(table, parts_log2, lists.pair_offsets, info_x.row_offsets,
+                                                       info_o.row_offsets, B * R, info_x.count)
 
     validate_contiguous(sparsity_layout_x, layout_cache["packed_indices_x"],
                         sparsity_layout_y, layout_cache["packed_indices_y"],

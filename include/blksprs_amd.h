@@ -208,24 +208,37 @@ int bsa_matmul(const void *x, const void *y, void *out, const int32_t *pair_offs
                const int32_t *pairs, const int32_t *block_order, int64_t nnz_o, int64_t nnz_x, int64_t nnz_y, int sbs, int dtype,
                int trans_x, int trans_y, bsa_stream_t stream);
 
+#define BSA_ROWS_RECORD_INTS 32
+
 /*
- * The same product for fp16 / bf16 operands with sbs == 64, organised by output block row: the x
- * blocks of a row are kept in LDS while the row's output blocks are computed.  x_row_offsets and
- * o_row_offsets are the int32 CSR row offsets (n_rows + 1 entries, rows = B * R) of the x layout
- * and of the output layout as bsa_lut_packed(row_len = ...) writes them.  A workgroup computes one
- * part of a row: the row's output blocks are cut into 2^parts_log2 runs of equal length (parts_log2
- * 0..3; more parts keep fewer y blocks in flight at the price of loading the x row once per part).
- * work_table (n_items int32) is the order in which parts are handed to workgroups: entry
- * row << parts_log2 | part, or -1 for nothing; every (row, part) once.  NULL (with parts_log2 == 0 and
- * n_items == n_rows): rows 0, 1, 2, ...  Workgroup g runs on XCD g % 8, so a table that gives position
- * 8 k + c to the k-th item of a contiguous eighth c of the rows, heaviest rows first, keeps the y
- * blocks in flight on one L2 few and the tail of the launch short.
+ * Layout-to-LUT step of bsa_matmul_rows (integer only): one record of BSA_ROWS_RECORD_INTS int32 per work
+ * table entry.  x_row_offsets and o_row_offsets are the int32 CSR row offsets (n_rows + 1 entries,
+ * rows = B * R) of the x layout and of the output layout as bsa_lut_packed(row_len = ...) writes them.  A
+ * workgroup of bsa_matmul_rows computes one part of a row: the row's output blocks are cut into
+ * 2^parts_log2 runs of equal length (parts_log2 0..3; more parts keep fewer y blocks in flight at the price of
+ * loading the x row once per part).  work_table (n_items int32) is the order in which parts are handed to
+ * workgroups: entry row << parts_log2 | part, or -1 for nothing; every (row, part) once.  NULL (with
+ * parts_log2 == 0 and n_items == n_rows): rows 0, 1, 2, ...  Workgroup g runs on XCD g % 8, so a table that
+ * gives position 8 k + c to the k-th item of a contiguous eighth c of the rows, heaviest rows first, keeps the
+ * y blocks in flight on one L2 few and the tail of the launch short.  A record holds the row (-1: nothing),
+ * the row's first x block and their number, and for each of the kernel's eight waves the run of output
+ * blocks it computes and the first pair of that run.  No counterpart in the reference, whose kernel
+ * (blksprs/ops/matmul.py:147-253) takes one output block per program.
+ */
+int bsa_matmul_rows_records(const int32_t *work_table, int64_t n_items, int parts_log2,
+                            const int32_t *pair_offsets, const int32_t *x_row_offsets,
+                            const int32_t *o_row_offsets, int64_t n_rows, int64_t nnz_x, int32_t *records,
+                            bsa_stream_t stream);
+
+/*
+ * The same product as bsa_matmul for fp16 / bf16 operands with sbs == 64, organised by output block row: the
+ * x blocks of a row are kept in LDS while the row's output blocks are computed.  records (n_items records
+ * from bsa_matmul_rows_records, built for the same pair_offsets) says what each workgroup computes.
  * Bit-identical results to bsa_matmul (same accumulation order).  Same reference counterpart as
  * bsa_matmul.
  */
 int bsa_matmul_rows(const void *x, const void *y, void *out, const int32_t *pair_offsets,
-                    const int32_t *pairs, const int32_t *x_row_offsets, const int32_t *o_row_offsets,
-                    const int32_t *work_table, int64_t n_items, int parts_log2, int64_t n_rows, int64_t nnz_o,
+                    const int32_t *pairs, const int32_t *records, int64_t n_items, int64_t nnz_o,
                     int64_t nnz_x, int64_t nnz_y, int sbs, int dtype, bsa_stream_t stream);
 
 /*
