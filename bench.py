@@ -46,7 +46,7 @@ TRAFFIC_KIB = {  # config: (FETCH_SIZE, WRITE_SIZE)
     "v1": (66312.1, 129576.0),
     "v2": (66851.5, 524499.4),
     "t1": (67086.4, 129576.0),
-    "l1": (262170.9, 72.5),
+    "l1": (262170.4, 68.6),
     "r1": (64865.6, 8192.0),
     "r2": (66875.5, 129576.0),
 }
