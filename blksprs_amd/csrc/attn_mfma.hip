@@ -485,6 +485,9 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
   BSA_PROBE_FLUSH(blockIdx.x * 2 * G + wave, lane);
   // ---- epilogue: O = O^T^T / l, lse = m + log2(l) ----
   if (!has_q) return;
+  // one reciprocal per row, then products: 64 IEEE divisions per lane cost ten instructions each, and the last
+  // bit they would buy is rounded away with the other fifteen when the quotient becomes a 16-bit value
+  const float inv_l = (l_i != 0.f) ? 1.f / l_i : 0.f;
 #pragma unroll
   for (int h = 0; h < NHV; ++h) {
     const int64_t po = a.pidx_o[row * NHV + h];
@@ -496,7 +499,7 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
       for (int q = 0; q < 4; ++q) {
         float v[4];
 #pragma unroll
-        for (int t = 0; t < 4; ++t) v[t] = (l_i != 0.f) ? oacc[h][db][4 * q + t] / l_i : 0.f;
+        for (int t = 0; t < 4; ++t) v[t] = oacc[h][db][4 * q + t] * inv_l;
         u32x2 w;
         w[0] = Tr::pack2(v[0], v[1]);
         w[1] = Tr::pack2(v[2], v[3]);
