@@ -45,6 +45,8 @@ SIGNATURES = {
     "bsa_lut_workspace_bytes": (c_size_t, [c_int64]),
     "bsa_lut_packed": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                c_size_t, c_void_p]),
+    "bsa_lut_packed_static_max_entries": (c_int64, []),
+    "bsa_lut_packed_static": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
     "bsa_lut_nonzero": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p]),
     "bsa_lut_csr_indices": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_void_p]),
     "bsa_lut_sorted_rows": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_void_p]),

@@ -6,6 +6,8 @@
 // layout of a million entries is 512 tiles.
 #include "common.h"
 
+#include <mutex>
+
 namespace {
 
 constexpr int kScanThreads = 256;
@@ -308,34 +310,104 @@ inline unsigned grid_for(int64_t n, int threads) { return (unsigned)bsa::cdiv(n,
 
 extern "C" size_t bsa_lut_workspace_bytes(int64_t n) { return scan_workspace_bytes(n); }
 
-extern "C" int bsa_lut_packed(const uint8_t *layout, int64_t n, int64_t row_len, int64_t *packed,
-                              int32_t *row_offsets, int64_t *stats_dev, int64_t *stats_host, void *workspace,
-                              size_t workspace_bytes, bsa_stream_t stream) {
-  BSA_REQUIRE(n >= 0 && row_len >= 0, "bsa_lut_packed: negative size");
-  BSA_REQUIRE(stats_dev != nullptr, "bsa_lut_packed: stats_dev is NULL");
-  BSA_REQUIRE(row_len == 0 || row_offsets != nullptr, "bsa_lut_packed: row_len given without row_offsets");
-  BSA_REQUIRE(row_len == 0 || n % row_len == 0, "bsa_lut_packed: n is not a multiple of row_len");
-  if (n / kScanTile >= 0x7fffffffLL) return bsa::fail(BSA_ELIMIT, "bsa_lut_packed: layout too large");
-  hipStream_t s = bsa::as_stream(stream);
+namespace {
+
+// The launches of the scan; tile_counts (int32) and tile_offsets (int64) hold one entry per tile of kScanTile
+// layout entries and are written before they are read.
+int lut_packed_launch(const char *who, const uint8_t *layout, int64_t n, int64_t row_len, int64_t *packed,
+                      int32_t *row_offsets, int64_t *stats_dev, int64_t *stats_host, int32_t *tile_counts,
+                      int64_t *tile_offsets, hipStream_t s) {
+  BSA_REQUIRE(n >= 0 && row_len >= 0, "%s: negative size", who);
+  BSA_REQUIRE(stats_dev != nullptr, "%s: stats_dev is NULL", who);
+  BSA_REQUIRE(row_len == 0 || row_offsets != nullptr, "%s: row_len given without row_offsets", who);
+  BSA_REQUIRE(row_len == 0 || n % row_len == 0, "%s: n is not a multiple of row_len", who);
+  if (n / kScanTile >= 0x7fffffffLL) return bsa::fail(BSA_ELIMIT, "%s: layout too large", who);
   if (n == 0) {
     // row_len > 0 with n == 0 still has the leading 0 (n_rows is 0 then).
     zero_stats_kernel<<<1, 64, 0, s>>>(stats_dev, row_len > 0 ? row_offsets : nullptr, 1);
     if (int rc = bsa::check_launch("zero_stats_kernel")) return rc;
     return fetch_stats(stats_dev, stats_host, s);
   }
-  BSA_REQUIRE(layout && packed, "bsa_lut_packed: NULL layout or output");
-  BSA_REQUIRE(workspace && workspace_bytes >= scan_workspace_bytes(n), "bsa_lut_packed: workspace too small");
-  ScanWorkspace w = carve(workspace, n);
+  BSA_REQUIRE(layout && packed, "%s: NULL layout or output", who);
+  BSA_REQUIRE(tile_counts && tile_offsets, "%s: no workspace", who);
   const int64_t tiles = bsa::cdiv(n, kScanTile);
   const int64_t n_rows = row_len > 0 ? n / row_len : 0;
-  tile_counts_kernel<uint8_t><<<(unsigned)tiles, kScanThreads, 0, s>>>(layout, n, w.tile_counts);
-  scan_tiles_kernel<<<1, kScanThreads, 0, s>>>(w.tile_counts, tiles, w.tile_offsets, stats_dev,
+  tile_counts_kernel<uint8_t><<<(unsigned)tiles, kScanThreads, 0, s>>>(layout, n, tile_counts);
+  scan_tiles_kernel<<<1, kScanThreads, 0, s>>>(tile_counts, tiles, tile_offsets, stats_dev,
                                                row_len > 0 ? row_offsets + n_rows : nullptr);
-  write_packed_kernel<<<(unsigned)tiles, kScanThreads, 0, s>>>(layout, n, w.tile_offsets, row_len, packed,
-                                                               row_offsets);
+  write_packed_kernel<<<(unsigned)tiles, kScanThreads, 0, s>>>(layout, n, tile_offsets, row_len, packed, row_offsets);
   if (row_len > 0) row_max_kernel<<<grid_for(n_rows, 256), 256, 0, s>>>(row_offsets, n_rows, stats_dev);
-  if (int rc = bsa::check_launch("bsa_lut_packed")) return rc;
+  if (int rc = bsa::check_launch(who)) return rc;
   return fetch_stats(stats_dev, stats_host, s);
+}
+
+}  // namespace
+
+extern "C" int bsa_lut_packed(const uint8_t *layout, int64_t n, int64_t row_len, int64_t *packed,
+                              int32_t *row_offsets, int64_t *stats_dev, int64_t *stats_host, void *workspace,
+                              size_t workspace_bytes, bsa_stream_t stream) {
+  BSA_REQUIRE(n <= 0 || (workspace && workspace_bytes >= scan_workspace_bytes(n)),
+              "bsa_lut_packed: workspace too small");
+  ScanWorkspace w = carve(workspace, n);
+  return lut_packed_launch("bsa_lut_packed", layout, n, row_len, packed, row_offsets, stats_dev, stats_host,
+                           n > 0 ? w.tile_counts : nullptr, n > 0 ? w.tile_offsets : nullptr, bsa::as_stream(stream));
+}
+
+// ---------------------------------------------------------------------------------------------------
+// bsa_lut_packed_static: the scan of bsa_lut_packed with its tile counts and tile offsets in a file-scope
+// device array instead of a caller-provided workspace, for callers that cannot allocate.
+namespace {
+
+constexpr int64_t kStaticMaxEntries = (int64_t)1 << 24;                  // layout entries per call
+constexpr int64_t kStaticMaxTiles = kStaticMaxEntries / kScanTile;       // 8192
+constexpr size_t kStaticScratchBytes = (size_t)kStaticMaxTiles * (4 + 8);  // 96 KiB per device
+
+}  // namespace
+
+// Every device the library runs on holds its own copy of this array, at its own address.
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex static_scratch_mutex;
+void *static_scratch_ptr[kMaxDevices] = {nullptr};
+
+// Device address of `scratch` on the current device (looked up once per device; the host-side name
+// of the array is not an address a kernel can use).
+int static_scratch(void **out) {
+  int dev = -1;
+  BSA_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return bsa::fail(BSA_ELIMIT, "bsa_lut_packed_static: device %d out of range", dev);
+  std::lock_guard<std::mutex> lock(static_scratch_mutex);
+  if (!static_scratch_ptr[dev]) {
+    void *p = nullptr;
+    BSA_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) return bsa::fail(BSA_ELAUNCH, "bsa_lut_packed_static: no device address for the scratch array");
+    static_scratch_ptr[dev] = p;
+  }
+  *out = static_scratch_ptr[dev];
+  return BSA_OK;
+}
+
+}  // namespace
+
+extern "C" int64_t bsa_lut_packed_static_max_entries(void) { return kStaticMaxEntries; }
+
+extern "C" int bsa_lut_packed_static(const uint8_t *layout, int64_t n, int64_t row_len, int64_t *packed,
+                                     int32_t *row_offsets, int64_t *stats_dev, bsa_stream_t stream) {
+  BSA_REQUIRE(n >= 0 && row_len >= 0, "bsa_lut_packed_static: negative size");
+  if (n > kStaticMaxEntries)
+    return bsa::fail(BSA_ELIMIT, "bsa_lut_packed_static: %lld layout entries exceed the static scratch (at most %lld)",
+                     (long long)n, (long long)kStaticMaxEntries);
+  void *ws = nullptr;
+  if (int rc = static_scratch(&ws)) return rc;
+  // Same launches as bsa_lut_packed; every tile count and tile offset that is read is written first by this
+  // call, so what an earlier call left in the array does not matter.
+  int32_t *tile_counts = static_cast<int32_t *>(ws);
+  int64_t *tile_offsets = reinterpret_cast<int64_t *>(static_cast<char *>(ws) + kStaticMaxTiles * 4);
+  return lut_packed_launch("bsa_lut_packed_static", layout, n, row_len, packed, row_offsets, stats_dev, nullptr,
+                           tile_counts, tile_offsets, bsa::as_stream(stream));
 }
 
 extern "C" int bsa_lut_nonzero(const int64_t *packed, int64_t B, int64_t R, int64_t C, int64_t *coords,

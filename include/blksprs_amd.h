@@ -68,6 +68,22 @@ int bsa_lut_packed(const uint8_t *layout, int64_t n, int64_t row_len, int64_t *p
                    void *workspace, size_t workspace_bytes, bsa_stream_t stream);
 
 /*
+ * bsa_lut_packed for callers that cannot allocate device memory (code under HIP graph capture, serving loops,
+ * harnesses that forbid hipMalloc): the same launches and the same results, but the scan's scratch (one int32
+ * count and one int64 offset per tile of 2048 layout entries) lives in a file-scope device array of 96 KiB that
+ * every device the library runs on holds until the process ends, so no workspace is passed and nothing is
+ * allocated or freed.  n may be at most bsa_lut_packed_static_max_entries() (2^24 layout entries); a larger n
+ * returns BSA_ELIMIT.  The counts stay on the device (stats_dev as in bsa_lut_packed; no host copy, no wait for
+ * the stream).  The first call on a device looks up the array's device address (hipGetSymbolAddress); make that
+ * call outside a capture.  All calls on one device share the array: the call overwrites every entry it reads,
+ * so nothing needs clearing between calls, but two calls that overlap on one device (different streams or
+ * threads) race.  This entry point has no counterpart in the reference.
+ */
+int64_t bsa_lut_packed_static_max_entries(void);
+int bsa_lut_packed_static(const uint8_t *layout, int64_t n, int64_t row_len, int64_t *packed,
+                          int32_t *row_offsets, int64_t *stats_dev, bsa_stream_t stream);
+
+/*
  * Coordinates of the active blocks, int64 [count, 3] = (b, r, c) in row-major
  * order: torch.nonzero(layout) of build_layout_indices
  * (blksprs/utils/tools.py:33-35), derived from the reverse index.
