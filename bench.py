@@ -6,8 +6,15 @@ A step is one pass of the hot path over one batch of synthetic, seeded input tha
 HBM, with the lookup tables built beforehand (their build time is reported separately).  The default
 workload is configuration 2 of BASELINE.json (bf16 block-sparse matmul, B=16, 4096^3, sbs 64, 25 % operand
 density, product output layout), the configuration the headline metric is quoted on; ``--config`` selects
-c1 (fp32 matmul 256^3), c3 (fp32 softmax), c4 / c4bwd (bf16 flash attention forward / forward+backward) or
-c5 (fp16 matmul, sbs 16) instead.  One JSON line is printed on stdout; everything else goes to stderr.
+c1 (fp32 matmul 256^3), c2bwd (the two backward products of c2), c3 / c3bwd (fp32 softmax forward / backward),
+c4 / c4bwd (bf16 flash attention forward / forward+backward), c5 (fp16 matmul, sbs 16) or one of the data
+movement rows instead.  Without ``--config`` the line also carries, under ``other_configs``, the roofline objects of
+c4 (forward), c3 and c5, timed in the same process.  One JSON line is printed on stdout; everything else goes to
+stderr.
+
+Every configuration is first checked on a sample against the CPU oracle (``correct``), then run untimed for 0.3 s
+(a card that has idled starts below its sustained clock), then timed.  ``launch_ms_flushed`` / ``frac_flushed``
+repeat the timing with 1 GiB written between launches, so that no launch finds its operands in the memory-side cache.
 
 The ``roofline`` object prices the dominant kernel against the roofline that bounds it, from the average
 launch duration measured with events on the launch stream; ``cpu_baseline`` times the CPU oracle on a
@@ -95,8 +102,35 @@ def _sleep_cycles_per_ms():
     return probe / max(a.elapsed_time(b), 1e-3)
 
 
+PREROLL_MS = 300.0   # untimed work in front of the warm-up steps, whatever --warmup says
+FLUSH_BYTES = 1 << 30  # written between launches of the flushed timing: 4x the 256 MB memory-side cache
+
+
+def preroll(step):
+    """Runs ``step`` untimed until the card has worked for PREROLL_MS: a card that has idled runs its first tens of
+    milliseconds below its sustained clock, and the driver's run has only a few warm-up steps.  Returns
+    (milliseconds, launches)."""
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    n = 0
+    while True:
+        for _ in range(20):
+            step()
+        n += 20
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3
+        if ms >= PREROLL_MS:
+            return ms, n
+
+
+def _percentile(sorted_values, q):
+    return sorted_values[min(len(sorted_values) - 1, int(q * len(sorted_values)))]
+
+
 def time_steps(step, steps, warmup):
-    """Returns (wall ms per step over exactly `steps` steps, mean and median per-launch ms from stream events).
+    """Times exactly ``steps`` steps after ``warmup`` untimed ones.  Returns a dict: wall ms per step, per-launch
+    mean / median / p20 / p80 from stream events (p20 and p80 as the reference's own timing helper reports them,
+    blksprs/utils/benchmarking.py:15, :22-23), and the host's enqueue time per step.
 
     The per-launch figure must not contain the time the card waits for the host: a step whose kernels are
     shorter than the host's work per call leaves the stream empty between launches, and an event recorded on an
@@ -134,14 +168,52 @@ def time_steps(step, steps, warmup):
                 e.record()
             torch.cuda.synchronize()
     per = sorted(s.elapsed_time(e) for s, e in ev)
-    return wall_ms, sum(per) / len(per), per[len(per) // 2], host_ms
+    return {"wall_ms": wall_ms, "mean_ms": sum(per) / len(per), "median_ms": per[len(per) // 2],
+            "p20_ms": _percentile(per, 0.2), "p80_ms": _percentile(per, 0.8), "host_ms": host_ms}
+
+
+def time_steps_flushed(step, steps, scratch):
+    """Mean per-launch ms with the caches emptied in front of every launch: FLUSH_BYTES are written between the
+    launches, outside the event pair (the fill also keeps the stream busy while the host enqueues the step).  What a
+    launch finds in the 256 MB memory-side cache and the L2s is then what the fill left, not its own operands from
+    the launch before."""
+    ev = _events(steps)
+    for i, (s, e) in enumerate(ev):
+        scratch.fill_(i & 1)
+        s.record()
+        step()
+        e.record()
+    torch.cuda.synchronize()
+    per = sorted(s.elapsed_time(e) for s, e in ev)
+    return sum(per) / len(per)
+
+
+def count_host_syncs(fn):
+    """Runs ``fn`` and returns (milliseconds, number of calls that made the host wait for the device, as torch's
+    sync debug mode reports them)."""
+    import warnings
+    torch.cuda.synchronize()
+    torch.cuda.set_sync_debug_mode("warn")
+    try:
+        with warnings.catch_warnings(record=True) as seen:
+            warnings.simplefilter("always")
+            t0 = time.perf_counter()
+            fn()
+            torch.cuda.set_sync_debug_mode("default")
+            torch.cuda.synchronize()
+            ms = (time.perf_counter() - t0) * 1e3
+    finally:
+        torch.cuda.set_sync_debug_mode("default")
+    return ms, sum("synchroniz" in str(w.message).lower() for w in seen)
 
 
 # --------------------------------------------------------------------------- workloads
 
 
-def matmul_workload(name, B, n, sbs, dtype, density, ensure_rows, value_scale, dev, cpu_sample_batches):
+def matmul_workload(name, B, n, sbs, dtype, density, ensure_rows, value_scale, dev, cpu_sample_batches,
+                    backward=False, check_batch=0):
     import blksprs_amd as bs
+    from blksprs_amd.ops.matmul import matmul_build_layout_cache
     from oracle import blksprs_oracle as orc
 
     g = torch.Generator().manual_seed(0)
@@ -153,29 +225,62 @@ def matmul_workload(name, B, n, sbs, dtype, density, ensure_rows, value_scale, d
     gd = torch.Generator(device=dev).manual_seed(1)
     x = (torch.randn((nnz_x, sbs, sbs), generator=gd, device=dev) * value_scale).to(dtype)
     y = torch.randn((nnz_y, sbs, sbs), generator=gd, device=dev).to(dtype)
+    go = (torch.randn((nnz_o, sbs, sbs), generator=gd, device=dev) / math.sqrt(n * sbs)).to(dtype)
 
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     cache = {}
     out = bs.ops.matmul(x, lxd, y, lyd, lod, sbs, layout_cache=cache)
     torch.cuda.synchronize()
-    lut_ms = (time.perf_counter() - t0) * 1e3
+    first_ms = (time.perf_counter() - t0) * 1e3  # holds the load of the library and of its code objects
+    # the lookup tables of a second, empty cache: what a new triple of layouts costs once the library is loaded
+    lut_ms, lut_syncs = count_host_syncs(lambda: matmul_build_layout_cache(None, lxd, lyd, lod))
     pairs = int(cache["contraction_pairs"].size(0))
     es = x.element_size()
     flops = pairs * 2.0 * sbs ** 3
     alg_bytes = (nnz_x + nnz_y + nnz_o) * sbs * sbs * es
     log(f"[{name}] nnz_x={nnz_x} nnz_y={nnz_y} nnz_o={nnz_o} ({nnz_o / (B * n * n):.1%} of output) "
         f"pairs={pairs} (mean {pairs / max(nnz_o, 1):.2f}/block) flops={flops / 1e9:.2f}G "
-        f"algorithmic bytes={alg_bytes / 1e6:.1f}MB; first call incl. LUT build {lut_ms:.2f} ms")
+        f"algorithmic bytes={alg_bytes / 1e6:.1f}MB; first call {first_ms:.2f} ms, lookup tables of a fresh cache "
+        f"{lut_ms:.2f} ms with {lut_syncs} host syncs")
 
     bs.utils.disable_validation()
+    if backward:
+        xg, yg = x.requires_grad_(True), y.requires_grad_(True)
+        graph_out = bs.ops.matmul(xg, lxd, yg, lyd, lod, sbs, layout_cache=cache)
 
-    def step():
-        return bs.ops.matmul(x, lxd, y, lyd, lod, sbs, layout_cache=cache)
+        def step():  # dX = dO Y^T and dY = X^T dO, nothing else
+            return torch.autograd.grad(graph_out, (xg, yg), go, retain_graph=True)
+
+        flops = 2.0 * flops
+        alg_bytes = (2 * nnz_o + 2 * nnz_x + 2 * nnz_y) * sbs * sbs * es
+    else:
+        def step():
+            return bs.ops.matmul(x, lxd, y, lyd, lod, sbs, layout_cache=cache)
+
+    def slices(b):
+        sl = lambda lay, t: t[int(lay[:b].sum()):int(lay[:b + 1].sum())].detach().cpu()
+        lo = lod.cpu()
+        return lo, sl(lx, x), sl(ly, y), sl(lo, go), sl
+
+    def check():
+        """Batch entry ``check_batch`` against the CPU oracle (fp64 accumulation of the rounded operands)."""
+        b = check_batch
+        lo, xs, ys, gs, sl = slices(b)
+        tol = 1e-5 if dtype == torch.float32 else 2e-2
+        close = lambda got, want: bool(torch.allclose(got.double().cpu(), want.double(), rtol=tol, atol=tol))
+        lxb, lyb, lob = lx[b:b + 1].numpy(), ly[b:b + 1].numpy(), lo[b:b + 1].numpy()
+        if not backward:
+            want = orc.matmul(xs.double(), lxb, ys.double(), lyb, lob, sbs, acc_dtype=torch.float64)
+            return close(sl(lo, step()), want)
+        x64, y64 = xs.double().requires_grad_(True), ys.double().requires_grad_(True)
+        orc.matmul(x64, lxb, y64, lyb, lob, sbs, acc_dtype=torch.float64).backward(gs.double())
+        dx, dy = step()
+        return close(sl(lx, dx), x64.grad) and close(sl(ly, dy), y64.grad)
 
     def cpu_baseline():
         nb = min(cpu_sample_batches, B)
-        sl = lambda lay, t: t[:int(lay[:nb].sum())].float().cpu()
+        sl = lambda lay, t: t[:int(lay[:nb].sum())].detach().float().cpu()
         lo = lod.cpu()
         xs, ys = sl(lx, x), sl(ly, y)
         reps, dt = _repeat_for(CPU_SAMPLE_SECONDS, lambda: orc.matmul(
@@ -183,15 +288,22 @@ def matmul_workload(name, B, n, sbs, dtype, density, ensure_rows, value_scale, d
         sample_pairs = int(torch.einsum("bik,bkj,bij->", lx[:nb].float(), ly[:nb].float(), lo[:nb].float()))
         return {"value": sample_pairs * 2.0 * sbs ** 3 / dt / 1e12, "unit": "TFLOP/s",
                 "cores": torch.get_num_threads(), "kind": "port",
-                "sample": f"{nb} of {B} batches x {reps} passes, dense-masked fp32 torch matmul + to_sparse, "
-                          f"{dt * reps:.1f} s"}
+                "sample": f"{'forward of ' if backward else ''}{nb} of {B} batches x {reps} passes, dense-masked fp32 "
+                          f"torch matmul + to_sparse, {dt * reps:.1f} s"}
 
     dt_name = {torch.bfloat16: "bf16", torch.float16: "f16", torch.float32: "f32"}[dtype]
+    if backward:
+        kernel = "matmul_mfma_kernel (two launches: dX with y read transposed, dY with x read transposed)"
+    elif sbs > 16:
+        kernel = "matmul_rows_kernel" if sbs == 64 and dtype != torch.float32 else "matmul_mfma_kernel"
+    else:
+        kernel = "matmul_small16_kernel" if dtype != torch.float32 else "matmul_small_kernel"
     return dict(step=step, flops=flops, alg_bytes=alg_bytes, dtype=dt_name, bound="hbm", cpu_baseline=cpu_baseline,
-                kernel=("matmul_rows_kernel" if sbs == 64 and dtype != torch.float32 else "matmul_mfma_kernel") if sbs > 16 else ("matmul_small16_kernel" if dtype != torch.float32 else "matmul_small_kernel"),
+                check=check, kernel=kernel,
                 config={"workload": name, "B": B, "M": n * sbs, "K": n * sbs, "N": n * sbs,
                         "sparsity_block_size": sbs, "density": density, "nnz_x": nnz_x, "nnz_y": nnz_y,
-                        "nnz_o": nnz_o, "block_pairs": pairs, "lut_build_ms": round(lut_ms, 3)})
+                        "nnz_o": nnz_o, "block_pairs": pairs, "first_call_ms": round(first_ms, 3),
+                        "lut_build_ms": round(lut_ms, 3), "lut_build_host_syncs": lut_syncs})
 
 
 def linear_workload(dev):
@@ -238,7 +350,7 @@ def linear_workload(dev):
                         "nnz_o": nnz_o})
 
 
-def softmax_workload(dev):
+def softmax_workload(dev, backward=False):
     import blksprs_amd as bs
     from oracle import blksprs_oracle as orc
 
@@ -249,28 +361,46 @@ def softmax_workload(dev):
     ld = layout.to(dev)
     nnz = int(layout.sum())
     x = torch.randn((nnz, sbs, sbs), device=dev) * 2.0  # N(0, 4): sigma = 2
+    go = torch.randn((nnz, sbs, sbs), device=dev)
     cache = {}
     bs.ops.softmax(x, ld, sbs, layout_cache=cache)
-    alg_bytes = 2 * nnz * sbs * sbs * 4
-    log(f"[c3] nnz={nnz} algorithmic bytes={alg_bytes / 1e6:.1f}MB")
+    lut_ms, lut_syncs = count_host_syncs(lambda: bs.ops.softmax(x, ld, sbs, layout_cache={}))
+    alg_bytes = (3 if backward else 2) * nnz * sbs * sbs * 4
+    log(f"[c3] nnz={nnz} algorithmic bytes={alg_bytes / 1e6:.1f}MB; call with a fresh cache {lut_ms:.2f} ms, "
+        f"{lut_syncs} host syncs")
     bs.utils.disable_validation()
+    if backward:
+        xg = x.requires_grad_(True)
+        graph_out = bs.ops.softmax(xg, ld, sbs, layout_cache=cache)
 
-    def step():
-        return bs.ops.softmax(x, ld, sbs, layout_cache=cache)
+        def step():  # reads y and dy, writes dx
+            return torch.autograd.grad(graph_out, xg, go, retain_graph=True)[0]
+    else:
+        def step():
+            return bs.ops.softmax(x, ld, sbs, layout_cache=cache)
+
+    def check():
+        """Batch entry 0 against the CPU oracle at rtol = atol = 1e-5."""
+        cnt = int(layout[:1].sum())
+        xs = x[:cnt].detach().cpu()
+        ys = orc.softmax(xs, layout[:1].numpy(), sbs)
+        want = orc.softmax_backward(go[:cnt].cpu(), ys, layout[:1].numpy(), sbs) if backward else ys
+        return bool(torch.allclose(step()[:cnt].cpu().double(), want.double(), rtol=1e-5, atol=1e-5))
 
     def cpu_baseline():
         nb = 8
         cnt = int(layout[:nb].sum())
-        xs = x[:cnt].cpu()
+        xs = x[:cnt].detach().cpu()
         reps, dt = _repeat_for(CPU_SAMPLE_SECONDS, lambda: orc.softmax(xs, layout[:nb].numpy(), sbs))
         return {"value": 2 * cnt * sbs * sbs * 4 / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(),
-                "kind": "port", "sample": f"{nb} of {B} batches x {reps} passes, dense -inf-masked torch softmax (fp64), "
-                                            f"{dt * reps:.1f} s"}
+                "kind": "port", "sample": f"{'forward of ' if backward else ''}{nb} of {B} batches x {reps} passes, "
+                                          f"dense -inf-masked torch softmax (fp64), {dt * reps:.1f} s"}
 
     return dict(step=step, flops=0.0, alg_bytes=alg_bytes, dtype="f32", bound="hbm", cpu_baseline=cpu_baseline,
-                kernel="softmax_fwd_kernel",
-                config={"workload": "c3_softmax_fp32", "B": B, "rows": n * sbs, "cols": n * sbs,
-                        "sparsity_block_size": sbs, "nnz": nnz})
+                check=check, kernel="softmax_bwd_kernel" if backward else "softmax_fwd_kernel",
+                config={"workload": "c3_softmax_fp32" + ("_backward" if backward else ""), "B": B, "rows": n * sbs,
+                        "cols": n * sbs, "sparsity_block_size": sbs, "nnz": nnz, "lut_build_ms": round(lut_ms, 3),
+                        "lut_build_host_syncs": lut_syncs})
 
 
 def movement_workload(dev, which):
@@ -304,8 +434,13 @@ def movement_workload(dev, which):
             return {"value": 2 * cnt * sbs * sbs * 2 / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(),
                     "kind": "port", "sample": f"{nb} of {B} batches x {reps} passes, per-block torch transpose, {dt * reps:.1f} s"}
 
+        def check():
+            cnt = int(layout[:1].sum())
+            want, _ = orc.transpose(x[:cnt].cpu(), layout[:1].numpy(), sbs)
+            return bool(torch.equal(step()[0][:cnt].cpu(), want))
+
         return dict(step=step, flops=0.0, alg_bytes=alg_bytes, dtype="bf16", bound="hbm", cpu_baseline=cpu_baseline,
-                    kernel="transpose_blocks16_kernel",
+                    check=check, kernel="transpose_blocks16_kernel",
                     config={"workload": "t1_transpose_bf16", "B": B, "rows": n * sbs, "cols": n * sbs,
                             "sparsity_block_size": sbs, "nnz": nnz})
     if which in ("row_sum", "row_add"):
@@ -326,8 +461,13 @@ def movement_workload(dev, which):
                         "cores": torch.get_num_threads(), "kind": "port",
                         "sample": f"{nb} of {B} batches x {reps} passes, per-block torch sums, {dt * reps:.1f} s"}
 
+            def check():
+                want = orc.row_wise_reduce(xs, lnp[:nb], sbs, "sum")[0]
+                got = step()[0][:want.size(0)].cpu()
+                return bool(torch.allclose(got.double(), want.double(), rtol=2e-2, atol=2e-2))
+
             return dict(step=step, flops=0.0, alg_bytes=alg_bytes, dtype="bf16", bound="hbm",
-                        cpu_baseline=cpu_baseline, kernel="row_reduce_kernel",
+                        cpu_baseline=cpu_baseline, check=check, kernel="row_reduce_kernel",
                         config={"workload": "r1_row_wise_sum_bf16", "B": B, "rows": n * sbs, "cols": n * sbs,
                                 "sparsity_block_size": sbs, "nnz": nnz})
         y = torch.randn((n_rows, sbs, 1), device=dev, dtype=torch.bfloat16, generator=gd)
@@ -343,8 +483,12 @@ def movement_workload(dev, which):
                     "kind": "port",
                     "sample": f"{nb} of {B} batches x {reps} passes, per-block torch adds, {dt * reps:.1f} s"}
 
+        def check():
+            want = orc.row_wise_add(xs, lnp[:nb], ys, sbs)
+            return bool(torch.allclose(step()[:cnt].cpu().double(), want.double(), rtol=2e-2, atol=2e-2))
+
         return dict(step=step, flops=0.0, alg_bytes=alg_bytes, dtype="bf16", bound="hbm", cpu_baseline=cpu_baseline,
-                    kernel="row_add_kernel",
+                    check=check, kernel="row_add_kernel",
                     config={"workload": "r2_row_wise_add_bf16", "B": B, "rows": n * sbs, "cols": n * sbs,
                             "sparsity_block_size": sbs, "nnz": nnz})
     dense = bs.ops.to_dense(x, ld, sbs)
@@ -368,6 +512,7 @@ def movement_workload(dev, which):
                         "kind": "port", "sample": f"{nb} of {B} batches x {reps} passes, torch reshape / permute / "
                                                   f"boolean index, {dt * reps:.1f} s"}
 
+            check = lambda: bool(torch.equal(step()[:cnt].cpu(), orc.to_sparse(ds, lnp[:nb], sbs)))
             kernel, workload = "to_sparse_kernel", "v1_to_sparse_bf16"
         else:
             bs.ops.to_dense(x, ld, sbs, layout_cache=cache)
@@ -385,9 +530,10 @@ def movement_workload(dev, which):
                         "sample": f"{nb} of {B} batches x {reps} passes, torch fill / boolean index / permute, "
                                   f"{dt * reps:.1f} s"}
 
+            check = lambda: bool(torch.equal(step()[:nb].cpu(), orc.to_dense(xs, lnp[:nb], sbs)))
             kernel, workload = "to_dense_kernel", "v2_to_dense_bf16"
         return dict(step=step, flops=0.0, alg_bytes=alg_bytes, dtype="bf16", bound="hbm", cpu_baseline=cpu_baseline,
-                    kernel=kernel, config={"workload": workload, "B": B, "rows": n * sbs, "cols": n * sbs,
+                    check=check, kernel=kernel, config={"workload": workload, "B": B, "rows": n * sbs, "cols": n * sbs,
                                            "sparsity_block_size": sbs, "nnz": nnz})
     alg_bytes = dense.numel() * 2 + B * n * n
 
@@ -401,8 +547,12 @@ def movement_workload(dev, which):
         return {"value": ds.numel() * 2 / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
                 "sample": f"{nb} of {B} batches x {reps} passes, torch != 0 and any over blocks, {dt * reps:.1f} s"}
 
+    def check():
+        want = torch.from_numpy(orc.build_sparsity_layout(dense[:1].cpu(), sbs))
+        return bool(torch.equal(step()[:1].cpu().to(torch.bool), want.to(torch.bool)))
+
     return dict(step=step, flops=0.0, alg_bytes=alg_bytes, dtype="bf16", bound="hbm", cpu_baseline=cpu_baseline,
-                kernel="layout_from_dense_kernel",
+                check=check, kernel="layout_from_dense_kernel",
                 config={"workload": "l1_build_sparsity_layout_bf16", "B": B, "rows": n * sbs, "cols": n * sbs,
                         "sparsity_block_size": sbs, "active_blocks": nnz})
 
@@ -449,6 +599,20 @@ def attention_workload(dev, backward):
             o.backward(d_o)
         return o
 
+    def check():
+        """Head 0 against the CPU oracle (dense masked attention, fp32 accumulation) at rtol = atol = 2e-2."""
+        cnt = int(lmask[:1].sum())
+        fl = full[:1].cpu().numpy()
+        leaves = [t[:n * nh].detach().float().cpu().requires_grad_(backward) for t in (q, k, v)]
+        want = orc.flash_attention(leaves[0], fl, leaves[1], fl, leaves[2], fl, la[:1].numpy(), sbs,
+                                   mask=mask[:cnt].cpu(), layout_mask=lmask[:1].numpy())
+        close = lambda got, ref: bool(torch.allclose(got[:n * nh].detach().float().cpu(), ref, rtol=2e-2, atol=2e-2))
+        ok = close(step(), want.detach())
+        if backward:
+            want.backward(d_o[:n * nh].float().cpu())
+            ok = ok and all(close(t.grad, ref.grad) for t, ref in zip((q, k, v), leaves))
+        return ok
+
     def cpu_baseline():
         heads = 1
         qs, ks, vs = (t[:heads * n * nh].detach().float().cpu() for t in (q, k, v))
@@ -463,7 +627,7 @@ def attention_workload(dev, backward):
                           f"{dt * reps:.1f} s"}
 
     return dict(step=step, flops=flops, alg_bytes=alg_bytes, dtype="bf16", bound="mfma", cpu_baseline=cpu_baseline,
-                executed_flops=flops * live_pairs / nnz,
+                check=check, executed_flops=flops * live_pairs / nnz,
                 kernel="attn_fwd_mfma_kernel" if not backward else
                 "attn_fwd_mfma_kernel + attn_bwd_delta_kernel + attn_bwd_kv8_kernel + attn_bwd_q_kernel (one step; the mask_dead / records / order kernels ran once, in the warm-up)",
                 config={"workload": "c4_flash_attention_bf16" + ("_fwd_bwd" if backward else "_fwd"),
@@ -475,9 +639,15 @@ def make_workload(name, dev):
     if name == "c1":
         return matmul_workload("c1_matmul_fp32", 2, 8, 32, torch.float32, 0.5, True, 1.0, dev, 2)
     if name == "c2":
-        return matmul_workload("c2_matmul_bf16", 16, 64, 64, torch.bfloat16, 0.25, False, 1.0 / 64.0, dev, 16)
+        return matmul_workload("c2_matmul_bf16", 16, 64, 64, torch.bfloat16, 0.25, False, 1.0 / 64.0, dev, 16,
+                               check_batch=3)
+    if name == "c2bwd":
+        return matmul_workload("c2_matmul_bf16_backward", 16, 64, 64, torch.bfloat16, 0.25, False, 1.0 / 64.0, dev,
+                               16, backward=True, check_batch=3)
     if name == "c3":
         return softmax_workload(dev)
+    if name == "c3bwd":
+        return softmax_workload(dev, backward=True)
     if name == "c4":
         return attention_workload(dev, backward=False)
     if name == "c4bwd":
@@ -501,14 +671,63 @@ def make_workload(name, dev):
     raise SystemExit(f"unknown config {name}")
 
 
+CONFIGS = ["c1", "c2", "c2bwd", "c3", "c3bwd", "c4", "c4bwd", "c5", "t1", "l1", "r1", "r2", "p1", "v1", "v2"]
+# the configurations a default run times behind the headline one, with fewer steps (their roofline objects ride
+# along in the same JSON line so that they are timed by whoever runs the script, not quoted from elsewhere)
+COMPANIONS = ["c4", "c3", "c5"]
+
+
+def measure(config, dev, steps, warmup, scratch):
+    """Builds the workload, checks a sample against the oracle, times it.  Returns (workload, result dict)."""
+    import blksprs_amd as bs
+
+    w = make_workload(config, dev)
+    try:
+        correct = w["check"]() if "check" in w else None
+    finally:
+        bs.utils.disable_validation()
+    preroll_ms, preroll_launches = preroll(w["step"])
+    t = time_steps(w["step"], steps, warmup)
+    flushed_ms = time_steps_flushed(w["step"], min(steps, 50), scratch)
+    mean_ms = t["mean_ms"]
+    if w["bound"] == "hbm":
+        gbs = w["alg_bytes"] / (mean_ms * 1e-3) / 1e9
+        roofline = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                    "frac": round(gbs / PEAK_HBM_GBS, 4)}
+        roofline["frac_flushed"] = round(w["alg_bytes"] / (flushed_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)
+    else:
+        ach = w["flops"] / (mean_ms * 1e-3) / 1e12
+        peak = PEAK_MFMA_TFLOPS[w["dtype"]]
+        roofline = {"bound": "mfma", "achieved": round(ach, 1), "peak": peak, "unit": "TFLOP/s",
+                    "frac": round(ach / peak, 4)}
+        roofline["frac_flushed"] = round(w["flops"] / (flushed_ms * 1e-3) / 1e12 / peak, 4)
+    if "executed_flops" in w:
+        # the matrix-core work the kernels really do (pairs that the mask rules out as a whole are skipped): this,
+        # not the metric's count over all pairs of the layout, is the utilisation of the matrix cores
+        executed = w["executed_flops"] / (mean_ms * 1e-3) / 1e12
+        roofline["achieved_executed"] = round(executed, 1)
+        roofline["frac_executed"] = round(executed / roofline["peak"], 4)
+    roofline["traffic"] = traffic_bytes(config)
+    roofline["algorithmic_bytes"] = int(w["alg_bytes"])
+    roofline["kernel"] = w["kernel"]
+    roofline["launch_ms_mean"] = round(mean_ms, 4)
+    roofline["launch_ms_median"] = round(t["median_ms"], 4)
+    roofline["launch_ms_p20"] = round(t["p20_ms"], 4)
+    roofline["launch_ms_p80"] = round(t["p80_ms"], 4)
+    roofline["launch_ms_flushed"] = round(flushed_ms, 4)  # caches emptied in front of every launch
+    roofline["host_ms_per_step"] = round(t["host_ms"], 4)  # what the host needs to enqueue one step
+    roofline["preroll_ms"] = round(preroll_ms, 1)
+    roofline["preroll_launches"] = preroll_launches
+    return w, {"wall_ms": t["wall_ms"], "roofline": roofline, "correct": correct}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    # the card needs about a hundred launches (some tens of milliseconds) to settle at its sustained clock:
-    # with 10 warm-up steps the first timed steps of configuration 2 still run 10 % slower
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=100)
-    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c4bwd", "c5", "t1", "l1", "r1", "r2", "p1", "v1", "v2"])
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--config", default=None, choices=CONFIGS,
+                    help="one configuration only; without it: c2 as the headline, then " + ", ".join(COMPANIONS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -518,41 +737,40 @@ def main():
         raise SystemExit("bench.py needs a GPU (the product has no CPU path)")
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    w = make_workload(args.config, dev)
-    wall_ms, mean_ms, median_ms, host_ms = time_steps(w["step"], args.steps, args.warmup)
+    scratch = torch.empty(FLUSH_BYTES, dtype=torch.uint8, device=dev)
+    headline = args.config or "c2"
+    w, r = measure(headline, dev, args.steps, args.warmup, scratch)
+    wall_ms = r["wall_ms"]
     tflops = w["flops"] / (wall_ms * 1e-3) / 1e12
-    gbs = w["alg_bytes"] / (mean_ms * 1e-3) / 1e9
-    if w["bound"] == "hbm":
-        roofline = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                    "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None}
-    else:
-        ach = w["flops"] / (mean_ms * 1e-3) / 1e12
-        peak = PEAK_MFMA_TFLOPS[w["dtype"]]
-        roofline = {"bound": "mfma", "achieved": round(ach, 1), "peak": peak, "unit": "TFLOP/s",
-                    "frac": round(ach / peak, 4), "traffic": None}
-    if "executed_flops" in w:
-        # the matrix-core work the kernels really do (pairs that the mask rules out as a whole are skipped)
-        executed = w["executed_flops"] / (mean_ms * 1e-3) / 1e12
-        roofline["achieved_executed"] = round(executed, 1)
-        roofline["frac_executed"] = round(executed / roofline["peak"], 4)
-    roofline["traffic"] = traffic_bytes(args.config)
-    roofline["algorithmic_bytes"] = int(w["alg_bytes"])
-    roofline["kernel"] = w["kernel"]
-    roofline["launch_ms_mean"] = round(mean_ms, 4)
-    roofline["launch_ms_median"] = round(median_ms, 4)
-    roofline["host_ms_per_step"] = round(host_ms, 4)  # what the host needs to enqueue one step
+    gbs = w["alg_bytes"] / (wall_ms * 1e-3) / 1e9
     line = {
         "metric": "effective TFLOP/s on nonzero blocks" if w["flops"] else "achieved GB/s on nonzero blocks",
         "value": round(tflops, 3) if w["flops"] else round(gbs, 1),
         "unit": "TFLOP/s" if w["flops"] else "GB/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall_ms, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": w["dtype"], "data": "synthetic",
-        "config": w["config"], "roofline": roofline,
+        "config": w["config"], "roofline": r["roofline"], "correct": r["correct"],
     }
     if w["flops"]:
         line["pct_of_mfma_peak"] = round(100.0 * tflops / PEAK_MFMA_TFLOPS[w["dtype"]], 2)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = w["cpu_baseline"]()
+    del w
+    if args.config is None:
+        others = {}
+        for name in COMPANIONS:
+            torch.cuda.empty_cache()
+            wo, ro = measure(name, dev, min(args.steps, 50), args.warmup, scratch)
+            entry = {"workload": wo["config"]["workload"], "dtype": wo["dtype"], "ms_per_step": round(ro["wall_ms"], 4),
+                     "roofline": ro["roofline"], "correct": ro["correct"]}
+            if wo["flops"]:
+                entry["tflops"] = round(wo["flops"] / (ro["wall_ms"] * 1e-3) / 1e12, 3)
+            for key in ("lut_build_ms", "lut_build_host_syncs"):
+                if key in wo["config"]:
+                    entry[key] = wo["config"][key]
+            others[name] = entry
+            del wo
+        line["other_configs"] = others
     print(json.dumps(line), flush=True)
 
 

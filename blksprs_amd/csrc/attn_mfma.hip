@@ -31,27 +31,6 @@
 // multiply V; the row sum uses the unrounded values.
 #include "attn_mfma_common.h"
 
-// Phase clocks for an offline timing harness; compiled out of the library.
-#ifdef BSA_ATTN_PROBE
-__device__ unsigned long long bsa_attn_probe[8 * 4096];
-#define BSA_PROBE_DECL unsigned long long probe_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0}, probe_t = __builtin_readcyclecounter()
-#define BSA_PROBE(slot)                                            \
-  do {                                                             \
-    const unsigned long long now_ = __builtin_readcyclecounter();  \
-    probe_acc[slot] += now_ - probe_t;                             \
-    probe_t = now_;                                                \
-  } while (0)
-#define BSA_PROBE_FLUSH(wg, lane_)                                                                   \
-  do {                                                                                               \
-    if ((wg) < 4096 && (lane_) == 0)                                                                 \
-      for (int i_ = 0; i_ < 8; ++i_) bsa_attn_probe[(wg) * 8 + i_] = probe_acc[i_];                 \
-  } while (0)
-#else
-#define BSA_PROBE_DECL
-#define BSA_PROBE(slot)
-#define BSA_PROBE_FLUSH(wg, lane_)
-#endif
-
 namespace bsa {
 namespace {
 
@@ -129,7 +108,6 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
   }
   const int qpos = (int)qb * kSbs + qi;
 
-  BSA_PROBE_DECL;
   if (k_begin < k_end) {
     u32x4 mask_a[2], mask_b[2];  // mask words of a tile as loaded: a = arrived, being judged; b = in flight
     // Per-tile facts travel through a short pipeline.  For tile j: its record is loaded while tile j-3 is
@@ -282,7 +260,6 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
     }
 
     for (int e = k_begin; e < k_end; ++e) {
-      BSA_PROBE(0);
       const int buf = (e - k_begin) & 1;
       // mask words of tile e+2, requested one tile ago
       mask_a[0] = mask_b[0];
@@ -299,7 +276,6 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
       Facts f3 = make_facts(r3);
       const int rv4 = load_record(clamp_e(e + 4));
       fetch_mask(f3.pm, mask_b);
-      BSA_PROBE(1);
 
       // tile e.  A tile in which every score of this wave's 32 rows is masked changes nothing: m stays, alpha
       // is 1, every p is 0.
@@ -344,7 +320,6 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
             __builtin_amdgcn_sched_barrier(0);
           }
         }
-        BSA_PROBE(2);
 
         // first batch of V fragments: in flight while the softmax runs
         constexpr int kVBatches = NHV * 4;  // batch g: head slice g / 4, key quarter g % 4, both column halves
@@ -460,7 +435,6 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
           for (int db = 0; db < 2; ++db) oacc[h][db] = Tr::mfma(vf[g & 1][db], pf[jq >> 1][jq & 1], oacc[h][db]);
           __builtin_amdgcn_sched_barrier(0);
         }
-        BSA_PROBE(3);
       }  // live
 
       // ---- the barrier ends the reads of tile e and publishes tile e+1 and the verdicts on tile e+2 ----
@@ -476,13 +450,10 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
       r1 = r2;
       r2 = r3;
       rv3 = rv4;
-      BSA_PROBE(4);
       __syncthreads();
-      BSA_PROBE(5);
     }
   }
 
-  BSA_PROBE_FLUSH(blockIdx.x * 2 * G + wave, lane);
   // ---- epilogue: O = O^T^T / l, lse = m + log2(l) ----
   if (!has_q) return;
   // one reciprocal per row, then products: 64 IEEE divisions per lane cost ten instructions each, and the last

@@ -73,8 +73,9 @@ typedef __attribute__((address_space(3))) void *lds_ptr_t;
 // Asynchronous copy of 64 x 16 bytes, global -> LDS: lane l's 16 bytes land at dst + 16 l (dst is wave
 // uniform).  Completion is counted by vmcnt like any vector load.  Written as inline assembly so that the
 // compiler's wait-count pass does not see it: it would otherwise wait for the copy in front of every later
-// LDS read, also reads of other LDS arrays.  m0 is reserved: the compiler sets it before each of its own
-// uses and keeps nothing in it across statements.  The caller waits (vmcnt(0)) before the data is read.  Copies
+// LDS read, also reads of other LDS arrays.  m0 is a reserved register for clang's AMDGPU backend (it is never allocated
+// to a value that lives across statements: the backend writes it immediately in front of each of its own uses,
+// and naming it in a clobber list is diagnosed as undefined behaviour), so overwriting it here is safe.  The caller waits (vmcnt(0)) before the data is read.  Copies
 // the compiler does not know about only make the waits it computes for its own loads longer, never shorter.
 // The source is base (wave uniform) + off (per lane, 32 bits).
 __device__ static inline void copy_1k_to_lds(const char *base, uint32_t off, char *dst) {

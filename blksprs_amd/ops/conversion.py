@@ -10,7 +10,7 @@ from torch import Tensor
 
 from .. import _capi
 from ..utils.blksprs_tensor import BlksprsTensor
-from ..utils.tools import (finalize_layout_cache, nonzero_from_packed, pack_layout, prepare_layout_cache)
+from ..utils.tools import (eager_only, finalize_layout_cache, nonzero_from_packed, pack_layout, prepare_layout_cache)
 from ..utils.validation import (ensure_contiguous, validate_contiguous, validate_device, validate_dimensions,
                                 validate_dtype_supported, validate_sparsity, validate_sparsity_block_size,
                                 validate_sparsity_dense)
@@ -95,7 +95,7 @@ def to_dense_build_layout_cache(layout_cache: dict | None, sparsity_layout: Tens
     return finalize_layout_cache(layout_cache)
 
 
-@torch.compiler.disable
+@eager_only
 @torch.amp.custom_fwd(device_type="cuda")
 def to_sparse(x: Tensor, sparsity_layout: Tensor,
               sparsity_block_size: int, layout_cache: dict | None = None) -> BlksprsTensor:
@@ -130,7 +130,7 @@ def to_sparse(x: Tensor, sparsity_layout: Tensor,
                                               sparsity_block_size, layout_cache["n_sparse_blocks"]))
 
 
-@torch.compiler.disable
+@eager_only
 @torch.amp.custom_fwd(device_type="cuda")
 def to_dense(x: BlksprsTensor, sparsity_layout: Tensor,
              sparsity_block_size: int, fill_value: float = 0, layout_cache: dict | None = None) -> Tensor:

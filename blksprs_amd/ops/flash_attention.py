@@ -18,11 +18,11 @@ from torch import Tensor
 from .. import _capi
 from ..layouting.sparsity_layout import build_sparsity_layout_matmul
 from ..utils.blksprs_tensor import BlksprsTensor
-from ..utils.tools import (INT32_INDEX_MAX, CacheHolder, as_base_tensor, cast_for_autocast, csr_indices_from_packed,
-                           finalize_layout_cache, pack_layout, prepare_layout_cache)
-from ..utils.validation import (ensure_contiguous, validate_binary, validate_contiguous, validate_device,
-                                validate_dimensions, validate_dtype_float, validate_shape, validate_sparsity,
-                                validate_sparsity_block_size, validate_sparsity_layout)
+from ..utils.tools import (CacheHolder, INT32_INDEX_MAX, as_base_tensor, cast_for_autocast, csr_indices_from_packed,
+                           eager_only, finalize_layout_cache, pack_layout, prepare_layout_cache)
+from ..utils.validation import (ensure_contiguous, mask_facts_enabled, validate_binary, validate_contiguous,
+                                validate_device, validate_dimensions, validate_dtype_float, validate_shape,
+                                validate_sparsity, validate_sparsity_block_size, validate_sparsity_layout)
 
 
 def _select_segmented_index_dtype(n_active_blocks: int, n_blocks_col: int) -> torch.dtype:
@@ -251,6 +251,22 @@ def _build_forward_records(layout_cache: dict, attention_layout: Tensor, n_batch
     return offsets, as_base_tensor(records), group_size
 
 
+class _Tables:
+    """The lookup tables of one attention layout cache as one object.  A forward pass hands this object, not the
+    caller's cache dict, to its backward pass: the dict may be emptied and refilled for other layouts between the
+    two (``prepare_layout_cache`` clears it in place), the object keeps what it was built with.  Nothing writes
+    to its tensors after they are built."""
+
+    _NAMES = ("n_sparse_blocks_o", "packed_indices_q", "packed_indices_k", "packed_indices_v", "packed_indices_o",
+              "packed_indices_mask", "packed_indices_bias", "key_offsets_i32", "key_indices_i32",
+              "query_offsets_i32", "query_indices_i32", "group_offsets", "group_records", "group_size")
+    __slots__ = _NAMES
+
+    def __init__(self, cache: dict):
+        for name in self._NAMES:
+            setattr(self, name, cache.get(name))
+
+
 class _MaskFacts:
     """What one mask tensor (and one tensor of causal lengths) adds to the layout metadata.
 
@@ -278,12 +294,14 @@ def _tensor_identity(t: Tensor | None):
 
 
 def _mask_facts(layout_cache: dict, attention_layout: Tensor, mask: Tensor | None, mask_bytes: Tensor | None,
-                lengths: Tensor | None, dims: tuple[int, int, int, int, int], sbs: int) -> _MaskFacts:
+                lengths: Tensor | None, dims: tuple[int, int, int, int, int], sbs: int) -> "_MaskFacts | None":
     """The facts for this mask in ``layout_cache``, renewed when another mask (or another version) arrives.
 
     The forward lists without dead pairs are built when a mask is seen for the second time in a row: a caller
     that brings a new mask with every call never pays for lists it would use once.
     """
+    if not mask_facts_enabled():
+        return None
     holder = layout_cache.get("mask_facts")
     if holder is None:
         holder = layout_cache["mask_facts"] = CacheHolder()
@@ -322,40 +340,42 @@ def _mask_facts(layout_cache: dict, attention_layout: Tensor, mask: Tensor | Non
 class _Meta:
     """Everything the kernels need besides the differentiable tensors."""
 
-    __slots__ = ("cache", "dims", "sbs", "scale", "mask", "causal_lengths", "has_bias", "facts")
+    __slots__ = ("tables", "dims", "sbs", "scale", "has_bias", "facts")
 
 
-def _fill_args(meta: "_Meta", q, k, v, bias) -> _capi.AttnArgs:
-    c = meta.cache
+def _fill_args(meta: "_Meta", q, k, v, bias, mask, causal_lengths) -> _capi.AttnArgs:
+    """``mask`` (one byte per element) and ``causal_lengths`` come from the caller at forward time and from
+    autograd's saved tensors at backward time, so a change in place between the two is an autograd error."""
+    c = meta.tables
     a = _capi.AttnArgs()
     B, nq, nk, nh, nhv = meta.dims
     a.B, a.nq, a.nk, a.nh, a.nhv = B, nq, nk, nh, nhv
     a.q, a.k, a.v = _capi.ptr(q), _capi.ptr(k), _capi.ptr(v)
     a.n_q_blocks, a.n_k_blocks, a.n_v_blocks = q.size(0), k.size(0), v.size(0)
-    a.n_o_blocks = c["n_sparse_blocks_o"]
-    a.pidx_q, a.pidx_k = _capi.ptr(c["packed_indices_q"]), _capi.ptr(c["packed_indices_k"])
-    a.pidx_v, a.pidx_o = _capi.ptr(c["packed_indices_v"]), _capi.ptr(c["packed_indices_o"])
+    a.n_o_blocks = c.n_sparse_blocks_o
+    a.pidx_q, a.pidx_k = _capi.ptr(c.packed_indices_q), _capi.ptr(c.packed_indices_k)
+    a.pidx_v, a.pidx_o = _capi.ptr(c.packed_indices_v), _capi.ptr(c.packed_indices_o)
     # int64 CSR metadata only exists beyond 2**31 - 1 blocks; the kernels index with int32
-    a.key_offsets = c["key_offsets_i32"].data_ptr()
-    a.key_indices = _capi.ptr(c["key_indices_i32"])
-    a.query_offsets = c["query_offsets_i32"].data_ptr()
-    a.query_indices = _capi.ptr(c["query_indices_i32"])
-    if "group_offsets" in c:
-        a.group_offsets = c["group_offsets"].data_ptr()
-        a.group_records = _capi.ptr(c["group_records"])
-        a.group_size = c["group_size"]
+    a.key_offsets = c.key_offsets_i32.data_ptr()
+    a.key_indices = _capi.ptr(c.key_indices_i32)
+    a.query_offsets = c.query_offsets_i32.data_ptr()
+    a.query_indices = _capi.ptr(c.query_indices_i32)
+    if c.group_offsets is not None:
+        a.group_offsets = c.group_offsets.data_ptr()
+        a.group_records = _capi.ptr(c.group_records)
+        a.group_size = c.group_size
         if meta.facts is not None and meta.facts.group_offsets is not None:
             a.group_offsets = meta.facts.group_offsets.data_ptr()
             a.group_records = _capi.ptr(meta.facts.group_records)
-    if meta.mask is not None:
-        a.mask, a.pidx_mask = _capi.ptr(meta.mask), _capi.ptr(c["packed_indices_mask"])
-        a.n_mask_blocks = meta.mask.size(0)
-        a.mask_kind = 1 if meta.mask.numel() else 0
+    if mask is not None:
+        a.mask, a.pidx_mask = _capi.ptr(mask), _capi.ptr(c.packed_indices_mask)
+        a.n_mask_blocks = mask.size(0)
+        a.mask_kind = 1 if mask.numel() else 0
     if meta.has_bias:
-        a.bias, a.pidx_bias = _capi.ptr(bias), _capi.ptr(c["packed_indices_bias"])
+        a.bias, a.pidx_bias = _capi.ptr(bias), _capi.ptr(c.packed_indices_bias)
         a.n_bias_blocks = bias.size(0)
-    if meta.causal_lengths is not None:
-        a.causal_lengths = meta.causal_lengths.data_ptr()
+    if causal_lengths is not None:
+        a.causal_lengths = causal_lengths.data_ptr()
     a.sbs = meta.sbs
     a.dtype = _capi.DTYPE_CODES[q.dtype]
     a.scale = meta.scale
@@ -364,34 +384,37 @@ def _fill_args(meta: "_Meta", q, k, v, bias) -> _capi.AttnArgs:
 
 class _FlashAttention(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, q, k, v, bias, meta: "_Meta"):
+    def forward(ctx, q, k, v, bias, mask, causal_lengths, meta: "_Meta"):
         B, nq, nk, nh, nhv = meta.dims
         sbs = meta.sbs
-        out = torch.empty((meta.cache["n_sparse_blocks_o"], sbs, sbs), dtype=q.dtype, device=q.device)
+        out = torch.empty((meta.tables.n_sparse_blocks_o, sbs, sbs), dtype=q.dtype, device=q.device)
         lse = torch.empty((B, nq, sbs), dtype=torch.float32, device=q.device)
-        args = _fill_args(meta, q, k, v, bias)
+        args = _fill_args(meta, q, k, v, bias, mask, causal_lengths)
         args.o, args.lse = _capi.ptr(out), _capi.ptr(lse)
         with torch.cuda.device(q.device):
             _capi.call("bsa_attn_fwd", ctypes.byref(args), _capi.stream(q.device))
-        ctx.save_for_backward(q, k, v, bias, out, lse)
+        # the mask and the lengths are saved like the operands (as the reference does,
+        # blksprs/ops/flash_attention.py:498-501): autograd then refuses a backward pass after either was
+        # changed in place
+        ctx.save_for_backward(q, k, v, bias, out, lse, mask, causal_lengths)
         ctx.meta = meta
         return out
 
     @staticmethod
     def backward(ctx, grad_output):
         grad_output = grad_output.contiguous()
-        q, k, v, bias, out, lse = ctx.saved_tensors
+        q, k, v, bias, out, lse, mask, causal_lengths = ctx.saved_tensors
         meta = ctx.meta
         B, nq, nk, nh, nhv = meta.dims
         dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
         delta = torch.empty((B, nq, meta.sbs), dtype=torch.float32, device=q.device)
         dbias = torch.empty(bias.shape, dtype=torch.float32, device=q.device) if meta.has_bias else None
-        args = _fill_args(meta, q, k, v, bias)
+        args = _fill_args(meta, q, k, v, bias, mask, causal_lengths)
         args.o, args.d_o, args.lse, args.delta = _capi.ptr(out), _capi.ptr(grad_output), _capi.ptr(lse), _capi.ptr(delta)
         args.dq, args.dk, args.dv, args.dbias = _capi.ptr(dq), _capi.ptr(dk), _capi.ptr(dv), _capi.ptr(dbias)
         # room for the records of the pairs that some score survives (built and used inside bsa_attn_bwd)
-        n_layout_blocks = meta.cache["key_indices_i32"].numel()
-        n_mask_blocks = meta.mask.size(0) if meta.mask is not None else 0
+        n_layout_blocks = meta.tables.key_indices_i32.numel()
+        n_mask_blocks = mask.size(0) if mask is not None else 0
         size = max(_capi.load().bsa_attn_bwd_scratch_bytes(B, nq, nk, n_layout_blocks, n_mask_blocks), 16)
         stream = _capi.stream(q.device)
         facts = meta.facts
@@ -407,10 +430,10 @@ class _FlashAttention(torch.autograd.Function):
         if facts is not None and not args.bwd_scratch_ready and not torch.cuda.is_current_stream_capturing():
             facts.bwd_scratch, facts.bwd_stream = scratch, stream
         grad_bias = dbias.to(bias.dtype) if meta.has_bias else None
-        return dq, dk, dv, grad_bias, None
+        return dq, dk, dv, grad_bias, None, None, None
 
 
-@torch.compiler.disable
+@eager_only
 @torch.amp.custom_fwd(device_type="cuda")
 def flash_attention(q: BlksprsTensor, sparsity_layout_q: Tensor,
                     k: BlksprsTensor, sparsity_layout_k: Tensor,
@@ -555,18 +578,17 @@ def flash_attention(q: BlksprsTensor, sparsity_layout_q: Tensor,
                 int(n_head_blocks_qk), int(n_head_blocks_v))
             layout_cache["group_offsets"], layout_cache["group_records"] = offsets, records
             layout_cache["group_size"] = group_size
+        layout_cache["tables"] = _Tables(layout_cache)
         finalize_layout_cache(layout_cache)
 
     meta = _Meta()
-    meta.cache = layout_cache
+    meta.tables = layout_cache["tables"]
     meta.dims = (int(n_batches), int(n_seq_blocks_q), int(n_seq_blocks_k), int(n_head_blocks_qk),
                  int(n_head_blocks_v))
     meta.sbs = sparsity_block_size
     meta.scale = scale
-    meta.mask = mask_bytes
-    meta.causal_lengths = lengths
     meta.has_bias = has_bias
     meta.facts = _mask_facts(layout_cache, attention_layout, attention_mask, mask_bytes, lengths, meta.dims,
                              sparsity_block_size)
 
-    return BlksprsTensor.wrap(_FlashAttention.apply(q, k, v, attention_bias, meta))
+    return BlksprsTensor.wrap(_FlashAttention.apply(q, k, v, attention_bias, mask_bytes, lengths, meta))

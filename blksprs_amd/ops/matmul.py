@@ -12,8 +12,8 @@ from torch import Tensor
 
 from .. import _capi
 from ..utils.blksprs_tensor import BlksprsTensor
-from ..utils.tools import (build_contraction_lists, cast_for_autocast, finalize_layout_cache, nonzero_from_packed,
-                           pack_layout, prepare_layout_cache)
+from ..utils.tools import (build_contraction_lists, cast_for_autocast, eager_only, finalize_layout_cache,
+                           nonzero_from_packed, pack_layout, prepare_layout_cache)
 from ..utils.validation import (ensure_contiguous, validate_contiguous, validate_device, validate_dimensions,
                                 validate_dtype_float, validate_shape, validate_sparsity, validate_sparsity_block_size,
                                 validate_sparsity_layout)
@@ -30,15 +30,15 @@ def _launch(x: Tensor, y: Tensor, pair_offsets: Tensor, pairs: Tensor, order: Te
     return out
 
 
-def _launch_rows(x: Tensor, y: Tensor, cache: dict, n_rows: int, sbs: int) -> Tensor:
+def _launch_rows(x: Tensor, y: Tensor, plan: "_Plan", sbs: int) -> Tensor:
     """Forward product by output block row (fp16 / bf16, sbs 64): x row panels stay in LDS."""
-    n_out = cache["n_sparse_blocks"]
+    n_out = plan.n_out
     out = torch.empty((n_out, sbs, sbs), dtype=x.dtype, device=x.device)
     if n_out:
         with torch.cuda.device(x.device):
             _capi.call("bsa_matmul_rows", _capi.ptr(x), _capi.ptr(y), out.data_ptr(),
-                       cache["contraction_offsets"].data_ptr(), _capi.ptr(cache["contraction_pairs"]),
-                       _capi.ptr(cache["row_records"]), cache["row_records"].size(0), n_out,
+                       plan.pair_offsets.data_ptr(), _capi.ptr(plan.pairs),
+                       _capi.ptr(plan.row_records), plan.row_records.size(0), n_out,
                        x.size(0), y.size(0), sbs, _capi.DTYPE_CODES[x.dtype], _capi.stream(x.device))
     return out
 
@@ -126,47 +126,71 @@ def _row_work_table(pair_offsets: Tensor, row_offsets_o: Tensor, rows_per_batch:
     return table
 
 
-def _backward_lists(layout_cache: dict, shape_x, shape_y):
-    """Contraction lists of dX = dO Y^T and dY = X^T dO, built once per cache."""
-    if "grad_x_pair_offsets" not in layout_cache:
+class _Plan:
+    """The lookup tables of one (x layout, y layout, output layout) triple as one object.  A forward pass hands
+    this object, not the caller's cache dict, to its backward pass: the dict may be emptied and filled for other
+    layouts between the two (``prepare_layout_cache`` clears it in place), the object keeps what it was built
+    with.  Nothing writes to its tensors after they are built."""
+
+    __slots__ = ("pair_offsets", "pairs", "block_order", "n_out", "n_x", "n_y", "row_records", "packed_x",
+                 "packed_y", "packed_o", "grad_lists")
+
+    def __init__(self, cache: dict):
+        self.pair_offsets, self.pairs = cache["contraction_offsets"], cache["contraction_pairs"]
+        self.block_order, self.row_records = cache["block_order"], cache["row_records"]
+        self.n_out, self.n_x, self.n_y = (cache["n_sparse_blocks"], cache["n_sparse_blocks_x"],
+                                          cache["n_sparse_blocks_y"])
+        self.packed_x, self.packed_y, self.packed_o = (cache["packed_indices_x"], cache["packed_indices_y"],
+                                                       cache["packed_indices_o"])
+        self.grad_lists = None
+
+
+def _backward_lists(plan: _Plan, shape_x, shape_y):
+    """Contraction lists of dX = dO Y^T and dY = X^T dO, built once per plan from the plan's own indices."""
+    if plan.grad_lists is None:
         B, R, K = (int(s) for s in shape_x)
         C = int(shape_y[2])
-        pidx_x = layout_cache["packed_indices_x"]
-        pidx_y = layout_cache["packed_indices_y"]
-        pidx_o = layout_cache["packed_indices_o"]
         # operand layouts seen by the builder: dO (B,R,C) times Y^T (B,C,K) -> (B,R,K)
-        pidx_yt = pidx_y.view(B, K, C).transpose(1, 2).contiguous().view(-1)
-        gx = build_contraction_lists(pidx_o, pidx_yt, pidx_x, B, R, C, K, layout_cache["n_sparse_blocks_x"])
+        pidx_yt = plan.packed_y.view(B, K, C).transpose(1, 2).contiguous().view(-1)
+        gx = build_contraction_lists(plan.packed_o, pidx_yt, plan.packed_x, B, R, C, K, plan.n_x)
         # X^T (B,K,R) times dO (B,R,C) -> (B,K,C)
-        pidx_xt = pidx_x.view(B, R, K).transpose(1, 2).contiguous().view(-1)
-        gy = build_contraction_lists(pidx_xt, pidx_o, pidx_y, B, K, R, C, layout_cache["n_sparse_blocks_y"])
-        layout_cache["grad_x_pair_offsets"], layout_cache["grad_x_pairs"] = gx.pair_offsets, gx.pairs
-        layout_cache["grad_y_pair_offsets"], layout_cache["grad_y_pairs"] = gy.pair_offsets, gy.pairs
+        pidx_xt = plan.packed_x.view(B, R, K).transpose(1, 2).contiguous().view(-1)
+        gy = build_contraction_lists(pidx_xt, plan.packed_o, plan.packed_y, B, K, R, C, plan.n_y)
+        plan.grad_lists = (gx.pair_offsets, gx.pairs, gy.pair_offsets, gy.pairs)
+    return plan.grad_lists
+
+
+def _publish_backward_lists(layout_cache: dict, plan: _Plan) -> None:
+    """Shows the plan's backward lists under the cache's own keys, while the cache still belongs to the plan."""
+    if layout_cache.get("plan") is plan and "grad_x_pair_offsets" not in layout_cache:
+        (layout_cache["grad_x_pair_offsets"], layout_cache["grad_x_pairs"], layout_cache["grad_y_pair_offsets"],
+         layout_cache["grad_y_pairs"]) = plan.grad_lists
         finalize_layout_cache(layout_cache)
-    return (layout_cache["grad_x_pair_offsets"], layout_cache["grad_x_pairs"],
-            layout_cache["grad_y_pair_offsets"], layout_cache["grad_y_pairs"])
 
 
 class _Matmul(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, y, layout_cache, shape_x, shape_y, sparsity_block_size):
+        plan = layout_cache["plan"]
         ctx.save_for_backward(x, y)
-        ctx.layout_cache = layout_cache
+        ctx.plan = plan
+        ctx.layout_cache = layout_cache  # only to publish the backward lists; never read for the computation
         ctx.shapes = (shape_x, shape_y)
         ctx.sparsity_block_size = sparsity_block_size
         if (sparsity_block_size == 64 and x.dtype in (torch.float16, torch.bfloat16)
-                and layout_cache["row_records"] is not None):
-            return _launch_rows(x, y, layout_cache, shape_x[0] * shape_x[1], sparsity_block_size)
-        return _launch(x, y, layout_cache["contraction_offsets"], layout_cache["contraction_pairs"],
-                       layout_cache["block_order"], layout_cache["n_sparse_blocks"], sparsity_block_size, False,
-                       False)
+                and plan.row_records is not None):
+            return _launch_rows(x, y, plan, sparsity_block_size)
+        return _launch(x, y, plan.pair_offsets, plan.pairs, plan.block_order, plan.n_out, sparsity_block_size,
+                       False, False)
 
     @staticmethod
     def backward(ctx, grad_output):
         grad_output = grad_output.contiguous()
         x, y = ctx.saved_tensors
         sbs = ctx.sparsity_block_size
-        gx_off, gx_pairs, gy_off, gy_pairs = _backward_lists(ctx.layout_cache, *ctx.shapes)
+        plan = ctx.plan
+        gx_off, gx_pairs, gy_off, gy_pairs = _backward_lists(plan, *ctx.shapes)
+        _publish_backward_lists(ctx.layout_cache, plan)
         grad_x = grad_y = None
         if ctx.needs_input_grad[0]:
             grad_x = _launch(grad_output, y, gx_off, gx_pairs, None, x.size(0), sbs, False, True)
@@ -212,6 +236,7 @@ def matmul_build_layout_cache(layout_cache: dict | None, sparsity_layout_x: Tens
             layout_cache["row_parts_log2"], layout_cache["row_work_table"] = parts_log2, table
             layout_cache["row_records"] = _row_records(table, parts_log2, lists.pair_offsets, info_x.row_offsets,
                                                        info_o.row_offsets, B * R, info_x.count)
+        layout_cache["plan"] = _Plan(layout_cache)
 
     validate_contiguous(sparsity_layout_x, layout_cache["packed_indices_x"],
                         sparsity_layout_y, layout_cache["packed_indices_y"],
@@ -219,7 +244,7 @@ def matmul_build_layout_cache(layout_cache: dict | None, sparsity_layout_x: Tens
     return finalize_layout_cache(layout_cache)
 
 
-@torch.compiler.disable
+@eager_only
 @torch.amp.custom_fwd(device_type="cuda")
 def matmul(x: BlksprsTensor, sparsity_layout_x: Tensor,
            y: BlksprsTensor, sparsity_layout_y: Tensor,

@@ -13,8 +13,8 @@ from torch import Tensor
 
 from .. import _capi
 from ..utils.blksprs_tensor import BlksprsTensor
-from ..utils.tools import (ceil_pow2, finalize_layout_cache, nonzero_from_packed, pack_layout, prepare_layout_cache,
-                           sorted_rows_from_offsets)
+from ..utils.tools import (ceil_pow2, eager_only, finalize_layout_cache, nonzero_from_packed, pack_layout,
+                           prepare_layout_cache, sorted_rows_from_offsets)
 from ..utils.validation import (ensure_contiguous, validate_contiguous, validate_device, validate_dimensions,
                                 validate_dtype_float_32, validate_sparsity, validate_sparsity_block_size)
 
@@ -101,7 +101,7 @@ def _run(x: Tensor, sparsity_layout: Tensor, sparsity_block_size: int, layout_ca
     return BlksprsTensor.wrap(_Softmax.apply(x, layout_cache["row_offsets"], n_rows, sparsity_block_size))
 
 
-@torch.compiler.disable
+@eager_only
 @torch.amp.custom_fwd(device_type="cuda")
 def softmax(x: BlksprsTensor, sparsity_layout: Tensor, sparsity_block_size: int,
             flag_fused: bool = True, layout_cache: dict | None = None) -> BlksprsTensor:
@@ -127,7 +127,7 @@ def softmax(x: BlksprsTensor, sparsity_layout: Tensor, sparsity_block_size: int,
     return softmax_regular(x, sparsity_layout, sparsity_block_size, layout_cache)
 
 
-@torch.compiler.disable
+@eager_only
 @torch.amp.custom_fwd(device_type="cuda")
 def softmax_regular(x: BlksprsTensor, sparsity_layout: Tensor, sparsity_block_size: int,
                     layout_cache: dict | None = None) -> BlksprsTensor:
@@ -139,7 +139,7 @@ def softmax_regular(x: BlksprsTensor, sparsity_layout: Tensor, sparsity_block_si
     return _run(x, sparsity_layout, sparsity_block_size, layout_cache)
 
 
-@torch.compiler.disable
+@eager_only
 @torch.amp.custom_fwd(device_type="cuda")
 def softmax_fused(x: BlksprsTensor, sparsity_layout: Tensor, sparsity_block_size: int,
                   layout_cache: dict | None = None) -> BlksprsTensor:

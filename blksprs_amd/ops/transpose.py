@@ -10,7 +10,7 @@ from torch import Tensor
 
 from .. import _capi
 from ..utils.blksprs_tensor import BlksprsTensor
-from ..utils.tools import (as_base_tensor, finalize_layout_cache, nonzero_from_packed, pack_layout,
+from ..utils.tools import (as_base_tensor, eager_only, finalize_layout_cache, nonzero_from_packed, pack_layout,
                            prepare_layout_cache)
 from ..utils.validation import (ensure_contiguous, validate_contiguous, validate_device, validate_dimensions,
                                 validate_dtype_supported, validate_sparsity, validate_sparsity_block_size)
@@ -43,7 +43,7 @@ class _Transpose(torch.autograd.Function):
         return grad, None, None, None, None, None
 
 
-@torch.compiler.disable
+@eager_only
 @torch.amp.custom_fwd(device_type="cuda")
 def transpose(x: BlksprsTensor, sparsity_layout: Tensor,
               sparsity_block_size: int, layout_cache: dict | None = None) -> tuple[BlksprsTensor, Tensor]:

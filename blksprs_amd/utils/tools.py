@@ -7,6 +7,7 @@ the observable results identical to the reference's torch formulations
 :159-287 for the shape and dtype helpers).
 """
 
+import functools
 from typing import Any
 
 import torch
@@ -313,6 +314,22 @@ def can_use_int32_indexing(*values: Tensor | int | None) -> bool:
         if n > INT32_INDEX_MAX:
             return False
     return True
+
+
+
+def eager_only(fn):
+    """Makes ``fn`` run outside ``torch.compile``: the returned entry point is an ordinary function whose only
+    statement calls ``torch.compiler.disable(fn)``.  A caller's compiled graph breaks at that call and resumes after
+    it (the reference's wrappers break the graph as well, at their validation and cache preparation).  Decorating
+    the public function with ``torch.compiler.disable`` itself is not enough: ``torch.compile(fn)`` unwraps a
+    disabled function it is handed directly and traces its body."""
+    disabled = torch.compiler.disable(fn)
+
+    @functools.wraps(fn)
+    def entry(*args, **kwargs):
+        return disabled(*args, **kwargs)
+
+    return entry
 
 
 def cast_for_autocast(*values: Tensor):

@@ -44,6 +44,24 @@ def enable_contiguous() -> None:
     _state.contiguous = True
 
 
+def mask_facts_enabled() -> bool:
+    return getattr(_state, "mask_facts", True)
+
+
+def disable_mask_facts() -> None:
+    """Turns off, for the calling thread, everything ``flash_attention`` keeps per mask tensor (the forward lists
+    without the pairs a mask's values rule out, the reuse of the backward records): every call then walks the
+    lists of the layouts alone and rebuilds the backward records.  For callers that rewrite a mask's memory
+    behind autograd's back (``.data``, a foreign kernel), which the version counter those facts are keyed on
+    does not see.  No counterpart in the reference, whose lists do not depend on mask values."""
+    _state.mask_facts = False
+
+
+def enable_mask_facts() -> None:
+    """Reverts :func:`disable_mask_facts` (calling thread only)."""
+    _state.mask_facts = True
+
+
 def _check(fn):
     """Turns ``fn`` into a no-op while validation is disabled."""
 

@@ -397,6 +397,27 @@ def test_attention_known_answers_from_reference_tests():
     assert torch.allclose(orc.to_dense(out, lv, sbs), mean, atol=1e-6)
 
 
+def test_attention_finite_bias_is_added_unscaled_before_the_softmax():
+    """A finite additive bias against ``F.scaled_dot_product_attention(attn_mask=bias)``, which adds a float
+    mask to the scaled scores: a bias multiplied by the scale, added after the softmax or subtracted would
+    differ.  Gradients of q, k, v and the bias against torch's own."""
+    g = torch.Generator().manual_seed(21)
+    sbs, B, S, D = 4, 2, 12, 8
+    lq, la = _full(B, S // sbs, D // sbs), _full(B, S // sbs, S // sbs)
+    dense = [torch.randn((B, S, D), generator=g, dtype=torch.float64).requires_grad_(True) for _ in range(3)]
+    bias = (3.0 * torch.randn((B, S, S), generator=g, dtype=torch.float64)).requires_grad_(True)
+    sparse = [orc.to_sparse_autograd(t, lq, sbs) for t in dense]
+    out = orc.flash_attention(sparse[0], lq, sparse[1], lq, sparse[2], lq, la, sbs, scale=0.3,
+                              bias=orc.to_sparse_autograd(bias, la, sbs), layout_bias=la, acc_dtype=torch.float64)
+    go = torch.randn((B, S, D), generator=g, dtype=torch.float64)
+    got = torch.autograd.grad(orc.to_dense_autograd(out, lq, sbs), (*dense, bias), go)
+    ref_in = [t.detach().clone().requires_grad_(True) for t in (*dense, bias)]
+    ref = F.scaled_dot_product_attention(ref_in[0], ref_in[1], ref_in[2], attn_mask=ref_in[3], scale=0.3)
+    assert torch.allclose(orc.to_dense(out.detach(), lq, sbs), ref.detach(), atol=1e-12)
+    for a, b in zip(got, torch.autograd.grad(ref, ref_in, go)):
+        assert torch.allclose(a, b, atol=1e-12)
+
+
 def test_attention_mask_bias_order_and_fully_masked_rows():
     g = torch.Generator().manual_seed(8)
     sbs, S = 4, 8
