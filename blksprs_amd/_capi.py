@@ -71,8 +71,8 @@ SIGNATURES = {
     "bsa_matmul": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int,
                            c_int, c_int, c_int, c_void_p]),
     "bsa_matmul_rows_records": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
-                                        c_void_p, c_void_p]),
-    "bsa_matmul_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
+                                        c_int64, c_void_p, c_void_p]),
+    "bsa_matmul_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int64,
                                 c_int64, c_int64, c_int, c_int, c_void_p]),
     "bsa_attn_fwd_records": (c_int, [ctypes.POINTER(AttnArgs), c_void_p, c_void_p, c_void_p]),
     "bsa_attn_mask_dead": (c_int, [c_void_p, c_int64, ctypes.c_int32, c_void_p, c_void_p]),

@@ -1,23 +1,29 @@
 // Row kernel of the block-sparse GEMM (16-bit operands, sbs == 64, untransposed operands): one workgroup of
-// 8 waves owns one block row (b, i) of the output.
+// 8 waves owns one part of a block row (b, i) of the output, at most 64 output blocks.
 //
 // x: the row's x blocks are consecutive in memory; up to 18 of them (144 KiB) are copied once into LDS by
 // asynchronous global -> LDS copies and stay there while the waves walk the row's output blocks, so x is
 // read from L2 once per row, and a wave never waits for x.  x blocks beyond the 18 resident ones are read
 // from global memory in fragment layout (slow path, rare).
 //
-// Work split: the row's output blocks are cut into 8 contiguous runs of about equal numbers of (x, y) pairs
-// (not of equal numbers of blocks), one run per wave; rows are handed to workgroups in the order the caller
-// gives (longest first keeps the tail of the launch short).
+// Work split: the part's output blocks are dealt to the 8 waves in ascending order, each to the wave that has
+// the least work so far (list scheduling over the blocks' numbers of (x, y) pairs, done once per layout by
+// bsa_matmul_rows_records, which leaves one 64-bit mask of blocks per wave in the row's record).  The waves
+// therefore move through the row's columns together: the y blocks in flight on a compute unit, and on the XCD
+// whose rows belong to one batch entry, lie in a narrow band of columns, and the waves of a workgroup end within
+// a block of each other.  Rows are handed to workgroups in the order the caller gives (longest first keeps the
+// tail of the launch short).
 //
-// y: only y blocks stream.  A wave walks its slice of the pair list as one flat sequence.  Each y block
-// travels global -> registers -> LDS -> matrix-core operand: two register slots of 8 KiB hold the y blocks of
-// the next two pairs, so a block is requested about one and a half pairs before it is used.  The loads are
-// issued from inline assembly and waited for with hand-placed s_waitcnt vmcnt(n): the compiler would join
-// the outstanding loads with vmcnt(0) at every branch.  vmcnt counts vector memory instructions in issue
-// order, so "all but the youngest n" is exact as long as n is not larger than the number of instructions
-// issued after the loads waited for; every n used below is such a lower bound (the other slot's 8 loads,
-// plus the 8 stores of an output block written since).
+// y: only y blocks stream.  A wave walks the pairs of its blocks as one flat sequence.  Which pair comes next
+// is scalar work that runs a pair ahead of everything else: the list entry of the next pair and the pair range
+// of the next block are requested (scalar loads) while the current entry is turned into addresses, so no load
+// of metadata is waited for.  Each y block travels global -> registers -> LDS -> matrix-core operand: two
+// register slots of 8 KiB hold the y blocks of the next two pairs, so a block is requested about one and a half
+// pairs before it is used.  The loads are issued from inline assembly and waited for with hand-placed
+// s_waitcnt vmcnt(n): the compiler would join the outstanding loads with vmcnt(0) at every branch.  vmcnt
+// counts vector memory instructions in issue order, so "all but the youngest n" is exact as long as n is not
+// larger than the number of instructions issued after the loads waited for; every n used below is such a lower
+// bound (the other slot's 8 loads, plus the 8 stores of an output block written since).
 //
 // Per pair, per quarter of the contraction (16 k): 2 KiB of the y block are written to the wave's LDS stage
 // as stored (k rows), and read back with the transposing LDS load, which delivers the matrix-core operand
@@ -28,7 +34,8 @@
 //
 // The product is formed transposed (y fragments as the A operand, x fragments as B), which leaves 4
 // consecutive output columns of one row in each lane; a finished block is rounded, passed through the stage
-// 16 rows at a time and written with 16-byte stores that cover whole rows.
+// 16 rows at a time and written with 16-byte stores that cover whole rows.  Output blocks without any pair are
+// written (zeros) before the walk starts.
 #include "attn_mfma_common.h"
 
 namespace {
@@ -208,19 +215,22 @@ __device__ __forceinline__ void rows_flush(f32x16 (&acc)[2][2], char *ob, char *
       for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
 }
 
-// What a workgroup needs to know about its part of a row, in one 128-byte record (one load, where walking the
-// tables is a chain of five dependent loads and a loop of ballots): the row, the x blocks of the row, and for
-// each of the eight waves its run of output blocks and the pairs of that run.  Wave w takes the output blocks
-// in front of which at least w / 8 and less than (w + 1) / 8 of the part's pairs lie.
+// What a workgroup needs to know about its part of a row, in one 128-byte record (one load): the row's x
+// blocks, the part's output blocks (at most 64), and for each of the eight waves the blocks it computes, as a
+// 64-bit mask over the part's blocks.  Blocks without pairs are in no mask.
 struct RowsRecord {
-  int32_t row;                    // -1: nothing to do
-  int32_t x_first, x_count;       // the row's blocks in x
+  int32_t row;                // -1: nothing to do
+  int32_t x_first, x_count;   // the row's blocks in x
+  int32_t o_first, o_count;   // the part's output blocks
+  uint32_t empty_blocks[2];   // mask of the part's blocks that have no pair (they are written as zeros)
   int32_t pad0;
-  int32_t block_begin[kWaves + 1];  // wave w: output blocks [block_begin[w], block_begin[w + 1])
-  int32_t pair_begin[kWaves + 1];   // pair_offsets at those blocks
-  int32_t pad1[32 - 4 - 2 * (kWaves + 1)];
+  uint32_t wave_blocks[kWaves][2];  // low and high word of wave w's mask
+  int32_t pad1[8];
 };
 static_assert(sizeof(RowsRecord) == BSA_ROWS_RECORD_INTS * 4, "record layout");
+
+// cost of an output block in the list scheduling, in units of half a pair: its pairs and one write
+constexpr int kBlockCost = 3;
 
 // one wave per work table entry
 __global__ __launch_bounds__(256) void rows_records_kernel(const int32_t *__restrict__ work_table, int64_t n_items,
@@ -247,52 +257,66 @@ __global__ __launch_bounds__(256) void rows_records_kernel(const int32_t *__rest
       n0 = first;
       n1 = last;
     }
+    n0 = __builtin_amdgcn_readfirstlane(n0);
+    n1 = __builtin_amdgcn_readfirstlane(n1);
+    if (n1 - n0 > 64) n1 = n0;  // the caller sizes the parts; a part that does not fit a mask is refused whole
     const int xs = x_row_offsets[row];
     int nx = x_row_offsets[row + 1] - xs;
     if (xs < 0 || nx < 0 || (int64_t)xs + nx > nnz_x) nx = 0;
-    const int row_p0 = pair_offsets[n0], row_p1 = pair_offsets[n1];
-    const int64_t span = row_p1 - row_p0;
-    // lane w < 8 counts the blocks in front of wave w's boundary: pair_offsets ascends, one ballot per 64 blocks
-    // for each boundary
-    int below[kWaves];
+    // lane i: number of pairs of block n0 + i
+    int my_pairs = 0;
+    if (n0 + lane < n1) my_pairs = pair_offsets[n0 + lane + 1] - pair_offsets[n0 + lane];
+    // blocks in ascending order, each to the wave with the least work so far (the lowest such wave)
+    int load[kWaves];
+    uint64_t blocks[kWaves];
 #pragma unroll
-    for (int w = 0; w < kWaves; ++w) below[w] = 0;
-    for (int base = n0; base < n1; base += 64) {
-      const int b = base + lane;
-      const int off = b < n1 ? pair_offsets[b] : 0x7fffffff;
+    for (int w = 0; w < kWaves; ++w) load[w] = 0, blocks[w] = 0;
+    for (int i = 0; i < n1 - n0; ++i) {
+      const int c = __builtin_amdgcn_readlane(my_pairs, i);
+      if (c <= 0) continue;
+      int best = 0, least = load[0];
 #pragma unroll
-      for (int w = 1; w < kWaves; ++w) {
-        const int lo = row_p0 + (int)((span * w + kWaves - 1) / kWaves);
-        below[w] += __builtin_popcountll(__ballot(off < lo));
-      }
+      for (int w = 1; w < kWaves; ++w)
+        if (load[w] < least) best = w, least = load[w];
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w)
+        if (w == best) load[w] += 2 * c + kBlockCost, blocks[w] |= 1ull << i;
     }
-    int begin = n0;  // boundary number lane (for lanes 0 .. 8)
-#pragma unroll
-    for (int w = 1; w < kWaves; ++w)
-      if (lane == w) begin = n0 + below[w];
-    if (lane >= kWaves) begin = n1;
-    const int pair_at = pair_offsets[begin];
-    const int moved = __shfl(begin, lane - 4), moved_pair = __shfl(pair_at, lane - 4 - (kWaves + 1));
+    const uint64_t empty = __ballot(n0 + lane < n1 && my_pairs <= 0);
     if (lane == 0) value = n0 >= n1 ? -1 : row;
+    else if (lane == 5) value = (int)(uint32_t)empty;
+    else if (lane == 6) value = (int)(uint32_t)(empty >> 32);
     else if (lane == 1) value = xs;
     else if (lane == 2) value = nx;
-    else if (lane >= 4 && lane < 4 + kWaves + 1) value = moved;
-    else if (lane >= 4 + kWaves + 1 && lane < 4 + 2 * (kWaves + 1)) value = moved_pair;
+    else if (lane == 3) value = n0;
+    else if (lane == 4) value = n1 - n0;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      if (lane == 8 + 2 * w) value = (int)(uint32_t)blocks[w];
+      if (lane == 9 + 2 * w) value = (int)(uint32_t)(blocks[w] >> 32);
+    }
   }
   if (lane < BSA_ROWS_RECORD_INTS) out[lane] = value;
 }
 
+// One pair of a wave's walk; everything here is wave uniform (scalar registers).
+struct PairItem {
+  const char *y;  // the y block (for an item past the end: the last block requested, so the load hits)
+  int xoff;       // offset of the x block in the panel, -1 if it is not resident
+  int px;         // packed index of the x block (range checked), for the read from global memory
+  int block;      // the output block the pair belongs to
+  bool last;      // the block's last pair: the block is written after it
+  bool valid;     // false: past the end of the wave's pairs
+};
+
+// One record: one part of a row.  `mine`: int (lane % 32) of the record.  Every wave of the workgroup passes the
+// same number of barriers (none when the record holds nothing, else two).
 template <typename Tr>
-__global__ __launch_bounds__(kWaves * 64, 1) void matmul_rows_kernel(
-    const char *__restrict__ x, const char *__restrict__ y, char *__restrict__ out,
-    const int32_t *__restrict__ pair_offsets, const int32_t *__restrict__ pairs,
-    const RowsRecord *__restrict__ records, int64_t nnz_x, int64_t nnz_y) {
-  extern __shared__ __attribute__((aligned(16))) char rows_smem[];
-  const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  // the grid has one workgroup per record; lane l < 32 fetches int l of it
-  const int32_t *rec = reinterpret_cast<const int32_t *>(records + blockIdx.x);
-  const int mine = rec[lane & 31];
+__device__ __forceinline__ void rows_part(const char *__restrict__ x, const char *__restrict__ y,
+                                          char *__restrict__ out, const int32_t *__restrict__ pair_offsets,
+                                          const int32_t *__restrict__ pairs, const int mine, int64_t nnz_o,
+                                          int64_t nnz_x, int64_t nnz_y, char *rows_smem, const int lane,
+                                          const int wave) {
   const int row = __builtin_amdgcn_readlane(mine, 0);
   if (row < 0) return;
   const int xs = __builtin_amdgcn_readlane(mine, 1);
@@ -312,58 +336,76 @@ __global__ __launch_bounds__(kWaves * 64, 1) void matmul_rows_kernel(
     for (int idx = wave; idx < nx * 8; idx += kWaves) copy_1k_to_lds(xsrc + idx * 1024, src_off, panel + idx * 1024);
   }
 
-  // this wave's run of output blocks and its pairs
-  const int wb0 = __builtin_amdgcn_readlane(mine, 4 + wave), wb1 = __builtin_amdgcn_readlane(mine, 5 + wave);
-  const int p_begin = __builtin_amdgcn_readlane(mine, 4 + kWaves + 1 + wave);
-  const int p_end = __builtin_amdgcn_readlane(mine, 5 + kWaves + 1 + wave);
+  // the part's output blocks, and this wave's share of them (a corrupt record must not turn into a wild access)
+  const int o_first = __builtin_amdgcn_readlane(mine, 3);
+  int o_count = __builtin_amdgcn_readlane(mine, 4);
+  if (o_first < 0 || o_count < 0 || o_count > 64 || (int64_t)o_first + o_count > nnz_o) o_count = 0;
+  uint64_t todo = ((uint64_t)(uint32_t)__builtin_amdgcn_readlane(mine, 9 + 2 * wave) << 32) |
+                  (uint32_t)__builtin_amdgcn_readlane(mine, 8 + 2 * wave);
+  todo &= o_count >= 64 ? ~0ull : (1ull << o_count) - 1;
 
-  // 64 entries of the pair list and 64 block boundaries at a time, one per lane.  A lane turns its entry into
-  // what the loop needs per pair (the address of the y block; the panel offset of the x block, or -1 if it is
-  // not resident), so that a pair costs a few v_readlane and no address arithmetic.
-  int win_base = p_begin, win_px = 0, win_xoff = 0;
-  uint32_t win_ylo = 0, win_yhi = 0;
-  int off_base = wb0, win_off = 0;
-  auto load_pair_window = [&](int base) {
-    win_base = base;
-    const int t = base + lane;
-    int px = 0, py = 0;
-    if (t < p_end) {
-      const int2 v = *reinterpret_cast<const int2 *>(pairs + 2 * (int64_t)t);
-      px = v.x;
-      py = v.y;
+  // output blocks without pairs: zeros, block first + 8 m + wave by this wave
+  {
+    uint64_t zeros = ((uint64_t)(uint32_t)__builtin_amdgcn_readlane(mine, 6) << 32) |
+                     (uint32_t)__builtin_amdgcn_readlane(mine, 5);
+    zeros &= o_count >= 64 ? ~0ull : (1ull << o_count) - 1;
+    zeros &= 0x0101010101010101ull << wave;
+    while (zeros) {
+      const int b = __builtin_ctzll(zeros);
+      zeros &= zeros - 1;
+      char *ob = out + (int64_t)(o_first + b) * 8192;
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        __builtin_nontemporal_store(u32x4{0, 0, 0, 0}, reinterpret_cast<u32x4 *>(ob + i * 1024 + lane * 16));
     }
+  }
+
+  // The walk over this wave's pairs, one step ahead of its use.  g_*: the block being walked and its pairs not
+  // yet handed out; n_*: the block after it, whose pair range was requested when g_* was entered; raw: the next
+  // pair to hand out, its list entry already requested.
+  auto pop_block = [&]() -> int {
+    if (!todo) return -1;
+    const int b = __builtin_ctzll(todo);
+    todo &= todo - 1;
+    return o_first + b;
+  };
+  int g_block = pop_block(), g_p = 0, g_pe = 0;
+  if (g_block >= 0) g_p = pair_offsets[g_block], g_pe = pair_offsets[g_block + 1];
+  int n_block = pop_block(), n_p = 0, n_pe = 0;
+  if (n_block >= 0) n_p = pair_offsets[n_block], n_pe = pair_offsets[n_block + 1];
+  int raw_px = 0, raw_py = 0, raw_block = 0;
+  bool raw_last = false, raw_valid = false;
+  auto advance = [&]() {
+    while (g_block >= 0 && g_p >= g_pe) {  // the block is used up (one turn, unless a record names an empty block)
+      g_block = n_block, g_p = n_p, g_pe = n_pe;
+      n_block = pop_block();
+      if (n_block >= 0) n_p = pair_offsets[n_block], n_pe = pair_offsets[n_block + 1];
+    }
+    raw_valid = g_block >= 0;
+    if (raw_valid) {
+      const int2 e = *reinterpret_cast<const int2 *>(pairs + 2 * (int64_t)g_p);
+      raw_px = e.x, raw_py = e.y, raw_block = g_block;
+      ++g_p;
+      raw_last = g_p >= g_pe;
+    }
+  };
+  const char *y_recent = y;
+  auto next_item = [&]() {
+    PairItem it;
+    it.valid = raw_valid;
+    it.block = raw_block;
+    it.last = raw_last;
     // a corrupt list must not turn into a wild read
-    const uint64_t ya = reinterpret_cast<uint64_t>(y) + (uint64_t)((py < 0 || py >= nnz_y) ? 0 : py) * 8192;
-    win_ylo = (uint32_t)ya;
-    win_yhi = (uint32_t)(ya >> 32);
-    win_px = (px < 0 || px >= nnz_x) ? 0 : px;
-    win_xoff = (unsigned)(px - xs) < (unsigned)nx ? (px - xs) * 8192 : -1;
-    // a use right here: the wait for the load lands inside this (rarely taken) branch, not at the join
-    asm volatile("" : "+v"(win_px), "+v"(win_xoff), "+v"(win_ylo), "+v"(win_yhi));
+    if (raw_valid) y_recent = y + (uint64_t)((raw_py < 0 || raw_py >= nnz_y) ? 0 : raw_py) * 8192;
+    it.y = y_recent;
+    it.px = (raw_px < 0 || raw_px >= nnz_x) ? 0 : raw_px;
+    it.xoff = (unsigned)(raw_px - xs) < (unsigned)nx ? (raw_px - xs) * 8192 : -1;
+    advance();
+    return it;
   };
-  auto load_offset_window = [&](int base) {
-    off_base = base;
-    const int n = base + lane;
-    win_off = pair_offsets[n <= wb1 ? n : wb1];
-    asm volatile("" : "+v"(win_off));
-  };
-  // end of the pair list of block n (n < wb1)
-  auto block_end = [&](int n) {
-    if (n + 1 - off_base >= 64) load_offset_window(n);
-    return __builtin_amdgcn_readlane(win_off, __builtin_amdgcn_readfirstlane(n + 1 - off_base));
-  };
-  // y block of pair t (clamped to the wave's last pair: the lookup stays in the window)
-  auto y_block_of = [&](int t) -> const char * {
-    t = t < p_end ? t : p_end - 1;
-    const int sel = __builtin_amdgcn_readfirstlane(t - win_base);
-    const uint32_t lo = __builtin_amdgcn_readlane(win_ylo, sel), hi = __builtin_amdgcn_readlane(win_yhi, sel);
-    return reinterpret_cast<const char *>(((uint64_t)hi << 32) | lo);
-  };
-  load_pair_window(p_begin);
-  load_offset_window(wb0);
+  advance();
 
   const uint32_t lane_lo = 16 * lane, lane_hi = 16 * lane + 4096;
-  const bool has_pairs = p_begin < p_end;
 
   LaneAddr la;
   {
@@ -386,6 +428,14 @@ __global__ __launch_bounds__(kWaves * 64, 1) void matmul_rows_kernel(
     for (int s = 0; s < 4; ++s) la.xoff[s] = li * 128 + (((2 * s + kg) ^ t_swizzle(li)) << 4);
   }
 
+  if (!raw_valid) {
+    // no pair for this wave: its panel pieces and zero blocks must still land before the others read the panel
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    __syncthreads();
+    return;
+  }
+
   f32x16 acc[2][2];  // [block along j][block along i]
 #pragma unroll
   for (int a = 0; a < 2; ++a)
@@ -394,71 +444,44 @@ __global__ __launch_bounds__(kWaves * 64, 1) void matmul_rows_kernel(
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
 
-  int cur = wb0;
-  int blk_end = cur < wb1 ? block_end(cur) : -1;
-  // writes the blocks that end at pair t (the first holds the sums, the others have no pairs: zeros)
-  auto flush_until = [&](int t) {
-    bool any = false;
-    while (cur < wb1 && blk_end == t) {
-      rows_flush<Tr>(acc, out + (int64_t)cur * 8192, stage, lane);
-      any = true;
-      ++cur;
-      blk_end = cur < wb1 ? block_end(cur) : -1;
-    }
-    return any;
-  };
-
-  if (!has_pairs) {
-    // only blocks without pairs (or none at all): wait for this wave's panel pieces, then write zeros
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    flush_until(p_begin);
-    return;
-  }
-
   // The registers of a slot are written by loads the compiler does not know of.  Two rules keep it from ever
   // touching them while a load is in flight: (1) no load sits in a branch of its own (a join could make the
-  // compiler copy the registers), so blocks are requested unconditionally, the last two requests of a wave
-  // repeat its last block; (2) every request is consumed, the last ones by the statement after the loop that
-  // passes both slots through (registers whose contents are never used may be reused at once).
+  // compiler copy the registers), so blocks are requested unconditionally, the requests past the end of a wave's
+  // pairs repeat its last block; (2) every request is consumed, the last ones by the statement after the loop
+  // that passes both slots through (registers whose contents are never used may be reused at once).
   YSlot slot_a, slot_b;
-  y_issue(slot_a, y_block_of(p_begin), lane_lo, lane_hi);
-  y_issue(slot_b, y_block_of(p_begin + 1), lane_lo, lane_hi);
+  PairItem item_a = next_item(), item_b = next_item();
+  y_issue(slot_a, item_a.y, lane_lo, lane_hi);
+  y_issue(slot_b, item_b.y, lane_lo, lane_hi);
   // everything requested so far has arrived: the panel pieces of this wave and both slots
   BSA_Y_WAIT(slot_a, 0);
   BSA_Y_TIE(slot_b);
   __syncthreads();
 
-  int t = p_begin;
   int flushed = 0;  // a block was written after the last pair
-  flush_until(t);   // blocks without pairs in front of the first pair
 
-  // x block of pair t (the window must hold it)
-  auto x_source_of = [&](int t) {
-    const int sel = __builtin_amdgcn_readfirstlane(t - win_base);
-    const int xoff = __builtin_amdgcn_readlane(win_xoff, sel);
+  auto x_source_of = [&](const PairItem &it) {
     XSource src;
-    src.resident = xoff >= 0;
-    src.lds = panel + (xoff >= 0 ? xoff : 0);
-    src.px = __builtin_amdgcn_readlane(win_px, sel);
+    src.resident = it.xoff >= 0;
+    src.lds = panel + (it.xoff >= 0 ? it.xoff : 0);
+    src.px = it.px;
     return src;
   };
 
-  // The loop is software pipelined across pairs: while the last two quarters of pair t are multiplied, the
-  // first two quarters of pair t + 1 are staged and their fragments read, so the matrix core does not wait
+  // The loop is software pipelined across pairs: while the last two quarters of a pair are multiplied, the
+  // first two quarters of the next pair are staged and their fragments read, so the matrix core does not wait
   // for LDS at the start of a pair.  f0 / f1 hold the fragments of the quarter multiplied next / after it.
   Frags f0, f1;
-  XSource x_cur = x_source_of(t);
+  XSource x_cur = x_source_of(item_a);
   stage_and_read<0>(f0, slot_a, x_cur, la, x, lane);
   stage_and_read<1>(f1, slot_a, x_cur, la, x, lane);
 
-  // pair t from slot `cur_slot` (its first two quarters are in f0 / f1 already); `next_slot` holds pair t + 1
-  auto do_pair = [&](YSlot &cur_slot, YSlot &next_slot) {
-    // the window must hold pairs t .. t + 2
-    if (t + 2 - win_base >= 64) load_pair_window(t);
-    const char *next = y_block_of(t + 2);
-    const bool more = t + 1 < p_end;
-    const XSource x_next = x_source_of(more ? t + 1 : t);
+  // the pair `cur` from `cur_slot` (its first two quarters are in f0 / f1 already); `next_slot` holds the pair
+  // `next`; at the end `cur` is the pair whose block has been requested into `cur_slot`
+  auto do_pair = [&](YSlot &cur_slot, PairItem &cur, YSlot &next_slot, const PairItem &next) {
+    const PairItem fresh = next_item();
+    const bool more = next.valid;
+    const XSource x_next = x_source_of(more ? next : cur);
     __builtin_amdgcn_sched_barrier(0);
     multiply<Tr>(acc, f0);
     stage_and_read<2>(f0, cur_slot, x_cur, la, x, lane);
@@ -466,7 +489,7 @@ __global__ __launch_bounds__(kWaves * 64, 1) void matmul_rows_kernel(
     multiply<Tr>(acc, f1);
     stage_and_read<3>(f1, cur_slot, x_cur, la, x, lane);
     // the slot's registers have been handed to the LDS writes: request the block of the pair after next
-    y_issue(cur_slot, next, lane_lo, lane_hi);
+    y_issue(cur_slot, fresh.y, lane_lo, lane_hi);
     __builtin_amdgcn_sched_barrier(0);
     multiply<Tr>(acc, f0);
     // younger than the next slot's loads (issued during the pair before this one): the 8 loads just issued,
@@ -482,31 +505,67 @@ __global__ __launch_bounds__(kWaves * 64, 1) void matmul_rows_kernel(
     multiply<Tr>(acc, f1);
     if (more) stage_and_read<1>(f1, next_slot, x_next, la, x, lane);
     x_cur = x_next;
-    ++t;
-    if (flush_until(t)) flushed = 1;
+    if (cur.last) {
+      rows_flush<Tr>(acc, out + (int64_t)cur.block * 8192, stage, lane);
+      flushed = 1;
+    }
+    cur = fresh;
   };
-  while (t < p_end) {
-    do_pair(slot_a, slot_b);
-    if (t >= p_end) break;
-    do_pair(slot_b, slot_a);
+  while (true) {
+    do_pair(slot_a, item_a, slot_b, item_b);
+    if (!item_b.valid) break;
+    do_pair(slot_b, item_b, slot_a, item_a);
+    if (!item_a.valid) break;
   }
   // the last requests land here
   BSA_Y_WAIT(slot_a, 0);
   BSA_Y_TIE(slot_b);
+  // the panel may be overwritten (by the next record's row) once every wave is done with it
+  __syncthreads();
+}
+
+// Workgroup g runs on XCD g % 8 and takes the records 8 (items_per_wg (g / 8) + r) + g % 8, r = 0 ..
+// items_per_wg - 1, one after the other: consecutive entries of its XCD's list in the work table.
+template <typename Tr>
+__global__ __launch_bounds__(kWaves * 64, 1) void matmul_rows_kernel(
+    const char *__restrict__ x, const char *__restrict__ y, char *__restrict__ out,
+    const int32_t *__restrict__ pair_offsets, const int32_t *__restrict__ pairs,
+    const RowsRecord *__restrict__ records, int64_t n_items, int items_per_wg, int64_t nnz_o, int64_t nnz_x,
+    int64_t nnz_y) {
+  extern __shared__ __attribute__((aligned(16))) char rows_smem[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int64_t group = blockIdx.x >> 3, xcd = blockIdx.x & 7;
+  // lane l < 32 fetches int l of a record; the next record is requested before the current one is worked on
+  auto fetch = [&](int r) {
+    const int64_t at = 8 * (group * items_per_wg + r) + xcd;
+    const int32_t *rec = reinterpret_cast<const int32_t *>(records + (at < n_items ? at : 0));
+    const int v = rec[lane & 31];
+    return at < n_items && r < items_per_wg ? v : -1;  // int 0 of a record: -1 means nothing to do
+  };
+  int mine = fetch(0);
+  for (int r = 0; r < items_per_wg; ++r) {
+    const int following = fetch(r + 1);
+    rows_part<Tr>(x, y, out, pair_offsets, pairs, mine, nnz_o, nnz_x, nnz_y, rows_smem, lane, wave);
+    mine = following;
+  }
 }
 
 template <typename Tr>
 int launch_rows(const void *x, const void *y, void *out, const int32_t *pair_offsets, const int32_t *pairs,
-                const int32_t *records, int64_t n_items, int64_t nnz_x, int64_t nnz_y, hipStream_t s) {
+                const int32_t *records, int64_t n_items, int items_per_wg, int64_t nnz_o, int64_t nnz_x,
+                int64_t nnz_y, hipStream_t s) {
   static bool configured = false;  // raising the dynamic LDS limit is per function, once per process
   if (!configured) {
     BSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&matmul_rows_kernel<Tr>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kRowsLds));
     configured = true;
   }
-  matmul_rows_kernel<Tr><<<(unsigned)n_items, kWaves * 64, kRowsLds, s>>>(
+  // groups of 8 * items_per_wg records, one workgroup per XCD and group
+  const int64_t groups = bsa::cdiv(n_items, (int64_t)8 * items_per_wg);
+  matmul_rows_kernel<Tr><<<(unsigned)(groups * 8), kWaves * 64, kRowsLds, s>>>(
       static_cast<const char *>(x), static_cast<const char *>(y), static_cast<char *>(out), pair_offsets, pairs,
-      reinterpret_cast<const RowsRecord *>(records), nnz_x, nnz_y);
+      reinterpret_cast<const RowsRecord *>(records), n_items, items_per_wg, nnz_o, nnz_x, nnz_y);
   return bsa::check_launch("matmul_rows_kernel");
 }
 
@@ -516,13 +575,16 @@ bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 
 
 extern "C" int bsa_matmul_rows_records(const int32_t *work_table, int64_t n_items, int parts_log2,
                                        const int32_t *pair_offsets, const int32_t *x_row_offsets,
-                                       const int32_t *o_row_offsets, int64_t n_rows, int64_t nnz_x,
-                                       int32_t *records, bsa_stream_t stream) {
+                                       const int32_t *o_row_offsets, int64_t n_rows, int64_t n_cols,
+                                       int64_t nnz_x, int32_t *records, bsa_stream_t stream) {
   const char *who = "bsa_matmul_rows_records";
   BSA_REQUIRE(parts_log2 >= 0 && parts_log2 <= 3, "%s: parts_log2 must be 0..3 (got %d)", who, parts_log2);
   BSA_REQUIRE(n_rows >= 0 && (n_rows << parts_log2) < 0x7fffffffLL, "%s: bad number of block rows", who);
   BSA_REQUIRE(n_items >= 0 && n_items < 0x7fffffffLL, "%s: bad number of table entries", who);
   BSA_REQUIRE(nnz_x >= 0, "%s: negative size", who);
+  BSA_REQUIRE(n_cols >= 0 && ((n_cols + (1 << parts_log2) - 1) >> parts_log2) <= 64,
+              "%s: a part of a row must hold at most 64 output blocks (%lld columns of blocks in %d parts)", who,
+              (long long)n_cols, 1 << parts_log2);
   BSA_REQUIRE(work_table != nullptr || (parts_log2 == 0 && n_items == n_rows),
               "%s: without a work table the rows are taken whole and in order", who);
   if (n_items == 0) return BSA_OK;
@@ -535,17 +597,20 @@ extern "C" int bsa_matmul_rows_records(const int32_t *work_table, int64_t n_item
 }
 
 extern "C" int bsa_matmul_rows(const void *x, const void *y, void *out, const int32_t *pair_offsets,
-                               const int32_t *pairs, const int32_t *records, int64_t n_items, int64_t nnz_o,
-                               int64_t nnz_x, int64_t nnz_y, int sbs, int dtype, bsa_stream_t stream) {
+                               const int32_t *pairs, const int32_t *records, int64_t n_items,
+                               int items_per_workgroup, int64_t nnz_o, int64_t nnz_x, int64_t nnz_y, int sbs,
+                               int dtype, bsa_stream_t stream) {
   BSA_REQUIRE(sbs == 64, "bsa_matmul_rows: sbs must be 64 (got %d)", sbs);
   BSA_REQUIRE(dtype == BSA_F16 || dtype == BSA_BF16, "bsa_matmul_rows: dtype must be fp16 or bf16 (got %d)", dtype);
   BSA_REQUIRE(nnz_o >= 0 && nnz_x >= 0 && nnz_y >= 0, "bsa_matmul_rows: negative size");
   BSA_REQUIRE(n_items >= 0 && n_items < 0x7fffffffLL, "bsa_matmul_rows: bad number of records");
+  BSA_REQUIRE(items_per_workgroup >= 1 && items_per_workgroup <= 64,
+              "bsa_matmul_rows: items_per_workgroup must be 1..64 (got %d)", items_per_workgroup);
   if (nnz_o == 0 || n_items == 0) return BSA_OK;
   BSA_REQUIRE(out && pair_offsets && records, "bsa_matmul_rows: NULL pointer");
   BSA_REQUIRE(aligned16(x) && aligned16(y) && aligned16(out), "bsa_matmul_rows: buffers must be 16-byte aligned");
   BSA_REQUIRE((reinterpret_cast<uintptr_t>(records) & 127) == 0, "bsa_matmul_rows: records must be 128-byte aligned");
   hipStream_t s = bsa::as_stream(stream);
-  if (dtype == BSA_BF16) return launch_rows<MBf16>(x, y, out, pair_offsets, pairs, records, n_items, nnz_x, nnz_y, s);
-  return launch_rows<MF16>(x, y, out, pair_offsets, pairs, records, n_items, nnz_x, nnz_y, s);
+  if (dtype == BSA_BF16) return launch_rows<MBf16>(x, y, out, pair_offsets, pairs, records, n_items, items_per_workgroup, nnz_o, nnz_x, nnz_y, s);
+  return launch_rows<MF16>(x, y, out, pair_offsets, pairs, records, n_items, items_per_workgroup, nnz_o, nnz_x, nnz_y, s);
 }

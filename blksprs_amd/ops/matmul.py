@@ -7,6 +7,8 @@ and is computed by ``bsa_matmul``.  The backward pass reads the saved operands
 transposed inside the kernel instead of materialising transposed copies.
 """
 
+import os
+
 import torch
 from torch import Tensor
 
@@ -38,7 +40,7 @@ def _launch_rows(x: Tensor, y: Tensor, plan: "_Plan", sbs: int) -> Tensor:
         with torch.cuda.device(x.device):
             _capi.call("bsa_matmul_rows", _capi.ptr(x), _capi.ptr(y), out.data_ptr(),
                        plan.pair_offsets.data_ptr(), _capi.ptr(plan.pairs),
-                       _capi.ptr(plan.row_records), plan.row_records.size(0), n_out,
+                       _capi.ptr(plan.row_records), plan.row_records.size(0), plan.row_items, n_out,
                        x.size(0), y.size(0), sbs, _capi.DTYPE_CODES[x.dtype], _capi.stream(x.device))
     return out
 
@@ -63,22 +65,34 @@ _N_XCD = 8
 _L2_BYTES = 4 << 20  # one XCD's L2
 
 
-def _row_parts_log2(n_rows: int, rows_per_batch: int, n_blocks_y: int, n_blocks_o: int, block_bytes: int) -> int:
-    """Into how many runs (as log2) the row kernel cuts the output blocks of a row.
+_MAX_PART_BLOCKS = 64  # a workgroup of the row kernel takes at most this many output blocks (one mask bit each)
 
-    The rows in flight on one XCD belong to one batch entry and stream through its y blocks.  When those do
-    not fit the XCD's L2, two column halves of the entry, one after the other, halve what is in flight (on
-    C2: 30 % fewer bytes fetched behind the L2, 2 % less time); the x row is then loaded twice, and with
-    four parts that costs more than it saves.  Rows too short to feed eight waves twice stay whole.
+
+def _row_parts_log2(n_rows: int, rows_per_batch: int, n_cols: int, n_blocks_y: int, n_blocks_o: int,
+                    block_bytes: int) -> int | None:
+    """Into how many runs (as log2) the row kernel cuts the output blocks of a row; ``None`` when a row does not
+    fit the kernel's eight parts.
+
+    The rows in flight on one XCD belong to one batch entry and walk its y blocks column by column, roughly in
+    step, so the y blocks in flight are a band of columns.  When an entry's y blocks are several times an
+    XCD's L2, two column halves of the entry, one after the other, halve the band; the x row is then loaded
+    twice, and with four parts that costs more than it saves.  Rows too short to feed eight waves twice stay
+    whole.  A part holds at most 64 blocks.
     """
     batches = max(n_rows // max(rows_per_batch, 1), 1)
     y_bytes_per_entry = n_blocks_y * block_bytes // batches
     blocks_per_row = n_blocks_o // max(n_rows, 1)
-    return 1 if y_bytes_per_entry > _L2_BYTES and blocks_per_row >= 32 else 0
+    parts_log2 = 1 if y_bytes_per_entry > 4 * _L2_BYTES and blocks_per_row >= 32 else 0
+    forced = os.environ.get("BLKSPRS_AMD_ROW_PARTS_LOG2")  # for measurements
+    if forced is not None:
+        parts_log2 = int(forced)
+    while parts_log2 <= 3 and -(-n_cols // (1 << parts_log2)) > _MAX_PART_BLOCKS:
+        parts_log2 += 1
+    return parts_log2 if parts_log2 <= 3 else None
 
 
 def _row_records(work_table: Tensor, parts_log2: int, pair_offsets: Tensor, row_offsets_x: Tensor,
-                 row_offsets_o: Tensor, n_rows: int, n_blocks_x: int) -> Tensor:
+                 row_offsets_o: Tensor, n_rows: int, n_cols: int, n_blocks_x: int) -> Tensor:
     """One record per work table entry with what a workgroup of the row kernel needs to know about its part of
     a row (``bsa_matmul_rows_records``): int32 ``[n_items, 32]``."""
     records = torch.empty((work_table.numel(), _capi.ROWS_RECORD_INTS), dtype=torch.int32,
@@ -86,12 +100,13 @@ def _row_records(work_table: Tensor, parts_log2: int, pair_offsets: Tensor, row_
     if work_table.numel():
         with torch.cuda.device(work_table.device):
             _capi.call("bsa_matmul_rows_records", _capi.ptr(work_table), work_table.numel(), parts_log2,
-                       pair_offsets.data_ptr(), row_offsets_x.data_ptr(), row_offsets_o.data_ptr(), n_rows,
+                       pair_offsets.data_ptr(), row_offsets_x.data_ptr(), row_offsets_o.data_ptr(), n_rows, n_cols,
                        n_blocks_x, _capi.ptr(records), _capi.stream(work_table.device))
     return records
 
 
-def _row_work_table(pair_offsets: Tensor, row_offsets_o: Tensor, rows_per_batch: int, parts_log2: int) -> Tensor:
+def _row_work_table(pair_offsets: Tensor, row_offsets_o: Tensor, rows_per_batch: int, parts_log2: int,
+                    pair_up: bool = False) -> Tensor:
     """Order in which the row kernel hands parts of output block rows to workgroups: int32 entries
     ``row << parts_log2 | part``, -1 for nothing.
 
@@ -99,7 +114,10 @@ def _row_work_table(pair_offsets: Tensor, row_offsets_o: Tensor, rows_per_batch:
     flight on one L2 belong to the same batch entry and stream through the same y blocks), and walks it batch
     entry by batch entry, part by part, rows with the most (x, y) pairs first, so that the last workgroups of a
     launch are the short ones.  The k-th item of eighth c sits at position 8 k + c; eighths with a row less end
-    in an empty entry.
+    in an empty entry.  With ``pair_up`` the rows of a batch entry alternate longest, shortest, second longest,
+    second shortest, ...: a workgroup that takes two consecutive entries of its XCD's list then has about the
+    same work as every other one, the workgroups of an XCD start and end their rows of one batch entry together
+    (they stream through the same y blocks at the same time), and a launch ends without a tail of short rows.
     """
     n_rows = row_offsets_o.numel() - 1
     parts = 1 << parts_log2
@@ -118,6 +136,17 @@ def _row_work_table(pair_offsets: Tensor, row_offsets_o: Tensor, rows_per_batch:
     heaviest = int(work.max())
     key = ((chunk_of_row[rows] * n_entries + entry) * parts + part) * (heaviest + 1) + (heaviest - work[rows])
     by_chunk = torch.argsort(key, stable=True)  # chunk-major, batch entry, part, work descending
+    if pair_up:
+        # within a (chunk, batch entry, part) group: longest, shortest, second longest, second shortest, ...
+        group_key = (key // (heaviest + 1))[by_chunk]
+        _, inverse, sizes_g = torch.unique_consecutive(group_key, return_inverse=True, return_counts=True)
+        starts = torch.cumsum(sizes_g, 0) - sizes_g
+        rank = torch.arange(rows.numel(), device=device) - starts[inverse]
+        m = sizes_g[inverse]
+        spot = torch.where(rank < (m + 1) // 2, 2 * rank, 2 * (m - 1 - rank) + 1)
+        reordered = torch.empty_like(by_chunk)
+        reordered[starts[inverse] + spot] = by_chunk
+        by_chunk = reordered
     chunk = chunk_of_row[rows][by_chunk]
     counts = sizes * parts
     within = torch.arange(rows.numel(), device=device) - (torch.cumsum(counts, 0) - counts)[chunk]
@@ -132,12 +161,13 @@ class _Plan:
     layouts between the two (``prepare_layout_cache`` clears it in place), the object keeps what it was built
     with.  Nothing writes to its tensors after they are built."""
 
-    __slots__ = ("pair_offsets", "pairs", "block_order", "n_out", "n_x", "n_y", "row_records", "packed_x",
-                 "packed_y", "packed_o", "grad_lists")
+    __slots__ = ("pair_offsets", "pairs", "block_order", "n_out", "n_x", "n_y", "row_records", "row_items",
+                 "packed_x", "packed_y", "packed_o", "grad_lists")
 
     def __init__(self, cache: dict):
         self.pair_offsets, self.pairs = cache["contraction_offsets"], cache["contraction_pairs"]
         self.block_order, self.row_records = cache["block_order"], cache["row_records"]
+        self.row_items = cache["row_items_per_workgroup"]
         self.n_out, self.n_x, self.n_y = (cache["n_sparse_blocks"], cache["n_sparse_blocks_x"],
                                           cache["n_sparse_blocks_y"])
         self.packed_x, self.packed_y, self.packed_o = (cache["packed_indices_x"], cache["packed_indices_y"],
@@ -230,12 +260,21 @@ def matmul_build_layout_cache(layout_cache: dict | None, sparsity_layout_x: Tens
         layout_cache["row_offsets_x"] = info_x.row_offsets
         layout_cache["row_offsets_o"] = info_o.row_offsets
         layout_cache["row_records"] = None
+        layout_cache["row_items_per_workgroup"] = 1
         if info_x.row_offsets is not None and info_o.row_offsets is not None:
-            parts_log2 = _row_parts_log2(B * R, R, info_y.count, info_o.count, 64 * 64 * 2)
-            table = _row_work_table(lists.pair_offsets, info_o.row_offsets, R, parts_log2)
-            layout_cache["row_parts_log2"], layout_cache["row_work_table"] = parts_log2, table
-            layout_cache["row_records"] = _row_records(table, parts_log2, lists.pair_offsets, info_x.row_offsets,
-                                                       info_o.row_offsets, B * R, info_x.count)
+            parts_log2 = _row_parts_log2(B * R, R, C, info_y.count, info_o.count, 64 * 64 * 2)
+            if parts_log2 is not None:
+                # One row per workgroup.  Two per workgroup, a long one and a short one (equal work for every
+                # workgroup, no tail of short rows), measured no faster on configuration 2: compute units differ
+                # in speed by +-12 % on equal work, which the hardware's hand-out of many small items evens out
+                # and a static split does not.  Kept switchable for measurements.
+                pair_up = (B * R << parts_log2) >= 1024 and os.environ.get("BLKSPRS_AMD_ROW_PAIRS", "0") == "1"
+                table = _row_work_table(lists.pair_offsets, info_o.row_offsets, R, parts_log2, pair_up)
+                layout_cache["row_parts_log2"], layout_cache["row_work_table"] = parts_log2, table
+                layout_cache["row_items_per_workgroup"] = 2 if pair_up else 1
+                layout_cache["row_records"] = _row_records(table, parts_log2, lists.pair_offsets,
+                                                           info_x.row_offsets, info_o.row_offsets, B * R, C,
+                                                           info_x.count)
         layout_cache["plan"] = _Plan(layout_cache)
 
     validate_contiguous(sparsity_layout_x, layout_cache["packed_indices_x"],

@@ -229,33 +229,37 @@ int bsa_matmul(const void *x, const void *y, void *out, const int32_t *pair_offs
 /*
  * Layout-to-LUT step of bsa_matmul_rows (integer only): one record of BSA_ROWS_RECORD_INTS int32 per work
  * table entry.  x_row_offsets and o_row_offsets are the int32 CSR row offsets (n_rows + 1 entries,
- * rows = B * R) of the x layout and of the output layout as bsa_lut_packed(row_len = ...) writes them.  A
- * workgroup of bsa_matmul_rows computes one part of a row: the row's output blocks are cut into
- * 2^parts_log2 runs of equal length (parts_log2 0..3; more parts keep fewer y blocks in flight at the price of
- * loading the x row once per part).  work_table (n_items int32) is the order in which parts are handed to
- * workgroups: entry row << parts_log2 | part, or -1 for nothing; every (row, part) once.  NULL (with
- * parts_log2 == 0 and n_items == n_rows): rows 0, 1, 2, ...  Workgroup g runs on XCD g % 8, so a table that
- * gives position 8 k + c to the k-th item of a contiguous eighth c of the rows, heaviest rows first, keeps the
- * y blocks in flight on one L2 few and the tail of the launch short.  A record holds the row (-1: nothing),
- * the row's first x block and their number, and for each of the kernel's eight waves the run of output
- * blocks it computes and the first pair of that run.  No counterpart in the reference, whose kernel
- * (blksprs/ops/matmul.py:147-253) takes one output block per program.
+ * rows = B * R) of the x layout and of the output layout as bsa_lut_packed(row_len = ...) writes them; n_cols
+ * is the number of block columns of the output layout.  A workgroup of bsa_matmul_rows computes one part of a
+ * row: the row's output blocks are cut into 2^parts_log2 runs of equal length (parts_log2 0..3; more parts keep
+ * fewer y blocks in flight at the price of loading the x row once per part); a part holds at most 64 blocks, so
+ * n_cols <= 64 << parts_log2 (BSA_EINVAL otherwise).  work_table (n_items int32) is the order in which parts
+ * are handed to workgroups: entry row << parts_log2 | part, or -1 for nothing; every (row, part) once.  NULL
+ * (with parts_log2 == 0 and n_items == n_rows): rows 0, 1, 2, ...  Workgroup g runs on XCD g % 8, so a table
+ * that gives position 8 k + c to the k-th item of a contiguous eighth c of the rows, heaviest rows first, keeps
+ * the y blocks in flight on one L2 few and the tail of the launch short.  A record holds the row (-1: nothing),
+ * the row's first x block and their number, the part's first output block and their number, the mask of the
+ * part's blocks without pairs, and for each of the kernel's eight waves the mask of the blocks it computes:
+ * the blocks in ascending order, each given to the wave with the fewest pairs so far.  No counterpart in the
+ * reference, whose kernel (blksprs/ops/matmul.py:147-253) takes one output block per program.
  */
 int bsa_matmul_rows_records(const int32_t *work_table, int64_t n_items, int parts_log2,
                             const int32_t *pair_offsets, const int32_t *x_row_offsets,
-                            const int32_t *o_row_offsets, int64_t n_rows, int64_t nnz_x, int32_t *records,
-                            bsa_stream_t stream);
+                            const int32_t *o_row_offsets, int64_t n_rows, int64_t n_cols, int64_t nnz_x,
+                            int32_t *records, bsa_stream_t stream);
 
 /*
  * The same product as bsa_matmul for fp16 / bf16 operands with sbs == 64, organised by output block row: the
  * x blocks of a row are kept in LDS while the row's output blocks are computed.  records (n_items records
- * from bsa_matmul_rows_records, built for the same pair_offsets) says what each workgroup computes.
- * Bit-identical results to bsa_matmul (same accumulation order).  Same reference counterpart as
- * bsa_matmul.
+ * from bsa_matmul_rows_records, built for the same pair_offsets) says what the workgroups compute: workgroup g
+ * takes items_per_workgroup records one after the other, the records 8 (items_per_workgroup (g / 8) + r) + g % 8
+ * (consecutive entries of the work table's list for XCD g % 8; a table that pairs a long row with a short one
+ * gives every workgroup the same amount of work).  Bit-identical results to bsa_matmul (same accumulation
+ * order).  Same reference counterpart as bsa_matmul.
  */
 int bsa_matmul_rows(const void *x, const void *y, void *out, const int32_t *pair_offsets,
-                    const int32_t *pairs, const int32_t *records, int64_t n_items, int64_t nnz_o,
-                    int64_t nnz_x, int64_t nnz_y, int sbs, int dtype, bsa_stream_t stream);
+                    const int32_t *pairs, const int32_t *records, int64_t n_items, int items_per_workgroup,
+                    int64_t nnz_o, int64_t nnz_x, int64_t nnz_y, int sbs, int dtype, bsa_stream_t stream);
 
 /*
  * Block gather with element transposition: out[o] = transpose(blocks[packed[(b * R + r) * C + c]]) with

@@ -67,10 +67,11 @@ def test_bad_arguments_of_the_neighbouring_entry_points_are_rejected_on_the_host
     assert lib.bsa_attn_bwd_scratch_bytes(2, 3, 5, 7, 11) == (2 * 32 * 7 + 68 * (2 * 3 + 2 * 5) + 11 + 15) // 16 * 16
     assert lib.bsa_attn_bwd_scratch_bytes(-1, 3, 5, 7, 11) == 0
     # records of the row kernel: parts_log2 in 0..3; without a table the rows are taken whole and in order
-    assert lib.bsa_matmul_rows_records(0, 4, 4, 0, 0, 0, 4, 0, 0, 0) == -1 and b"parts_log2" in lib.bsa_last_error()
-    assert lib.bsa_matmul_rows_records(0, 8, 1, 0, 0, 0, 4, 0, 0, 0) == -1 and b"work table" in lib.bsa_last_error()
-    assert lib.bsa_matmul_rows_records(0, 0, 0, 0, 0, 0, 0, 0, 0, 0) == 0
-    assert lib.bsa_matmul_rows(0, 0, 0, 0, 0, 0, 4, 4, 1, 1, 32, _capi.BF16, 0) == -1 and b"sbs must be 64" in lib.bsa_last_error()
+    assert lib.bsa_matmul_rows_records(0, 4, 4, 0, 0, 0, 4, 4, 0, 0, 0) == -1 and b"parts_log2" in lib.bsa_last_error()
+    assert lib.bsa_matmul_rows_records(0, 8, 1, 0, 0, 0, 4, 4, 0, 0, 0) == -1 and b"work table" in lib.bsa_last_error()
+    assert lib.bsa_matmul_rows_records(0, 8, 1, 0, 0, 0, 4, 129, 0, 0, 0) == -1 and b"at most 64" in lib.bsa_last_error()
+    assert lib.bsa_matmul_rows_records(0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0) == 0
+    assert lib.bsa_matmul_rows(0, 0, 0, 0, 0, 0, 4, 1, 4, 1, 1, 32, _capi.BF16, 0) == -1 and b"sbs must be 64" in lib.bsa_last_error()
     # mask blocks that mask everything: 64 x 64 blocks only, no mask blocks is nothing to do
     assert lib.bsa_attn_mask_dead(0, 1, 32, 0, 0) == -1 and b"64 x 64" in lib.bsa_last_error()
     assert lib.bsa_attn_mask_dead(0, 1, 64, 0, 0) == -1 and b"NULL" in lib.bsa_last_error()

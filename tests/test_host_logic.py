@@ -201,10 +201,22 @@ def test_row_work_table_holds_every_part_once_and_keeps_eighths_together():
             assert order == sorted(order)
             start += size
     assert mm._row_work_table(torch.zeros(1, dtype=torch.int32), torch.zeros(1, dtype=torch.int32), 1, 1).numel() == 0
-    # two parts only when an entry's y blocks overflow one L2 and the rows are long enough to feed the waves twice
-    assert mm._row_parts_log2(1024, 64, 16287, 64370, 8192) == 1      # configuration 2
-    assert mm._row_parts_log2(1024, 64, 4096, 64370, 8192) == 0       # y of an entry fits
-    assert mm._row_parts_log2(1024, 64, 16287, 16000, 8192) == 0      # short rows
+    # two parts only when an entry's y blocks are several times one L2 and the rows are long enough to feed the
+    # waves twice
+    assert mm._row_parts_log2(1024, 64, 64, 16287, 64370, 8192) == 0      # configuration 2: 8 MB per entry
+    assert mm._row_parts_log2(1024, 64, 64, 4 * 16287, 64370, 8192) == 1  # 32 MB per entry
+    assert mm._row_parts_log2(1024, 64, 64, 4 * 16287, 16000, 8192) == 0  # short rows
+    # with pair_up a group's rows alternate longest, shortest, second longest, second shortest, ...: 16 rows of one
+    # batch entry, two per XCD, the work ascending with the row: every XCD's list is (its longer row, its shorter)
+    ascending = torch.cumsum(torch.arange(17, dtype=torch.int32) * 3, 0).to(torch.int32)
+    paired = mm._row_work_table(ascending, torch.arange(17, dtype=torch.int32), 16, 0, pair_up=True)
+    plain = mm._row_work_table(ascending, torch.arange(17, dtype=torch.int32), 16, 0)
+    for c in range(8):
+        assert paired[c::8].tolist() == [2 * c + 1, 2 * c] == plain[c::8].tolist()
+    # one XCD list of 5 rows (40 rows, one batch entry): longest, shortest, second longest, second shortest, middle
+    offsets = torch.cumsum(torch.arange(41, dtype=torch.int32), 0).to(torch.int32)
+    paired = mm._row_work_table(offsets, torch.arange(41, dtype=torch.int32), 40, 0, pair_up=True)
+    assert paired[0::8].tolist() == [4, 0, 3, 1, 2]
 
 
 def test_library_operators_are_registered_with_shape_functions():
