@@ -36,7 +36,7 @@ class AttnArgs(ctypes.Structure):
 
 
 ATTN_RECORD_INTS = 16  # BSA_ATTN_RECORD_INTS
-ROWS_RECORD_INTS = 32  # BSA_ROWS_RECORD_INTS
+ROWS_RECORD_INTS = 128  # BSA_ROWS_RECORD_INTS
 
 # name -> (restype, argtypes); must list every symbol of include/blksprs_amd.h
 SIGNATURES = {

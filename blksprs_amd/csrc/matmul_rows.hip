@@ -215,17 +215,19 @@ __device__ __forceinline__ void rows_flush(f32x16 (&acc)[2][2], char *ob, char *
       for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
 }
 
-// What a workgroup needs to know about its part of a row, in one 128-byte record (one load): the row's x
-// blocks, the part's output blocks (at most 64), and for each of the eight waves the blocks it computes, as a
-// 64-bit mask over the part's blocks.  Blocks without pairs are in no mask.
+// What a workgroup needs to know about its part of a row, in one 512-byte record (two loads per lane, the
+// first instructions of the kernel): the row's x blocks, the part's output blocks (at most 64) with their
+// pair ranges, and for each of the eight waves the blocks it computes, as a 64-bit mask over the part's blocks.
+// Blocks without pairs are in no mask.  With the pair ranges in the record the kernel reads no offsets table.
 struct RowsRecord {
   int32_t row;                // -1: nothing to do
   int32_t x_first, x_count;   // the row's blocks in x
   int32_t o_first, o_count;   // the part's output blocks
   uint32_t empty_blocks[2];   // mask of the part's blocks that have no pair (they are written as zeros)
-  int32_t pad0;
+  int32_t pairs_end;          // end of the pair list of the part's last block
   uint32_t wave_blocks[kWaves][2];  // low and high word of wave w's mask
-  int32_t pad1[8];
+  int32_t pad[40];
+  int32_t pairs_begin[64];    // start of the pair list of block o_first + i (it ends where the next one starts)
 };
 static_assert(sizeof(RowsRecord) == BSA_ROWS_RECORD_INTS * 4, "record layout");
 
@@ -246,7 +248,7 @@ __global__ __launch_bounds__(256) void rows_records_kernel(const int32_t *__rest
   item = __builtin_amdgcn_readfirstlane(item);
   const int part = item & ((1 << parts_log2) - 1);
   const int row = item < 0 ? -1 : item >> parts_log2;
-  int value = 0;  // lane l writes int l of the record
+  int value = 0, offset = 0;  // lane l writes ints l and 64 + l of the record
   if (row < 0 || row >= n_rows) {  // nothing, or a corrupt table (which must not turn into a wild read)
     if (lane == 0) value = -1;
   } else {
@@ -263,9 +265,13 @@ __global__ __launch_bounds__(256) void rows_records_kernel(const int32_t *__rest
     const int xs = x_row_offsets[row];
     int nx = x_row_offsets[row + 1] - xs;
     if (xs < 0 || nx < 0 || (int64_t)xs + nx > nnz_x) nx = 0;
-    // lane i: number of pairs of block n0 + i
+    // lane i: pair range of block n0 + i
     int my_pairs = 0;
-    if (n0 + lane < n1) my_pairs = pair_offsets[n0 + lane + 1] - pair_offsets[n0 + lane];
+    const int pairs_end = pair_offsets[n1];
+    if (n0 + lane < n1) {
+      offset = pair_offsets[n0 + lane];
+      my_pairs = pair_offsets[n0 + lane + 1] - offset;
+    }
     // blocks in ascending order, each to the wave with the least work so far (the lowest such wave)
     int load[kWaves];
     uint64_t blocks[kWaves];
@@ -284,19 +290,21 @@ __global__ __launch_bounds__(256) void rows_records_kernel(const int32_t *__rest
     }
     const uint64_t empty = __ballot(n0 + lane < n1 && my_pairs <= 0);
     if (lane == 0) value = n0 >= n1 ? -1 : row;
-    else if (lane == 5) value = (int)(uint32_t)empty;
-    else if (lane == 6) value = (int)(uint32_t)(empty >> 32);
     else if (lane == 1) value = xs;
     else if (lane == 2) value = nx;
     else if (lane == 3) value = n0;
     else if (lane == 4) value = n1 - n0;
+    else if (lane == 5) value = (int)(uint32_t)empty;
+    else if (lane == 6) value = (int)(uint32_t)(empty >> 32);
+    else if (lane == 7) value = pairs_end;
 #pragma unroll
     for (int w = 0; w < kWaves; ++w) {
       if (lane == 8 + 2 * w) value = (int)(uint32_t)blocks[w];
       if (lane == 9 + 2 * w) value = (int)(uint32_t)(blocks[w] >> 32);
     }
   }
-  if (lane < BSA_ROWS_RECORD_INTS) out[lane] = value;
+  out[lane] = value;
+  out[64 + lane] = offset;
 }
 
 // One pair of a wave's walk; everything here is wave uniform (scalar registers).
@@ -309,14 +317,15 @@ struct PairItem {
   bool valid;     // false: past the end of the wave's pairs
 };
 
-// One record: one part of a row.  `mine`: int (lane % 32) of the record.  Every wave of the workgroup passes the
+// One record: one part of a row.  `mine`: int `lane` of the record, `offs`: int 64 + lane (the pair list of
+// the part's block `lane` starts there).  Every wave of the workgroup passes the
 // same number of barriers (none when the record holds nothing, else two).
 template <typename Tr>
 __device__ __forceinline__ void rows_part(const char *__restrict__ x, const char *__restrict__ y,
                                           char *__restrict__ out, const int32_t *__restrict__ pair_offsets,
-                                          const int32_t *__restrict__ pairs, const int mine, int64_t nnz_o,
-                                          int64_t nnz_x, int64_t nnz_y, char *rows_smem, const int lane,
-                                          const int wave) {
+                                          const int32_t *__restrict__ pairs, const int mine, const int offs,
+                                          int64_t nnz_o, int64_t nnz_x, int64_t nnz_y, char *rows_smem,
+                                          const int lane, const int wave) {
   const int row = __builtin_amdgcn_readlane(mine, 0);
   if (row < 0) return;
   const int xs = __builtin_amdgcn_readlane(mine, 1);
@@ -360,50 +369,80 @@ __device__ __forceinline__ void rows_part(const char *__restrict__ x, const char
     }
   }
 
-  // The walk over this wave's pairs, one step ahead of its use.  g_*: the block being walked and its pairs not
-  // yet handed out; n_*: the block after it, whose pair range was requested when g_* was entered; raw: the next
-  // pair to hand out, its list entry already requested.
-  auto pop_block = [&]() -> int {
-    if (!todo) return -1;
-    const int b = __builtin_ctzll(todo);
-    todo &= todo - 1;
-    return o_first + b;
+  // The walk over this wave's pairs is scalar work without a branch: `todo` holds the wave's blocks from the
+  // one being walked on (its lowest set bit), [w_p, w_pe) are that block's pairs from the one handed out last.
+  // step() moves to the next pair and requests its list entry; entry_to_item() turns the entry into addresses.
+  // In the loop the two are called a whole pair of matrix products apart.  The entry is requested by a vector
+  // load (every lane the same 8 bytes) from inline assembly and waited for with vmcnt like the y blocks: a
+  // scalar load would share its counter with the LDS reads and, returning out of order, make every wait for an
+  // LDS read a wait for the load as well.  Only the first three entries of a wave, in front of the loop, come
+  // by scalar loads (behind the panel copies, a counted vector load would have to wait for those).
+  const int pairs_end = __builtin_amdgcn_readlane(mine, 7);
+  auto range_of = [&](int b, int &p, int &pe) {  // pair range of the part's block b (0 .. 63)
+    p = __builtin_amdgcn_readlane(offs, b);
+    const int next = __builtin_amdgcn_readlane(offs, (b + 1) & 63);
+    pe = b + 1 < o_count ? next : pairs_end;
   };
-  int g_block = pop_block(), g_p = 0, g_pe = 0;
-  if (g_block >= 0) g_p = pair_offsets[g_block], g_pe = pair_offsets[g_block + 1];
-  int n_block = pop_block(), n_p = 0, n_pe = 0;
-  if (n_block >= 0) n_p = pair_offsets[n_block], n_pe = pair_offsets[n_block + 1];
-  int raw_px = 0, raw_py = 0, raw_block = 0;
+  int w_p = 0, w_pe = 0;
+  if (todo) range_of(__builtin_ctzll(todo), w_p, w_pe);
+  w_p -= 1;  // nothing handed out yet
+  // what a step leaves for entry_to_item(): the entry (requested) and the facts known without it
+  u32x2 raw_entry = {0, 0};
+  int raw_block = 0;
   bool raw_last = false, raw_valid = false;
-  auto advance = [&]() {
-    while (g_block >= 0 && g_p >= g_pe) {  // the block is used up (one turn, unless a record names an empty block)
-      g_block = n_block, g_p = n_p, g_pe = n_pe;
-      n_block = pop_block();
-      if (n_block >= 0) n_p = pair_offsets[n_block], n_pe = pair_offsets[n_block + 1];
-    }
-    raw_valid = g_block >= 0;
-    if (raw_valid) {
-      const int2 e = *reinterpret_cast<const int2 *>(pairs + 2 * (int64_t)g_p);
-      raw_px = e.x, raw_py = e.y, raw_block = g_block;
-      ++g_p;
-      raw_last = g_p >= g_pe;
-    }
+  uint32_t lane_zero = 0;
+  asm volatile("" : "+v"(lane_zero));
+  auto advance = [&]() -> const int32_t * {  // returns where the next pair's entry lies
+    const int p1 = w_p + 1;
+    const bool block_done = p1 >= w_pe && todo != 0;
+    const uint64_t rest = block_done ? todo & (todo - 1) : todo;
+    const int b = rest ? __builtin_ctzll(rest) : 0;
+    int bp, bpe;
+    range_of(b, bp, bpe);
+    w_p = block_done ? bp : p1;
+    w_pe = block_done ? bpe : w_pe;
+    todo = rest;
+    raw_valid = rest != 0;
+    raw_block = o_first + b;
+    raw_last = w_p + 1 >= w_pe;
+    // past the end the last entry is requested again (the request must not depend on a branch)
+    const int at = raw_valid ? w_p : (pairs_end > 0 ? pairs_end - 1 : 0);
+    return pairs + 2 * (int64_t)(at < 0 ? 0 : at);
+  };
+  auto step_scalar = [&]() {
+    const int32_t *src = advance();
+    uint64_t e;  // spelled out: the compiler would pick a vector load, since the entry is kept in vector registers
+    asm volatile("s_load_dwordx2 %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(e) : "s"(src) : "memory");
+    raw_entry = u32x2{(uint32_t)e, (uint32_t)(e >> 32)};
+  };
+  auto step = [&]() {
+    const int32_t *src = advance();
+    asm volatile("s_nop 4\n\tglobal_load_dwordx2 %0, %1, %2" : "=v"(raw_entry) : "v"(lane_zero), "s"(src) : "memory");
   };
   const char *y_recent = y;
-  auto next_item = [&]() {
+  auto entry_to_item = [&]() {
     PairItem it;
     it.valid = raw_valid;
     it.block = raw_block;
     it.last = raw_last;
+    const int px = __builtin_amdgcn_readfirstlane((int)raw_entry[0]);
+    const int py = __builtin_amdgcn_readfirstlane((int)raw_entry[1]);
     // a corrupt list must not turn into a wild read
-    if (raw_valid) y_recent = y + (uint64_t)((raw_py < 0 || raw_py >= nnz_y) ? 0 : raw_py) * 8192;
+    if (raw_valid) y_recent = y + (uint64_t)((py < 0 || py >= nnz_y) ? 0 : py) * 8192;
     it.y = y_recent;
-    it.px = (raw_px < 0 || raw_px >= nnz_x) ? 0 : raw_px;
-    it.xoff = (unsigned)(raw_px - xs) < (unsigned)nx ? (raw_px - xs) * 8192 : -1;
-    advance();
+    it.px = (px < 0 || px >= nnz_x) ? 0 : px;
+    it.xoff = (unsigned)(px - xs) < (unsigned)nx ? (px - xs) * 8192 : -1;
     return it;
   };
-  advance();
+  if (!todo) {
+    // no block for this wave (none of its blocks has a pair: the list of pairs may be empty, so nothing is read
+    // from it): its panel pieces and zero blocks must still land before the others read the panel
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    __syncthreads();
+    return;
+  }
+  step_scalar();
 
   const uint32_t lane_lo = 16 * lane, lane_hi = 16 * lane + 4096;
 
@@ -428,14 +467,6 @@ __device__ __forceinline__ void rows_part(const char *__restrict__ x, const char
     for (int s = 0; s < 4; ++s) la.xoff[s] = li * 128 + (((2 * s + kg) ^ t_swizzle(li)) << 4);
   }
 
-  if (!raw_valid) {
-    // no pair for this wave: its panel pieces and zero blocks must still land before the others read the panel
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    __syncthreads();
-    return;
-  }
-
   f32x16 acc[2][2];  // [block along j][block along i]
 #pragma unroll
   for (int a = 0; a < 2; ++a)
@@ -450,7 +481,11 @@ __device__ __forceinline__ void rows_part(const char *__restrict__ x, const char
   // pairs repeat its last block; (2) every request is consumed, the last ones by the statement after the loop
   // that passes both slots through (registers whose contents are never used may be reused at once).
   YSlot slot_a, slot_b;
-  PairItem item_a = next_item(), item_b = next_item();
+  PairItem item_a = entry_to_item();
+  step_scalar();
+  PairItem item_b = entry_to_item();
+  step_scalar();
+  PairItem upcoming = entry_to_item();  // the pair after item_b
   y_issue(slot_a, item_a.y, lane_lo, lane_hi);
   y_issue(slot_b, item_b.y, lane_lo, lane_hi);
   // everything requested so far has arrived: the panel pieces of this wave and both slots
@@ -460,28 +495,28 @@ __device__ __forceinline__ void rows_part(const char *__restrict__ x, const char
 
   int flushed = 0;  // a block was written after the last pair
 
-  auto x_source_of = [&](const PairItem &it) {
-    XSource src;
-    src.resident = it.xoff >= 0;
-    src.lds = panel + (it.xoff >= 0 ? it.xoff : 0);
-    src.px = it.px;
-    return src;
-  };
-
   // The loop is software pipelined across pairs: while the last two quarters of a pair are multiplied, the
   // first two quarters of the next pair are staged and their fragments read, so the matrix core does not wait
   // for LDS at the start of a pair.  f0 / f1 hold the fragments of the quarter multiplied next / after it.
+  // Past the end of the wave's pairs the staging goes on with the block requested last (no branch; the
+  // fragments are not used).
   Frags f0, f1;
-  XSource x_cur = x_source_of(item_a);
+  XSource x_cur;
+  x_cur.resident = item_a.xoff >= 0;
+  x_cur.lds = panel + (item_a.xoff >= 0 ? item_a.xoff : 0);
+  x_cur.px = item_a.px;
   stage_and_read<0>(f0, slot_a, x_cur, la, x, lane);
   stage_and_read<1>(f1, slot_a, x_cur, la, x, lane);
 
   // the pair `cur` from `cur_slot` (its first two quarters are in f0 / f1 already); `next_slot` holds the pair
   // `next`; at the end `cur` is the pair whose block has been requested into `cur_slot`
   auto do_pair = [&](YSlot &cur_slot, PairItem &cur, YSlot &next_slot, const PairItem &next) {
-    const PairItem fresh = next_item();
-    const bool more = next.valid;
-    const XSource x_next = x_source_of(more ? next : cur);
+    const PairItem fresh = upcoming;
+    step();  // requests the list entry of the pair after `fresh`; it is read at the end of this pair
+    XSource x_next;
+    x_next.resident = next.xoff >= 0;
+    x_next.lds = panel + (next.xoff >= 0 ? next.xoff : 0);
+    x_next.px = next.px;
     __builtin_amdgcn_sched_barrier(0);
     multiply<Tr>(acc, f0);
     stage_and_read<2>(f0, cur_slot, x_cur, la, x, lane);
@@ -493,18 +528,23 @@ __device__ __forceinline__ void rows_part(const char *__restrict__ x, const char
     __builtin_amdgcn_sched_barrier(0);
     multiply<Tr>(acc, f0);
     // younger than the next slot's loads (issued during the pair before this one): the 8 loads just issued,
-    // and the 8 stores of a block written after that pair
+    // the request of the list entry at the top of this pair, and the 8 stores of a block written after that pair
     if (flushed)
-      asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+      asm volatile("s_waitcnt vmcnt(17)" ::: "memory");
     else
-      asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+      asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
     BSA_Y_TIE(next_slot);
     flushed = 0;
-    if (more) stage_and_read<0>(f0, next_slot, x_next, la, x, lane);
+    stage_and_read<0>(f0, next_slot, x_next, la, x, lane);
     __builtin_amdgcn_sched_barrier(0);
     multiply<Tr>(acc, f1);
-    if (more) stage_and_read<1>(f1, next_slot, x_next, la, x, lane);
+    stage_and_read<1>(f1, next_slot, x_next, la, x, lane);
     x_cur = x_next;
+    // the list entry requested at the top of this pair: only the slot's 8 loads are younger.  One statement on
+    // the straight path: the entry's registers pass through it, and with a wait in either branch of the test
+    // below the compiler would merge two copies of them, made while the load may still be in flight.
+    asm volatile("s_waitcnt vmcnt(8)" : "+v"(raw_entry) : : "memory");
+    upcoming = entry_to_item();
     if (cur.last) {
       rows_flush<Tr>(acc, out + (int64_t)cur.block * 8192, stage, lane);
       flushed = 1;
@@ -536,18 +576,23 @@ __global__ __launch_bounds__(kWaves * 64, 1) void matmul_rows_kernel(
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int64_t group = blockIdx.x >> 3, xcd = blockIdx.x & 7;
-  // lane l < 32 fetches int l of a record; the next record is requested before the current one is worked on
-  auto fetch = [&](int r) {
+  // lane l fetches ints l and 64 + l of a record; the next record is requested before the current one is worked on
+  auto fetch = [&](int r, int &head, int &offs) {
     const int64_t at = 8 * (group * items_per_wg + r) + xcd;
-    const int32_t *rec = reinterpret_cast<const int32_t *>(records + (at < n_items ? at : 0));
-    const int v = rec[lane & 31];
-    return at < n_items && r < items_per_wg ? v : -1;  // int 0 of a record: -1 means nothing to do
+    const bool there = at < n_items && r < items_per_wg;
+    const int32_t *rec = reinterpret_cast<const int32_t *>(records + (there ? at : 0));
+    head = rec[lane];
+    offs = rec[64 + lane];
+    if (!there) head = -1;  // int 0 of a record: -1 means nothing to do
   };
-  int mine = fetch(0);
+  int mine, offs;
+  fetch(0, mine, offs);
   for (int r = 0; r < items_per_wg; ++r) {
-    const int following = fetch(r + 1);
-    rows_part<Tr>(x, y, out, pair_offsets, pairs, mine, nnz_o, nnz_x, nnz_y, rows_smem, lane, wave);
-    mine = following;
+    int mine_next, offs_next;
+    fetch(r + 1, mine_next, offs_next);
+    rows_part<Tr>(x, y, out, pair_offsets, pairs, mine, offs, nnz_o, nnz_x, nnz_y, rows_smem, lane, wave);
+    mine = mine_next;
+    offs = offs_next;
   }
 }
 

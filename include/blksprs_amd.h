@@ -224,7 +224,7 @@ int bsa_matmul(const void *x, const void *y, void *out, const int32_t *pair_offs
                const int32_t *pairs, const int32_t *block_order, int64_t nnz_o, int64_t nnz_x, int64_t nnz_y, int sbs, int dtype,
                int trans_x, int trans_y, bsa_stream_t stream);
 
-#define BSA_ROWS_RECORD_INTS 32
+#define BSA_ROWS_RECORD_INTS 128
 
 /*
  * Layout-to-LUT step of bsa_matmul_rows (integer only): one record of BSA_ROWS_RECORD_INTS int32 per work
@@ -239,8 +239,9 @@ int bsa_matmul(const void *x, const void *y, void *out, const int32_t *pair_offs
  * that gives position 8 k + c to the k-th item of a contiguous eighth c of the rows, heaviest rows first, keeps
  * the y blocks in flight on one L2 few and the tail of the launch short.  A record holds the row (-1: nothing),
  * the row's first x block and their number, the part's first output block and their number, the mask of the
- * part's blocks without pairs, and for each of the kernel's eight waves the mask of the blocks it computes:
- * the blocks in ascending order, each given to the wave with the fewest pairs so far.  No counterpart in the
+ * part's blocks without pairs, the pair range of every block of the part, and for each of the kernel's eight
+ * waves the mask of the blocks it computes: the blocks in ascending order, each given to the wave with the
+ * fewest pairs so far.  No counterpart in the
  * reference, whose kernel (blksprs/ops/matmul.py:147-253) takes one output block per program.
  */
 int bsa_matmul_rows_records(const int32_t *work_table, int64_t n_items, int parts_log2,
