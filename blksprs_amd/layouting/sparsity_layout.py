@@ -94,7 +94,7 @@ def build_sparsity_layout_matmul(sparsity_layout_x: Tensor, sparsity_layout_y: T
     out = torch.empty((B, R, C), dtype=torch.bool, device=dev)
     if out.numel():
         lx, ly = _layout_bytes(sparsity_layout_x), _layout_bytes(sparsity_layout_y)
-        with torch.cuda.device(dev):
+        with _capi.on_device(dev):
             _capi.call("bsa_layout_matmul", _capi.ptr(lx), _capi.ptr(ly), B, R, K, C,
                        out.view(torch.uint8).data_ptr(), _capi.stream(dev))
     return as_base_tensor(out)

@@ -30,7 +30,7 @@ def _single_full_block(sparsity_layout: Tensor) -> bool:
 def _launch_to_sparse(x: Tensor, layout_indices: Tensor, sbs: int, n_sparse_blocks: int) -> Tensor:
     out = torch.empty((n_sparse_blocks, sbs, sbs), dtype=x.dtype, device=x.device)
     if n_sparse_blocks:
-        with torch.cuda.device(x.device):
+        with _capi.on_device(x.device):
             _capi.call("bsa_to_sparse", x.data_ptr(), layout_indices.data_ptr(), out.data_ptr(), n_sparse_blocks,
                        x.size(1), x.size(2), sbs, x.element_size(), _capi.stream(x.device))
     return out
@@ -40,7 +40,7 @@ def _launch_to_dense(x: Tensor, shape, packed_indices: Tensor, sbs: int, fill_va
     B, R, C = (int(s) for s in shape)
     out = torch.empty((B, R * sbs, C * sbs), dtype=x.dtype, device=x.device)
     if out.numel():
-        with torch.cuda.device(x.device):
+        with _capi.on_device(x.device):
             _capi.call("bsa_to_dense", _capi.ptr(x), packed_indices.data_ptr(), out.data_ptr(), B, R, C, x.size(0),
                        sbs, x.element_size(), _fill_bits(fill_value, x.dtype), _capi.stream(x.device))
     return out

@@ -245,7 +245,7 @@ def _build_forward_records(layout_cache: dict, attention_layout: Tensor, n_batch
     if "packed_indices_bias" in layout_cache:
         a.pidx_bias = _capi.ptr(layout_cache["packed_indices_bias"])
     a.group_offsets, a.group_size = offsets.data_ptr(), group_size
-    with torch.cuda.device(entries.device):
+    with _capi.on_device(entries.device):
         _capi.check(_capi.load().bsa_attn_fwd_records(ctypes.byref(a), _capi.ptr(entries), _capi.ptr(records),
                                                       _capi.stream(entries.device)), "bsa_attn_fwd_records")
     return offsets, as_base_tensor(records), group_size
@@ -319,7 +319,7 @@ def _mask_facts(layout_cache: dict, attention_layout: Tensor, mask: Tensor | Non
         live_layout = attention_layout.reshape(B, nq, nk) != 0
         if has_mask:
             dead = torch.empty(mask_bytes.size(0), dtype=torch.uint8, device=device)
-            with torch.cuda.device(device):
+            with _capi.on_device(device):
                 _capi.call("bsa_attn_mask_dead", _capi.ptr(mask_bytes), mask_bytes.size(0), mask_bytes.size(-1),
                            _capi.ptr(dead), _capi.stream(device))
             block_of_pair = layout_cache["packed_indices_mask"].reshape(B, nq, nk)
@@ -391,7 +391,7 @@ class _FlashAttention(torch.autograd.Function):
         lse = torch.empty((B, nq, sbs), dtype=torch.float32, device=q.device)
         args = _fill_args(meta, q, k, v, bias, mask, causal_lengths)
         args.o, args.lse = _capi.ptr(out), _capi.ptr(lse)
-        with torch.cuda.device(q.device):
+        with _capi.on_device(q.device):
             _capi.call("bsa_attn_fwd", ctypes.byref(args), _capi.stream(q.device))
         # the mask and the lengths are saved like the operands (as the reference does,
         # blksprs/ops/flash_attention.py:498-501): autograd then refuses a backward pass after either was
@@ -425,7 +425,7 @@ class _FlashAttention(torch.autograd.Function):
         if not args.bwd_scratch_ready:
             scratch = torch.empty(size, dtype=torch.uint8, device=q.device)
         args.bwd_scratch, args.n_layout_blocks = scratch.data_ptr(), n_layout_blocks
-        with torch.cuda.device(q.device):
+        with _capi.on_device(q.device):
             _capi.call("bsa_attn_bwd", ctypes.byref(args), stream)
         if facts is not None and not args.bwd_scratch_ready and not torch.cuda.is_current_stream_capturing():
             facts.bwd_scratch, facts.bwd_stream = scratch, stream

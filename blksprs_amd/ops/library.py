@@ -62,7 +62,7 @@ def _to_dense_shape(x, sparsity_layout, packed_indices, sparsity_block_size, fil
 
 def _softmax_fused_forward(x: Tensor, row_offsets: Tensor, n_rows: int, sparsity_block_size: int) -> Tensor:
     out = torch.empty_like(x)
-    with torch.cuda.device(x.device):
+    with _capi.on_device(x.device):
         _capi.call("bsa_softmax_fwd", x.data_ptr(), out.data_ptr(), row_offsets.data_ptr(), n_rows, x.size(0),
                    sparsity_block_size, _capi.stream(x.device))
     return out
@@ -71,7 +71,7 @@ def _softmax_fused_forward(x: Tensor, row_offsets: Tensor, n_rows: int, sparsity
 def _softmax_fused_backward(grad_output: Tensor, o: Tensor, row_offsets: Tensor, n_rows: int,
                             sparsity_block_size: int) -> Tensor:
     grad_x = torch.empty_like(o)
-    with torch.cuda.device(o.device):
+    with _capi.on_device(o.device):
         _capi.call("bsa_softmax_bwd", grad_output.data_ptr(), o.data_ptr(), grad_x.data_ptr(),
                    row_offsets.data_ptr(), n_rows, o.size(0), sparsity_block_size, _capi.stream(o.device))
     return grad_x

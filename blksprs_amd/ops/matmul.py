@@ -18,14 +18,14 @@ from ..utils.tools import (build_contraction_lists, cast_for_autocast, eager_onl
                            nonzero_from_packed, pack_layout, prepare_layout_cache)
 from ..utils.validation import (ensure_contiguous, validate_contiguous, validate_device, validate_dimensions,
                                 validate_dtype_float, validate_shape, validate_sparsity, validate_sparsity_block_size,
-                                validate_sparsity_layout)
+                                validate_sparsity_layout, validation_enabled)
 
 
 def _launch(x: Tensor, y: Tensor, pair_offsets: Tensor, pairs: Tensor, order: Tensor | None, n_out: int, sbs: int,
             trans_x: bool, trans_y: bool) -> Tensor:
     out = torch.empty((n_out, sbs, sbs), dtype=x.dtype, device=x.device)
     if n_out:
-        with torch.cuda.device(x.device):
+        with _capi.on_device(x.device):
             _capi.call("bsa_matmul", _capi.ptr(x), _capi.ptr(y), out.data_ptr(), pair_offsets.data_ptr(),
                        _capi.ptr(pairs), _capi.ptr(order), n_out, x.size(0), y.size(0), sbs,
                        _capi.DTYPE_CODES[x.dtype], int(trans_x), int(trans_y), _capi.stream(x.device))
@@ -37,7 +37,7 @@ def _launch_rows(x: Tensor, y: Tensor, plan: "_Plan", sbs: int) -> Tensor:
     n_out = plan.n_out
     out = torch.empty((n_out, sbs, sbs), dtype=x.dtype, device=x.device)
     if n_out:
-        with torch.cuda.device(x.device):
+        with _capi.on_device(x.device):
             _capi.call("bsa_matmul_rows", _capi.ptr(x), _capi.ptr(y), out.data_ptr(),
                        plan.pair_offsets.data_ptr(), _capi.ptr(plan.pairs),
                        _capi.ptr(plan.row_records), plan.row_records.size(0), plan.row_items, n_out,
@@ -98,7 +98,7 @@ def _row_records(work_table: Tensor, parts_log2: int, pair_offsets: Tensor, row_
     records = torch.empty((work_table.numel(), _capi.ROWS_RECORD_INTS), dtype=torch.int32,
                           device=work_table.device)
     if work_table.numel():
-        with torch.cuda.device(work_table.device):
+        with _capi.on_device(work_table.device):
             _capi.call("bsa_matmul_rows_records", _capi.ptr(work_table), work_table.numel(), parts_log2,
                        pair_offsets.data_ptr(), row_offsets_x.data_ptr(), row_offsets_o.data_ptr(), n_rows, n_cols,
                        n_blocks_x, _capi.ptr(records), _capi.stream(work_table.device))
@@ -198,6 +198,14 @@ def _publish_backward_lists(layout_cache: dict, plan: _Plan) -> None:
         finalize_layout_cache(layout_cache)
 
 
+def _forward(x: Tensor, y: Tensor, plan: _Plan, sparsity_block_size: int) -> Tensor:
+    if (sparsity_block_size == 64 and x.dtype in (torch.float16, torch.bfloat16)
+            and plan.row_records is not None):
+        return _launch_rows(x, y, plan, sparsity_block_size)
+    return _launch(x, y, plan.pair_offsets, plan.pairs, plan.block_order, plan.n_out, sparsity_block_size,
+                   False, False)
+
+
 class _Matmul(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, y, layout_cache, shape_x, shape_y, sparsity_block_size):
@@ -207,11 +215,7 @@ class _Matmul(torch.autograd.Function):
         ctx.layout_cache = layout_cache  # only to publish the backward lists; never read for the computation
         ctx.shapes = (shape_x, shape_y)
         ctx.sparsity_block_size = sparsity_block_size
-        if (sparsity_block_size == 64 and x.dtype in (torch.float16, torch.bfloat16)
-                and plan.row_records is not None):
-            return _launch_rows(x, y, plan, sparsity_block_size)
-        return _launch(x, y, plan.pair_offsets, plan.pairs, plan.block_order, plan.n_out, sparsity_block_size,
-                       False, False)
+        return _forward(x, y, plan, sparsity_block_size)
 
     @staticmethod
     def backward(ctx, grad_output):
@@ -309,25 +313,30 @@ def matmul(x: BlksprsTensor, sparsity_layout_x: Tensor,
     x, y = ensure_contiguous(x, y)
     x, y = cast_for_autocast(x, y)
 
-    validate_dimensions(x, y)
-    validate_contiguous(x, y, sparsity_layout_output)
-    validate_dtype_float(x, y)
-    validate_device(x, y, sparsity_layout_output)
-    validate_sparsity(sparsity_block_size, (x, sparsity_layout_x), (y, sparsity_layout_y))
-    validate_sparsity_layout(sparsity_layout_output)
+    if validation_enabled():  # every check below is a no-op otherwise
+        validate_dimensions(x, y)
+        validate_contiguous(x, y, sparsity_layout_output)
+        validate_dtype_float(x, y)
+        validate_device(x, y, sparsity_layout_output)
+        validate_sparsity(sparsity_block_size, (x, sparsity_layout_x), (y, sparsity_layout_y))
+        validate_sparsity_layout(sparsity_layout_output)
     if sparsity_layout_x.size(0) != sparsity_layout_y.size(0):
         raise ValueError("Batch dimensions of tensors must match")
     if sparsity_layout_x.size(-1) != sparsity_layout_y.size(-2):
         raise ValueError("Inner dimensions of tensors must match")
-    validate_shape(
-        sparsity_layout_output,
-        (sparsity_layout_x.size(0), sparsity_layout_x.size(1), sparsity_layout_y.size(2)),
-        "Output sparsity layout",
-    )
-    validate_sparsity_block_size(sparsity_block_size, x, y)
+    if validation_enabled():
+        validate_shape(
+            sparsity_layout_output,
+            (sparsity_layout_x.size(0), sparsity_layout_x.size(1), sparsity_layout_y.size(2)),
+            "Output sparsity layout",
+        )
+        validate_sparsity_block_size(sparsity_block_size, x, y)
 
     layout_cache = matmul_build_layout_cache(layout_cache, sparsity_layout_x, sparsity_layout_y,
                                              sparsity_layout_output)
 
+    if not (torch.is_grad_enabled() and (x.requires_grad or y.requires_grad)):
+        # nothing to differentiate: the launch itself, without the autograd machinery around it
+        return BlksprsTensor.wrap(_forward(x, y, layout_cache["plan"], sparsity_block_size))
     return BlksprsTensor.wrap(_Matmul.apply(x, y, layout_cache, tuple(sparsity_layout_x.shape),
                                             tuple(sparsity_layout_y.shape), sparsity_block_size))

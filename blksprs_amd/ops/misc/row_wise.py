@@ -94,7 +94,7 @@ def _reduce(x: Tensor, sparsity_layout: Tensor, sparsity_block_size: int, flag_s
     n_rows = int(sparsity_layout.size(0)) * int(sparsity_layout.size(1))
     with torch.no_grad():
         out = torch.empty((tables.n_rows_active, sparsity_block_size, columns), dtype=x.dtype, device=x.device)
-        with torch.cuda.device(x.device):
+        with _capi.on_device(x.device):
             _capi.call("bsa_row_reduce", x.data_ptr(), tables.row_offsets.data_ptr(), tables.packed_rows.data_ptr(),
                        _capi.ptr(out), n_rows, tables.n_rows_active, x.size(0), sparsity_block_size,
                        _capi.DTYPE_CODES[x.dtype], op, int(flag_slice_only), _capi.stream(x.device))
@@ -178,7 +178,7 @@ def row_wise_add(x: BlksprsTensor, sparsity_layout_x: Tensor, y: Tensor,
         out = torch.empty_like(as_base_tensor(x))
         if x.size(0):
             coords = tables.coords(sparsity_layout_x.shape)
-            with torch.cuda.device(x.device):
+            with _capi.on_device(x.device):
                 _capi.call("bsa_row_add", x.data_ptr(), coords.data_ptr(), tables.packed_rows.data_ptr(), _capi.ptr(y),
                            out.data_ptr(), x.size(0), y.size(0), int(sparsity_layout_x.size(0)),
                            int(sparsity_layout_x.size(1)), int(y.size(-1)), sparsity_block_size,

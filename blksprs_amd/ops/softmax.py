@@ -25,7 +25,7 @@ class _Softmax(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, row_offsets, n_rows, sparsity_block_size):
         out = torch.empty_like(x)
-        with torch.cuda.device(x.device):
+        with _capi.on_device(x.device):
             _capi.call("bsa_softmax_fwd", x.data_ptr(), out.data_ptr(), row_offsets.data_ptr(), n_rows, x.size(0),
                        sparsity_block_size, _capi.stream(x.device))
         ctx.save_for_backward(out, row_offsets)
@@ -38,7 +38,7 @@ class _Softmax(torch.autograd.Function):
         grad_output = grad_output.contiguous()
         out, row_offsets = ctx.saved_tensors
         grad_x = torch.empty_like(out)
-        with torch.cuda.device(out.device):
+        with _capi.on_device(out.device):
             _capi.call("bsa_softmax_bwd", grad_output.data_ptr(), out.data_ptr(), grad_x.data_ptr(),
                        row_offsets.data_ptr(), ctx.n_rows, out.size(0), ctx.sparsity_block_size,
                        _capi.stream(out.device))

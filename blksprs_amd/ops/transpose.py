@@ -21,7 +21,7 @@ def _launch(x: Tensor, sparsity_layout_t: Tensor, layout_indices: Tensor, packed
     out = torch.empty((n_sparse_blocks, sbs, sbs), dtype=x.dtype, device=x.device)
     if n_sparse_blocks:
         B, R, C = (int(s) for s in sparsity_layout_t.shape)
-        with torch.cuda.device(x.device):
+        with _capi.on_device(x.device):
             _capi.call("bsa_transpose_blocks", _capi.ptr(x), layout_indices.data_ptr(), packed_indices.data_ptr(),
                        out.data_ptr(), n_sparse_blocks, x.size(0), B, R, C, sbs, x.element_size(),
                        _capi.stream(x.device))

@@ -23,7 +23,8 @@ _KEY = "_blksprs_cache_key"
 _REFS = "_blksprs_cache_refs"
 _STATE = "_blksprs_cache_state"
 _CHECKED = "_blksprs_cache_checked"  # number of entries when the recorded state was last found valid
-_PRIVATE = frozenset((_KEY, _REFS, _STATE, _CHECKED))
+_WATCH = "_blksprs_cache_watch"      # the recorded state once more, in a form that is cheap to compare
+_PRIVATE = frozenset((_KEY, _REFS, _STATE, _CHECKED, _WATCH))
 
 
 def as_base_tensor(value: Tensor) -> Tensor:
@@ -86,7 +87,7 @@ def pack_layout(layout: Tensor, row_len: int = 0) -> PackedLayout:
     lib = _capi.load()
     ws_bytes = lib.bsa_lut_workspace_bytes(n)
     workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
-    with torch.cuda.device(dev):
+    with _capi.on_device(dev):
         _capi.call("bsa_lut_packed", _capi.ptr(lay), n, row_len, _capi.ptr(packed),
                    row_offsets.data_ptr() if row_offsets is not None else 0,
                    stats_dev.data_ptr(), stats_host.data_ptr(), _capi.ptr(workspace), ws_bytes, _capi.stream(dev))
@@ -103,7 +104,7 @@ def nonzero_from_packed(packed: Tensor, shape, count: int) -> Tensor:
     B, R, C = (int(s) for s in shape)
     coords = torch.empty((count, 3), dtype=torch.int64, device=packed.device)
     if count:
-        with torch.cuda.device(packed.device):
+        with _capi.on_device(packed.device):
             _capi.call("bsa_lut_nonzero", packed.data_ptr(), B, R, C, coords.data_ptr(), _capi.stream(packed.device))
     return coords
 
@@ -118,7 +119,7 @@ def csr_indices_from_packed(packed: Tensor, n_cols: int, count: int) -> Tensor:
     """int32 column ids of the active blocks, row by row."""
     indices = torch.empty(count, dtype=torch.int32, device=packed.device)
     if count:
-        with torch.cuda.device(packed.device):
+        with _capi.on_device(packed.device):
             _capi.call("bsa_lut_csr_indices", packed.data_ptr(), packed.numel(), n_cols, indices.data_ptr(),
                        _capi.stream(packed.device))
     return indices
@@ -128,7 +129,7 @@ def sorted_rows_from_offsets(row_offsets: Tensor, n_rows: int, n_cols: int) -> T
     """Per-row descending sort of the reverse index (active first), int64 flat."""
     out = torch.empty(n_rows * n_cols, dtype=torch.int64, device=row_offsets.device)
     if out.numel():
-        with torch.cuda.device(out.device):
+        with _capi.on_device(out.device):
             _capi.call("bsa_lut_sorted_rows", row_offsets.data_ptr(), n_rows, n_cols, out.data_ptr(),
                        _capi.stream(out.device))
     return out
@@ -157,7 +158,7 @@ def build_contraction_lists(pidx_x: Tensor, pidx_y: Tensor, pidx_o: Tensor, B: i
     lib = _capi.load()
     ws_bytes = lib.bsa_lut_workspace_bytes(n)
     workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
-    with torch.cuda.device(dev):
+    with _capi.on_device(dev):
         st = _capi.stream(dev)
         _capi.call("bsa_lut_contraction_offsets", _capi.ptr(pidx_x), _capi.ptr(pidx_y), _capi.ptr(pidx_o),
                    B, R, K, C, mask_x.data_ptr(), mask_y.data_ptr(), pos_offsets.data_ptr(),
@@ -175,12 +176,6 @@ def build_contraction_lists(pidx_x: Tensor, pidx_y: Tensor, pidx_o: Tensor, B: i
 
 # --------------------------------------------------------------------------- layout cache
 
-def _tensor_signature(value: Tensor, version):
-    # torch.Size and the stride tuple compare and hash like plain tuples
-    return ("tensor", id(value), version, value.shape, value.stride(), value.dtype, value.device,
-            value.requires_grad)
-
-
 def prepare_layout_cache(layout_cache: LayoutCache | None, operation: str, *values: object) -> LayoutCache:
     """Returns ``layout_cache`` ready for ``operation``, emptied first if it belongs to other inputs.
 
@@ -194,7 +189,7 @@ def prepare_layout_cache(layout_cache: LayoutCache | None, operation: str, *valu
         layout_cache = {}
     key, refs = layout_cache_key(operation, *values)
     recorded = layout_cache.get(_STATE)
-    stale = (layout_cache.get(_KEY) != key or recorded is None or _snapshot(layout_cache) != recorded)
+    stale = layout_cache.get(_KEY) != key or recorded is None or not _unchanged(layout_cache, recorded)
     if stale:
         layout_cache.clear()
         layout_cache[_KEY] = key
@@ -209,19 +204,23 @@ def prepare_layout_cache(layout_cache: LayoutCache | None, operation: str, *valu
 def layout_cache_key(operation: str, *values: object) -> tuple[tuple, tuple]:
     """The key ``prepare_layout_cache`` files a cache under, and the tensors it depends on."""
     refs: list[Tensor] = []
-    never_equal = object()
+    parts = [_signature(v, refs) for v in values]
+    return (operation, tuple(parts)), tuple(refs)
 
-    def signature(value):
-        if isinstance(value, Tensor):
-            refs.append(value)
-            return _tensor_signature(value, never_equal if torch.is_inference(value) else int(value._version))
-        if isinstance(value, (tuple, list, Size)):
-            return tuple(signature(v) for v in value)
-        if isinstance(value, dict):
-            return tuple(sorted((k, signature(v)) for k, v in value.items()))
-        return value
 
-    return (operation, tuple(signature(v) for v in values)), tuple(refs)
+def _signature(value, refs: list):
+    if isinstance(value, Tensor):
+        refs.append(value)
+        # an inference tensor has no version counter: a fresh object never equals an earlier key
+        version = object() if value.is_inference() else value._version
+        # torch.Size and the stride tuple compare and hash like plain tuples
+        return ("tensor", id(value), version, value.shape, value.stride(), value.dtype, value.device,
+                value.requires_grad)
+    if isinstance(value, (tuple, list, Size)):
+        return tuple(_signature(v, refs) for v in value)
+    if isinstance(value, dict):
+        return tuple(sorted((k, _signature(v, refs)) for k, v in value.items()))
+    return value
 
 
 class CacheHolder:
@@ -243,7 +242,43 @@ def finalize_layout_cache(layout_cache: LayoutCache) -> LayoutCache:
         return layout_cache
     layout_cache[_STATE] = _snapshot(layout_cache)
     layout_cache[_CHECKED] = None
+    layout_cache[_WATCH] = None
+    layout_cache[_WATCH] = _watch_list(layout_cache)
     return layout_cache
+
+
+def _watch_list(layout_cache: LayoutCache) -> tuple:
+    """The recorded state as ``(number of entries, [(key, object, version or None), ...])`` when every entry is a
+    tensor with a version counter or a value that is compared by identity; ``None`` when some entry needs the full
+    comparison (containers, inference tensors)."""
+    entries = []
+    for key, value in layout_cache.items():
+        if key in _PRIVATE:
+            continue
+        if isinstance(value, Tensor):
+            if torch.is_inference(value):
+                return None
+            entries.append((key, value, value._version))
+        elif isinstance(value, (dict, tuple, list, Size, PackedLayout, ContractionLists)):
+            return None
+        else:
+            entries.append((key, value, None))
+    return len(layout_cache), tuple(entries)
+
+
+def _unchanged(layout_cache: LayoutCache, recorded: tuple) -> bool:
+    """Whether the cache holds what it held when its state was recorded: every entry the same object with the same
+    version counter (this runs on every call of an operator that is handed a cache)."""
+    watch = layout_cache.get(_WATCH)
+    if watch is None or len(layout_cache) != watch[0]:
+        return _snapshot(layout_cache) == recorded
+    get = layout_cache.get
+    for key, value, version in watch[1]:
+        current = get(key, _PRIVATE)
+        if current is not value or (version is not None and current._version != version):
+            # an equal value under another identity (an int, say) is no change: let the full comparison decide
+            return _snapshot(layout_cache) == recorded
+    return True
 
 
 def _snapshot(layout_cache: LayoutCache) -> tuple:

@@ -20,6 +20,9 @@ def _validation_enabled() -> bool:
     return getattr(_state, "validation", True)
 
 
+validation_enabled = _validation_enabled
+
+
 def _contiguous_enabled() -> bool:
     return getattr(_state, "contiguous", True)
 
