@@ -635,6 +635,75 @@ def attention_workload(dev, backward):
                         "layout_blocks": nnz, "mask": "explicit causal blocks"})
 
 
+def reference_attention_benchmark(dev, m=2048):
+    """The reference's own attention benchmark (test/cases/test_blocksparse.py:1481-1579): fp32, batch * heads = 8,
+    sequence ``m``, head_dim 64, sbs 32, half of the attention layout's blocks active (every row at least one).  The
+    step is ``flash_attention``; the same result by ``matmul -> scale -> softmax -> matmul`` of this library is timed
+    next to it (``unfused_ms``), and the reference asserts flash <= 1.1 x unfused."""
+    import blksprs_amd as bs
+    from oracle import blksprs_oracle as orc
+
+    bh, hd, sbs = 8, 64, 32
+    n, nh = m // sbs, hd // sbs
+    g = torch.Generator().manual_seed(0)
+    la = orc.random_layout((bh, n, n), 0.5, g, ensure_rows=True).to(dev)
+    lqkv = torch.ones((bh, n, nh), dtype=torch.bool, device=dev)
+    gd = torch.Generator(device=dev).manual_seed(1)
+    q, k, v = (bs.ops.to_sparse(torch.randn((bh, m, hd), generator=gd, device=dev), lqkv, sbs) for _ in range(3))
+    k_t, lkt = bs.ops.transpose(k, lqkv, sbs)
+    lo = bs.layouting.build_sparsity_layout_matmul(la, lqkv)
+    scale = 1.0 / hd ** 0.5
+    caches = [{}, {}, {}, {}]
+
+    def unfused():
+        scores = bs.ops.matmul(q, lqkv, k_t, lkt, la, sbs, layout_cache=caches[0]) * scale
+        probs = bs.ops.softmax(scores, la, sbs, layout_cache=caches[1])
+        return bs.ops.matmul(probs, la, v, lqkv, lo, sbs, layout_cache=caches[2])
+
+    def step():
+        return bs.ops.flash_attention(q, lqkv, k, lqkv, v, lqkv, la, sbs, scale=scale, layout_cache=caches[3])
+
+    same = bool(torch.allclose(unfused(), step(), rtol=1e-4, atol=1e-4))
+    bs.utils.disable_validation()
+    for _ in range(20):
+        unfused()
+    torch.cuda.synchronize()
+    ev = _events(20)
+    for s_, e_ in ev:
+        s_.record()
+        unfused()
+        e_.record()
+    torch.cuda.synchronize()
+    unfused_ms = sorted(a.elapsed_time(b) for a, b in ev)[10]
+    nnz = int(la.sum())
+    flops = nnz * 4.0 * sbs * sbs * hd
+    alg_bytes = 4 * bh * m * hd * 4
+
+    def check():
+        """Batch entry 0 against the CPU oracle at rtol = atol = 1e-5, and flash against the unfused path."""
+        cnt = n * nh
+        fl = lqkv[:1].cpu().numpy()
+        want = orc.flash_attention(q[:cnt].cpu(), fl, k[:cnt].cpu(), fl, v[:cnt].cpu(), fl, la[:1].cpu().numpy(), sbs,
+                                   scale=scale)
+        return same and bool(torch.allclose(step()[:cnt].cpu(), want, rtol=1e-5, atol=1e-5))
+
+    def cpu_baseline():
+        cnt = n * nh
+        fl = lqkv[:1].cpu().numpy()
+        qs, ks, vs, lay = q[:cnt].cpu(), k[:cnt].cpu(), v[:cnt].cpu(), la[:1].cpu().numpy()
+        reps, dt = _repeat_for(CPU_SAMPLE_SECONDS, lambda: orc.flash_attention(qs, fl, ks, fl, vs, fl, lay, sbs,
+                                                                                scale=scale))
+        return {"value": int(la[:1].sum()) * 4.0 * sbs * sbs * hd / dt / 1e12, "unit": "TFLOP/s",
+                "cores": torch.get_num_threads(), "kind": "port",
+                "sample": f"1 of {bh} heads x {reps} passes, dense masked fp32 torch attention, {dt * reps:.1f} s"}
+
+    return dict(step=step, flops=flops, alg_bytes=alg_bytes, dtype="f32", bound="mfma", cpu_baseline=cpu_baseline,
+                check=check, kernel="attn_fwd kernel of the fp32 path",
+                config={"workload": "a1_flash_attention_fp32_reference_benchmark", "batch_heads": bh, "seq": m,
+                        "head_dim": hd, "sparsity_block_size": sbs, "layout_blocks": nnz,
+                        "unfused_ms": round(unfused_ms, 4)})
+
+
 def make_workload(name, dev):
     if name == "c1":
         return matmul_workload("c1_matmul_fp32", 2, 8, 32, torch.float32, 0.5, True, 1.0, dev, 2)
@@ -652,6 +721,8 @@ def make_workload(name, dev):
         return attention_workload(dev, backward=False)
     if name == "c4bwd":
         return attention_workload(dev, backward=True)
+    if name == "a1":
+        return reference_attention_benchmark(dev)
     if name == "c5":
         return matmul_workload("c5_matmul_fp16", 64, 128, 16, torch.float16, 0.05, True, 1.0, dev, 8)
     if name == "t1":
@@ -671,7 +742,7 @@ def make_workload(name, dev):
     raise SystemExit(f"unknown config {name}")
 
 
-CONFIGS = ["c1", "c2", "c2bwd", "c3", "c3bwd", "c4", "c4bwd", "c5", "t1", "l1", "r1", "r2", "p1", "v1", "v2"]
+CONFIGS = ["a1", "c1", "c2", "c2bwd", "c3", "c3bwd", "c4", "c4bwd", "c5", "t1", "l1", "r1", "r2", "p1", "v1", "v2"]
 # the configurations a default run times behind the headline one, with fewer steps (their roofline objects ride
 # along in the same JSON line so that they are timed by whoever runs the script, not quoted from elsewhere)
 COMPANIONS = ["c4", "c3", "c5"]

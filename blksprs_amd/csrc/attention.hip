@@ -1,5 +1,7 @@
-// C ABI of block-sparse flash attention: argument checks and the choice between the
-// MFMA kernels (16-bit operands, sbs 32/64) and the generic kernels (everything else).
+// C ABI of block-sparse flash attention: argument checks and the choice between the 16-bit matrix-core kernels
+// (16-bit operands, 64 x 64 blocks, at most two head slices), the fp32 matrix-core forward kernel (every other
+// operand type and block size) and the generic kernels (what neither takes, and the backward pass of what the
+// first does not take).
 #include "attn_common.h"
 
 namespace {
@@ -45,7 +47,8 @@ int check_args(const char *who, const bsa_attn_args *a, bool backward) {
 extern "C" int bsa_attn_fwd(const bsa_attn_args *args, bsa_stream_t stream) {
   if (int rc = check_args("bsa_attn_fwd", args, false)) return rc;
   hipStream_t s = bsa::as_stream(stream);
-  int rc = bsa::attn_fwd_mfma(*args, s);
+  int rc = bsa::attn_fwd_mfma(*args, s);          // 16-bit operands, 64 x 64 blocks
+  if (rc == 1) rc = bsa::attn_fwd_f32mma(*args, s);  // everything else, on the fp32 matrix-core instruction
   if (rc == 1) rc = bsa::attn_fwd_generic(*args, s);
   return rc;
 }

@@ -92,6 +92,18 @@ def test_rectangular_sparse_heads_and_custom_output_layout(device, dtype):
               custom_o=True, use_mask=True, use_bias=True, scale=0.37)
 
 
+@pytest.mark.parametrize("dtype,sbs", [(torch.float32, 16), (torch.float32, 64), (torch.bfloat16, 32), (torch.float16, 16)])
+@pytest.mark.parametrize("nh,nhv", [(4, 3), (1, 4), (3, 5)])
+def test_many_head_slices_and_long_key_lists(device, dtype, sbs, nh, nhv):
+    """The fp32 matrix-core forward kernel: key lists longer than its groups of waves (9 key blocks for 2 or 4
+    groups, rows with a single key block next to them), three and four value head slices (the kernel is built for
+    1, 2 and 4), and five, which it leaves to the generic kernel; sparse head layouts, mask, bias and causal
+    lengths together."""
+    _run_case(device, dtype, sbs, B=2, nq=5, nk=9, nh=nh, nhv=nhv, density=0.55, seed=sbs + nh, use_mask=True,
+              use_bias=True, sparse_heads=True, custom_o=True)
+    _run_case(device, dtype, sbs, B=1, nq=9, nk=9, nh=nh, nhv=nhv, density=0.3, seed=sbs + nhv, use_causal=True)
+
+
 def test_bigbird_layout_with_causal_mask_head_dim_128(device):
     """Config 4's shape at reduced batch and length: bf16, sbs 64, head_dim 128, BigBird layout, causal mask."""
     B, n, sbs, nh = 2, 16, 64, 2
