@@ -635,7 +635,7 @@ def attention_workload(dev, backward):
                         "layout_blocks": nnz, "mask": "explicit causal blocks"})
 
 
-def reference_attention_benchmark(dev, m=2048):
+def reference_attention_benchmark(dev, m=2048, backward=False):
     """The reference's own attention benchmark (test/cases/test_blocksparse.py:1481-1579): fp32, batch * heads = 8,
     sequence ``m``, head_dim 64, sbs 32, half of the attention layout's blocks active (every row at least one).  The
     step is ``flash_attention``; the same result by ``matmul -> scale -> softmax -> matmul`` of this library is timed
@@ -650,20 +650,35 @@ def reference_attention_benchmark(dev, m=2048):
     lqkv = torch.ones((bh, n, nh), dtype=torch.bool, device=dev)
     gd = torch.Generator(device=dev).manual_seed(1)
     q, k, v = (bs.ops.to_sparse(torch.randn((bh, m, hd), generator=gd, device=dev), lqkv, sbs) for _ in range(3))
+    d_o = torch.randn(q.shape, generator=gd, device=dev)
+    if backward:
+        q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
     k_t, lkt = bs.ops.transpose(k, lqkv, sbs)
     lo = bs.layouting.build_sparsity_layout_matmul(la, lqkv)
     scale = 1.0 / hd ** 0.5
     caches = [{}, {}, {}, {}]
 
     def unfused():
-        scores = bs.ops.matmul(q, lqkv, k_t, lkt, la, sbs, layout_cache=caches[0]) * scale
+        k_now, _ = bs.ops.transpose(k, lqkv, sbs) if backward else (k_t, None)
+        scores = bs.ops.matmul(q, lqkv, k_now, lkt, la, sbs, layout_cache=caches[0]) * scale
         probs = bs.ops.softmax(scores, la, sbs, layout_cache=caches[1])
-        return bs.ops.matmul(probs, la, v, lqkv, lo, sbs, layout_cache=caches[2])
+        out = bs.ops.matmul(probs, la, v, lqkv, lo, sbs, layout_cache=caches[2])
+        if backward:
+            q.grad = k.grad = v.grad = None
+            out.backward(d_o)
+        return out
 
     def step():
-        return bs.ops.flash_attention(q, lqkv, k, lqkv, v, lqkv, la, sbs, scale=scale, layout_cache=caches[3])
+        out = bs.ops.flash_attention(q, lqkv, k, lqkv, v, lqkv, la, sbs, scale=scale, layout_cache=caches[3])
+        if backward:
+            q.grad = k.grad = v.grad = None
+            out.backward(d_o)
+        return out
 
-    same = bool(torch.allclose(unfused(), step(), rtol=1e-4, atol=1e-4))
+    unfused_out = unfused().detach()
+    unfused_grads = [t.grad.clone() for t in (q, k, v)] if backward else []
+    same = bool(torch.allclose(unfused_out, step().detach(), rtol=1e-4, atol=1e-4))
+    same = same and all(torch.allclose(g, t.grad, rtol=1e-3, atol=1e-4) for g, t in zip(unfused_grads, (q, k, v)))
     bs.utils.disable_validation()
     for _ in range(20):
         unfused()
@@ -676,21 +691,27 @@ def reference_attention_benchmark(dev, m=2048):
     torch.cuda.synchronize()
     unfused_ms = sorted(a.elapsed_time(b) for a, b in ev)[10]
     nnz = int(la.sum())
-    flops = nnz * 4.0 * sbs * sbs * hd
-    alg_bytes = 4 * bh * m * hd * 4
+    flops = nnz * 4.0 * sbs * sbs * hd * (3.5 if backward else 1.0)
+    alg_bytes = (9 if backward else 4) * bh * m * hd * 4
 
     def check():
-        """Batch entry 0 against the CPU oracle at rtol = atol = 1e-5, and flash against the unfused path."""
+        """Batch entry 0 against the CPU oracle at rtol = atol = 1e-5 (gradients: 2e-5 on O(1) values), and flash
+        against the unfused path."""
         cnt = n * nh
         fl = lqkv[:1].cpu().numpy()
-        want = orc.flash_attention(q[:cnt].cpu(), fl, k[:cnt].cpu(), fl, v[:cnt].cpu(), fl, la[:1].cpu().numpy(), sbs,
-                                   scale=scale)
-        return same and bool(torch.allclose(step()[:cnt].cpu(), want, rtol=1e-5, atol=1e-5))
+        leaves = [t[:cnt].detach().cpu().requires_grad_(backward) for t in (q, k, v)]
+        want = orc.flash_attention(leaves[0], fl, leaves[1], fl, leaves[2], fl, la[:1].cpu().numpy(), sbs, scale=scale)
+        ok = same and bool(torch.allclose(step()[:cnt].detach().cpu(), want.detach(), rtol=1e-5, atol=1e-5))
+        if backward:
+            want.backward(d_o[:cnt].cpu())
+            ok = ok and all(torch.allclose(t.grad[:cnt].cpu(), ref.grad, rtol=2e-5, atol=2e-5)
+                            for t, ref in zip((q, k, v), leaves))
+        return ok
 
     def cpu_baseline():
         cnt = n * nh
         fl = lqkv[:1].cpu().numpy()
-        qs, ks, vs, lay = q[:cnt].cpu(), k[:cnt].cpu(), v[:cnt].cpu(), la[:1].cpu().numpy()
+        qs, ks, vs, lay = (*(t[:cnt].detach().cpu() for t in (q, k, v)), la[:1].cpu().numpy())
         reps, dt = _repeat_for(CPU_SAMPLE_SECONDS, lambda: orc.flash_attention(qs, fl, ks, fl, vs, fl, lay, sbs,
                                                                                 scale=scale))
         return {"value": int(la[:1].sum()) * 4.0 * sbs * sbs * hd / dt / 1e12, "unit": "TFLOP/s",
@@ -698,8 +719,9 @@ def reference_attention_benchmark(dev, m=2048):
                 "sample": f"1 of {bh} heads x {reps} passes, dense masked fp32 torch attention, {dt * reps:.1f} s"}
 
     return dict(step=step, flops=flops, alg_bytes=alg_bytes, dtype="f32", bound="mfma", cpu_baseline=cpu_baseline,
-                check=check, kernel="attn_fwd kernel of the fp32 path",
-                config={"workload": "a1_flash_attention_fp32_reference_benchmark", "batch_heads": bh, "seq": m,
+                check=check, kernel="attn_fwd_f32mma_kernel" + (" + attn_f32mma_delta / dkdv / dq kernels" if backward else ""),
+                config={"workload": "a1_flash_attention_fp32_reference_benchmark" + ("_fwd_bwd" if backward else ""),
+                        "batch_heads": bh, "seq": m,
                         "head_dim": hd, "sparsity_block_size": sbs, "layout_blocks": nnz,
                         "unfused_ms": round(unfused_ms, 4)})
 
@@ -723,6 +745,8 @@ def make_workload(name, dev):
         return attention_workload(dev, backward=True)
     if name == "a1":
         return reference_attention_benchmark(dev)
+    if name == "a1bwd":
+        return reference_attention_benchmark(dev, backward=True)
     if name == "c5":
         return matmul_workload("c5_matmul_fp16", 64, 128, 16, torch.float16, 0.05, True, 1.0, dev, 8)
     if name == "t1":
@@ -742,7 +766,7 @@ def make_workload(name, dev):
     raise SystemExit(f"unknown config {name}")
 
 
-CONFIGS = ["a1", "c1", "c2", "c2bwd", "c3", "c3bwd", "c4", "c4bwd", "c5", "t1", "l1", "r1", "r2", "p1", "v1", "v2"]
+CONFIGS = ["a1", "a1bwd", "c1", "c2", "c2bwd", "c3", "c3bwd", "c4", "c4bwd", "c5", "t1", "l1", "r1", "r2", "p1", "v1", "v2"]
 # the configurations a default run times behind the headline one, with fewer steps (their roofline objects ride
 # along in the same JSON line so that they are timed by whoever runs the script, not quoted from elsewhere)
 COMPANIONS = ["c4", "c3", "c5"]

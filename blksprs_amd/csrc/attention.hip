@@ -1,7 +1,6 @@
 // C ABI of block-sparse flash attention: argument checks and the choice between the 16-bit matrix-core kernels
-// (16-bit operands, 64 x 64 blocks, at most two head slices), the fp32 matrix-core forward kernel (every other
-// operand type and block size) and the generic kernels (what neither takes, and the backward pass of what the
-// first does not take).
+// (16-bit operands, 64 x 64 blocks, at most two head slices), the fp32 matrix-core kernels (every other operand
+// type and block size) and the generic kernels (what neither takes: more head slices than fit LDS).
 #include "attn_common.h"
 
 namespace {
@@ -93,6 +92,7 @@ extern "C" int bsa_attn_bwd(const bsa_attn_args *args, bsa_stream_t stream) {
   BSA_REQUIRE((reinterpret_cast<uintptr_t>(args->bwd_scratch) & 15) == 0, "bsa_attn_bwd: bwd_scratch must be 16-byte aligned");
   hipStream_t s = bsa::as_stream(stream);
   int rc = bsa::attn_bwd_mfma(*args, s);
+  if (rc == 1) rc = bsa::attn_bwd_f32mma(*args, s);
   if (rc == 1) rc = bsa::attn_bwd_generic(*args, s);
   return rc;
 }
