@@ -252,6 +252,47 @@ __global__ __launch_bounds__(64 * kWaves) void softmax_bwd_kernel(const float *_
     return;
   }
 
+  if (units <= kMaxUnits) {
+    // middle rows: y stays in registers, the gradient passes twice in chunks (once for the row's sum, once for the
+    // result): 1.5 instead of 2 reads of the row's 2 x 16 bytes per element
+    float4 yv[kMaxUnits];
+    load_row(yv, yr, units, g);
+    float s = 0.f;
+#pragma unroll
+    for (int c = 0; c < kMaxUnits; c += kChunk) {
+      if (c < units) {
+        const int count = units - c < kChunk ? units - c : kChunk;
+        float4 gv[kChunk];
+        load_chunk(gv, gr, c, count, g);
+#pragma unroll
+        for (int j = 0; j < kChunk; ++j)
+          if (j < count)
+            s += (yv[c + j].x * gv[j].x + yv[c + j].y * gv[j].y) + (yv[c + j].z * gv[j].z + yv[c + j].w * gv[j].w);
+      }
+    }
+    s = lanes_sum(s, g.lpr);
+#pragma unroll
+    for (int c = 0; c < kMaxUnits; c += kChunk) {
+      if (c < units) {
+        const int count = units - c < kChunk ? units - c : kChunk;
+        float4 gv[kChunk];
+        load_chunk(gv, gr, c, count, g);
+#pragma unroll
+        for (int j = 0; j < kChunk; ++j) {
+          if (j < count) {
+            float4 o;
+            o.x = yv[c + j].x * (gv[j].x - s);
+            o.y = yv[c + j].y * (gv[j].y - s);
+            o.z = yv[c + j].z * (gv[j].z - s);
+            o.w = yv[c + j].w * (gv[j].w - s);
+            store_streaming(dr + unit_offset(c + j, g), o);
+          }
+        }
+      }
+    }
+    return;
+  }
+
   // long rows: two passes in chunks whose loads are all issued before the first one is used
   float s = 0.f;
   for (int u0 = 0; u0 < units; u0 += kChunk) {
