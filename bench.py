@@ -46,10 +46,12 @@ PEAK_MFMA_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}
 # what leaves an L2, so reads served by the memory-side cache are included.  Not re-measured by this script.
 TRAFFIC_KIB = {  # config: (FETCH_SIZE, WRITE_SIZE)
     "c1": (616.2, 476.0),
-    "c2": (347206.9, 514967.2),
+    "c2": (376348.9, 514961.6),
     "c3": (148153.3, 296259.0),
     "c4": (238469.4, 133139.0),
     "c5": (28438.4, 143960.0),
+    "c3bwd": (369125.1, 296130.4),
+    "a1": (38057.2, 4160.0),
     "v1": (66312.1, 129576.0),
     "v2": (66851.5, 524499.4),
     "t1": (67086.4, 129576.0),
