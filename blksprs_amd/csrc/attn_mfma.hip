@@ -442,6 +442,13 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
       vote(f2, e + 2);
       // The rows this wave copied have to be in LDS; the loads issued after the copies (a record, two mask
       // loads if the tile has a mask block) may stay in flight.  vmcnt(3) / vmcnt(1), other counters untouched.
+      // The counts follow this iteration's issue order at the top of the loop: copy_k / copy_v (the asynchronous
+      // copies of tile e + 1), then load_record (one vector load, the record of tile e + 4), then fetch_mask,
+      // which issues two loads only when the record of tile e + 3 names a mask block (f3.pm >= 0).  vmcnt
+      // retires in issue order, so "at most 1 (3) outstanding" leaves exactly those younger loads in flight.
+      // The bias loads of the tile are consumed (and so waited for by the compiler) inside the tile.  A load
+      // added after the copies and not consumed before this point would make these waits too lax by one: it has
+      // to be added to both counts.
       if (f3.pm >= 0) __builtin_amdgcn_s_waitcnt(0x0F73);
       else __builtin_amdgcn_s_waitcnt(0x0F71);
       f0 = f1;

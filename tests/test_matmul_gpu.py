@@ -234,6 +234,42 @@ def test_row_panel_kernel_is_bit_identical_to_the_tile_kernel(device, dtype, dim
     assert_close(out, _oracle(x.cpu(), lx.cpu(), y.cpu(), ly.cpu(), lo.cpu(), sbs), 2e-2, "row panel vs oracle")
 
 
+@pytest.mark.parametrize("parts_log2,items", [(0, 1), (1, 1), (2, 3), (0, 2), (3, 2)])
+def test_row_kernel_parts_and_records_per_workgroup(device, parts_log2, items):
+    """The row kernel through the C ABI with rows cut into 1, 2, 4 and 8 column parts and with one, two and
+    three records per workgroup (a workgroup then works through consecutive entries of its XCD's list, the
+    last workgroups through fewer): the same bits as the tile kernel.  120 block columns: parts of up to 64
+    blocks (one mask bit each) and of 15; a work table in reversed order with empty entries."""
+    import importlib
+    from blksprs_amd import _capi
+    from blksprs_amd.utils.tools import build_contraction_lists, pack_layout
+    mm = importlib.import_module("blksprs_amd.ops.matmul")
+    B, R, K, C, sbs = 2, 5, 6, 120, 64
+    if (C + (1 << parts_log2) - 1) >> parts_log2 > 64:
+        parts_log2 += 1  # whole rows of 120 blocks do not fit a record: the entry point refuses them (below)
+        with pytest.raises(RuntimeError, match="at most 64"):
+            _capi.call("bsa_matmul_rows_records", 0, B * R, 0, 8, 8, 8, B * R, C, 0, 8, 0)
+    lx, ly = rand_layout((B, R, K), 0.6, seed=1).to(device), rand_layout((B, K, C), 0.5, seed=2).to(device)
+    lo = rand_layout((B, R, C), 0.7, seed=3).to(device)
+    x = rand_blocks(int(lx.sum()), sbs, torch.bfloat16, 4, 1.0 / math.sqrt(K * sbs)).to(device)
+    y = rand_blocks(int(ly.sum()), sbs, torch.bfloat16, 5).to(device)
+    info_x, info_y, info_o = pack_layout(lx, row_len=K), pack_layout(ly), pack_layout(lo, row_len=C)
+    lists = build_contraction_lists(info_x.packed, info_y.packed, info_o.packed, B, R, K, C, info_o.count)
+    table = mm._row_work_table(lists.pair_offsets, info_o.row_offsets, R, parts_log2, pair_up=items == 2)
+    table = torch.cat([table.flip(0), torch.full((5,), -1, dtype=torch.int32, device=device)])
+    records = mm._row_records(table, parts_log2, lists.pair_offsets, info_x.row_offsets, info_o.row_offsets, B * R, C,
+                              info_x.count)
+    out = torch.full((info_o.count, sbs, sbs), float("nan"), dtype=torch.bfloat16, device=device)
+    _capi.call("bsa_matmul_rows", x.data_ptr(), y.data_ptr(), out.data_ptr(), lists.pair_offsets.data_ptr(),
+               _capi.ptr(lists.pairs), records.data_ptr(), records.size(0), items, info_o.count, x.size(0), y.size(0),
+               sbs, _capi.BF16, _capi.stream(device))
+    ref = torch.empty_like(out)
+    _capi.call("bsa_matmul", x.data_ptr(), y.data_ptr(), ref.data_ptr(), lists.pair_offsets.data_ptr(),
+               _capi.ptr(lists.pairs), 0, info_o.count, x.size(0), y.size(0), sbs, _capi.BF16, 0, 0,
+               _capi.stream(device))
+    assert torch.equal(out, ref)
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("trans", ["nn", "grads"])
 @pytest.mark.parametrize("dims,density", [
