@@ -15,7 +15,7 @@ from torch import Tensor
 from .. import _capi
 from ..utils.blksprs_tensor import BlksprsTensor
 from ..utils.tools import (build_contraction_lists, cast_for_autocast, eager_only, finalize_layout_cache,
-                           nonzero_from_packed, pack_layout, prepare_layout_cache)
+                           nonzero_from_packed, pack_layouts, prepare_layout_cache)
 from ..utils.validation import (ensure_contiguous, validate_contiguous, validate_device, validate_dimensions,
                                 validate_dtype_float, validate_shape, validate_sparsity, validate_sparsity_block_size,
                                 validate_sparsity_layout, validation_enabled)
@@ -48,13 +48,14 @@ def _launch_rows(x: Tensor, y: Tensor, plan: "_Plan", sbs: int) -> Tensor:
 _SUPER_TILE = 16
 
 
-def _block_order(layout_indices: Tensor) -> Tensor:
-    """Work order of the output blocks: 16 x 16 super-tiles of the block grid, columns of super-tiles
-    fastest, so that the blocks in flight on one L2 share x row panels and y column panels."""
+def _block_order(layout_indices: Tensor, n_rows: int, n_cols: int) -> Tensor:
+    """Work order of the output blocks of a layout with ``n_rows`` x ``n_cols`` blocks per batch entry: 16 x 16
+    super-tiles of the block grid, columns of super-tiles fastest, so that the blocks in flight on one L2 share
+    x row panels and y column panels."""
     b, i, j = layout_indices[:, 0], layout_indices[:, 1], layout_indices[:, 2]
     t = _SUPER_TILE
-    n_i = int(i.max().item()) // t + 1 if i.numel() else 1
-    n_j = int(j.max().item()) // t + 1 if j.numel() else 1
+    n_i = max(-(-n_rows // t), 1)
+    n_j = max(-(-n_cols // t), 1)
     key = ((b * n_i + i // t) * n_j + j // t) * (t * t) + (i % t) * t + (j % t)
     return torch.argsort(key, stable=True).to(torch.int32)
 
@@ -106,7 +107,7 @@ def _row_records(work_table: Tensor, parts_log2: int, pair_offsets: Tensor, row_
 
 
 def _row_work_table(pair_offsets: Tensor, row_offsets_o: Tensor, rows_per_batch: int, parts_log2: int,
-                    pair_up: bool = False) -> Tensor:
+                    pair_up: bool = False, max_work: int | None = None) -> Tensor:
     """Order in which the row kernel hands parts of output block rows to workgroups: int32 entries
     ``row << parts_log2 | part``, -1 for nothing.
 
@@ -118,6 +119,8 @@ def _row_work_table(pair_offsets: Tensor, row_offsets_o: Tensor, rows_per_batch:
     second shortest, ...: a workgroup that takes two consecutive entries of its XCD's list then has about the
     same work as every other one, the workgroups of an XCD start and end their rows of one batch entry together
     (they stream through the same y blocks at the same time), and a launch ends without a tail of short rows.
+    ``max_work`` is a bound on the pairs of one row that the caller knows without asking the device (inner
+    blocks times output columns); without it the largest count is read back, which waits for the stream.
     """
     n_rows = row_offsets_o.numel() - 1
     parts = 1 << parts_log2
@@ -127,13 +130,14 @@ def _row_work_table(pair_offsets: Tensor, row_offsets_o: Tensor, rows_per_batch:
     ends = pair_offsets[row_offsets_o.long()]
     work = (ends[1:] - ends[:-1]).long()
     small, extra = divmod(n_rows, _N_XCD)
-    sizes = torch.tensor([small + (c < extra) for c in range(_N_XCD)], device=device)
+    chunk_sizes = [small + (c < extra) for c in range(_N_XCD)]
+    sizes = torch.tensor(chunk_sizes, device=device)
     chunk_of_row = torch.repeat_interleave(torch.arange(_N_XCD, device=device), sizes)
     rows = torch.arange(n_rows, device=device).repeat_interleave(parts)
     part = torch.arange(parts, device=device).repeat(n_rows)
     entry = rows // max(rows_per_batch, 1)
     n_entries = n_rows // max(rows_per_batch, 1) + 1
-    heaviest = int(work.max())
+    heaviest = int(work.max()) if max_work is None else int(max_work)
     key = ((chunk_of_row[rows] * n_entries + entry) * parts + part) * (heaviest + 1) + (heaviest - work[rows])
     by_chunk = torch.argsort(key, stable=True)  # chunk-major, batch entry, part, work descending
     if pair_up:
@@ -150,7 +154,7 @@ def _row_work_table(pair_offsets: Tensor, row_offsets_o: Tensor, rows_per_batch:
     chunk = chunk_of_row[rows][by_chunk]
     counts = sizes * parts
     within = torch.arange(rows.numel(), device=device) - (torch.cumsum(counts, 0) - counts)[chunk]
-    table = torch.full((int(counts.max()) * _N_XCD,), -1, dtype=torch.int32, device=device)
+    table = torch.full((max(chunk_sizes) * parts * _N_XCD,), -1, dtype=torch.int32, device=device)
     table[within * _N_XCD + chunk] = ((rows[by_chunk] << parts_log2) | part[by_chunk]).to(torch.int32)
     return table
 
@@ -247,8 +251,8 @@ def matmul_build_layout_cache(layout_cache: dict | None, sparsity_layout_x: Tens
     if "contraction_pairs" not in layout_cache:
         B, R, K = (int(s) for s in sparsity_layout_x.shape)
         C = int(sparsity_layout_y.size(2))
-        info_x, info_y = pack_layout(sparsity_layout_x, row_len=K), pack_layout(sparsity_layout_y)
-        info_o = pack_layout(sparsity_layout_output, row_len=C)
+        info_x, info_y, info_o = pack_layouts((sparsity_layout_x, K), (sparsity_layout_y, 0),
+                                              (sparsity_layout_output, C))
         lists = build_contraction_lists(info_x.packed, info_y.packed, info_o.packed, B, R, K, C, info_o.count)
         layout_cache["packed_indices_x"] = info_x.packed
         layout_cache["packed_indices_y"] = info_y.packed
@@ -260,7 +264,7 @@ def matmul_build_layout_cache(layout_cache: dict | None, sparsity_layout_x: Tens
         layout_cache["n_sparse_blocks_y"] = info_y.count
         layout_cache["contraction_offsets"] = lists.pair_offsets
         layout_cache["contraction_pairs"] = lists.pairs
-        layout_cache["block_order"] = _block_order(layout_cache["layout_indices_o"])
+        layout_cache["block_order"] = _block_order(layout_cache["layout_indices_o"], R, C)
         layout_cache["row_offsets_x"] = info_x.row_offsets
         layout_cache["row_offsets_o"] = info_o.row_offsets
         layout_cache["row_records"] = None
@@ -273,7 +277,7 @@ def matmul_build_layout_cache(layout_cache: dict | None, sparsity_layout_x: Tens
                 # in speed by +-12 % on equal work, which the hardware's hand-out of many small items evens out
                 # and a static split does not.  Kept switchable for measurements.
                 pair_up = (B * R << parts_log2) >= 1024 and os.environ.get("BLKSPRS_AMD_ROW_PAIRS", "0") == "1"
-                table = _row_work_table(lists.pair_offsets, info_o.row_offsets, R, parts_log2, pair_up)
+                table = _row_work_table(lists.pair_offsets, info_o.row_offsets, R, parts_log2, pair_up, max_work=K * C)
                 layout_cache["row_parts_log2"], layout_cache["row_work_table"] = parts_log2, table
                 layout_cache["row_items_per_workgroup"] = 2 if pair_up else 1
                 layout_cache["row_records"] = _row_records(table, parts_log2, lists.pair_offsets,

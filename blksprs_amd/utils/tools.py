@@ -70,28 +70,40 @@ class PackedLayout:
         self.packed, self.count, self.row_offsets, self.max_per_row = packed, count, row_offsets, max_per_row
 
 
-def pack_layout(layout: Tensor, row_len: int = 0) -> PackedLayout:
-    """Scans a layout on the device: reverse index, block count and optional CSR row offsets.
+def pack_layouts(*specs) -> list:
+    """Scans several layouts on the device, ``specs`` being ``(layout, row_len)`` pairs: reverse index, block
+    count and optional CSR row offsets of each.
 
-    One stream synchronisation (the count sizes the caller's next allocation).
+    One stream synchronisation for all of them (the counts size the caller's next allocations).
     """
-    _require_device(layout)
-    lay = _layout_bytes(layout)
-    n = lay.numel()
-    dev = lay.device
-    packed = torch.empty(n, dtype=torch.int64, device=dev)
-    n_rows = n // row_len if row_len > 0 else 0
-    row_offsets = torch.empty(n_rows + 1, dtype=torch.int32, device=dev) if row_len > 0 else None
-    stats_dev = torch.empty(2, dtype=torch.int64, device=dev)
-    stats_host = torch.empty(2, dtype=torch.int64, pin_memory=True)
     lib = _capi.load()
-    ws_bytes = lib.bsa_lut_workspace_bytes(n)
-    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
-    with _capi.on_device(dev):
-        _capi.call("bsa_lut_packed", _capi.ptr(lay), n, row_len, _capi.ptr(packed),
-                   row_offsets.data_ptr() if row_offsets is not None else 0,
-                   stats_dev.data_ptr(), stats_host.data_ptr(), _capi.ptr(workspace), ws_bytes, _capi.stream(dev))
-    return PackedLayout(packed, int(stats_host[0]), row_offsets, int(stats_host[1]))
+    results = []
+    stats_dev = None
+    for number, (layout, row_len) in enumerate(specs):
+        _require_device(layout)
+        lay = _layout_bytes(layout)
+        n = lay.numel()
+        dev = lay.device
+        if stats_dev is None:
+            stats_dev = torch.empty((len(specs), 2), dtype=torch.int64, device=dev)
+        packed = torch.empty(n, dtype=torch.int64, device=dev)
+        n_rows = n // row_len if row_len > 0 else 0
+        row_offsets = torch.empty(n_rows + 1, dtype=torch.int32, device=dev) if row_len > 0 else None
+        ws_bytes = lib.bsa_lut_workspace_bytes(n)
+        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        with _capi.on_device(dev):
+            _capi.call("bsa_lut_packed", _capi.ptr(lay), n, row_len, _capi.ptr(packed),
+                       row_offsets.data_ptr() if row_offsets is not None else 0,
+                       stats_dev[number].data_ptr(), 0, _capi.ptr(workspace), ws_bytes, _capi.stream(dev))
+        results.append((packed, row_offsets))
+    stats = stats_dev.tolist() if results else []
+    return [PackedLayout(packed, int(count), row_offsets, int(longest))
+            for (packed, row_offsets), (count, longest) in zip(results, stats)]
+
+
+def pack_layout(layout: Tensor, row_len: int = 0) -> PackedLayout:
+    """``pack_layouts`` for one layout."""
+    return pack_layouts((layout, row_len))[0]
 
 
 def build_packed_indices(sparsity_layout: Tensor) -> Tensor:

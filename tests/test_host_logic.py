@@ -183,6 +183,9 @@ def test_row_work_table_holds_every_part_once_and_keeps_eighths_together():
         pair_offsets = torch.cumsum(torch.randint(0, 6, (n_rows * blocks_per_row + 1,), generator=g), 0).to(torch.int32)
         work = (pair_offsets[row_offsets.long()][1:] - pair_offsets[row_offsets.long()][:-1]).tolist()
         table = mm._row_work_table(pair_offsets, row_offsets, rows_per_batch, parts_log2)
+        # a bound on a row's pairs that the caller knows in advance gives the same table as the measured maximum
+        assert torch.equal(table, mm._row_work_table(pair_offsets, row_offsets, rows_per_batch, parts_log2,
+                                                     max_work=5 * blocks_per_row + 100))
         parts = 1 << parts_log2
         assert table.dtype == torch.int32 and table.numel() % 8 == 0
         live = table[table >= 0].long()
