@@ -46,7 +46,7 @@ PEAK_MFMA_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}
 # what leaves an L2, so reads served by the memory-side cache are included.  Not re-measured by this script.
 TRAFFIC_KIB = {  # config: (FETCH_SIZE, WRITE_SIZE)
     "c1": (616.2, 476.0),
-    "c2": (376348.9, 514961.6),
+    "c2": (337914.7, 514960.1),
     "c3": (148153.3, 296259.0),
     "c4": (238469.4, 133139.0),
     "c5": (28438.4, 143960.0),

@@ -226,7 +226,8 @@ struct RowsRecord {
   uint32_t empty_blocks[2];   // mask of the part's blocks that have no pair (they are written as zeros)
   int32_t pairs_end;          // end of the pair list of the part's last block
   uint32_t wave_blocks[kWaves][2];  // low and high word of wave w's mask
-  int32_t pad[40];
+  int32_t downward;           // the waves take their blocks from the highest column down
+  int32_t pad[39];
   int32_t pairs_begin[64];    // start of the pair list of block o_first + i (it ends where the next one starts)
 };
 static_assert(sizeof(RowsRecord) == BSA_ROWS_RECORD_INTS * 4, "record layout");
@@ -246,6 +247,8 @@ __global__ __launch_bounds__(256) void rows_records_kernel(const int32_t *__rest
   int32_t *out = reinterpret_cast<int32_t *>(records + at);
   int item = work_table ? work_table[at] : (int)at;
   item = __builtin_amdgcn_readfirstlane(item);
+  const int downward = item >= 0 ? (item >> 30) & 1 : 0;
+  if (item >= 0) item &= ~BSA_ROWS_DOWNWARD;
   const int part = item & ((1 << parts_log2) - 1);
   const int row = item < 0 ? -1 : item >> parts_log2;
   int value = 0, offset = 0;  // lane l writes ints l and 64 + l of the record
@@ -297,6 +300,7 @@ __global__ __launch_bounds__(256) void rows_records_kernel(const int32_t *__rest
     else if (lane == 5) value = (int)(uint32_t)empty;
     else if (lane == 6) value = (int)(uint32_t)(empty >> 32);
     else if (lane == 7) value = pairs_end;
+    else if (lane == 24) value = downward;
 #pragma unroll
     for (int w = 0; w < kWaves; ++w) {
       if (lane == 8 + 2 * w) value = (int)(uint32_t)blocks[w];
@@ -370,7 +374,7 @@ __device__ __forceinline__ void rows_part(const char *__restrict__ x, const char
   }
 
   // The walk over this wave's pairs is scalar work without a branch: `todo` holds the wave's blocks from the
-  // one being walked on (its lowest set bit), [w_p, w_pe) are that block's pairs from the one handed out last.
+  // one being walked on (its lowest set bit, or its highest when the part is walked downward), [w_p, w_pe) are that block's pairs from the one handed out last.
   // step() moves to the next pair and requests its list entry; entry_to_item() turns the entry into addresses.
   // In the loop the two are called a whole pair of matrix products apart.  The entry is requested by a vector
   // load (every lane the same 8 bytes) from inline assembly and waited for with vmcnt like the y blocks: a
@@ -383,8 +387,12 @@ __device__ __forceinline__ void rows_part(const char *__restrict__ x, const char
     const int next = __builtin_amdgcn_readlane(offs, (b + 1) & 63);
     pe = b + 1 < o_count ? next : pairs_end;
   };
+  // A wave takes its blocks in ascending order of the column, or (downward) in descending order; the pairs of a
+  // block are always walked in ascending order of k.
+  const bool downward = __builtin_amdgcn_readlane(mine, 24) != 0;
+  auto next_block = [&](uint64_t blocks) { return downward ? 63 - __builtin_clzll(blocks) : __builtin_ctzll(blocks); };
   int w_p = 0, w_pe = 0;
-  if (todo) range_of(__builtin_ctzll(todo), w_p, w_pe);
+  if (todo) range_of(next_block(todo), w_p, w_pe);
   w_p -= 1;  // nothing handed out yet
   // what a step leaves for entry_to_item(): the entry (requested) and the facts known without it
   u32x2 raw_entry = {0, 0};
@@ -395,8 +403,9 @@ __device__ __forceinline__ void rows_part(const char *__restrict__ x, const char
   auto advance = [&]() -> const int32_t * {  // returns where the next pair's entry lies
     const int p1 = w_p + 1;
     const bool block_done = p1 >= w_pe && todo != 0;
-    const uint64_t rest = block_done ? todo & (todo - 1) : todo;
-    const int b = rest ? __builtin_ctzll(rest) : 0;
+    const uint64_t without = downward ? todo & ~(1ull << (63 - __builtin_clzll(todo | 1))) : todo & (todo - 1);
+    const uint64_t rest = block_done ? without : todo;
+    const int b = rest ? next_block(rest) : 0;
     int bp, bpe;
     range_of(b, bp, bpe);
     w_p = block_done ? bp : p1;
@@ -624,7 +633,7 @@ extern "C" int bsa_matmul_rows_records(const int32_t *work_table, int64_t n_item
                                        int64_t nnz_x, int32_t *records, bsa_stream_t stream) {
   const char *who = "bsa_matmul_rows_records";
   BSA_REQUIRE(parts_log2 >= 0 && parts_log2 <= 3, "%s: parts_log2 must be 0..3 (got %d)", who, parts_log2);
-  BSA_REQUIRE(n_rows >= 0 && (n_rows << parts_log2) < 0x7fffffffLL, "%s: bad number of block rows", who);
+  BSA_REQUIRE(n_rows >= 0 && (n_rows << parts_log2) < (int64_t)BSA_ROWS_DOWNWARD, "%s: bad number of block rows", who);
   BSA_REQUIRE(n_items >= 0 && n_items < 0x7fffffffLL, "%s: bad number of table entries", who);
   BSA_REQUIRE(nnz_x >= 0, "%s: negative size", who);
   BSA_REQUIRE(n_cols >= 0 && ((n_cols + (1 << parts_log2) - 1) >> parts_log2) <= 64,

@@ -106,8 +106,12 @@ def _row_records(work_table: Tensor, parts_log2: int, pair_offsets: Tensor, row_
     return records
 
 
+_ROWS_DOWNWARD = 1 << 30  # BSA_ROWS_DOWNWARD
+_CUS_PER_XCD = 32
+
+
 def _row_work_table(pair_offsets: Tensor, row_offsets_o: Tensor, rows_per_batch: int, parts_log2: int,
-                    pair_up: bool = False, max_work: int | None = None) -> Tensor:
+                    pair_up: bool = False, max_work: int | None = None, sweep: int = 0) -> Tensor:
     """Order in which the row kernel hands parts of output block rows to workgroups: int32 entries
     ``row << parts_log2 | part``, -1 for nothing.
 
@@ -119,6 +123,10 @@ def _row_work_table(pair_offsets: Tensor, row_offsets_o: Tensor, rows_per_batch:
     second shortest, ...: a workgroup that takes two consecutive entries of its XCD's list then has about the
     same work as every other one, the workgroups of an XCD start and end their rows of one batch entry together
     (they stream through the same y blocks at the same time), and a launch ends without a tail of short rows.
+    With ``sweep`` > 0 the items of one (XCD, batch entry, part) group alternate their direction every ``sweep``
+    items: the first ``sweep`` walk their columns upward, the next ``sweep`` (which start as those end, on the
+    same compute units) downward, and so on: a part that starts finds the y blocks its predecessors read last
+    still in the L2.
     ``max_work`` is a bound on the pairs of one row that the caller knows without asking the device (inner
     blocks times output columns); without it the largest count is read back, which waits for the stream.
     """
@@ -155,7 +163,13 @@ def _row_work_table(pair_offsets: Tensor, row_offsets_o: Tensor, rows_per_batch:
     counts = sizes * parts
     within = torch.arange(rows.numel(), device=device) - (torch.cumsum(counts, 0) - counts)[chunk]
     table = torch.full((max(chunk_sizes) * parts * _N_XCD,), -1, dtype=torch.int32, device=device)
-    table[within * _N_XCD + chunk] = ((rows[by_chunk] << parts_log2) | part[by_chunk]).to(torch.int32)
+    items = (rows[by_chunk] << parts_log2) | part[by_chunk]
+    if sweep > 0:
+        group_key = (key // (heaviest + 1))[by_chunk]
+        _, inverse, sizes_g = torch.unique_consecutive(group_key, return_inverse=True, return_counts=True)
+        rank = torch.arange(rows.numel(), device=device) - (torch.cumsum(sizes_g, 0) - sizes_g)[inverse]
+        items = items | (((rank // sweep) & 1) * _ROWS_DOWNWARD)
+    table[within * _N_XCD + chunk] = items.to(torch.int32)
     return table
 
 
@@ -277,7 +291,9 @@ def matmul_build_layout_cache(layout_cache: dict | None, sparsity_layout_x: Tens
                 # in speed by +-12 % on equal work, which the hardware's hand-out of many small items evens out
                 # and a static split does not.  Kept switchable for measurements.
                 pair_up = (B * R << parts_log2) >= 1024 and os.environ.get("BLKSPRS_AMD_ROW_PAIRS", "0") == "1"
-                table = _row_work_table(lists.pair_offsets, info_o.row_offsets, R, parts_log2, pair_up, max_work=K * C)
+                sweep = int(os.environ.get("BLKSPRS_AMD_ROW_SWEEP", _CUS_PER_XCD))  # 0: every part upward
+                table = _row_work_table(lists.pair_offsets, info_o.row_offsets, R, parts_log2, pair_up,
+                                        max_work=K * C, sweep=0 if pair_up else sweep)
                 layout_cache["row_parts_log2"], layout_cache["row_work_table"] = parts_log2, table
                 layout_cache["row_items_per_workgroup"] = 2 if pair_up else 1
                 layout_cache["row_records"] = _row_records(table, parts_log2, lists.pair_offsets,

@@ -225,6 +225,7 @@ int bsa_matmul(const void *x, const void *y, void *out, const int32_t *pair_offs
                int trans_x, int trans_y, bsa_stream_t stream);
 
 #define BSA_ROWS_RECORD_INTS 128
+#define BSA_ROWS_DOWNWARD (1 << 30)
 
 /*
  * Layout-to-LUT step of bsa_matmul_rows (integer only): one record of BSA_ROWS_RECORD_INTS int32 per work
@@ -234,7 +235,10 @@ int bsa_matmul(const void *x, const void *y, void *out, const int32_t *pair_offs
  * row: the row's output blocks are cut into 2^parts_log2 runs of equal length (parts_log2 0..3; more parts keep
  * fewer y blocks in flight at the price of loading the x row once per part); a part holds at most 64 blocks, so
  * n_cols <= 64 << parts_log2 (BSA_EINVAL otherwise).  work_table (n_items int32) is the order in which parts
- * are handed to workgroups: entry row << parts_log2 | part, or -1 for nothing; every (row, part) once.  NULL
+ * are handed to workgroups: entry row << parts_log2 | part, or -1 for nothing; every (row, part) once; with
+ * BSA_ROWS_DOWNWARD or'ed in, the part's blocks are computed from the highest column down (same results: the
+ * order of the products inside a block does not change), so that a part that starts when its neighbours on the
+ * XCD end finds the y blocks of the high columns still in the L2.  NULL
  * (with parts_log2 == 0 and n_items == n_rows): rows 0, 1, 2, ...  Workgroup g runs on XCD g % 8, so a table
  * that gives position 8 k + c to the k-th item of a contiguous eighth c of the rows, heaviest rows first, keeps
  * the y blocks in flight on one L2 few and the tail of the launch short.  A record holds the row (-1: nothing),

@@ -186,6 +186,19 @@ def test_row_work_table_holds_every_part_once_and_keeps_eighths_together():
         # a bound on a row's pairs that the caller knows in advance gives the same table as the measured maximum
         assert torch.equal(table, mm._row_work_table(pair_offsets, row_offsets, rows_per_batch, parts_log2,
                                                      max_work=5 * blocks_per_row + 100))
+        # with a sweep every second run of `sweep` items of a (XCD, batch entry, part) group carries the downward flag
+        swept = mm._row_work_table(pair_offsets, row_offsets, rows_per_batch, parts_log2, sweep=3)
+        assert torch.equal(torch.where(swept >= 0, swept & ~mm._ROWS_DOWNWARD, swept), table)
+        for c in range(8):
+            run, last_group = 0, None
+            for e in swept[c::8].tolist():
+                if e < 0:
+                    continue
+                plain = e & ~mm._ROWS_DOWNWARD
+                group = ((plain >> parts_log2) // rows_per_batch, plain & ((1 << parts_log2) - 1))
+                run = run + 1 if group == last_group else 0
+                last_group = group
+                assert bool(e & mm._ROWS_DOWNWARD) == bool((run // 3) & 1)
         parts = 1 << parts_log2
         assert table.dtype == torch.int32 and table.numel() % 8 == 0
         live = table[table >= 0].long()

@@ -239,7 +239,9 @@ def test_row_kernel_parts_and_records_per_workgroup(device, parts_log2, items):
     """The row kernel through the C ABI with rows cut into 1, 2, 4 and 8 column parts and with one, two and
     three records per workgroup (a workgroup then works through consecutive entries of its XCD's list, the
     last workgroups through fewer): the same bits as the tile kernel.  120 block columns: parts of up to 64
-    blocks (one mask bit each) and of 15; a work table in reversed order with empty entries."""
+    blocks (one mask bit each) and of 15; a work table in reversed order with empty entries.  Every second item
+    of a group walks its columns downward (the flag in the table entry), which changes the order of the blocks
+    and not the bits."""
     import importlib
     from blksprs_amd import _capi
     from blksprs_amd.utils.tools import build_contraction_lists, pack_layout
@@ -255,7 +257,9 @@ def test_row_kernel_parts_and_records_per_workgroup(device, parts_log2, items):
     y = rand_blocks(int(ly.sum()), sbs, torch.bfloat16, 5).to(device)
     info_x, info_y, info_o = pack_layout(lx, row_len=K), pack_layout(ly), pack_layout(lo, row_len=C)
     lists = build_contraction_lists(info_x.packed, info_y.packed, info_o.packed, B, R, K, C, info_o.count)
-    table = mm._row_work_table(lists.pair_offsets, info_o.row_offsets, R, parts_log2, pair_up=items == 2)
+    table = mm._row_work_table(lists.pair_offsets, info_o.row_offsets, R, parts_log2, pair_up=items == 2,
+                               sweep=0 if items == 2 else 1)
+    assert items == 2 or int((table >= mm._ROWS_DOWNWARD).sum()) > 0
     table = torch.cat([table.flip(0), torch.full((5,), -1, dtype=torch.int32, device=device)])
     records = mm._row_records(table, parts_log2, lists.pair_offsets, info_x.row_offsets, info_o.row_offsets, B * R, C,
                               info_x.count)
