@@ -191,9 +191,11 @@ def time_steps_flushed(step, steps, scratch):
 
 
 def count_host_syncs(fn):
-    """Runs ``fn`` and returns (milliseconds, number of calls that made the host wait for the device, as torch's
-    sync debug mode reports them)."""
+    """Runs ``fn`` and returns (milliseconds, number of calls that made the host wait for the device: those torch's
+    sync debug mode reports plus the library calls that wait for the stream themselves)."""
     import warnings
+    from blksprs_amd import _capi
+    inside_library = _capi.host_waits
     torch.cuda.synchronize()
     torch.cuda.set_sync_debug_mode("warn")
     try:
@@ -206,7 +208,7 @@ def count_host_syncs(fn):
             ms = (time.perf_counter() - t0) * 1e3
     finally:
         torch.cuda.set_sync_debug_mode("default")
-    return ms, sum("synchroniz" in str(w.message).lower() for w in seen)
+    return ms, sum("synchroniz" in str(w.message).lower() for w in seen) + _capi.host_waits - inside_library
 
 
 # --------------------------------------------------------------------------- workloads

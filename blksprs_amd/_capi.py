@@ -128,7 +128,16 @@ def stream(device) -> int:
     return torch._C._cuda_getCurrentRawStream(torch.cuda.current_device() if index is None else index)
 
 
+# entry points that wait for the stream when their `stats_host` argument (at the given position) is not NULL
+_WAITS_WITH_STATS_HOST = {"bsa_lut_packed": 6, "bsa_lut_contraction_offsets": 11}
+host_waits = 0  # calls so far that made the host wait for the device inside the library
+
+
 def call(name: str, *args) -> None:
+    global host_waits
+    at = _WAITS_WITH_STATS_HOST.get(name)
+    if at is not None and args[at]:
+        host_waits += 1
     check(getattr(load(), name)(*args), name)
 
 

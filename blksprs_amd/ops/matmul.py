@@ -138,36 +138,39 @@ def _row_work_table(pair_offsets: Tensor, row_offsets_o: Tensor, rows_per_batch:
     ends = pair_offsets[row_offsets_o.long()]
     work = (ends[1:] - ends[:-1]).long()
     small, extra = divmod(n_rows, _N_XCD)
-    chunk_sizes = [small + (c < extra) for c in range(_N_XCD)]
-    sizes = torch.tensor(chunk_sizes, device=device)
-    chunk_of_row = torch.repeat_interleave(torch.arange(_N_XCD, device=device), sizes)
-    rows = torch.arange(n_rows, device=device).repeat_interleave(parts)
+    # chunk c holds small + 1 rows for c < extra and small rows after that: plain arithmetic, nothing is copied
+    # to the device
+    all_rows = torch.arange(n_rows, device=device)
+    long_rows = extra * (small + 1)
+    chunk_of_row = torch.where(all_rows < long_rows, all_rows // (small + 1),
+                               extra + (all_rows - long_rows) // max(small, 1))
+    rows = all_rows.repeat_interleave(parts)
     part = torch.arange(parts, device=device).repeat(n_rows)
     entry = rows // max(rows_per_batch, 1)
     n_entries = n_rows // max(rows_per_batch, 1) + 1
     heaviest = int(work.max()) if max_work is None else int(max_work)
     key = ((chunk_of_row[rows] * n_entries + entry) * parts + part) * (heaviest + 1) + (heaviest - work[rows])
     by_chunk = torch.argsort(key, stable=True)  # chunk-major, batch entry, part, work descending
+    # position of every item inside its (chunk, batch entry, part) group, and the group's size (the number of
+    # groups is known here, so nothing is read back)
+    group = (key // (heaviest + 1))[by_chunk]
+    sizes_g = torch.zeros(_N_XCD * n_entries * parts, dtype=torch.int64, device=device)
+    sizes_g.scatter_add_(0, group, torch.ones_like(group))
+    starts = torch.cumsum(sizes_g, 0) - sizes_g
+    rank = torch.arange(rows.numel(), device=device) - starts[group]
     if pair_up:
-        # within a (chunk, batch entry, part) group: longest, shortest, second longest, second shortest, ...
-        group_key = (key // (heaviest + 1))[by_chunk]
-        _, inverse, sizes_g = torch.unique_consecutive(group_key, return_inverse=True, return_counts=True)
-        starts = torch.cumsum(sizes_g, 0) - sizes_g
-        rank = torch.arange(rows.numel(), device=device) - starts[inverse]
-        m = sizes_g[inverse]
+        # within a group: longest, shortest, second longest, second shortest, ...
+        m = sizes_g[group]
         spot = torch.where(rank < (m + 1) // 2, 2 * rank, 2 * (m - 1 - rank) + 1)
         reordered = torch.empty_like(by_chunk)
-        reordered[starts[inverse] + spot] = by_chunk
+        reordered[starts[group] + spot] = by_chunk
         by_chunk = reordered
     chunk = chunk_of_row[rows][by_chunk]
-    counts = sizes * parts
-    within = torch.arange(rows.numel(), device=device) - (torch.cumsum(counts, 0) - counts)[chunk]
-    table = torch.full((max(chunk_sizes) * parts * _N_XCD,), -1, dtype=torch.int32, device=device)
+    first_of_chunk = (chunk * small + torch.clamp(chunk, max=extra)) * parts
+    within = torch.arange(rows.numel(), device=device) - first_of_chunk
+    table = torch.full(((small + (extra > 0)) * parts * _N_XCD,), -1, dtype=torch.int32, device=device)
     items = (rows[by_chunk] << parts_log2) | part[by_chunk]
     if sweep > 0:
-        group_key = (key // (heaviest + 1))[by_chunk]
-        _, inverse, sizes_g = torch.unique_consecutive(group_key, return_inverse=True, return_counts=True)
-        rank = torch.arange(rows.numel(), device=device) - (torch.cumsum(sizes_g, 0) - sizes_g)[inverse]
         items = items | (((rank // sweep) & 1) * _ROWS_DOWNWARD)
     table[within * _N_XCD + chunk] = items.to(torch.int32)
     return table
@@ -358,5 +361,11 @@ def matmul(x: BlksprsTensor, sparsity_layout_x: Tensor,
     if not (torch.is_grad_enabled() and (x.requires_grad or y.requires_grad)):
         # nothing to differentiate: the launch itself, without the autograd machinery around it
         return BlksprsTensor.wrap(_forward(x, y, layout_cache["plan"], sparsity_block_size))
-    return BlksprsTensor.wrap(_Matmul.apply(x, y, layout_cache, tuple(sparsity_layout_x.shape),
-                                            tuple(sparsity_layout_y.shape), sparsity_block_size))
+    shape_x, shape_y = tuple(sparsity_layout_x.shape), tuple(sparsity_layout_y.shape)
+    plan = layout_cache["plan"]
+    if plan.grad_lists is None:
+        # the lists of the two backward products are built with the first forward pass that will need them, so
+        # that no backward pass waits for the device
+        _backward_lists(plan, shape_x, shape_y)
+        _publish_backward_lists(layout_cache, plan)
+    return BlksprsTensor.wrap(_Matmul.apply(x, y, layout_cache, shape_x, shape_y, sparsity_block_size))
