@@ -820,6 +820,36 @@ def measure(config, dev, steps, warmup, scratch):
     return w, {"wall_ms": t["wall_ms"], "roofline": roofline, "correct": correct}
 
 
+def measured_ceilings(dev):
+    """What plain library kernels reach on this card, next to the published peaks the roofline fractions use: a
+    dense bf16 and fp32 GEMM of 8192^3 through torch (hipBLASLt / rocBLAS) and a device-to-device copy of 2 GiB."""
+    def timed(fn, reps):
+        for _ in range(3):
+            fn()
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+        for s, e in ev:
+            s.record()
+            fn()
+            e.record()
+        torch.cuda.synchronize()
+        return sorted(s.elapsed_time(e) for s, e in ev)[reps // 2]
+
+    out = {}
+    n = 8192
+    for name, dtype in (("dense_gemm_bf16_tflops", torch.bfloat16), ("dense_gemm_fp32_tflops", torch.float32)):
+        a = torch.randn((n, n), device=dev, dtype=dtype)
+        b = torch.randn((n, n), device=dev, dtype=dtype)
+        c = torch.empty((n, n), device=dev, dtype=dtype)
+        ms = timed(lambda: torch.matmul(a, b, out=c), 10)
+        out[name] = round(2.0 * n ** 3 / (ms * 1e-3) / 1e12, 1)
+        del a, b, c
+    src = torch.empty(2 << 30, dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    ms = timed(lambda: dst.copy_(src), 10)
+    out["copy_2gib_read_plus_write_gbs"] = round(2.0 * src.numel() / (ms * 1e-3) / 1e9, 1)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -870,6 +900,9 @@ def main():
             others[name] = entry
             del wo
         line["other_configs"] = others
+        del scratch
+        torch.cuda.empty_cache()
+        line["measured_ceilings"] = measured_ceilings(dev)
     print(json.dumps(line), flush=True)
 
 
