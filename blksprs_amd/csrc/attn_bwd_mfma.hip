@@ -43,6 +43,8 @@ constexpr bool kSplitKeyPass = false;
 // dK and dV by two teams of four waves in one workgroup of eight (the default); the two switches above
 // choose among the four-wave kernels otherwise
 constexpr bool kEightWaves = true;
+// the eight-wave kernel by workgroups that stay for the whole launch and walk key block after key block
+constexpr bool kKvWalk = true;
 
 // One 64 x 64 16-bit block, global -> LDS, by the NW (4 or 8) waves of a workgroup: wave w copies rows
 // (64 / NW) w .. with asynchronous 1 KiB copies (eight rows each); lane l supplies the chunk that belongs at
@@ -97,6 +99,13 @@ __device__ __forceinline__ void staged_products(Load load, Multiply multiply) {
   }
 }
 
+// workgroups per XCD of the dK / dV kernel whose workgroups stay for the whole launch: one per compute unit
+constexpr int kCusPerXcd = 32;
+__host__ __device__ inline int64_t kv_slots(int64_t key_rows) {
+  const int64_t chunk = (key_rows + 7) / 8;
+  return chunk < kCusPerXcd ? chunk : kCusPerXcd;
+}
+
 // XCD-aware row of a workgroup: every XCD gets a contiguous range of rows, so that the blocks in flight on one
 // L2 belong to the same batch entries
 __device__ inline int64_t xcd_row() { return (int64_t)(blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3); }
@@ -104,21 +113,27 @@ __device__ inline int64_t xcd_row() { return (int64_t)(blockIdx.x & 7) * (gridDi
 // sum of the accumulators of wave pairs (w, w ^ partner_bit): the wave with the bit set writes, the other adds
 template <int N>
 __device__ inline void reduce_partner(f32x16 (&acc)[N], float *lds, bool writer, int slot, int lane) {
-  // slot: which pair of waves (0 or 1); layout [slot][n][r][lane]
-  float *base = lds + (size_t)slot * N * 16 * 64 + lane;
+  // slot: which pair of waves (0 or 1); layout [slot][n][r / 4][lane][r % 4]: 128-bit accesses, a wave's lanes side
+  // by side
+  f32x4 *base = reinterpret_cast<f32x4 *>(lds + (size_t)slot * N * 16 * 64) + lane;
   __syncthreads();  // the tile buffers are free
   if (writer) {
 #pragma unroll
     for (int n = 0; n < N; ++n)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) base[(n * 16 + r) * 64] = acc[n][r];
+      for (int q = 0; q < 4; ++q)
+        base[(n * 4 + q) * 64] = f32x4{acc[n][4 * q], acc[n][4 * q + 1], acc[n][4 * q + 2], acc[n][4 * q + 3]};
   }
   __syncthreads();
   if (!writer) {
 #pragma unroll
     for (int n = 0; n < N; ++n)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[n][r] += base[(n * 16 + r) * 64];
+      for (int q = 0; q < 4; ++q) {
+        const f32x4 v = base[(n * 4 + q) * 64];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) acc[n][4 * q + t] += v[t];
+      }
   }
 }
 
@@ -148,6 +163,7 @@ struct BwdLists {
   // query row, K and V for a key row; -1: none).  Everything a workgroup has to know before its first tile
   // comes with one load.
   int32_t *q_head, *k_head;
+  int32_t *kv_tickets;             // [16]: per XCD, the next position of its eighth of the key rows to hand out
   uint8_t *mask_dead;              // [n_mask_blocks]
 };
 
@@ -159,7 +175,8 @@ __host__ __device__ inline BwdLists bwd_lists(const bsa_attn_args &a) {
   L.query_end = L.key_end + a.B * a.nq;
   L.q_head = L.query_end + a.B * a.nk;
   L.k_head = L.q_head + 16 * a.B * a.nq;
-  L.mask_dead = reinterpret_cast<uint8_t *>(L.k_head + 16 * a.B * a.nk);
+  L.kv_tickets = L.k_head + 16 * a.B * a.nk;
+  L.mask_dead = reinterpret_cast<uint8_t *>(L.kv_tickets + 16);
   return L;
 }
 
@@ -311,6 +328,9 @@ template <typename Tr>
 __global__ __launch_bounds__(kBwdThreads) void attn_bwd_delta_kernel(bsa_attn_args a) {
   const int64_t row = blockIdx.x;  // b * nq + qb
   const int tid = threadIdx.x;
+  // the dK / dV kernel that follows hands out key rows by tickets: the workgroups of an XCD start with the
+  // positions 0 .. slots - 1 of its eighth, the next one to hand out is `slots`
+  if (row == 0 && tid < 8) bwd_lists(a).kv_tickets[tid] = (int32_t)kv_slots(a.B * a.nk);
   const int i = tid >> 2, part = tid & 3;
   float acc = 0.f;
   for (int64_t h = 0; h < a.nhv; ++h) {
@@ -332,6 +352,132 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_delta_kernel(bsa_attn_ar
   acc += __shfl_xor(acc, 1);
   acc += __shfl_xor(acc, 2);
   if (part == 0) a.delta[row * kSbs + i] = acc;
+}
+
+// The work of one wave on one tile (a query block in LDS at `base`, this wave's quadrant of the 64 x 64 scores):
+// S and dP, P and dS, then dV^T += dO^T P and / or dK^T += Q^T dS.  mbits: the mask bytes of this lane's 16
+// scores, one bit each (0 when the tile has no mask block).
+template <typename Tr, int NH, int NHV, bool DK, bool DV>
+__device__ __forceinline__ void kv_tile(const bsa_attn_args &a, const char *base, const int qb, const int64_t pm,
+                                        const int64_t pb, const uint32_t mbits, const bool causal, const int seq_len,
+                                        const int kb, const int kpos, const float qk_scale, const int wi, const int wj,
+                                        const int li, const int kg, const int lane, const u32x4 (&kfr)[NH][4],
+                                        const u32x4 (&vfr)[NHV][4], f32x16 (&dkacc)[DK ? NH * 2 : 1],
+                                        f32x16 (&dvacc)[DV ? NHV * 2 : 1]) {
+  constexpr int kQRows = 0, kDoRows = NH * kBlockBytes, kStats = (NH + NHV) * kBlockBytes;
+  // A quadrant whose every score is masked has P = dS = 0: nothing to add, nothing to compute.
+  bool live = true;
+  if (pm >= 0) live = !__all(mbits == 0xffffu);
+  if (causal) {
+    const int k_first = (int)kb * kSbs + 32 * wj, q_first = qb * kSbs + 32 * wi;
+    if (k_first > q_first + 31 || q_first >= seq_len || k_first >= seq_len) live = false;
+  }
+  if (live) {
+    // ---- S and dP of this wave's quadrant ----
+    f32x16 sacc, dpacc;
+  #pragma unroll
+    for (int r = 0; r < 16; ++r) sacc[r] = dpacc[r] = 0.f;
+    staged_products<NH + (DK ? NHV : 0)>(
+        [&](int k, u32x4(&f)[4]) {
+          const char *src = base + (k < NH ? kQRows + k * kBlockBytes : kDoRows + (k - NH) * kBlockBytes);
+  #pragma unroll
+          for (int s = 0; s < 4; ++s) f[s] = frag_rows(src, 32 * wi + li, 2 * s + kg);
+        },
+        [&](int k, u32x4(&f)[4]) {
+  #pragma unroll
+          for (int s = 0; s < 4; ++s) {
+            if (k < NH) sacc = Tr::mfma(f[s], kfr[k < NH ? k : 0][s], sacc);
+            else dpacc = Tr::mfma(f[s], vfr[k < NH ? 0 : k - NH][s], dpacc);
+          }
+        });
+
+    // ---- P and dS; element r: query 32 wi + 8 (r / 4) + 4 kg + r % 4 ----
+    const float *stats = reinterpret_cast<const float *>(base + kStats);
+    // the bias elements are read where they are used: a bias is rare, its registers are not
+    uint32_t bias_c[16];
+    if (pb >= 0) {
+      const uint16_t *bp = static_cast<const uint16_t *>(a.bias) + pb * (kSbs * kSbs) +
+                           (32 * wi + 4 * kg) * kSbs + 32 * wj + li;
+  #pragma unroll
+      for (int r = 0; r < 16; ++r) bias_c[r] = bp[(8 * (r >> 2) + (r & 3)) * kSbs];
+    }
+    float p[16], ds[16];
+    // Most tiles have no bias, no mask block and lie where the causal predicate holds for every score: they
+    // take the plain path.  The conditions are the same for the whole wave.
+    auto probabilities = [&](auto plain_tag) {
+      constexpr bool kPlain = decltype(plain_tag)::value;
+  #pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int i0 = 32 * wi + 8 * q + 4 * kg;
+        const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(stats + i0);
+        const f32x4 del4 = *reinterpret_cast<const f32x4 *>(stats + kSbs + i0);
+  #pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const int r = 4 * q + t;
+          float s = sacc[r] * qk_scale;
+          if constexpr (!kPlain) {
+            if (pb >= 0) s = s + Tr::widen((uint16_t)bias_c[r]) * kLog2e;
+            if (causal) {
+              const int qpos = qb * kSbs + i0 + t;
+              s = (kpos > qpos || qpos >= seq_len || kpos >= seq_len) ? -INFINITY : s;
+            }
+            if (pm >= 0) s = ((mbits >> r) & 1u) ? -INFINITY : s;
+          }
+          p[r] = __builtin_amdgcn_exp2f(s - lse4[t]);
+          ds[r] = p[r] * (dpacc[r] - del4[t]);
+        }
+      }
+    };
+    bool plain = pb < 0 && pm < 0;
+    if (causal) {
+      // every key of the quadrant at or before every query of it, and all of them inside the sequence
+      const int k_last = (int)kb * kSbs + 32 * wj + 31, q_first = qb * kSbs + 32 * wi;
+      plain = plain && k_last <= q_first && q_first + 31 < seq_len;
+    }
+    if (plain) probabilities(std::true_type{});
+    else probabilities(std::false_type{});
+    if (DK && a.dbias != nullptr && pb >= 0) {
+      // every (query block, key block) pair is visited once, so this is a plain store
+      float *dbp = a.dbias + pb * (kSbs * kSbs) + (32 * wi + 4 * kg) * kSbs + 32 * wj + li;
+  #pragma unroll
+      for (int r = 0; r < 16; ++r) dbp[(8 * (r >> 2) + (r & 3)) * kSbs] = ds[r];
+    }
+    u32x4 pf[2], dsf[2];
+  #pragma unroll
+    for (int u = 0; u < 2; ++u)
+  #pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        pf[u][t] = Tr::pack2(p[8 * u + 2 * t], p[8 * u + 2 * t + 1]);
+        dsf[u][t] = Tr::pack2(ds[8 * u + 2 * t], ds[8 * u + 2 * t + 1]);
+      }
+
+    // ---- dV^T += dO^T P, dK^T += Q^T dS over this wave's 32 queries ----
+    const int col_t = 16 * ((lane >> 4) & 1);
+    if constexpr (DV) {
+      staged_products<NHV>(
+          [&](int h, u32x4(&f)[4]) {
+  #pragma unroll
+            for (int i = 0; i < 4; ++i)
+              f[i] = frag_cols_t(base + kDoRows + h * kBlockBytes, 32 * wi + 16 * (i & 1) + 4 * kg, 32 * (i >> 1) + col_t, lane);
+          },
+          [&](int h, u32x4(&f)[4]) {
+  #pragma unroll
+            for (int i = 0; i < 4; ++i) dvacc[2 * h + (i >> 1)] = Tr::mfma(f[i], pf[i & 1], dvacc[2 * h + (i >> 1)]);
+          });
+    }
+    if constexpr (DK) {
+      staged_products<NH>(
+          [&](int h, u32x4(&f)[4]) {
+  #pragma unroll
+            for (int i = 0; i < 4; ++i)
+              f[i] = frag_cols_t(base + kQRows + h * kBlockBytes, 32 * wi + 16 * (i & 1) + 4 * kg, 32 * (i >> 1) + col_t, lane);
+          },
+          [&](int h, u32x4(&f)[4]) {
+  #pragma unroll
+            for (int i = 0; i < 4; ++i) dkacc[2 * h + (i >> 1)] = Tr::mfma(f[i], dsf[i & 1], dkacc[2 * h + (i >> 1)]);
+          });
+    }
+  }  // live
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -488,119 +634,8 @@ __device__ __forceinline__ void attn_bwd_kv_body(const bsa_attn_args &a, char *s
       if (more) fetch(rec, buf ^ 1);
       rec = load_record(clamp_e(e + 2));
 
-      // A quadrant whose every score is masked has P = dS = 0: nothing to add, nothing to compute.
-      bool live = true;
-      if (pm >= 0) live = !__all(mbits == 0xffffu);
-      if (causal) {
-        const int k_first = (int)kb * kSbs + 32 * wj, q_first = qb * kSbs + 32 * wi;
-        if (k_first > q_first + 31 || q_first >= seq_len || k_first >= seq_len) live = false;
-      }
-      if (live) {
-        // ---- S and dP of this wave's quadrant ----
-        f32x16 sacc, dpacc;
-  #pragma unroll
-        for (int r = 0; r < 16; ++r) sacc[r] = dpacc[r] = 0.f;
-        staged_products<NH + (DK ? NHV : 0)>(
-            [&](int k, u32x4(&f)[4]) {
-              const char *src = base + (k < NH ? kQRows + k * kBlockBytes : kDoRows + (k - NH) * kBlockBytes);
-  #pragma unroll
-              for (int s = 0; s < 4; ++s) f[s] = frag_rows(src, 32 * wi + li, 2 * s + kg);
-            },
-            [&](int k, u32x4(&f)[4]) {
-  #pragma unroll
-              for (int s = 0; s < 4; ++s) {
-                if (k < NH) sacc = Tr::mfma(f[s], kfr[k < NH ? k : 0][s], sacc);
-                else dpacc = Tr::mfma(f[s], vfr[k < NH ? 0 : k - NH][s], dpacc);
-              }
-            });
-
-        // ---- P and dS; element r: query 32 wi + 8 (r / 4) + 4 kg + r % 4 ----
-        const float *stats = reinterpret_cast<const float *>(base + kStats);
-        // the bias elements are read where they are used: a bias is rare, its registers are not
-        uint32_t bias_c[16];
-        if (pb >= 0) {
-          const uint16_t *bp = static_cast<const uint16_t *>(a.bias) + pb * (kSbs * kSbs) +
-                               (32 * wi + 4 * kg) * kSbs + 32 * wj + li;
-  #pragma unroll
-          for (int r = 0; r < 16; ++r) bias_c[r] = bp[(8 * (r >> 2) + (r & 3)) * kSbs];
-        }
-        float p[16], ds[16];
-        // Most tiles have no bias, no mask block and lie where the causal predicate holds for every score: they
-        // take the plain path.  The conditions are the same for the whole wave.
-        auto probabilities = [&](auto plain_tag) {
-          constexpr bool kPlain = decltype(plain_tag)::value;
-  #pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const int i0 = 32 * wi + 8 * q + 4 * kg;
-            const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(stats + i0);
-            const f32x4 del4 = *reinterpret_cast<const f32x4 *>(stats + kSbs + i0);
-  #pragma unroll
-            for (int t = 0; t < 4; ++t) {
-              const int r = 4 * q + t;
-              float s = sacc[r] * qk_scale;
-              if constexpr (!kPlain) {
-                if (pb >= 0) s = s + Tr::widen((uint16_t)bias_c[r]) * kLog2e;
-                if (causal) {
-                  const int qpos = qb * kSbs + i0 + t;
-                  s = (kpos > qpos || qpos >= seq_len || kpos >= seq_len) ? -INFINITY : s;
-                }
-                if (pm >= 0) s = ((mbits >> r) & 1u) ? -INFINITY : s;
-              }
-              p[r] = __builtin_amdgcn_exp2f(s - lse4[t]);
-              ds[r] = p[r] * (dpacc[r] - del4[t]);
-            }
-          }
-        };
-        bool plain = pb < 0 && pm < 0;
-        if (causal) {
-          // every key of the quadrant at or before every query of it, and all of them inside the sequence
-          const int k_last = (int)kb * kSbs + 32 * wj + 31, q_first = qb * kSbs + 32 * wi;
-          plain = plain && k_last <= q_first && q_first + 31 < seq_len;
-        }
-        if (plain) probabilities(std::true_type{});
-        else probabilities(std::false_type{});
-        if (DK && a.dbias != nullptr && pb >= 0) {
-          // every (query block, key block) pair is visited once, so this is a plain store
-          float *dbp = a.dbias + pb * (kSbs * kSbs) + (32 * wi + 4 * kg) * kSbs + 32 * wj + li;
-  #pragma unroll
-          for (int r = 0; r < 16; ++r) dbp[(8 * (r >> 2) + (r & 3)) * kSbs] = ds[r];
-        }
-        u32x4 pf[2], dsf[2];
-  #pragma unroll
-        for (int u = 0; u < 2; ++u)
-  #pragma unroll
-          for (int t = 0; t < 4; ++t) {
-            pf[u][t] = Tr::pack2(p[8 * u + 2 * t], p[8 * u + 2 * t + 1]);
-            dsf[u][t] = Tr::pack2(ds[8 * u + 2 * t], ds[8 * u + 2 * t + 1]);
-          }
-
-        // ---- dV^T += dO^T P, dK^T += Q^T dS over this wave's 32 queries ----
-        const int col_t = 16 * ((lane >> 4) & 1);
-        if constexpr (DV) {
-          staged_products<NHV>(
-              [&](int h, u32x4(&f)[4]) {
-  #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                  f[i] = frag_cols_t(base + kDoRows + h * kBlockBytes, 32 * wi + 16 * (i & 1) + 4 * kg, 32 * (i >> 1) + col_t, lane);
-              },
-              [&](int h, u32x4(&f)[4]) {
-  #pragma unroll
-                for (int i = 0; i < 4; ++i) dvacc[2 * h + (i >> 1)] = Tr::mfma(f[i], pf[i & 1], dvacc[2 * h + (i >> 1)]);
-              });
-        }
-        if constexpr (DK) {
-          staged_products<NH>(
-              [&](int h, u32x4(&f)[4]) {
-  #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                  f[i] = frag_cols_t(base + kQRows + h * kBlockBytes, 32 * wi + 16 * (i & 1) + 4 * kg, 32 * (i >> 1) + col_t, lane);
-              },
-              [&](int h, u32x4(&f)[4]) {
-  #pragma unroll
-                for (int i = 0; i < 4; ++i) dkacc[2 * h + (i >> 1)] = Tr::mfma(f[i], dsf[i & 1], dkacc[2 * h + (i >> 1)]);
-              });
-        }
-      }  // live
+      kv_tile<Tr, NH, NHV, DK, DV>(a, base, qb, pm, pb, mbits, causal, seq_len, (int)kb, kpos, qk_scale, wi, wj, li, kg,
+                                   lane, kfr, vfr, dkacc, dvacc);
 
       // ---- tile e+1 into the other buffer; the barrier also ends the reads of tile e ----
       if (more) stage(buf ^ 1);
@@ -652,6 +687,300 @@ __global__ __launch_bounds__(kBwdThreads, (DK &&DV) ? 1 : 2) void attn_bwd_kv_ke
   attn_bwd_kv_body<Tr, NH, NHV, DK, DV, 4>(a, smem, reinterpret_cast<float *>(smem), wave, wave);
 }
 
+// dK / dV with eight waves (two teams, as below) by workgroups that stay for the whole launch and walk one key
+// block after the other without draining the pipeline of tiles in between.  A workgroup without tiles still costs
+// 8 us (the chain header -> K / V fragments, records -> first tile, and at the end the sum over the wave pairs and
+// the stores), a third of the time of a key block with 8 live pairs.  Here, while key block n is walked:
+//   - the position of block n + 2 is drawn (one atomic add on the XCD's ticket counter by one lane; key rows are
+//     handed out longest first, so a workgroup that drew a long one simply draws fewer);
+//   - the header of block n + 1 is loaded (every wave its own copy);
+//   - K and V of block n + 1 are copied into an LDS region (R) of their own, from which the fragments are read
+//     when block n is done;
+//   - the first tile of block n + 1 is copied into the free tile buffer during the last tile of block n.
+// R also takes the partial sums of the wave pairs at the end of a block (after the next block's fragments have
+// been read from it).  All conditions below are the same for the eight waves of a workgroup (they depend on headers
+// and records only), so every wave passes the same barriers.
+template <typename Tr, int NH, int NHV, bool DK, bool DV>
+__device__ __forceinline__ void attn_bwd_kv8_walk(const bsa_attn_args &a, char *smem, int wave, int quad) {
+  constexpr int kQRows = 0, kDoRows = NH * kBlockBytes, kStats = (NH + NHV) * kBlockBytes,
+                kMask = kStats + kStatBytes;
+  constexpr int kBufBytes = kMask + kSbs * kSbs;
+  constexpr int kSlices = NH > NHV ? NH : NHV;
+  constexpr int kTeamFloats = 2 * kSlices * 2 * 16 * 64;  // partial sums of one team
+  char *region = smem + 2 * kBufBytes;                     // R: K / V of the next block, then the partial sums
+  float *reduce_lds = reinterpret_cast<float *>(region) + (DK ? kTeamFloats : 0);
+  int *mailbox = reinterpret_cast<int *>(region + 2 * kTeamFloats * 4);
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int li = lane & 31, kg = lane >> 5;
+  const int wi = quad & 1, wj = quad >> 1;
+  const int64_t rows = a.B * a.nk, chunk = (rows + 7) / 8;
+  const int64_t first = (int64_t)(blockIdx.x & 7) * chunk;  // this XCD's eighth: positions first .. first + chunk - 1
+  const BwdLists lists = bwd_lists(a);
+  const int32_t *recs = reinterpret_cast<const int32_t *>(lists.query_rec);
+  const float qk_scale = a.scale * kLog2e;
+  const bool causal = a.causal_lengths != nullptr;
+  auto valid_ticket = [&](int t) { return t >= 0 && t < chunk && first + t < rows; };
+  auto load_head = [&](int t) {
+    int v = -1;
+    if (valid_ticket(t) && lane < 16) v = lists.k_head[(first + t) * 16 + lane];
+    return v;
+  };
+  auto draw = [&]() {  // one lane of the workgroup draws; -1 elsewhere
+    int t = -1;
+    if (tid == 0) t = atomicAdd(lists.kv_tickets + (blockIdx.x & 7), 1);
+    return t;
+  };
+
+  // ---- the first block: nothing to overlap with
+  int t_cur = (int)(blockIdx.x >> 3);
+  if (!valid_ticket(t_cur)) return;  // same for the whole workgroup
+  int drawn = draw();                // the position of the second block
+  int head = load_head(t_cur);
+  if (tid == 0) mailbox[0] = drawn;
+  __syncthreads();
+  int t_next = first_lane(mailbox[0]);
+  __syncthreads();  // the mailbox may be written again
+
+  u32x4 kfr[NH][4], vfr[NHV][4];
+  {
+#pragma unroll
+    for (int h = 0; h < NH; ++h)
+      load_resident(kfr[h], a.k, __builtin_amdgcn_readlane(head, 11 + h), a.n_k_blocks, 32 * wj + li, kg);
+#pragma unroll
+    for (int h = 0; h < NHV; ++h) {
+      if constexpr (DK) load_resident(vfr[h], a.v, __builtin_amdgcn_readlane(head, 13 + h), a.n_v_blocks, 32 * wj + li, kg);
+      else {
+#pragma unroll
+        for (int s4 = 0; s4 < 4; ++s4) vfr[h][s4] = u32x4{0u, 0u, 0u, 0u};
+      }
+    }
+  }
+  f32x16 dkacc[DK ? NH * 2 : 1], dvacc[DV ? NHV * 2 : 1];
+  auto clear = [&]() {
+    if constexpr (DK) {
+#pragma unroll
+      for (int n = 0; n < NH * 2; ++n)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dkacc[n][r] = 0.f;
+    }
+    if constexpr (DV) {
+#pragma unroll
+      for (int n = 0; n < NHV * 2; ++n)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dvacc[n][r] = 0.f;
+    }
+  };
+  clear();
+
+  // registers of the tile in flight (the blocks themselves go straight to LDS)
+  float stat = 0.f;  // thread t < 64: lse of query t; 64 <= t < 128: delta of query t - 64
+  int qb_nxt = 0, pm_nxt = -1, pb_nxt = -1;
+  // requests the tile of record `rec` (field i in lane i) of batch entry `batch` into tile buffer `buf`
+  auto fetch = [&](int rec, int buf, int64_t batch) {
+    const int qb = __builtin_amdgcn_readlane(rec, 0);
+    qb_nxt = qb;
+    char *base = smem + first_lane(buf) * kBufBytes;  // the same for the whole wave: said so explicitly
+#pragma unroll
+    for (int h = 0; h < NH; ++h) {
+      const int pq = __builtin_amdgcn_readlane(rec, 1 + h);
+      copy_block<8>(static_cast<const char *>(a.q) + (int64_t)(pq >= 0 ? pq : 0) * kBlockBytes, pq >= 0,
+                    base + kQRows + h * kBlockBytes, wave, lane, tid);
+    }
+#pragma unroll
+    for (int h = 0; h < NHV; ++h) {
+      const int po = __builtin_amdgcn_readlane(rec, 3 + h);
+      copy_block<8>(static_cast<const char *>(a.d_o) + (int64_t)(po >= 0 ? po : 0) * kBlockBytes, po >= 0,
+                    base + kDoRows + h * kBlockBytes, wave, lane, tid);
+    }
+    const int64_t qrow = batch * a.nq + qb;
+    if (tid < 64) stat = a.lse[qrow * kSbs + tid];
+    else if (tid < 128) stat = a.delta[qrow * kSbs + tid - 64];
+    pm_nxt = __builtin_amdgcn_readlane(rec, 5);
+    pb_nxt = __builtin_amdgcn_readlane(rec, 6);
+    if (pm_nxt >= 0 && wave < 4)
+      copy_1k_to_lds(static_cast<const char *>(a.mask) + (int64_t)pm_nxt * (kSbs * kSbs) + wave * 1024, lane * 16,
+                     base + kMask + wave * 1024);
+  };
+  // the statistics of the tile go to LDS through a register; then every copy of this wave has to have landed
+  auto stage = [&](int buf) {
+    char *base = smem + buf * kBufBytes;
+    if (tid < 128) reinterpret_cast<float *>(base + kStats)[tid] = (tid < 64 && stat == -INFINITY) ? INFINITY : stat;
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+  };
+  // K and V of the block with header `h` into R
+  auto prefetch_kv = [&](int h) {
+#pragma unroll
+    for (int s2 = 0; s2 < NH; ++s2) {
+      const int pk = __builtin_amdgcn_readlane(h, 11 + s2);
+      copy_block<8>(static_cast<const char *>(a.k) + (int64_t)(pk >= 0 ? pk : 0) * kBlockBytes, pk >= 0,
+                    region + s2 * kBlockBytes, wave, lane, tid);
+    }
+#pragma unroll
+    for (int s2 = 0; s2 < NHV; ++s2) {
+      const int pv = __builtin_amdgcn_readlane(h, 13 + s2);
+      copy_block<8>(static_cast<const char *>(a.v) + (int64_t)(pv >= 0 ? pv : 0) * kBlockBytes, pv >= 0,
+                    region + (NH + s2) * kBlockBytes, wave, lane, tid);
+    }
+  };
+
+  int buf = 0;            // the tile buffer of the current block's next tile
+  bool staged = false;    // that tile has been requested and published already (during the block before)
+  while (true) {
+    buf = first_lane(buf);
+    // ---- facts of the current block
+    const uint32_t krow = (uint32_t)__builtin_amdgcn_readlane(head, 8), nk32 = (uint32_t)a.nk;  // int32 in the header
+    const int64_t b = krow / nk32, kb = krow % nk32;
+    const int q_begin = __builtin_amdgcn_readlane(head, 9), q_end = __builtin_amdgcn_readlane(head, 10);
+    int seq_len = 0;
+    if (causal) {
+      const int64_t len = a.causal_lengths[b];
+      seq_len = len < 0 ? 0 : (len > 0x7fffffffLL ? 0x7fffffff : (int)len);
+    }
+    const int kpos = (int)kb * kSbs + 32 * wj + li;
+    const bool has_next = valid_ticket(t_next);
+    // ---- for the blocks after this one: draw the position of the one after next, load the next header
+    drawn = has_next ? draw() : -1;
+    const int head_next = load_head(t_next);  // -1 in every lane when there is no next block
+    int64_t b_next = 0;
+    int q_begin_next = 0, q_end_next = 0;
+    bool kv_requested = false;
+
+    auto load_record = [&](int pos) -> int {
+      int v = -1;
+      if (lane < 8) v = recs[(int64_t)pos * 8 + lane];
+      return v;
+    };
+    auto clamp_e = [&](int e) { return e < q_end ? e : q_end - 1; };
+
+    if (q_begin < q_end) {
+      int rec = load_record(clamp_e(q_begin + 1));
+      if (!staged) {
+        fetch(head, buf, b);
+        stage(buf);
+        __syncthreads();
+      }
+      for (int e = q_begin; e < q_end; ++e) {
+        const char *base = smem + buf * kBufBytes;
+        const int qb = qb_nxt;
+        const int64_t pm = pm_nxt, pb = pb_nxt;
+        uint32_t mbits = 0;
+        if (pm >= 0) {
+          const uint8_t *mp = reinterpret_cast<const uint8_t *>(base + kMask) + (32 * wi + 4 * kg) * kSbs + 32 * wj + li;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) mbits |= (uint32_t)mp[(8 * (r >> 2) + (r & 3)) * kSbs] << r;
+        }
+        const bool more = e + 1 < q_end;
+        bool next_tile = more;
+        if (e == q_begin + 1 && has_next) {
+          // R is free (a barrier has passed since the partial sums of the block before were read) and the next
+          // header has arrived (the wait at the end of the first tile covers its load)
+          prefetch_kv(head_next);
+          kv_requested = true;
+        }
+        // the next tile into the free buffer: the next one of this block, or (last tile) the first one of the next
+        // block; one call for both, so that the copies are in the code once
+        int rec_use = rec;
+        int64_t batch_use = b;
+        if (!more && has_next) {
+          b_next = (uint32_t)__builtin_amdgcn_readlane(head_next, 8) / (uint32_t)a.nk;
+          q_begin_next = __builtin_amdgcn_readlane(head_next, 9);
+          q_end_next = __builtin_amdgcn_readlane(head_next, 10);
+          next_tile = q_begin_next < q_end_next;
+          rec_use = head_next;
+          batch_use = b_next;
+        }
+        if (next_tile) fetch(rec_use, buf ^ 1, batch_use);
+        rec = load_record(clamp_e(e + 2));
+
+        kv_tile<Tr, NH, NHV, DK, DV>(a, base, qb, pm, pb, mbits, causal, seq_len, (int)kb, kpos, qk_scale, wi, wj, li,
+                                     kg, lane, kfr, vfr, dkacc, dvacc);
+
+        if (next_tile) stage(buf ^ 1);
+        else __builtin_amdgcn_s_waitcnt(0x0F70);  // whatever this wave has requested (K / V of the next block) has landed
+        __syncthreads();
+        buf ^= 1;
+        staged = next_tile && !more;
+      }
+    } else {
+      staged = false;
+    }
+
+    // ---- end of the block
+    if (has_next && !kv_requested) {
+      // a block of fewer than two tiles: nothing was overlapped
+      __syncthreads();  // R is free
+      prefetch_kv(head_next);
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+      __syncthreads();
+    }
+    // the stationary block's packed indices, before `head` is replaced
+    int64_t pk[NH], pv[NHV];
+#pragma unroll
+    for (int h = 0; h < NH; ++h) pk[h] = __builtin_amdgcn_readlane(head, 11 + h);
+#pragma unroll
+    for (int h = 0; h < NHV; ++h) pv[h] = __builtin_amdgcn_readlane(head, 13 + h);
+    if (has_next) {
+      // the next block's fragments: this wave's keys j = 32 wj + li (every wave reads R; the first barrier of the
+      // sum below ends these reads before R is written)
+#pragma unroll
+      for (int h = 0; h < NH; ++h)
+#pragma unroll
+        for (int s4 = 0; s4 < 4; ++s4) kfr[h][s4] = frag_rows(region + h * kBlockBytes, 32 * wj + li, 2 * s4 + kg);
+      if constexpr (DK) {
+#pragma unroll
+        for (int h = 0; h < NHV; ++h)
+#pragma unroll
+          for (int s4 = 0; s4 < 4; ++s4) vfr[h][s4] = frag_rows(region + (NH + h) * kBlockBytes, 32 * wj + li, 2 * s4 + kg);
+      }
+    }
+    if (tid == 0) mailbox[0] = drawn;  // published by the barriers of the sum
+    // ---- add the two query halves, scale, store
+    if constexpr (DK) reduce_partner(dkacc, reduce_lds, wi == 1, wj, lane);
+    if constexpr (DV) reduce_partner(dvacc, reduce_lds, wi == 1, wj, lane);
+    const int t_after = first_lane(mailbox[0]);
+    if (wi == 0) {
+      // lane: key 32 wj + li; register 4 q + t of half db: column 32 db + 8 q + 4 kg + t
+#pragma unroll
+      for (int h = 0; h < (DK ? NH : 0); ++h) {
+        if (pk[h] < 0) continue;
+        char *op = static_cast<char *>(a.dk) + pk[h] * kBlockBytes + (32 * wj + li) * 128 + kg * 8;
+#pragma unroll
+        for (int db = 0; db < 2; ++db)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const f32x16 &acc = dkacc[2 * h + db];
+            u32x2 w;
+            w[0] = Tr::pack2(acc[4 * q] * a.scale, acc[4 * q + 1] * a.scale);
+            w[1] = Tr::pack2(acc[4 * q + 2] * a.scale, acc[4 * q + 3] * a.scale);
+            *reinterpret_cast<u32x2 *>(op + 64 * db + 16 * q) = w;
+          }
+      }
+#pragma unroll
+      for (int h = 0; h < (DV ? NHV : 0); ++h) {
+        if (pv[h] < 0) continue;
+        char *op = static_cast<char *>(a.dv) + pv[h] * kBlockBytes + (32 * wj + li) * 128 + kg * 8;
+#pragma unroll
+        for (int db = 0; db < 2; ++db)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const f32x16 &acc = dvacc[2 * h + db];
+            u32x2 w;
+            w[0] = Tr::pack2(acc[4 * q], acc[4 * q + 1]);
+            w[1] = Tr::pack2(acc[4 * q + 2], acc[4 * q + 3]);
+            *reinterpret_cast<u32x2 *>(op + 64 * db + 16 * q) = w;
+          }
+      }
+    }
+    if (!has_next) break;
+    clear();
+    head = head_next;
+    t_cur = t_next;
+    t_next = t_after;
+    __syncthreads();  // the mailbox and the partial sums have been read
+  }
+}
+
 // Eight waves: waves 0 .. 3 accumulate dV, waves 4 .. 7 dK and dBias, two waves per SIMD.  Each team fits 256
 // registers per lane, which the two sets of accumulators in one wave do not; the tile is fetched once for both.
 constexpr int kKv8Threads = 512;
@@ -663,6 +992,14 @@ __global__ __launch_bounds__(kKv8Threads, 1) void attn_bwd_kv8_kernel(bsa_attn_a
   float *reduce_lds = reinterpret_cast<float *>(smem) + (wave >> 2) * (2 * (NH > NHV ? NH : NHV) * 2 * 16 * 64);
   if (wave < 4) attn_bwd_kv_body<Tr, NH, NHV, false, true, 8>(a, smem, reduce_lds, wave, wave & 3);
   else attn_bwd_kv_body<Tr, NH, NHV, true, false, 8>(a, smem, reduce_lds, wave, wave & 3);
+}
+
+template <typename Tr, int NH, int NHV>
+__global__ __launch_bounds__(kKv8Threads, 1) void attn_bwd_kv8_walk_kernel(bsa_attn_args a) {
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  const int wave = first_lane((int)threadIdx.x >> 6);
+  if (wave < 4) attn_bwd_kv8_walk<Tr, NH, NHV, false, true>(a, smem, wave, wave & 3);
+  else attn_bwd_kv8_walk<Tr, NH, NHV, true, false>(a, smem, wave, wave & 3);
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -932,7 +1269,16 @@ int launch_bwd(const bsa_attn_args &a, hipStream_t s) {
   }
   if (krows > 0) {
     constexpr int lds = 2 * ((NH + NHV) * kBlockBytes + kStatBytes + kSbs * kSbs);
-    if (kEightWaves) {
+    if (kEightWaves && kKvWalk && qrows > 0) {
+      // tile buffers, the region of the next block's K / V and of the partial sums of both teams, the mailbox
+      constexpr int kSlices = NH > NHV ? NH : NHV;
+      constexpr int lds_walk = lds + 2 * (2 * kSlices * 2 * 16 * 64) * 4 + 64;
+      static_assert((NH + NHV) * kBlockBytes <= 2 * (2 * kSlices * 2 * 16 * 64) * 4, "K and V fit the region");
+      BSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_bwd_kv8_walk_kernel<Tr, NH, NHV>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds_walk));
+      attn_bwd_kv8_walk_kernel<Tr, NH, NHV><<<(unsigned)(kv_slots(krows) * 8), kKv8Threads, lds_walk, s>>>(a);
+      if (int rc = check_launch("attn_bwd_kv8_walk_kernel")) return rc;
+    } else if (kEightWaves) {
       constexpr int lds8 = lds > 65536 ? lds : 65536;  // the tile buffers; at the end, the partial sums of both teams
       BSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_bwd_kv8_kernel<Tr, NH, NHV>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds8));
@@ -982,7 +1328,8 @@ int attn_mask_dead(const void *mask, int64_t n_mask_blocks, uint8_t *dead, hipSt
 }
 
 size_t attn_bwd_scratch_bytes(int64_t B, int64_t nq, int64_t nk, int64_t n_layout_blocks, int64_t n_mask_blocks) {
-  const size_t bytes = 2 * sizeof(BwdRecord) * (size_t)n_layout_blocks + (4 + 64) * (size_t)(B * nq + B * nk) + (size_t)n_mask_blocks;
+  const size_t bytes = 2 * sizeof(BwdRecord) * (size_t)n_layout_blocks + (4 + 64) * (size_t)(B * nq + B * nk) + 64 +
+                       (size_t)n_mask_blocks;
   return (bytes + 15) & ~(size_t)15;
 }
 

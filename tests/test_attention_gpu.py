@@ -104,6 +104,20 @@ def test_many_head_slices_and_long_key_lists(device, dtype, sbs, nh, nhv):
     _run_case(device, dtype, sbs, B=1, nq=9, nk=9, nh=nh, nhv=nhv, density=0.3, seed=sbs + nhv, use_causal=True)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("use_mask,use_bias,use_causal,nh,nhv", [(False, False, False, 2, 2), (True, True, False, 1, 2),
+                                                               (False, False, True, 2, 1)])
+def test_dk_dv_of_more_key_blocks_than_workgroups(device, dtype, use_mask, use_bias, use_causal, nh, nhv):
+    """The dK / dV kernel keeps one workgroup per compute unit for the whole launch; a workgroup walks key block
+    after key block (drawn by ticket), with the next block's K / V and first tile requested during the current
+    one.  400 (or 270) key rows are 50 (34) per XCD against 32 workgroups; at 8 % density most key blocks are attended by no
+    query block or by one (blocks without tiles and with a single tile take paths of their own), a few by
+    several."""
+    B, nq, nk = (3, 90, 90) if use_causal else (4, 12, 100)  # the native causal predicate wants a square layout
+    _run_case(device, dtype, 64, B, nq, nk, nh, nhv, 0.08, seed=23, use_mask=use_mask, use_bias=use_bias,
+              use_causal=use_causal)
+
+
 def test_bigbird_layout_with_causal_mask_head_dim_128(device):
     """Config 4's shape at reduced batch and length: bf16, sbs 64, head_dim 128, BigBird layout, causal mask."""
     B, n, sbs, nh = 2, 16, 64, 2
