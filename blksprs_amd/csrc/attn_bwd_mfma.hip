@@ -480,6 +480,155 @@ __device__ __forceinline__ void kv_tile(const bsa_attn_args &a, const char *base
   }  // live
 }
 
+// The same tile with the work split between the two teams of the eight-wave kernel: the dV team (DV) computes S
+// and P, leaves P (fp32, as computed) in LDS for the wave of the dK team that owns the same quadrant, and adds
+// dV^T += dO^T P; the dK team (DK) computes dP meanwhile, reads P, forms dS = P (dP - delta) and adds
+// dK^T += Q^T dS.  Each team then issues 16 products per tile (24 and 16 when both compute S) and only one of them
+// the exponentials; the results are the same bits.  One barrier in the middle of the tile, passed by every wave
+// whether its quadrant is live or not, hands P over; p_lds: this quadrant's 4 KiB, lane's slot ([q][lane] of 16
+// bytes).  The next P is written after the barrier that ends the tile, when this one has been read.
+template <typename Tr, int NH, int NHV, bool DK, bool DV>
+__device__ __forceinline__ void kv_tile_teams(const bsa_attn_args &a, const char *base, const int qb, const int64_t pm,
+                                              const int64_t pb, const uint32_t mbits, const bool causal,
+                                              const int seq_len, const int kb, const int kpos, const float qk_scale,
+                                              const int wi, const int wj, const int li, const int kg, const int lane,
+                                              const u32x4 (&kfr)[NH][4], const u32x4 (&vfr)[NHV][4],
+                                              f32x16 (&dkacc)[DK ? NH * 2 : 1], f32x16 (&dvacc)[DV ? NHV * 2 : 1],
+                                              f32x4 *p_lds) {
+  static_assert(DK != DV, "one team each");
+  constexpr int kQRows = 0, kDoRows = NH * kBlockBytes, kStats = (NH + NHV) * kBlockBytes;
+  bool live = true;
+  if (pm >= 0) live = !__all(mbits == 0xffffu);
+  if (causal) {
+    const int k_first = (int)kb * kSbs + 32 * wj, q_first = qb * kSbs + 32 * wi;
+    if (k_first > q_first + 31 || q_first >= seq_len || k_first >= seq_len) live = false;
+  }
+  const float *stats = reinterpret_cast<const float *>(base + kStats);
+  const int col_t = 16 * ((lane >> 4) & 1);
+  if constexpr (DV) {
+    u32x4 pf[2];
+    if (live) {
+      f32x16 sacc;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
+      staged_products<NH>(
+          [&](int k, u32x4(&f)[4]) {
+#pragma unroll
+            for (int s = 0; s < 4; ++s) f[s] = frag_rows(base + kQRows + k * kBlockBytes, 32 * wi + li, 2 * s + kg);
+          },
+          [&](int k, u32x4(&f)[4]) {
+#pragma unroll
+            for (int s = 0; s < 4; ++s) sacc = Tr::mfma(f[s], kfr[k][s], sacc);
+          });
+      // ---- P; element r: query 32 wi + 8 (r / 4) + 4 kg + r % 4 ----
+      uint32_t bias_c[16];
+      if (pb >= 0) {
+        const uint16_t *bp = static_cast<const uint16_t *>(a.bias) + pb * (kSbs * kSbs) +
+                             (32 * wi + 4 * kg) * kSbs + 32 * wj + li;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) bias_c[r] = bp[(8 * (r >> 2) + (r & 3)) * kSbs];
+      }
+      float p[16];
+      auto probabilities = [&](auto plain_tag) {
+        constexpr bool kPlain = decltype(plain_tag)::value;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int i0 = 32 * wi + 8 * q + 4 * kg;
+          const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(stats + i0);
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            const int r = 4 * q + t;
+            float s = sacc[r] * qk_scale;
+            if constexpr (!kPlain) {
+              if (pb >= 0) s = s + Tr::widen((uint16_t)bias_c[r]) * kLog2e;
+              if (causal) {
+                const int qpos = qb * kSbs + i0 + t;
+                s = (kpos > qpos || qpos >= seq_len || kpos >= seq_len) ? -INFINITY : s;
+              }
+              if (pm >= 0) s = ((mbits >> r) & 1u) ? -INFINITY : s;
+            }
+            p[r] = __builtin_amdgcn_exp2f(s - lse4[t]);
+          }
+        }
+      };
+      bool plain = pb < 0 && pm < 0;
+      if (causal) {
+        const int k_last = (int)kb * kSbs + 32 * wj + 31, q_first = qb * kSbs + 32 * wi;
+        plain = plain && k_last <= q_first && q_first + 31 < seq_len;
+      }
+      if (plain) probabilities(std::true_type{});
+      else probabilities(std::false_type{});
+#pragma unroll
+      for (int q = 0; q < 4; ++q) p_lds[q * 64] = f32x4{p[4 * q], p[4 * q + 1], p[4 * q + 2], p[4 * q + 3]};
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) pf[u][t] = Tr::pack2(p[8 * u + 2 * t], p[8 * u + 2 * t + 1]);
+    }
+    __syncthreads();  // P is in LDS
+    if (live) {
+      staged_products<NHV>(
+          [&](int h, u32x4(&f)[4]) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              f[i] = frag_cols_t(base + kDoRows + h * kBlockBytes, 32 * wi + 16 * (i & 1) + 4 * kg, 32 * (i >> 1) + col_t, lane);
+          },
+          [&](int h, u32x4(&f)[4]) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) dvacc[2 * h + (i >> 1)] = Tr::mfma(f[i], pf[i & 1], dvacc[2 * h + (i >> 1)]);
+          });
+    }
+  } else {
+    f32x16 dpacc;
+    if (live) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) dpacc[r] = 0.f;
+      staged_products<NHV>(
+          [&](int k, u32x4(&f)[4]) {
+#pragma unroll
+            for (int s = 0; s < 4; ++s) f[s] = frag_rows(base + kDoRows + k * kBlockBytes, 32 * wi + li, 2 * s + kg);
+          },
+          [&](int k, u32x4(&f)[4]) {
+#pragma unroll
+            for (int s = 0; s < 4; ++s) dpacc = Tr::mfma(f[s], vfr[k][s], dpacc);
+          });
+    }
+    __syncthreads();  // P is in LDS
+    if (live) {
+      float ds[16];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int i0 = 32 * wi + 8 * q + 4 * kg;
+        const f32x4 del4 = *reinterpret_cast<const f32x4 *>(stats + kSbs + i0);
+        const f32x4 p4 = p_lds[q * 64];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) ds[4 * q + t] = p4[t] * (dpacc[4 * q + t] - del4[t]);
+      }
+      if (a.dbias != nullptr && pb >= 0) {
+        // every (query block, key block) pair is visited once, so this is a plain store
+        float *dbp = a.dbias + pb * (kSbs * kSbs) + (32 * wi + 4 * kg) * kSbs + 32 * wj + li;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dbp[(8 * (r >> 2) + (r & 3)) * kSbs] = ds[r];
+      }
+      u32x4 dsf[2];
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) dsf[u][t] = Tr::pack2(ds[8 * u + 2 * t], ds[8 * u + 2 * t + 1]);
+      staged_products<NH>(
+          [&](int h, u32x4(&f)[4]) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              f[i] = frag_cols_t(base + kQRows + h * kBlockBytes, 32 * wi + 16 * (i & 1) + 4 * kg, 32 * (i >> 1) + col_t, lane);
+          },
+          [&](int h, u32x4(&f)[4]) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) dkacc[2 * h + (i >> 1)] = Tr::mfma(f[i], dsf[i & 1], dkacc[2 * h + (i >> 1)]);
+          });
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------------------------------------
 // dK and dBias (DK) and / or dV (DV) of one key block.  The two are launched as separate passes: each then fits
 // two workgroups per CU (the combined kernel needs more than 256 registers per lane), which more than pays
@@ -710,6 +859,8 @@ __device__ __forceinline__ void attn_bwd_kv8_walk(const bsa_attn_args &a, char *
   char *region = smem + 2 * kBufBytes;                     // R: K / V of the next block, then the partial sums
   float *reduce_lds = reinterpret_cast<float *>(region) + (DK ? kTeamFloats : 0);
   int *mailbox = reinterpret_cast<int *>(region + 2 * kTeamFloats * 4);
+  // P of the tile, handed from the dV team to the dK team: [quadrant][4][lane] of 16 bytes
+  f32x4 *p_lds = reinterpret_cast<f32x4 *>(region + 2 * kTeamFloats * 4 + 64) + quad * 4 * 64 + (threadIdx.x & 63);
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int li = lane & 31, kg = lane >> 5;
@@ -774,7 +925,7 @@ __device__ __forceinline__ void attn_bwd_kv8_walk(const bsa_attn_args &a, char *
   clear();
 
   // registers of the tile in flight (the blocks themselves go straight to LDS)
-  float stat = 0.f;  // thread t < 64: lse of query t; 64 <= t < 128: delta of query t - 64
+  float stat = 0.f;  // thread 256 + t, t < 64: lse of query t; 320 + t: delta of query t
   int qb_nxt = 0, pm_nxt = -1, pb_nxt = -1;
   // requests the tile of record `rec` (field i in lane i) of batch entry `batch` into tile buffer `buf`
   auto fetch = [&](int rec, int buf, int64_t batch) {
@@ -787,25 +938,30 @@ __device__ __forceinline__ void attn_bwd_kv8_walk(const bsa_attn_args &a, char *
       copy_block<8>(static_cast<const char *>(a.q) + (int64_t)(pq >= 0 ? pq : 0) * kBlockBytes, pq >= 0,
                     base + kQRows + h * kBlockBytes, wave, lane, tid);
     }
-#pragma unroll
-    for (int h = 0; h < NHV; ++h) {
-      const int po = __builtin_amdgcn_readlane(rec, 3 + h);
-      copy_block<8>(static_cast<const char *>(a.d_o) + (int64_t)(po >= 0 ? po : 0) * kBlockBytes, po >= 0,
-                    base + kDoRows + h * kBlockBytes, wave, lane, tid);
-    }
+    // The dV team has the longer first half of a tile (S and P against dP): the dO blocks, the statistics and the
+    // mask block are fetched by the dK team alone (waves 4 .. 7), the Q blocks by all eight waves.
     const int64_t qrow = batch * a.nq + qb;
-    if (tid < 64) stat = a.lse[qrow * kSbs + tid];
-    else if (tid < 128) stat = a.delta[qrow * kSbs + tid - 64];
     pm_nxt = __builtin_amdgcn_readlane(rec, 5);
     pb_nxt = __builtin_amdgcn_readlane(rec, 6);
-    if (pm_nxt >= 0 && wave < 4)
-      copy_1k_to_lds(static_cast<const char *>(a.mask) + (int64_t)pm_nxt * (kSbs * kSbs) + wave * 1024, lane * 16,
-                     base + kMask + wave * 1024);
+    if (wave >= 4) {
+#pragma unroll
+      for (int h = 0; h < NHV; ++h) {
+        const int po = __builtin_amdgcn_readlane(rec, 3 + h);
+        copy_block<4>(static_cast<const char *>(a.d_o) + (int64_t)(po >= 0 ? po : 0) * kBlockBytes, po >= 0,
+                      base + kDoRows + h * kBlockBytes, wave - 4, lane, tid - 256);
+      }
+      if (tid < 320) stat = a.lse[qrow * kSbs + tid - 256];
+      else if (tid < 384) stat = a.delta[qrow * kSbs + tid - 320];
+      if (pm_nxt >= 0)
+        copy_1k_to_lds(static_cast<const char *>(a.mask) + (int64_t)pm_nxt * (kSbs * kSbs) + (wave - 4) * 1024, lane * 16,
+                       base + kMask + (wave - 4) * 1024);
+    }
   };
   // the statistics of the tile go to LDS through a register; then every copy of this wave has to have landed
   auto stage = [&](int buf) {
     char *base = smem + buf * kBufBytes;
-    if (tid < 128) reinterpret_cast<float *>(base + kStats)[tid] = (tid < 64 && stat == -INFINITY) ? INFINITY : stat;
+    if (tid >= 256 && tid < 384)
+      reinterpret_cast<float *>(base + kStats)[tid - 256] = (tid < 320 && stat == -INFINITY) ? INFINITY : stat;
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
   };
   // K and V of the block with header `h` into R
@@ -893,8 +1049,8 @@ __device__ __forceinline__ void attn_bwd_kv8_walk(const bsa_attn_args &a, char *
         if (next_tile) fetch(rec_use, buf ^ 1, batch_use);
         rec = load_record(clamp_e(e + 2));
 
-        kv_tile<Tr, NH, NHV, DK, DV>(a, base, qb, pm, pb, mbits, causal, seq_len, (int)kb, kpos, qk_scale, wi, wj, li,
-                                     kg, lane, kfr, vfr, dkacc, dvacc);
+        kv_tile_teams<Tr, NH, NHV, DK, DV>(a, base, qb, pm, pb, mbits, causal, seq_len, (int)kb, kpos, qk_scale, wi, wj,
+                                           li, kg, lane, kfr, vfr, dkacc, dvacc, p_lds);
 
         if (next_tile) stage(buf ^ 1);
         else __builtin_amdgcn_s_waitcnt(0x0F70);  // whatever this wave has requested (K / V of the next block) has landed
@@ -1270,9 +1426,9 @@ int launch_bwd(const bsa_attn_args &a, hipStream_t s) {
   if (krows > 0) {
     constexpr int lds = 2 * ((NH + NHV) * kBlockBytes + kStatBytes + kSbs * kSbs);
     if (kEightWaves && kKvWalk && qrows > 0) {
-      // tile buffers, the region of the next block's K / V and of the partial sums of both teams, the mailbox
+      // tile buffers, the region of the next block's K / V and of the partial sums of both teams, the mailbox, P
       constexpr int kSlices = NH > NHV ? NH : NHV;
-      constexpr int lds_walk = lds + 2 * (2 * kSlices * 2 * 16 * 64) * 4 + 64;
+      constexpr int lds_walk = lds + 2 * (2 * kSlices * 2 * 16 * 64) * 4 + 64 + 4 * 4 * 64 * 16;  // + P of a tile
       static_assert((NH + NHV) * kBlockBytes <= 2 * (2 * kSlices * 2 * 16 * 64) * 4, "K and V fit the region");
       BSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_bwd_kv8_walk_kernel<Tr, NH, NHV>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds_walk));
