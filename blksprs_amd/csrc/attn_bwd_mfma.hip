@@ -106,6 +106,23 @@ __host__ __device__ inline int64_t kv_slots(int64_t key_rows) {
   return chunk < kCusPerXcd ? chunk : kCusPerXcd;
 }
 
+// The same run with the fragments of stage 0 already requested by the caller (`first`), so that their latency
+// lies behind whatever the caller did in between.
+template <int K, typename Load, typename Multiply>
+__device__ __forceinline__ void staged_products_from(const u32x4 (&first)[4], Load load, Multiply multiply) {
+  u32x4 f[2][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) f[0][i] = first[i];
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    if (k + 1 < K) load(k + 1, f[(k + 1) & 1]);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(f[k & 1][i]));
+    multiply(k, f[k & 1]);
+  }
+}
+
 // XCD-aware row of a workgroup: every XCD gets a contiguous range of rows, so that the blocks in flight on one
 // L2 belong to the same batch entries
 __device__ inline int64_t xcd_row() { return (int64_t)(blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3); }
@@ -480,152 +497,193 @@ __device__ __forceinline__ void kv_tile(const bsa_attn_args &a, const char *base
   }  // live
 }
 
-// The same tile with the work split between the two teams of the eight-wave kernel: the dV team (DV) computes S
-// and P, leaves P (fp32, as computed) in LDS for the wave of the dK team that owns the same quadrant, and adds
+// A tile with the work split between the two teams of the eight-wave kernel: the dV team (DV) computes S and P,
+// leaves P (fp32, as computed) in LDS for the wave of the dK team that owns the same quadrant, and adds
 // dV^T += dO^T P; the dK team (DK) computes dP meanwhile, reads P, forms dS = P (dP - delta) and adds
 // dK^T += Q^T dS.  Each team then issues 16 products per tile (24 and 16 when both compute S) and only one of them
 // the exponentials; the results are the same bits.  One barrier in the middle of the tile, passed by every wave
 // whether its quadrant is live or not, hands P over; p_lds: this quadrant's 4 KiB, lane's slot ([q][lane] of 16
 // bytes).  The next P is written after the barrier that ends the tile, when this one has been read.
-template <typename Tr, int NH, int NHV, bool DK, bool DV>
-__device__ __forceinline__ void kv_tile_teams(const bsa_attn_args &a, const char *base, const int qb, const int64_t pm,
-                                              const int64_t pb, const uint32_t mbits, const bool causal,
-                                              const int seq_len, const int kb, const int kpos, const float qk_scale,
-                                              const int wi, const int wj, const int li, const int kg, const int lane,
-                                              const u32x4 (&kfr)[NH][4], const u32x4 (&vfr)[NHV][4],
-                                              f32x16 (&dkacc)[DK ? NH * 2 : 1], f32x16 (&dvacc)[DV ? NHV * 2 : 1],
-                                              f32x4 *p_lds) {
-  static_assert(DK != DV, "one team each");
-  constexpr int kQRows = 0, kDoRows = NH * kBlockBytes, kStats = (NH + NHV) * kBlockBytes;
+// The tile comes in three calls, so that the caller can put other work behind the LDS reads that open each half:
+// kv_first_frags requests the fragments the first products start with (the caller then requests the next tile),
+// kv_first_half ends by requesting those of the second half (the caller then passes the barrier).
+
+// A quadrant whose every score is masked has P = dS = 0: nothing to add, nothing to compute.
+__device__ __forceinline__ bool kv_quadrant_live(const int64_t pm, const uint32_t mbits, const bool causal, const int kb,
+                                                 const int qb, const int seq_len, const int wi, const int wj) {
   bool live = true;
   if (pm >= 0) live = !__all(mbits == 0xffffu);
   if (causal) {
-    const int k_first = (int)kb * kSbs + 32 * wj, q_first = qb * kSbs + 32 * wi;
+    const int k_first = kb * kSbs + 32 * wj, q_first = qb * kSbs + 32 * wi;
     if (k_first > q_first + 31 || q_first >= seq_len || k_first >= seq_len) live = false;
   }
+  return live;
+}
+
+// stage 0 of the first products: rows of Q (dV team: S) or of dO (dK team: dP)
+template <int NH, bool DK>
+__device__ __forceinline__ void kv_first_frags(u32x4 (&f0)[4], const char *base, const int wi, const int li, const int kg) {
+  const char *src = base + (DK ? NH * kBlockBytes : 0);
+#pragma unroll
+  for (int s = 0; s < 4; ++s) f0[s] = frag_rows(src, 32 * wi + li, 2 * s + kg);
+}
+
+// what a wave carries over the barrier in the middle of the tile
+struct KvCarry {
+  u32x4 g0[4];   // stage 0 of the second products: columns of dO (dV team) or of Q (dK team)
+  u32x4 pf[2];   // dV team: P as operand
+  f32x16 dpacc;  // dK team: dP
+};
+
+template <typename Tr, int NH, int NHV, bool DK, bool DV>
+__device__ __forceinline__ void kv_first_half(KvCarry &c, const u32x4 (&f0)[4], const bool live, const bsa_attn_args &a,
+                                              const char *base, const int qb, const int64_t pm, const int64_t pb,
+                                              const uint32_t mbits, const bool causal, const int seq_len, const int kb,
+                                              const int kpos, const float qk_scale, const int wi, const int wj,
+                                              const int li, const int kg, const int lane, const u32x4 (&kfr)[NH][4],
+                                              const u32x4 (&vfr)[NHV][4], f32x4 *p_lds) {
+  static_assert(DK != DV, "one team each");
+  constexpr int kQRows = 0, kDoRows = NH * kBlockBytes, kStats = (NH + NHV) * kBlockBytes;
+  if (!live) return;
   const float *stats = reinterpret_cast<const float *>(base + kStats);
   const int col_t = 16 * ((lane >> 4) & 1);
   if constexpr (DV) {
-    u32x4 pf[2];
-    if (live) {
-      f32x16 sacc;
+    f32x16 sacc;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
-      staged_products<NH>(
-          [&](int k, u32x4(&f)[4]) {
+    for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
+    staged_products_from<NH>(
+        f0,
+        [&](int k, u32x4(&f)[4]) {
 #pragma unroll
-            for (int s = 0; s < 4; ++s) f[s] = frag_rows(base + kQRows + k * kBlockBytes, 32 * wi + li, 2 * s + kg);
-          },
-          [&](int k, u32x4(&f)[4]) {
+          for (int s = 0; s < 4; ++s) f[s] = frag_rows(base + kQRows + k * kBlockBytes, 32 * wi + li, 2 * s + kg);
+        },
+        [&](int k, u32x4(&f)[4]) {
 #pragma unroll
-            for (int s = 0; s < 4; ++s) sacc = Tr::mfma(f[s], kfr[k][s], sacc);
-          });
-      // ---- P; element r: query 32 wi + 8 (r / 4) + 4 kg + r % 4 ----
-      uint32_t bias_c[16];
-      if (pb >= 0) {
-        const uint16_t *bp = static_cast<const uint16_t *>(a.bias) + pb * (kSbs * kSbs) +
-                             (32 * wi + 4 * kg) * kSbs + 32 * wj + li;
+          for (int s = 0; s < 4; ++s) sacc = Tr::mfma(f[s], kfr[k][s], sacc);
+        });
+    // the fragments the dV products start with: in flight while P is formed
 #pragma unroll
-        for (int r = 0; r < 16; ++r) bias_c[r] = bp[(8 * (r >> 2) + (r & 3)) * kSbs];
-      }
-      float p[16];
-      auto probabilities = [&](auto plain_tag) {
-        constexpr bool kPlain = decltype(plain_tag)::value;
+    for (int i = 0; i < 4; ++i)
+      c.g0[i] = frag_cols_t(base + kDoRows, 32 * wi + 16 * (i & 1) + 4 * kg, 32 * (i >> 1) + col_t, lane);
+    // ---- P; element r: query 32 wi + 8 (r / 4) + 4 kg + r % 4 ----
+    uint32_t bias_c[16];
+    if (pb >= 0) {
+      const uint16_t *bp = static_cast<const uint16_t *>(a.bias) + pb * (kSbs * kSbs) +
+                           (32 * wi + 4 * kg) * kSbs + 32 * wj + li;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int i0 = 32 * wi + 8 * q + 4 * kg;
-          const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(stats + i0);
-#pragma unroll
-          for (int t = 0; t < 4; ++t) {
-            const int r = 4 * q + t;
-            float s = sacc[r] * qk_scale;
-            if constexpr (!kPlain) {
-              if (pb >= 0) s = s + Tr::widen((uint16_t)bias_c[r]) * kLog2e;
-              if (causal) {
-                const int qpos = qb * kSbs + i0 + t;
-                s = (kpos > qpos || qpos >= seq_len || kpos >= seq_len) ? -INFINITY : s;
-              }
-              if (pm >= 0) s = ((mbits >> r) & 1u) ? -INFINITY : s;
-            }
-            p[r] = __builtin_amdgcn_exp2f(s - lse4[t]);
-          }
-        }
-      };
-      bool plain = pb < 0 && pm < 0;
-      if (causal) {
-        const int k_last = (int)kb * kSbs + 32 * wj + 31, q_first = qb * kSbs + 32 * wi;
-        plain = plain && k_last <= q_first && q_first + 31 < seq_len;
-      }
-      if (plain) probabilities(std::true_type{});
-      else probabilities(std::false_type{});
-#pragma unroll
-      for (int q = 0; q < 4; ++q) p_lds[q * 64] = f32x4{p[4 * q], p[4 * q + 1], p[4 * q + 2], p[4 * q + 3]};
-#pragma unroll
-      for (int u = 0; u < 2; ++u)
-#pragma unroll
-        for (int t = 0; t < 4; ++t) pf[u][t] = Tr::pack2(p[8 * u + 2 * t], p[8 * u + 2 * t + 1]);
+      for (int r = 0; r < 16; ++r) bias_c[r] = bp[(8 * (r >> 2) + (r & 3)) * kSbs];
     }
-    __syncthreads();  // P is in LDS
-    if (live) {
-      staged_products<NHV>(
-          [&](int h, u32x4(&f)[4]) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-              f[i] = frag_cols_t(base + kDoRows + h * kBlockBytes, 32 * wi + 16 * (i & 1) + 4 * kg, 32 * (i >> 1) + col_t, lane);
-          },
-          [&](int h, u32x4(&f)[4]) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) dvacc[2 * h + (i >> 1)] = Tr::mfma(f[i], pf[i & 1], dvacc[2 * h + (i >> 1)]);
-          });
-    }
-  } else {
-    f32x16 dpacc;
-    if (live) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) dpacc[r] = 0.f;
-      staged_products<NHV>(
-          [&](int k, u32x4(&f)[4]) {
-#pragma unroll
-            for (int s = 0; s < 4; ++s) f[s] = frag_rows(base + kDoRows + k * kBlockBytes, 32 * wi + li, 2 * s + kg);
-          },
-          [&](int k, u32x4(&f)[4]) {
-#pragma unroll
-            for (int s = 0; s < 4; ++s) dpacc = Tr::mfma(f[s], vfr[k][s], dpacc);
-          });
-    }
-    __syncthreads();  // P is in LDS
-    if (live) {
-      float ds[16];
+    float p[16];
+    auto probabilities = [&](auto plain_tag) {
+      constexpr bool kPlain = decltype(plain_tag)::value;
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int i0 = 32 * wi + 8 * q + 4 * kg;
-        const f32x4 del4 = *reinterpret_cast<const f32x4 *>(stats + kSbs + i0);
-        const f32x4 p4 = p_lds[q * 64];
+        const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(stats + i0);
 #pragma unroll
-        for (int t = 0; t < 4; ++t) ds[4 * q + t] = p4[t] * (dpacc[4 * q + t] - del4[t]);
+        for (int t = 0; t < 4; ++t) {
+          const int r = 4 * q + t;
+          float s = sacc[r] * qk_scale;
+          if constexpr (!kPlain) {
+            if (pb >= 0) s = s + Tr::widen((uint16_t)bias_c[r]) * kLog2e;
+            if (causal) {
+              const int qpos = qb * kSbs + i0 + t;
+              s = (kpos > qpos || qpos >= seq_len || kpos >= seq_len) ? -INFINITY : s;
+            }
+            if (pm >= 0) s = ((mbits >> r) & 1u) ? -INFINITY : s;
+          }
+          p[r] = __builtin_amdgcn_exp2f(s - lse4[t]);
+        }
       }
-      if (a.dbias != nullptr && pb >= 0) {
-        // every (query block, key block) pair is visited once, so this is a plain store
-        float *dbp = a.dbias + pb * (kSbs * kSbs) + (32 * wi + 4 * kg) * kSbs + 32 * wj + li;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) dbp[(8 * (r >> 2) + (r & 3)) * kSbs] = ds[r];
-      }
-      u32x4 dsf[2];
-#pragma unroll
-      for (int u = 0; u < 2; ++u)
-#pragma unroll
-        for (int t = 0; t < 4; ++t) dsf[u][t] = Tr::pack2(ds[8 * u + 2 * t], ds[8 * u + 2 * t + 1]);
-      staged_products<NH>(
-          [&](int h, u32x4(&f)[4]) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-              f[i] = frag_cols_t(base + kQRows + h * kBlockBytes, 32 * wi + 16 * (i & 1) + 4 * kg, 32 * (i >> 1) + col_t, lane);
-          },
-          [&](int h, u32x4(&f)[4]) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) dkacc[2 * h + (i >> 1)] = Tr::mfma(f[i], dsf[i & 1], dkacc[2 * h + (i >> 1)]);
-          });
+    };
+    // Most tiles have no bias, no mask block and lie where the causal predicate holds for every score: they take
+    // the plain path.  The conditions are the same for the whole wave.
+    bool plain = pb < 0 && pm < 0;
+    if (causal) {
+      const int k_last = kb * kSbs + 32 * wj + 31, q_first = qb * kSbs + 32 * wi;
+      plain = plain && k_last <= q_first && q_first + 31 < seq_len;
     }
+    if (plain) probabilities(std::true_type{});
+    else probabilities(std::false_type{});
+#pragma unroll
+    for (int q = 0; q < 4; ++q) p_lds[q * 64] = f32x4{p[4 * q], p[4 * q + 1], p[4 * q + 2], p[4 * q + 3]};
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int t = 0; t < 4; ++t) c.pf[u][t] = Tr::pack2(p[8 * u + 2 * t], p[8 * u + 2 * t + 1]);
+  } else {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) c.dpacc[r] = 0.f;
+    staged_products_from<NHV>(
+        f0,
+        [&](int k, u32x4(&f)[4]) {
+#pragma unroll
+          for (int s = 0; s < 4; ++s) f[s] = frag_rows(base + kDoRows + k * kBlockBytes, 32 * wi + li, 2 * s + kg);
+        },
+        [&](int k, u32x4(&f)[4]) {
+#pragma unroll
+          for (int s = 0; s < 4; ++s) c.dpacc = Tr::mfma(f[s], vfr[k][s], c.dpacc);
+        });
+    // the fragments the dK products start with: in flight across the barrier and while dS is formed
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      c.g0[i] = frag_cols_t(base + kQRows, 32 * wi + 16 * (i & 1) + 4 * kg, 32 * (i >> 1) + col_t, lane);
+  }
+}
+
+template <typename Tr, int NH, int NHV, bool DK, bool DV>
+__device__ __forceinline__ void kv_second_half(const KvCarry &c, const bool live, const bsa_attn_args &a, const char *base,
+                                               const int64_t pb, const int wi, const int wj, const int li, const int kg,
+                                               const int lane, f32x16 (&dkacc)[DK ? NH * 2 : 1],
+                                               f32x16 (&dvacc)[DV ? NHV * 2 : 1], const f32x4 *p_lds) {
+  constexpr int kQRows = 0, kDoRows = NH * kBlockBytes, kStats = (NH + NHV) * kBlockBytes;
+  if (!live) return;
+  const int col_t = 16 * ((lane >> 4) & 1);
+  if constexpr (DV) {
+    staged_products_from<NHV>(
+        c.g0,
+        [&](int h, u32x4(&f)[4]) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            f[i] = frag_cols_t(base + kDoRows + h * kBlockBytes, 32 * wi + 16 * (i & 1) + 4 * kg, 32 * (i >> 1) + col_t, lane);
+        },
+        [&](int h, u32x4(&f)[4]) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) dvacc[2 * h + (i >> 1)] = Tr::mfma(f[i], c.pf[i & 1], dvacc[2 * h + (i >> 1)]);
+        });
+  } else {
+    const float *stats = reinterpret_cast<const float *>(base + kStats);
+    float ds[16];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int i0 = 32 * wi + 8 * q + 4 * kg;
+      const f32x4 del4 = *reinterpret_cast<const f32x4 *>(stats + kSbs + i0);
+      const f32x4 p4 = p_lds[q * 64];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) ds[4 * q + t] = p4[t] * (c.dpacc[4 * q + t] - del4[t]);
+    }
+    if (a.dbias != nullptr && pb >= 0) {
+      // every (query block, key block) pair is visited once, so this is a plain store
+      float *dbp = a.dbias + pb * (kSbs * kSbs) + (32 * wi + 4 * kg) * kSbs + 32 * wj + li;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) dbp[(8 * (r >> 2) + (r & 3)) * kSbs] = ds[r];
+    }
+    u32x4 dsf[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int t = 0; t < 4; ++t) dsf[u][t] = Tr::pack2(ds[8 * u + 2 * t], ds[8 * u + 2 * t + 1]);
+    staged_products_from<NH>(
+        c.g0,
+        [&](int h, u32x4(&f)[4]) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            f[i] = frag_cols_t(base + kQRows + h * kBlockBytes, 32 * wi + 16 * (i & 1) + 4 * kg, 32 * (i >> 1) + col_t, lane);
+        },
+        [&](int h, u32x4(&f)[4]) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) dkacc[2 * h + (i >> 1)] = Tr::mfma(f[i], dsf[i & 1], dkacc[2 * h + (i >> 1)]);
+        });
   }
 }
 
@@ -1026,6 +1084,10 @@ __device__ __forceinline__ void attn_bwd_kv8_walk(const bsa_attn_args &a, char *
 #pragma unroll
           for (int r = 0; r < 16; ++r) mbits |= (uint32_t)mp[(8 * (r >> 2) + (r & 3)) * kSbs] << r;
         }
+        const bool live = kv_quadrant_live(pm, mbits, causal, (int)kb, qb, seq_len, wi, wj);
+        // the fragments the tile's first products start with: their latency lies behind the requests for the next tile
+        u32x4 f0[4];
+        kv_first_frags<NH, DK>(f0, base, wi, li, kg);
         const bool more = e + 1 < q_end;
         bool next_tile = more;
         if (e == q_begin + 1 && has_next) {
@@ -1049,8 +1111,11 @@ __device__ __forceinline__ void attn_bwd_kv8_walk(const bsa_attn_args &a, char *
         if (next_tile) fetch(rec_use, buf ^ 1, batch_use);
         rec = load_record(clamp_e(e + 2));
 
-        kv_tile_teams<Tr, NH, NHV, DK, DV>(a, base, qb, pm, pb, mbits, causal, seq_len, (int)kb, kpos, qk_scale, wi, wj,
-                                           li, kg, lane, kfr, vfr, dkacc, dvacc, p_lds);
+        KvCarry carry;
+        kv_first_half<Tr, NH, NHV, DK, DV>(carry, f0, live, a, base, qb, pm, pb, mbits, causal, seq_len, (int)kb, kpos,
+                                           qk_scale, wi, wj, li, kg, lane, kfr, vfr, p_lds);
+        __syncthreads();  // P is in LDS
+        kv_second_half<Tr, NH, NHV, DK, DV>(carry, live, a, base, pb, wi, wj, li, kg, lane, dkacc, dvacc, p_lds);
 
         if (next_tile) stage(buf ^ 1);
         else __builtin_amdgcn_s_waitcnt(0x0F70);  // whatever this wave has requested (K / V of the next block) has landed
