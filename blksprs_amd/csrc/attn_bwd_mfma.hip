@@ -984,6 +984,14 @@ __device__ __forceinline__ void attn_bwd_kv8_walk(const bsa_attn_args &a, char *
 
   // registers of the tile in flight (the blocks themselves go straight to LDS)
   float stat = 0.f;  // thread 256 + t, t < 64: lse of query t; 320 + t: delta of query t
+  // The record of the tile after next (field i in lanes i, 8 + i, ...), requested from inline assembly: between the
+  // request and the wait in stage() nothing touches the register.
+  int rec_in_flight = -1;
+  const int32_t *const recs_lane = recs + (lane & 7);
+  auto request_record = [&](int pos) {
+    const int32_t *src = recs_lane + (int64_t)pos * 8;
+    asm volatile("global_load_dword %0, %1, off" : "+v"(rec_in_flight) : "v"(src) : "memory");
+  };
   int qb_nxt = 0, pm_nxt = -1, pb_nxt = -1;
   // requests the tile of record `rec` (field i in lane i) of batch entry `batch` into tile buffer `buf`
   auto fetch = [&](int rec, int buf, int64_t batch) {
@@ -998,7 +1006,6 @@ __device__ __forceinline__ void attn_bwd_kv8_walk(const bsa_attn_args &a, char *
     }
     // The dV team has the longer first half of a tile (S and P against dP): the dO blocks, the statistics and the
     // mask block are fetched by the dK team alone (waves 4 .. 7), the Q blocks by all eight waves.
-    const int64_t qrow = batch * a.nq + qb;
     pm_nxt = __builtin_amdgcn_readlane(rec, 5);
     pb_nxt = __builtin_amdgcn_readlane(rec, 6);
     if (wave >= 4) {
@@ -1008,19 +1015,33 @@ __device__ __forceinline__ void attn_bwd_kv8_walk(const bsa_attn_args &a, char *
         copy_block<4>(static_cast<const char *>(a.d_o) + (int64_t)(po >= 0 ? po : 0) * kBlockBytes, po >= 0,
                       base + kDoRows + h * kBlockBytes, wave - 4, lane, tid - 256);
       }
-      if (tid < 320) stat = a.lse[qrow * kSbs + tid - 256];
-      else if (tid < 384) stat = a.delta[qrow * kSbs + tid - 320];
       if (pm_nxt >= 0)
         copy_1k_to_lds(static_cast<const char *>(a.mask) + (int64_t)pm_nxt * (kSbs * kSbs) + (wave - 4) * 1024, lane * 16,
                        base + kMask + (wave - 4) * 1024);
     }
   };
+  // The statistics of the tile of record `rec`: wave 4 requests the lse of its 64 queries, wave 5 their delta (the
+  // other waves the lse as well, and drop it).  Requested from inline assembly like the copies: a load the compiler
+  // knows of makes it wait for everything in flight (vmcnt(0)) at the next join, the copies included, which would
+  // put the whole latency of the next tile in front of this tile's products.  Called on the straight path only (a
+  // request in a branch of its own would let the compiler move the register at the join, with the load in flight);
+  // when there is no next tile the record is the last valid one and the value is not used.
+  auto request_stat = [&](int rec, int64_t batch) {
+    const int64_t qrow = batch * a.nq + __builtin_amdgcn_readlane(rec, 0);
+    const float *src = (wave == 5 ? a.delta : a.lse) + qrow * kSbs + lane;
+    asm volatile("global_load_dword %0, %1, off" : "+v"(stat) : "v"(src) : "memory");
+  };
   // the statistics of the tile go to LDS through a register; then every copy of this wave has to have landed
   auto stage = [&](int buf) {
     char *base = smem + buf * kBufBytes;
+    // everything this wave has requested has landed: its copies, the statistics, the record of the tile after
+    // (the builtin, so that the compiler knows that nothing it has requested itself is pending either: a load it
+    // believes to be in flight at the top of the loop makes it wait, with vmcnt(0), in front of the first product of
+    // every tile, and that wait would include the copies of the next tile)
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    asm volatile("" : "+v"(stat), "+v"(rec_in_flight) : : "memory");
     if (tid >= 256 && tid < 384)
       reinterpret_cast<float *>(base + kStats)[tid - 256] = (tid < 320 && stat == -INFINITY) ? INFINITY : stat;
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
   };
   // K and V of the block with header `h` into R
   auto prefetch_kv = [&](int h) {
@@ -1038,6 +1059,9 @@ __device__ __forceinline__ void attn_bwd_kv8_walk(const bsa_attn_args &a, char *
     }
   };
 
+  // the first block's fragments have arrived: from here on the compiler has no load of its own in flight when a
+  // tile starts (see stage())
+  __builtin_amdgcn_s_waitcnt(0x0F70);
   int buf = 0;            // the tile buffer of the current block's next tile
   bool staged = false;    // that tile has been requested and published already (during the block before)
   while (true) {
@@ -1060,20 +1084,19 @@ __device__ __forceinline__ void attn_bwd_kv8_walk(const bsa_attn_args &a, char *
     int q_begin_next = 0, q_end_next = 0;
     bool kv_requested = false;
 
-    auto load_record = [&](int pos) -> int {
-      int v = -1;
-      if (lane < 8) v = recs[(int64_t)pos * 8 + lane];
-      return v;
-    };
     auto clamp_e = [&](int e) { return e < q_end ? e : q_end - 1; };
 
     if (q_begin < q_end) {
-      int rec = load_record(clamp_e(q_begin + 1));
+      // the record of the block's second tile: with the first tile staged during the block before, it was
+      // requested (and waited for) there as well
       if (!staged) {
+        request_record(clamp_e(q_begin + 1));
         fetch(head, buf, b);
-        stage(buf);
+        request_stat(head, b);
+        stage(buf);  // waits for the two requests above inside this branch
         __syncthreads();
       }
+      int rec = rec_in_flight;
       for (int e = q_begin; e < q_end; ++e) {
         const char *base = smem + buf * kBufBytes;
         const int qb = qb_nxt;
@@ -1109,7 +1132,10 @@ __device__ __forceinline__ void attn_bwd_kv8_walk(const bsa_attn_args &a, char *
           batch_use = b_next;
         }
         if (next_tile) fetch(rec_use, buf ^ 1, batch_use);
-        rec = load_record(clamp_e(e + 2));
+        request_stat(rec_use, batch_use);
+        // the record of the tile after that one: of this block, or the second one of the next block
+        request_record((!more && next_tile) ? (q_begin_next + 1 < q_end_next ? q_begin_next + 1 : q_end_next - 1)
+                                            : clamp_e(e + 2));
 
         KvCarry carry;
         kv_first_half<Tr, NH, NHV, DK, DV>(carry, f0, live, a, base, qb, pm, pb, mbits, causal, seq_len, (int)kb, kpos,
@@ -1118,7 +1144,11 @@ __device__ __forceinline__ void attn_bwd_kv8_walk(const bsa_attn_args &a, char *
         kv_second_half<Tr, NH, NHV, DK, DV>(carry, live, a, base, pb, wi, wj, li, kg, lane, dkacc, dvacc, p_lds);
 
         if (next_tile) stage(buf ^ 1);
-        else __builtin_amdgcn_s_waitcnt(0x0F70);  // whatever this wave has requested (K / V of the next block) has landed
+        else {  // K / V of the next block, the record
+          __builtin_amdgcn_s_waitcnt(0x0F70);
+          asm volatile("" : "+v"(rec_in_flight) : : "memory");
+        }
+        rec = rec_in_flight;
         __syncthreads();
         buf ^= 1;
         staged = next_tile && !more;
