@@ -46,7 +46,7 @@ PEAK_MFMA_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}
 # what leaves an L2, so reads served by the memory-side cache are included.  Not re-measured by this script.
 TRAFFIC_KIB = {  # config: (FETCH_SIZE, WRITE_SIZE)
     "c1": (616.2, 476.0),
-    "c2": (337914.7, 514960.1),
+    "c2": (338582.0, 514960.1),
     "c3": (148153.3, 296259.0),
     "c4": (238469.4, 133139.0),
     "c5": (28438.4, 143960.0),
@@ -773,7 +773,7 @@ def make_workload(name, dev):
 CONFIGS = ["a1", "a1bwd", "c1", "c2", "c2bwd", "c3", "c3bwd", "c4", "c4bwd", "c5", "t1", "l1", "r1", "r2", "p1", "v1", "v2"]
 # the configurations a default run times behind the headline one, with fewer steps (their roofline objects ride
 # along in the same JSON line so that they are timed by whoever runs the script, not quoted from elsewhere)
-COMPANIONS = ["c4", "c3", "c5"]
+COMPANIONS = ["c4", "c4bwd", "c3", "c5"]
 
 
 def measure(config, dev, steps, warmup, scratch):
