@@ -335,7 +335,9 @@ typedef struct bsa_attn_args {
   int64_t n_layout_blocks;
   /* Non-zero: bwd_scratch still holds what an earlier bsa_attn_bwd call wrote for the same layouts, packed
    * indices, head counts, mask values and causal lengths (the records depend on nothing else), and the call
-   * reads it without writing it again. */
+   * reads it without writing it again.  Either way every call writes 64 bytes of the scratch (the tickets by
+   * which its dK / dV kernel hands key rows to the workgroups that stay for the launch), so two calls that
+   * overlap in time (different streams) need a scratch each. */
   int64_t bwd_scratch_ready;
 } bsa_attn_args;
 
