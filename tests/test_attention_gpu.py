@@ -324,7 +324,8 @@ def test_config4_full_size_against_sampled_oracle_rows_and_invariants(device):
     """Configuration 4 at full size (bf16, 64 heads, 8192 positions, head_dim 128, sbs 64, BigBird layout with
     causal mask blocks), where the oracle cannot run whole.  A query block row depends only on its own row of
     the layout, so the oracle is run on single rows (1 x 1 x 128 layouts against all keys of the head) and gives
-    the exact output and dQ of those rows.  Everything else is held to invariants of attention:
+    the exact output and dQ of those rows; a key block's dK and dV depend only on the rows that attend to it, so
+    the oracle on the sub-layout of those rows gives them exactly.  Everything else is held to invariants of attention:
     rows of P sum to 1, hence with V = 1 the output is 1 and sum_k dV[k, f] = sum_q dO[q, f];
     rows of dS sum to 0, hence sum_k dK[k, f] = 0; and two runs give identical bits (no atomics)."""
     BH, n, sbs, nh = 64, 128, 64, 2
@@ -370,6 +371,29 @@ def test_config4_full_size_against_sampled_oracle_rows_and_invariants(device):
         assert_close(out[rows], ref, 2e-2, f"O head {h} row {i}")
         ref.backward(go[rows].cpu().double())
         assert_close(dq[rows], q64.grad, 2e-2, f"dQ head {h} row {i}")
+
+    # sampled key blocks against the oracle (dK and dV): a key block's gradients come from the query block rows that
+    # attend to it, and those rows need all of their keys (for their softmax): the oracle runs on the sub-layout
+    # of exactly those rows, whose dK / dV of that key block are then complete.  Key block 1 is a global one (every
+    # later query block attends to it), the others have a handful of rows.
+    for h, j in ((0, 5), (21, 1), (63, 127), (40, 64)):
+        rows_of = torch.nonzero(la[h, :, j]).flatten()
+        head = slice(h * n * nh, (h + 1) * n * nh)
+        pick = torch.cat([torch.arange((h * n + int(i)) * nh, (h * n + int(i) + 1) * nh) for i in rows_of])
+        sub_layout = la[h, rows_of][None]
+        sub_lmask = lmask[h, rows_of][None]
+        mask_at = torch.cat([mask_offsets[(h * n + int(i)) * n + torch.nonzero(lmask[h, int(i)]).flatten()] for i in rows_of])
+        mk = mask[mask_at.to(device)].cpu() if len(mask_at) else None
+        ones = lambda a, b: torch.ones((1, a, b), dtype=torch.bool).numpy()
+        k64 = k[head].detach().cpu().double().requires_grad_(True)
+        v64 = v[head].detach().cpu().double().requires_grad_(True)
+        ref = orc.flash_attention(q[pick.to(device)].detach().cpu().double(), ones(len(rows_of), nh), k64, ones(n, nh),
+                                  v64, ones(n, nh), sub_layout.numpy(), sbs, mask=mk,
+                                  layout_mask=sub_lmask.numpy() if mk is not None else None, acc_dtype=torch.float64)
+        ref.backward(go[pick.to(device)].cpu().double())
+        mine = slice((h * n + j) * nh, (h * n + j + 1) * nh)
+        assert_close(dk[mine], k64.grad[j * nh:(j + 1) * nh], 2e-2, f"dK head {h} key block {j}")
+        assert_close(dv[mine], v64.grad[j * nh:(j + 1) * nh], 2e-2, f"dV head {h} key block {j}")
 
     # invariants over all heads
     with torch.no_grad():
