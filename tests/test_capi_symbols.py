@@ -63,8 +63,9 @@ def test_bad_arguments_of_the_neighbouring_entry_points_are_rejected_on_the_host
     assert lib.bsa_transpose_blocks(0, 0, 0, 0, 0, 0, 1, 1, 1, 64, 2, 0) == 0
     assert lib.bsa_layout_from_dense(0, 0, 1, 1, 1, 64, 1, 1, 0) == -1 and b"1 byte" in lib.bsa_last_error()
     assert lib.bsa_layout_from_dense(0, 0, 0, 1, 1, 64, 2, 1, 0) == 0
-    # scratch of the attention backward: 2 x 32 bytes per layout block, (4 + 64) per row, one per mask block
-    assert lib.bsa_attn_bwd_scratch_bytes(2, 3, 5, 7, 11) == (2 * 32 * 7 + 68 * (2 * 3 + 2 * 5) + 11 + 15) // 16 * 16
+    # scratch of the attention backward: 2 x 32 bytes per layout block, (4 + 64) per row, 64 bytes of tickets, one
+    # byte per mask block
+    assert lib.bsa_attn_bwd_scratch_bytes(2, 3, 5, 7, 11) == (2 * 32 * 7 + 68 * (2 * 3 + 2 * 5) + 64 + 11 + 15) // 16 * 16
     assert lib.bsa_attn_bwd_scratch_bytes(-1, 3, 5, 7, 11) == 0
     # records of the row kernel: parts_log2 in 0..3; without a table the rows are taken whole and in order
     assert lib.bsa_matmul_rows_records(0, 4, 4, 0, 0, 0, 4, 4, 0, 0, 0) == -1 and b"parts_log2" in lib.bsa_last_error()
