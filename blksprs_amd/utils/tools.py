@@ -24,7 +24,8 @@ _REFS = "_blksprs_cache_refs"
 _STATE = "_blksprs_cache_state"
 _CHECKED = "_blksprs_cache_checked"  # number of entries when the recorded state was last found valid
 _WATCH = "_blksprs_cache_watch"      # the recorded state once more, in a form that is cheap to compare
-_PRIVATE = frozenset((_KEY, _REFS, _STATE, _CHECKED, _WATCH))
+_SAME = "_blksprs_cache_same"        # the key once more, in a form that is cheap to compare (see _same_inputs)
+_PRIVATE = frozenset((_KEY, _REFS, _STATE, _CHECKED, _WATCH, _SAME))
 
 
 def as_base_tensor(value: Tensor) -> Tensor:
@@ -199,18 +200,50 @@ def prepare_layout_cache(layout_cache: LayoutCache | None, operation: str, *valu
     """
     if layout_cache is None:
         layout_cache = {}
-    key, refs = layout_cache_key(operation, *values)
     recorded = layout_cache.get(_STATE)
-    stale = layout_cache.get(_KEY) != key or recorded is None or not _unchanged(layout_cache, recorded)
+    if recorded is not None and _same_inputs(layout_cache.get(_SAME), operation, values):
+        stale = not _unchanged(layout_cache, recorded)
+        key = refs = None
+    else:
+        key, refs = layout_cache_key(operation, *values)
+        stale = layout_cache.get(_KEY) != key or recorded is None or not _unchanged(layout_cache, recorded)
     if stale:
+        if key is None:
+            key, refs = layout_cache_key(operation, *values)
         layout_cache.clear()
         layout_cache[_KEY] = key
         # holding the sources keeps their ids from being reused by other tensors
         layout_cache[_REFS] = refs
+        layout_cache[_SAME] = _same_inputs_record(operation, values)
     else:
         layout_cache.setdefault(_CHECKED, None)  # counted by len() below
         layout_cache[_CHECKED] = len(layout_cache)
     return layout_cache
+
+
+def _same_inputs_record(operation: str, values: tuple):
+    """What ``_same_inputs`` compares against, or ``None`` when some value is not a tensor with a version counter
+    (the full key decides then)."""
+    entries = []
+    for v in values:
+        if not isinstance(v, Tensor) or v.is_inference():
+            return None
+        entries.append((v, v._version, v.data_ptr(), v.requires_grad, v.shape))
+    return operation, tuple(entries)
+
+
+def _same_inputs(record, operation: str, values: tuple) -> bool:
+    """True when every value is the very tensor object the cache was filed under, not modified in place since (its
+    version counter), at the same address, of the same shape and with the same ``requires_grad``: the full key
+    (``layout_cache_key``) is then the recorded one, since the stride, dtype and device of an object only change
+    together with its version counter or its storage.  False means "compare the full key", not "different"."""
+    if record is None or record[0] != operation or len(record[1]) != len(values):
+        return False
+    for (tensor, version, address, requires_grad, shape), v in zip(record[1], values):
+        if (v is not tensor or v._version != version or v.data_ptr() != address or v.requires_grad != requires_grad
+                or v.shape != shape):
+            return False
+    return True
 
 
 def layout_cache_key(operation: str, *values: object) -> tuple[tuple, tuple]:
