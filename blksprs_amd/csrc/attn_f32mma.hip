@@ -51,9 +51,21 @@ struct Row4 {
   }
 };
 
-// value of the other lane groups' lanes of the same query row
-__device__ inline float across16(float v) { return __shfl_xor(v, 16); }
-__device__ inline float across32(float v) { return __shfl_xor(v, 32); }
+// This lane's value and the value of lane ^ 16 (lane ^ 32), as (the one from the lower, the one from the upper
+// group of 16 (32) lanes): v_permlane16_swap / v_permlane32_swap trade the odd groups of the first operand for the
+// even groups of the second, so with the same value in both operands one result holds the even groups' values
+// twice and the other the odd groups'.  One instruction, where a shuffle goes through LDS.
+__device__ inline void pair16(float v, float &lower, float &upper) {
+  // spelled out: both operands are read and written, and they must be two registers that hold the same value
+  lower = upper = v;
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(lower), "+v"(upper));
+}
+__device__ inline void pair32(float v, float &lower, float &upper) {
+  lower = upper = v;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(lower), "+v"(upper));
+}
+// the larger of two values, NaN if either is
+__device__ inline float nan_max(float a, float b) { return (b > a || b != b) ? b : a; }
 
 template <int SBS>
 struct F32mmaShape {
@@ -178,10 +190,11 @@ __global__ __launch_bounds__(F32mmaShape<SBS>::kThreads) void attn_fwd_f32mma_ke
       }
       // ---- online softmax of the row (its 4 lane groups hold different keys)
       {
-        const float o1 = across16(tile_max);
-        tile_max = (o1 > tile_max || o1 != o1) ? o1 : tile_max;
-        const float o2 = across32(tile_max);
-        tile_max = (o2 > tile_max || o2 != o2) ? o2 : tile_max;
+        float lower, upper;
+        pair16(tile_max, lower, upper);
+        tile_max = nan_max(lower, upper);
+        pair32(tile_max, lower, upper);
+        tile_max = nan_max(lower, upper);
       }
       const float m_new = (tile_max > row_m || tile_max != tile_max) ? tile_max : row_m;
       const bool nothing = m_new == -INFINITY;  // the row has seen no key so far
@@ -229,8 +242,13 @@ __global__ __launch_bounds__(F32mmaShape<SBS>::kThreads) void attn_fwd_f32mma_ke
   }
   // ---- the row's sum over its four lane groups; then the groups' results are merged: every group leaves
   // (m, l, O) of its rows in LDS, group 0 rescales them to the common maximum and adds them up
-  row_l += across16(row_l);
-  row_l += across32(row_l);
+  {
+    float lower, upper;
+    pair16(row_l, lower, upper);
+    row_l = lower + upper;
+    pair32(row_l, lower, upper);
+    row_l = lower + upper;
+  }
   constexpr int kRowFloats = NHV * SBS + 2;
   float *merge = f32mma_smem;  // [group][SBS][kRowFloats]
   __syncthreads();               // tiles and query slices are no longer read

@@ -386,7 +386,7 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
         float m_blk = sv[0];
   #pragma unroll
         for (int x = 1; x < 32; ++x) m_blk = fmaxf(m_blk, sv[x]);
-        m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 32)) * cc;
+        m_blk = max_across32(m_blk) * cc;
         // The reference maximum m_i of the exponentials only follows the running maximum when that has grown by
         // more than kRescaleStep since the last update (for some row of the wave): in between, probabilities may
         // exceed 1 (by at most 2^kRescaleStep) and the accumulators need no rescaling.  o and lse do not depend on
@@ -412,8 +412,7 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
           sv[x] = __builtin_amdgcn_exp2f(fmaf(sv[x], cc, -m_sub));
           sum += sv[x];
         }
-        sum += __shfl_xor(sum, 32);
-        l_i += sum;
+        l_i += sum;  // of this lane's 32 keys: the two halves of a row are added once, in the epilogue
 
         u32x4 pf[2][2];
   #pragma unroll
@@ -465,6 +464,7 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
   if (!has_q) return;
   // one reciprocal per row, then products: 64 IEEE divisions per lane cost ten instructions each, and the last
   // bit they would buy is rounded away with the other fifteen when the quotient becomes a 16-bit value
+  l_i = sum_across32(l_i);
   const float inv_l = (l_i != 0.f) ? 1.f / l_i : 0.f;
 #pragma unroll
   for (int h = 0; h < NHV; ++h) {

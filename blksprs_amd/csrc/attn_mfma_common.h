@@ -67,6 +67,21 @@ __device__ static inline u32x4 frag_cols_t(const char *lds, int row0, int col0, 
   return u32x4{l2[0], l2[1], h2[0], h2[1]};
 }
 
+// The values of lanes l and l ^ 32 of a wave, combined: one v_permlane32_swap (lanes 32 .. 63 of the first operand
+// trade places with lanes 0 .. 31 of the second; with the same value in both, one result holds the lower half's
+// values in both halves and the other the upper half's), no trip through LDS as a shuffle takes.  Every lane gets
+// lower (op) upper, so for a sum both lanes of a pair hold the same bits.
+__device__ static inline float max_across32(float v) {
+  float lower = v, upper = v;  // spelled out: two registers that hold the same value, both read and written
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(lower), "+v"(upper));
+  return fmaxf(lower, upper);
+}
+__device__ static inline float sum_across32(float v) {
+  float lower = v, upper = v;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(lower), "+v"(upper));
+  return lower + upper;
+}
+
 __device__ static inline int first_lane(int v) { return __builtin_amdgcn_readfirstlane(v); }
 typedef __attribute__((address_space(3))) void *lds_ptr_t;
 
