@@ -22,13 +22,41 @@ struct RowGeom {
   int groups_log2;  // wave tasks per block row = sbs * lpr / 64, as log2
 };
 
-__device__ inline float lanes_max(float v, int lpr) {
-  for (int d = 1; d < lpr; d <<= 1) v = fmaxf(v, __shfl_xor(v, d));
+// The reductions over the lpr lanes of an element row, without a trip through LDS (a shuffle computes a lane
+// address, goes through LDS and waits for it).  Steps 1 and 2 exchange inside a group of four lanes (DPP quad_perm);
+// after them the four lanes of a group agree, so mirroring a half row (lane i <-> 7 - i) pairs every group with its
+// neighbour and mirroring a row (i <-> 15 - i) pairs the two halves of 16 lanes: partners other than those of an
+// xor exchange, holding the same values.  Steps 16 and 32 trade register halves (v_permlane16_swap /
+// v_permlane32_swap with the same value in both operands: one result holds the even groups' values twice, the other
+// the odd groups').  Every step combines a value with its partner's by a commutative operation, so all lanes of a
+// row end with the same bits, as with xor shuffles.
+template <int CTRL>
+__device__ inline float dpp_partner(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+template <typename Op>
+__device__ inline float lanes_reduce(float v, int lpr, Op op) {
+  if (lpr > 1) v = op(v, dpp_partner<0xB1>(v));   // quad_perm [1, 0, 3, 2]
+  if (lpr > 2) v = op(v, dpp_partner<0x4E>(v));   // quad_perm [2, 3, 0, 1]
+  if (lpr > 4) v = op(v, dpp_partner<0x141>(v));  // row_half_mirror
+  if (lpr > 8) v = op(v, dpp_partner<0x140>(v));  // row_mirror
+  if (lpr > 16) {
+    float lower = v, upper = v;
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(lower), "+v"(upper));
+    v = op(lower, upper);
+  }
+  if (lpr > 32) {
+    float lower = v, upper = v;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(lower), "+v"(upper));
+    v = op(lower, upper);
+  }
   return v;
 }
+__device__ inline float lanes_max(float v, int lpr) {
+  return lanes_reduce(v, lpr, [](float a, float b) { return fmaxf(a, b); });
+}
 __device__ inline float lanes_sum(float v, int lpr) {
-  for (int d = 1; d < lpr; d <<= 1) v += __shfl_xor(v, d);
-  return v;
+  return lanes_reduce(v, lpr, [](float a, float b) { return a + b; });
 }
 
 // float offset of unit u, relative to the first block of the row and to the lane's own offset (the same for every
