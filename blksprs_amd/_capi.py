@@ -133,12 +133,19 @@ _WAITS_WITH_STATS_HOST = {"bsa_lut_packed": 6, "bsa_lut_contraction_offsets": 11
 host_waits = 0  # calls so far that made the host wait for the device inside the library
 
 
+_bound = {}  # entry point name -> bound foreign function (looked up once)
+
+
 def call(name: str, *args) -> None:
     global host_waits
-    at = _WAITS_WITH_STATS_HOST.get(name)
-    if at is not None and args[at]:
+    fn = _bound.get(name)
+    if fn is None:
+        fn = _bound[name] = getattr(load(), name)
+    if name in _WAITS_WITH_STATS_HOST and args[_WAITS_WITH_STATS_HOST[name]]:
         host_waits += 1
-    check(getattr(load(), name)(*args), name)
+    rc = fn(*args)
+    if rc != 0:
+        check(rc, name)
 
 
 class on_device:

@@ -26,7 +26,8 @@ def _launch(x: Tensor, y: Tensor, pair_offsets: Tensor, pairs: Tensor, order: Te
     out = torch.empty((n_out, sbs, sbs), dtype=x.dtype, device=x.device)
     if n_out:
         with _capi.on_device(x.device):
-            _capi.call("bsa_matmul", _capi.ptr(x), _capi.ptr(y), out.data_ptr(), pair_offsets.data_ptr(),
+            # x and y may be empty (no block at all): the library never reads an operand of zero blocks
+            _capi.call("bsa_matmul", x.data_ptr(), y.data_ptr(), out.data_ptr(), pair_offsets.data_ptr(),
                        _capi.ptr(pairs), _capi.ptr(order), n_out, x.size(0), y.size(0), sbs,
                        _capi.DTYPE_CODES[x.dtype], int(trans_x), int(trans_y), _capi.stream(x.device))
     return out

@@ -404,9 +404,14 @@ def eager_only(fn):
     the public function with ``torch.compiler.disable`` itself is not enough: ``torch.compile(fn)`` unwraps a
     disabled function it is handed directly and traces its body."""
     disabled = torch.compiler.disable(fn)
+    is_compiling = torch.compiler.is_compiling
 
     @functools.wraps(fn)
     def entry(*args, **kwargs):
+        # outside a trace the body is called as it is (the wrapper that keeps a trace out costs two microseconds
+        # per call); while this function is being traced the test is true and the trace ends at the call below
+        if not is_compiling():
+            return fn(*args, **kwargs)
         return disabled(*args, **kwargs)
 
     return entry

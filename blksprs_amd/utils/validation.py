@@ -80,6 +80,8 @@ def _check(fn):
 def ensure_contiguous(*tensors: Tensor):
     """Returns the operands made contiguous unless that was switched off."""
     if _contiguous_enabled():
+        if len(tensors) == 2:  # the common call, without a generator
+            return tensors[0].contiguous(), tensors[1].contiguous()
         tensors = tuple(t.contiguous() for t in tensors)
     return tensors[0] if len(tensors) == 1 else tensors
 
