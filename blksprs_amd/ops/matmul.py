@@ -14,8 +14,9 @@ from torch import Tensor
 
 from .. import _capi
 from ..utils.blksprs_tensor import BlksprsTensor
-from ..utils.tools import (build_contraction_lists, cast_for_autocast, eager_only, finalize_layout_cache,
-                           nonzero_from_packed, pack_layouts, prepare_layout_cache)
+from ..utils.tools import (build_contraction_lists, cast_for_autocast, count_contraction_pairs, eager_only,
+                           finalize_layout_cache, nonzero_from_packed, pack_layouts, prepare_layout_cache,
+                           write_contraction_pairs)
 from ..utils.validation import (ensure_contiguous, validate_contiguous, validate_device, validate_dimensions,
                                 validate_dtype_float, validate_shape, validate_sparsity, validate_sparsity_block_size,
                                 validate_sparsity_layout, validation_enabled)
@@ -204,10 +205,11 @@ def _backward_lists(plan: _Plan, shape_x, shape_y):
         C = int(shape_y[2])
         # operand layouts seen by the builder: dO (B,R,C) times Y^T (B,C,K) -> (B,R,K)
         pidx_yt = plan.packed_y.view(B, K, C).transpose(1, 2).contiguous().view(-1)
-        gx = build_contraction_lists(plan.packed_o, pidx_yt, plan.packed_x, B, R, C, K, plan.n_x)
         # X^T (B,K,R) times dO (B,R,C) -> (B,K,C)
         pidx_xt = plan.packed_x.view(B, R, K).transpose(1, 2).contiguous().view(-1)
-        gy = build_contraction_lists(pidx_xt, plan.packed_o, plan.packed_y, B, K, R, C, plan.n_y)
+        # both products' pair counts come back in one read
+        gx, gy = build_contraction_lists((plan.packed_o, pidx_yt, plan.packed_x, B, R, C, K, plan.n_x),
+                                         (pidx_xt, plan.packed_o, plan.packed_y, B, K, R, C, plan.n_y))
         plan.grad_lists = (gx.pair_offsets, gx.pairs, gy.pair_offsets, gy.pairs)
     return plan.grad_lists
 
@@ -269,9 +271,13 @@ def matmul_build_layout_cache(layout_cache: dict | None, sparsity_layout_x: Tens
     if "contraction_pairs" not in layout_cache:
         B, R, K = (int(s) for s in sparsity_layout_x.shape)
         C = int(sparsity_layout_y.size(2))
-        info_x, info_y, info_o = pack_layouts((sparsity_layout_x, K), (sparsity_layout_y, 0),
-                                              (sparsity_layout_output, C))
-        lists = build_contraction_lists(info_x.packed, info_y.packed, info_o.packed, B, R, K, C, info_o.count)
+        # the three scans and the count of the product's block pairs are launched one after the other, and
+        # their results (block counts, longest rows, number of pairs) come back in ONE read
+        counted = []
+        (info_x, info_y, info_o), (n_pairs, _) = pack_layouts(
+            (sparsity_layout_x, K), (sparsity_layout_y, 0), (sparsity_layout_output, C),
+            then=lambda packed: (counted.append(count_contraction_pairs(*packed, B, R, K, C)), counted[0].stats_dev)[1])
+        lists = write_contraction_pairs(counted[0], int(n_pairs), info_o.count)
         layout_cache["packed_indices_x"] = info_x.packed
         layout_cache["packed_indices_y"] = info_y.packed
         layout_cache["packed_indices_o"] = info_o.packed

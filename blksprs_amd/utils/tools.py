@@ -71,11 +71,14 @@ class PackedLayout:
         self.packed, self.count, self.row_offsets, self.max_per_row = packed, count, row_offsets, max_per_row
 
 
-def pack_layouts(*specs) -> list:
+def pack_layouts(*specs, then=None):
     """Scans several layouts on the device, ``specs`` being ``(layout, row_len)`` pairs: reverse index, block
     count and optional CSR row offsets of each.
 
-    One stream synchronisation for all of them (the counts size the caller's next allocations).
+    One stream synchronisation for all of them (the counts size the caller's next allocations).  ``then``, if
+    given, is called with the reverse indices before that synchronisation: it launches what depends on them
+    alone and returns an int64 device tensor of its own statistics, which are read back in the same transfer;
+    the function then returns ``(infos, statistics as a list)``.
     """
     lib = _capi.load()
     results = []
@@ -97,9 +100,17 @@ def pack_layouts(*specs) -> list:
                        row_offsets.data_ptr() if row_offsets is not None else 0,
                        stats_dev[number].data_ptr(), 0, _capi.ptr(workspace), ws_bytes, _capi.stream(dev))
         results.append((packed, row_offsets))
-    stats = stats_dev.tolist() if results else []
-    return [PackedLayout(packed, int(count), row_offsets, int(longest))
-            for (packed, row_offsets), (count, longest) in zip(results, stats)]
+    if then is None:
+        stats = stats_dev.tolist() if results else []
+        extra = None
+    else:
+        more = then([packed for packed, _ in results])
+        both = torch.cat([stats_dev.reshape(-1), more.reshape(-1)]).tolist()
+        stats = [both[2 * i:2 * i + 2] for i in range(len(results))]
+        extra = both[2 * len(results):]
+    infos = [PackedLayout(packed, int(count), row_offsets, int(longest))
+             for (packed, row_offsets), (count, longest) in zip(results, stats)]
+    return infos if then is None else (infos, extra)
 
 
 def pack_layout(layout: Tensor, row_len: int = 0) -> PackedLayout:
@@ -157,34 +168,62 @@ class ContractionLists:
         self.pair_offsets, self.pairs, self.n_pairs = pair_offsets, pairs, n_pairs
 
 
-def build_contraction_lists(pidx_x: Tensor, pidx_y: Tensor, pidx_o: Tensor, B: int, R: int, K: int, C: int,
-                            nnz_o: int) -> ContractionLists:
-    """Builds, on the device, for every active output block the ascending-k list of block pairs to multiply."""
+class _ContractionCounts:
+    """What phase 1 of the contraction lists leaves on the device for phase 2."""
+
+    __slots__ = ("operands", "dims", "mask_x", "mask_y", "pos_offsets", "stats_dev")
+
+
+def count_contraction_pairs(pidx_x: Tensor, pidx_y: Tensor, pidx_o: Tensor, B: int, R: int, K: int,
+                            C: int) -> _ContractionCounts:
+    """Phase 1 of the contraction lists (``bsa_lut_contraction_offsets``), launched without waiting for it: the
+    total number of pairs lies in ``stats_dev[0]`` on the device."""
     dev = pidx_o.device
     n = B * R * C
     W = (K + 63) // 64
-    mask_x = torch.empty(max(B * R * W, 1), dtype=torch.int64, device=dev)
-    mask_y = torch.empty(max(B * C * W, 1), dtype=torch.int64, device=dev)
-    pos_offsets = torch.empty(n + 1, dtype=torch.int32, device=dev)
-    stats_dev = torch.empty(2, dtype=torch.int64, device=dev)
-    stats_host = torch.empty(2, dtype=torch.int64, pin_memory=True)
-    lib = _capi.load()
-    ws_bytes = lib.bsa_lut_workspace_bytes(n)
+    c = _ContractionCounts()
+    c.operands, c.dims = (pidx_x, pidx_y, pidx_o), (B, R, K, C)
+    c.mask_x = torch.empty(max(B * R * W, 1), dtype=torch.int64, device=dev)
+    c.mask_y = torch.empty(max(B * C * W, 1), dtype=torch.int64, device=dev)
+    c.pos_offsets = torch.empty(n + 1, dtype=torch.int32, device=dev)
+    c.stats_dev = torch.empty(2, dtype=torch.int64, device=dev)
+    ws_bytes = _capi.load().bsa_lut_workspace_bytes(n)
     workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     with _capi.on_device(dev):
-        st = _capi.stream(dev)
         _capi.call("bsa_lut_contraction_offsets", _capi.ptr(pidx_x), _capi.ptr(pidx_y), _capi.ptr(pidx_o),
-                   B, R, K, C, mask_x.data_ptr(), mask_y.data_ptr(), pos_offsets.data_ptr(),
-                   stats_dev.data_ptr(), stats_host.data_ptr(), workspace.data_ptr(), ws_bytes, st)
-        total = int(stats_host[0])
-        if total > INT32_INDEX_MAX:
-            raise RuntimeError(f"block-sparse product has {total} block pairs; at most {INT32_INDEX_MAX} are supported")
-        pair_offsets = torch.empty(nnz_o + 1, dtype=torch.int32, device=dev)
-        pairs = torch.empty((total, 2), dtype=torch.int32, device=dev)
+                   B, R, K, C, c.mask_x.data_ptr(), c.mask_y.data_ptr(), c.pos_offsets.data_ptr(),
+                   c.stats_dev.data_ptr(), 0, workspace.data_ptr(), ws_bytes, _capi.stream(dev))
+    return c
+
+
+def write_contraction_pairs(c: _ContractionCounts, total: int, nnz_o: int) -> ContractionLists:
+    """Phase 2: the lists themselves, ``total`` being the number of pairs phase 1 counted."""
+    if total > INT32_INDEX_MAX:
+        raise RuntimeError(f"block-sparse product has {total} block pairs; at most {INT32_INDEX_MAX} are supported")
+    pidx_x, pidx_y, pidx_o = c.operands
+    B, R, K, C = c.dims
+    dev = pidx_o.device
+    pair_offsets = torch.empty(nnz_o + 1, dtype=torch.int32, device=dev)
+    pairs = torch.empty((total, 2), dtype=torch.int32, device=dev)
+    with _capi.on_device(dev):
         _capi.call("bsa_lut_contraction_pairs", _capi.ptr(pidx_x), _capi.ptr(pidx_y), _capi.ptr(pidx_o),
-                   B, R, K, C, mask_x.data_ptr(), mask_y.data_ptr(), pos_offsets.data_ptr(), nnz_o,
-                   pair_offsets.data_ptr(), _capi.ptr(pairs), st)
+                   B, R, K, C, c.mask_x.data_ptr(), c.mask_y.data_ptr(), c.pos_offsets.data_ptr(), nnz_o,
+                   pair_offsets.data_ptr(), _capi.ptr(pairs), _capi.stream(dev))
     return ContractionLists(pair_offsets, pairs, total)
+
+
+def build_contraction_lists(*products) -> "ContractionLists | list":
+    """Builds, on the device, for every active output block the ascending-k list of block pairs to multiply.
+
+    ``build_contraction_lists(pidx_x, pidx_y, pidx_o, B, R, K, C, nnz_o)`` for one product, or one such tuple per
+    product for several: their pair counts are read back together, one wait for the stream in all."""
+    one = not isinstance(products[0], tuple)
+    if one:
+        products = (products,)
+    counted = [count_contraction_pairs(*p[:7]) for p in products]
+    totals = torch.stack([c.stats_dev[0] for c in counted]).tolist()
+    lists = [write_contraction_pairs(c, int(total), p[7]) for c, total, p in zip(counted, totals, products)]
+    return lists[0] if one else lists
 
 
 # --------------------------------------------------------------------------- layout cache
