@@ -19,7 +19,8 @@ from .. import _capi
 from ..layouting.sparsity_layout import build_sparsity_layout_matmul
 from ..utils.blksprs_tensor import BlksprsTensor
 from ..utils.tools import (CacheHolder, INT32_INDEX_MAX, as_base_tensor, cast_for_autocast, csr_indices_from_packed,
-                           eager_only, finalize_layout_cache, pack_layout, prepare_layout_cache)
+                           PackedLayout, eager_only, finalize_layout_cache, nonzero_from_packed, pack_layout,
+                           pack_layouts, prepare_layout_cache)
 from ..utils.validation import (ensure_contiguous, mask_facts_enabled, validate_binary, validate_contiguous,
                                 validate_device, validate_dimensions, validate_dtype_float, validate_shape,
                                 validate_sparsity, validate_sparsity_block_size, validate_sparsity_layout)
@@ -33,18 +34,20 @@ def _select_segmented_index_dtype(n_active_blocks: int, n_blocks_col: int) -> to
 
 
 def _build_segmented_indices(attention_layout: Tensor, n_batches: int, n_blocks_row: int,
-                             n_blocks_col: int) -> tuple[Tensor, Tensor, int]:
+                             n_blocks_col: int, info=None) -> tuple[Tensor, Tensor, int]:
     """CSR adjacency of a ``(B, rows, cols)`` layout: ``(indices, offsets, max_blocks_per_row)``.
 
     ``offsets`` has ``B * rows + 1`` entries with a leading 0, ``indices`` lists the active columns of each row
-    in ascending order.  Empty and all-zero layouts yield ``(empty, zeros, 1)``.
+    in ascending order.  Empty and all-zero layouts yield ``(empty, zeros, 1)``.  ``info``: the layout's scan with
+    row offsets (``pack_layouts``), when the caller has made it together with others.
     """
     device = attention_layout.device
     n_rows = n_batches * n_blocks_row
     if attention_layout.numel() == 0:
         return (torch.empty(0, dtype=torch.int32, device=device),
                 torch.zeros(n_rows + 1, dtype=torch.int32, device=device), 1)
-    info = pack_layout(attention_layout, row_len=n_blocks_col)
+    if info is None:
+        info = pack_layout(attention_layout, row_len=n_blocks_col)
     if info.max_per_row == 0:
         return (torch.empty(0, dtype=torch.int32, device=device),
                 torch.zeros(n_rows + 1, dtype=torch.int32, device=device), 1)
@@ -57,7 +60,7 @@ def _build_segmented_indices(attention_layout: Tensor, n_batches: int, n_blocks_
 
 
 def _build_group_lists(attention_layout: Tensor, n_batches: int, n_blocks_row: int,
-                       n_blocks_col: int) -> tuple[Tensor, Tensor, int]:
+                       n_blocks_col: int, info=None) -> tuple[Tensor, Tensor, int]:
     """The attention layout as lists over pairs of neighbouring query blocks: ``(offsets, entries, group_size)``.
 
     A group is the pair of query blocks ``(2p, 2p+1)`` and its list the union of their key lists.  ``entries``
@@ -65,19 +68,31 @@ def _build_group_lists(attention_layout: Tensor, n_batches: int, n_blocks_row: i
     ``offsets`` has ``B * ceil(rows / 2) + 1`` int32 entries.  The forward kernel gives a pair to one workgroup,
     which fetches a K / V block both query blocks need once.  These lists have no counterpart in the reference.
     """
-    device = attention_layout.device
+    even, odd, union = _group_union(attention_layout, n_batches, n_blocks_row, n_blocks_col)
+    if info is None:
+        info = pack_layout(union, row_len=n_blocks_col)
+    # coordinates of the union's blocks from its scan (no read of the device: the count is known)
+    where = nonzero_from_packed(info.packed, union.shape, info.count)
+    flags = even[where[:, 0], where[:, 1], where[:, 2]].to(torch.int32) \
+        | (odd[where[:, 0], where[:, 1], where[:, 2]].to(torch.int32) << 1)
+    entries = (where[:, 2].to(torch.int32) | (flags << 28)).contiguous()
+    return as_base_tensor(info.row_offsets), as_base_tensor(entries), 2
+
+
+def _grouped_lists_apply(n_blocks_col, n_head_blocks, n_head_blocks_v) -> bool:
+    """Whether the matrix-core forward kernel's lists over pairs of query blocks can exist for these shapes (the
+    block size, which the cache builder does not know, has to be 64 as well)."""
+    return (n_head_blocks is not None and n_head_blocks_v is not None and n_blocks_col < (1 << 28)
+            and n_head_blocks <= 2 and n_head_blocks_v <= 2)
+
+
+def _group_union(attention_layout: Tensor, n_batches: int, n_blocks_row: int, n_blocks_col: int):
+    """``(even rows, odd rows, their union)`` of the attention layout as boolean ``(B, ceil(rows / 2), cols)``."""
     active = attention_layout.reshape(n_batches, n_blocks_row, n_blocks_col) != 0
     if n_blocks_row % 2:
         active = torch.cat([active, torch.zeros_like(active[:, :1])], dim=1)
     even, odd = active[:, 0::2], active[:, 1::2]
-    union = even | odd
-    where = torch.nonzero(union)
-    flags = even[where[:, 0], where[:, 1], where[:, 2]].to(torch.int32) \
-        | (odd[where[:, 0], where[:, 1], where[:, 2]].to(torch.int32) << 1)
-    entries = (where[:, 2].to(torch.int32) | (flags << 28)).contiguous()
-    offsets = torch.zeros(union.size(0) * union.size(1) + 1, dtype=torch.int32, device=device)
-    offsets[1:] = torch.cumsum(union.sum(dim=-1).reshape(-1), dim=0).to(torch.int32)
-    return as_base_tensor(offsets), as_base_tensor(entries), 2
+    return even, odd, (even | odd).contiguous()
 
 
 def flash_attention_build_layout_cache(attention_layout: Tensor,
@@ -174,30 +189,51 @@ def flash_attention_build_layout_cache(attention_layout: Tensor,
             layout_cache["sparsity_layout_o"] = build_sparsity_layout_matmul(attention_layout, sparsity_layout_v)
     resolved_o = layout_cache.get("sparsity_layout_o")
 
+    # Every layout this cache still has to scan, in ONE batch: the scans are queued one after the other and their
+    # counts come back in one read (a cold cache scans eight layouts; one by one that was eight waits).
+    wanted = []  # (what for, layout, row length)
+    if "key_indices" not in layout_cache and attention_layout.numel():
+        wanted.append(("keys", attention_layout, n_seq_blocks_k))
+    transposed = None
+    if "query_indices" not in layout_cache:
+        transposed = as_base_tensor(attention_layout.transpose(1, 2).contiguous())
+        if transposed.numel():
+            wanted.append(("queries", transposed, n_seq_blocks_q))
+    for name, layout in (("q", sparsity_layout_q), ("k", sparsity_layout_k), ("v", sparsity_layout_v),
+                         ("mask", sparsity_layout_mask), ("bias", sparsity_layout_bias), ("o", resolved_o)):
+        if layout is not None and f"packed_indices_{name}" not in layout_cache:
+            wanted.append((name, layout, 0))
+    if ("key_offsets_i32" not in layout_cache and _grouped_lists_apply(n_seq_blocks_k, n_head_blocks,
+                                                                       n_head_blocks_v)
+            and attention_layout.numel()):
+        wanted.append(("groups", _group_union(attention_layout, int(n_batches), int(n_seq_blocks_q),
+                                              int(n_seq_blocks_k))[2], n_seq_blocks_k))
+    scans = dict(zip((w[0] for w in wanted), pack_layouts(*((w[1], w[2]) for w in wanted)))) if wanted else {}
+
     if "key_indices" not in layout_cache:
         indices, offsets, longest = _build_segmented_indices(attention_layout, n_batches, n_seq_blocks_q,
-                                                             n_seq_blocks_k)
+                                                             n_seq_blocks_k, scans.get("keys"))
         layout_cache["key_indices"], layout_cache["key_offsets"] = indices, offsets
         layout_cache["max_keys_per_query"] = longest
 
     if "query_indices" not in layout_cache:
-        transposed = as_base_tensor(attention_layout.transpose(1, 2).contiguous())
-        indices, offsets, longest = _build_segmented_indices(transposed, n_batches, n_seq_blocks_k, n_seq_blocks_q)
+        indices, offsets, longest = _build_segmented_indices(transposed, n_batches, n_seq_blocks_k, n_seq_blocks_q,
+                                                             scans.get("queries"))
         layout_cache["query_indices"], layout_cache["query_offsets"] = indices, offsets
         layout_cache["max_queries_per_key"] = longest
 
-    for name, layout in (("q", sparsity_layout_q), ("k", sparsity_layout_k), ("v", sparsity_layout_v),
-                         ("mask", sparsity_layout_mask), ("bias", sparsity_layout_bias)):
-        if layout is not None and f"packed_indices_{name}" not in layout_cache:
-            info = pack_layout(layout)
+    for name in ("q", "k", "v", "mask", "bias", "o"):
+        info = scans.get(name)
+        if info is not None:
             layout_cache[f"packed_indices_{name}"] = info.packed
-            if name == "q":
-                layout_cache["n_sparse_blocks_q"] = info.count
-
-    if "packed_indices_o" not in layout_cache and resolved_o is not None:
-        info = pack_layout(resolved_o)
-        layout_cache["packed_indices_o"] = info.packed
-        layout_cache["n_sparse_blocks_o"] = info.count
+            if name in ("q", "o"):
+                layout_cache[f"n_sparse_blocks_{name}"] = info.count
+    if "groups" in scans:
+        # the scan of the union of neighbouring query rows, from which the operator makes the lists of the
+        # matrix-core forward kernel when the block size is 64
+        info = scans["groups"]
+        layout_cache["group_union_packed"], layout_cache["group_union_offsets"] = info.packed, info.row_offsets
+        layout_cache["group_union_count"] = info.count
 
     tensors = [v for v in layout_cache.values() if isinstance(v, Tensor)]
     if tensors:
@@ -232,10 +268,15 @@ def _as_index(t: Tensor | None, dtype: torch.dtype) -> Tensor | None:
 
 
 def _build_forward_records(layout_cache: dict, attention_layout: Tensor, n_batches: int, nq: int, nk: int,
-                           nh: int, nhv: int) -> tuple[Tensor, Tensor, int]:
+                           nh: int, nhv: int, own_layout: bool = False) -> tuple[Tensor, Tensor, int]:
     """``(group_offsets, group_records, group_size)``: the lists the matrix-core forward kernel walks, for an
-    attention layout and a layout cache that already holds the packed indices."""
-    offsets, entries, group_size = _build_group_lists(attention_layout, n_batches, nq, nk)
+    attention layout and a layout cache that already holds the packed indices.  ``own_layout``: the layout is
+    the one the cache was built for."""
+    info = None
+    if own_layout and "group_union_packed" in layout_cache:  # scanned with the cache's other layouts
+        info = PackedLayout(layout_cache["group_union_packed"], layout_cache["group_union_count"],
+                            layout_cache["group_union_offsets"], 0)
+    offsets, entries, group_size = _build_group_lists(attention_layout, n_batches, nq, nk, info)
     records = torch.zeros(entries.numel() * _capi.ATTN_RECORD_INTS, dtype=torch.int32, device=entries.device)
     a = _capi.AttnArgs()
     a.B, a.nq, a.nk, a.nh, a.nhv = n_batches, nq, nk, nh, nhv
@@ -575,7 +616,7 @@ def flash_attention(q: BlksprsTensor, sparsity_layout_q: Tensor,
                 and n_head_blocks_qk <= 2 and n_head_blocks_v <= 2 and sparsity_block_size == 64):
             offsets, records, group_size = _build_forward_records(
                 layout_cache, attention_layout, int(n_batches), int(n_seq_blocks_q), int(n_seq_blocks_k),
-                int(n_head_blocks_qk), int(n_head_blocks_v))
+                int(n_head_blocks_qk), int(n_head_blocks_v), own_layout=True)
             layout_cache["group_offsets"], layout_cache["group_records"] = offsets, records
             layout_cache["group_size"] = group_size
         layout_cache["tables"] = _Tables(layout_cache)

@@ -10,7 +10,7 @@ from torch import Tensor
 
 from .. import _capi
 from ..utils.blksprs_tensor import BlksprsTensor
-from ..utils.tools import (as_base_tensor, eager_only, finalize_layout_cache, nonzero_from_packed, pack_layout,
+from ..utils.tools import (as_base_tensor, eager_only, finalize_layout_cache, nonzero_from_packed, pack_layouts,
                            prepare_layout_cache)
 from ..utils.validation import (ensure_contiguous, validate_contiguous, validate_device, validate_dimensions,
                                 validate_dtype_supported, validate_sparsity, validate_sparsity_block_size)
@@ -87,16 +87,22 @@ def transpose_build_layout_cache(layout_cache: dict | None, sparsity_layout: Ten
             sparsity_layout_t = sparsity_layout_t.clone()
         layout_cache["sparsity_layout_t"] = sparsity_layout_t
 
-    if "packed_indices" not in layout_cache or "n_sparse_blocks" not in layout_cache:
-        info = pack_layout(sparsity_layout)
-        layout_cache["packed_indices"] = (info.packed.reshape(sparsity_layout.size())
-                                          .transpose(-1, -2).contiguous().reshape(-1))
-        layout_cache["n_sparse_blocks"] = info.count
-
-    if "layout_indices" not in layout_cache:
-        info_t = pack_layout(layout_cache["sparsity_layout_t"])
-        layout_cache["layout_indices"] = nonzero_from_packed(info_t.packed, layout_cache["sparsity_layout_t"].shape,
-                                                             info_t.count)
+    need_packed = "packed_indices" not in layout_cache or "n_sparse_blocks" not in layout_cache
+    need_indices = "layout_indices" not in layout_cache
+    if need_packed or need_indices:
+        # both scans in one batch: their counts come back in one read
+        specs = ([(sparsity_layout, 0)] if need_packed else []) + \
+                ([(layout_cache["sparsity_layout_t"], 0)] if need_indices else [])
+        infos = pack_layouts(*specs)
+        if need_packed:
+            info = infos[0]
+            layout_cache["packed_indices"] = (info.packed.reshape(sparsity_layout.size())
+                                              .transpose(-1, -2).contiguous().reshape(-1))
+            layout_cache["n_sparse_blocks"] = info.count
+        if need_indices:
+            info_t = infos[-1]
+            layout_cache["layout_indices"] = nonzero_from_packed(info_t.packed,
+                                                                 layout_cache["sparsity_layout_t"].shape, info_t.count)
 
     validate_contiguous(layout_cache["sparsity_layout_t"], layout_cache["layout_indices"],
                         layout_cache["packed_indices"])
