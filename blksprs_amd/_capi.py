@@ -70,6 +70,10 @@ SIGNATURES = {
     "bsa_softmax_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p]),
     "bsa_matmul": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int,
                            c_int, c_int, c_int, c_void_p]),
+    "bsa_lut_order_workspace_bytes": (c_size_t, [c_int64]),
+    "bsa_lut_block_order": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "bsa_lut_row_work_table": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int, c_int, c_int64, c_int, c_void_p,
+                                       c_int64, c_void_p, c_size_t, c_void_p]),
     "bsa_matmul_rows_records": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
                                         c_int64, c_void_p, c_void_p]),
     "bsa_matmul_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int64,

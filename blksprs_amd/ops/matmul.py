@@ -53,13 +53,17 @@ _SUPER_TILE = 16
 def _block_order(layout_indices: Tensor, n_rows: int, n_cols: int) -> Tensor:
     """Work order of the output blocks of a layout with ``n_rows`` x ``n_cols`` blocks per batch entry: 16 x 16
     super-tiles of the block grid, columns of super-tiles fastest, so that the blocks in flight on one L2 share
-    x row panels and y column panels."""
-    b, i, j = layout_indices[:, 0], layout_indices[:, 1], layout_indices[:, 2]
-    t = _SUPER_TILE
-    n_i = max(-(-n_rows // t), 1)
-    n_j = max(-(-n_cols // t), 1)
-    key = ((b * n_i + i // t) * n_j + j // t) * (t * t) + (i % t) * t + (j % t)
-    return torch.argsort(key, stable=True).to(torch.int32)
+    x row panels and y column panels (``bsa_lut_block_order``: built on the device, nothing is read back)."""
+    layout_indices = layout_indices.contiguous()  # torch.nonzero hands out column-major results
+    n = layout_indices.size(0)
+    order = torch.empty(n, dtype=torch.int32, device=layout_indices.device)
+    if n:
+        ws_bytes = _capi.load().bsa_lut_order_workspace_bytes(n)
+        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=layout_indices.device)
+        with _capi.on_device(layout_indices.device):
+            _capi.call("bsa_lut_block_order", layout_indices.data_ptr(), n, n_rows, n_cols, _SUPER_TILE,
+                       order.data_ptr(), workspace.data_ptr(), ws_bytes, _capi.stream(layout_indices.device))
+    return order
 
 
 _N_XCD = 8
@@ -113,9 +117,10 @@ _CUS_PER_XCD = 32
 
 
 def _row_work_table(pair_offsets: Tensor, row_offsets_o: Tensor, rows_per_batch: int, parts_log2: int,
-                    pair_up: bool = False, max_work: int | None = None, sweep: int = 0) -> Tensor:
+                    pair_up: bool = False, max_work: int = 0, sweep: int = 0) -> Tensor:
     """Order in which the row kernel hands parts of output block rows to workgroups: int32 entries
-    ``row << parts_log2 | part``, -1 for nothing.
+    ``row << parts_log2 | part``, -1 for nothing (``bsa_lut_row_work_table``: built on the device, nothing is read
+    back).
 
     Workgroup ``g`` runs on XCD ``g % 8``.  Every XCD gets one contiguous eighth of the rows (so the rows in
     flight on one L2 belong to the same batch entry and stream through the same y blocks), and walks it batch
@@ -130,51 +135,19 @@ def _row_work_table(pair_offsets: Tensor, row_offsets_o: Tensor, rows_per_batch:
     same compute units) downward, and so on: a part that starts finds the y blocks its predecessors read last
     still in the L2.
     ``max_work`` is a bound on the pairs of one row that the caller knows without asking the device (inner
-    blocks times output columns); without it the largest count is read back, which waits for the stream.
+    blocks times output columns).
     """
     n_rows = row_offsets_o.numel() - 1
     parts = 1 << parts_log2
     device = row_offsets_o.device
-    if n_rows == 0:
-        return torch.empty(0, dtype=torch.int32, device=device)
-    ends = pair_offsets[row_offsets_o.long()]
-    work = (ends[1:] - ends[:-1]).long()
-    small, extra = divmod(n_rows, _N_XCD)
-    # chunk c holds small + 1 rows for c < extra and small rows after that: plain arithmetic, nothing is copied
-    # to the device
-    all_rows = torch.arange(n_rows, device=device)
-    long_rows = extra * (small + 1)
-    chunk_of_row = torch.where(all_rows < long_rows, all_rows // (small + 1),
-                               extra + (all_rows - long_rows) // max(small, 1))
-    rows = all_rows.repeat_interleave(parts)
-    part = torch.arange(parts, device=device).repeat(n_rows)
-    entry = rows // max(rows_per_batch, 1)
-    n_entries = n_rows // max(rows_per_batch, 1) + 1
-    heaviest = int(work.max()) if max_work is None else int(max_work)
-    key = ((chunk_of_row[rows] * n_entries + entry) * parts + part) * (heaviest + 1) + (heaviest - work[rows])
-    by_chunk = torch.argsort(key, stable=True)  # chunk-major, batch entry, part, work descending
-    # position of every item inside its (chunk, batch entry, part) group, and the group's size (the number of
-    # groups is known here, so nothing is read back)
-    group = (key // (heaviest + 1))[by_chunk]
-    sizes_g = torch.zeros(_N_XCD * n_entries * parts, dtype=torch.int64, device=device)
-    sizes_g.scatter_add_(0, group, torch.ones_like(group))
-    starts = torch.cumsum(sizes_g, 0) - sizes_g
-    rank = torch.arange(rows.numel(), device=device) - starts[group]
-    if pair_up:
-        # within a group: longest, shortest, second longest, second shortest, ...
-        m = sizes_g[group]
-        spot = torch.where(rank < (m + 1) // 2, 2 * rank, 2 * (m - 1 - rank) + 1)
-        reordered = torch.empty_like(by_chunk)
-        reordered[starts[group] + spot] = by_chunk
-        by_chunk = reordered
-    chunk = chunk_of_row[rows][by_chunk]
-    first_of_chunk = (chunk * small + torch.clamp(chunk, max=extra)) * parts
-    within = torch.arange(rows.numel(), device=device) - first_of_chunk
-    table = torch.full(((small + (extra > 0)) * parts * _N_XCD,), -1, dtype=torch.int32, device=device)
-    items = (rows[by_chunk] << parts_log2) | part[by_chunk]
-    if sweep > 0:
-        items = items | (((rank // sweep) & 1) * _ROWS_DOWNWARD)
-    table[within * _N_XCD + chunk] = items.to(torch.int32)
+    table = torch.empty((-(-n_rows // _N_XCD)) * parts * _N_XCD, dtype=torch.int32, device=device)
+    if n_rows > 0:
+        ws_bytes = _capi.load().bsa_lut_order_workspace_bytes(n_rows * parts)
+        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=device)
+        with _capi.on_device(device):
+            _capi.call("bsa_lut_row_work_table", pair_offsets.data_ptr(), row_offsets_o.data_ptr(), n_rows,
+                       rows_per_batch, parts_log2, int(pair_up), int(max_work), int(sweep), table.data_ptr(),
+                       table.numel(), workspace.data_ptr(), ws_bytes, _capi.stream(device))
     return table
 
 

@@ -224,6 +224,34 @@ int bsa_matmul(const void *x, const void *y, void *out, const int32_t *pair_offs
                const int32_t *pairs, const int32_t *block_order, int64_t nnz_o, int64_t nnz_x, int64_t nnz_y, int sbs, int dtype,
                int trans_x, int trans_y, bsa_stream_t stream);
 
+/*
+ * Work orders of the matmul kernels, built on the device without a read by the host (integer only; a stable sort by a
+ * key computed from tables already on the device).  workspace: bsa_lut_order_workspace_bytes(n) bytes, 256-byte
+ * aligned, n = the number of items sorted (blocks, or n_rows << parts_log2).  No counterpart in the reference, whose
+ * kernels take output blocks in launch order (blksprs/ops/matmul.py:88-128); an order changes which blocks are in
+ * flight together, never a result.
+ *
+ * bsa_lut_block_order: order (int32 [n], a permutation) lists the n active blocks of a layout, given by their
+ * coordinates layout_indices (int64 [n, 3]: batch, row, column, as bsa_lut_nonzero writes them), by super-tiles of
+ * tile x tile blocks of the n_rows x n_cols block grid: the super-tiles of a batch entry row by row, the blocks of
+ * a super-tile row by row.  It is the block_order argument of bsa_matmul.
+ *
+ * bsa_lut_row_work_table: the work_table argument of bsa_matmul_rows_records (see there for the entries' format
+ * and for why the order is what it is): table_len = 8 * ceil(n_rows / 8) << parts_log2 entries; every XCD's
+ * contiguous eighth of the rows batch entry by batch entry (rows_per_batch rows each), part by part, the rows
+ * with the most (x, y) pairs first (pair_offsets, row_offsets_o as for bsa_matmul_rows_records; max_work: a bound
+ * on the pairs of one row, e.g. inner blocks times output columns).  pair_up != 0: within such a group longest,
+ * shortest, second longest, ...; sweep > 0: every second run of `sweep` entries of a group carries
+ * BSA_ROWS_DOWNWARD.
+ */
+size_t bsa_lut_order_workspace_bytes(int64_t n);
+int bsa_lut_block_order(const int64_t *layout_indices, int64_t n, int64_t n_rows, int64_t n_cols, int tile,
+                        int32_t *order, void *workspace, size_t workspace_bytes, bsa_stream_t stream);
+int bsa_lut_row_work_table(const int32_t *pair_offsets, const int32_t *row_offsets_o, int64_t n_rows,
+                           int64_t rows_per_batch, int parts_log2, int pair_up, int64_t max_work, int sweep,
+                           int32_t *table, int64_t table_len, void *workspace, size_t workspace_bytes,
+                           bsa_stream_t stream);
+
 #define BSA_ROWS_RECORD_INTS 128
 #define BSA_ROWS_DOWNWARD (1 << 30)
 

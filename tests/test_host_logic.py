@@ -173,9 +173,14 @@ def test_unknown_autotune_mode_is_rejected():
 def test_row_work_table_holds_every_part_once_and_keeps_eighths_together():
     """The table of the row kernel: entries row << parts_log2 | part, the k-th item of the c-th contiguous
     eighth of the rows at position 8 k + c, -1 where an eighth has a row less; inside an eighth batch entries
-    ascend, parts ascend inside an entry, and inside a part the rows with the most pairs come first."""
+    ascend, parts ascend inside an entry, and inside a part the rows with the most pairs come first.  Checked
+    here on the restatement in torch that the device builder is held to bit for bit (test_lut_gpu.py)."""
     import importlib
-    mm = importlib.import_module("blksprs_amd.ops.matmul")
+    from types import SimpleNamespace
+    from tests import helpers
+    real = importlib.import_module("blksprs_amd.ops.matmul")
+    mm = SimpleNamespace(_row_work_table=helpers.expected_row_work_table, _ROWS_DOWNWARD=helpers.ROWS_DOWNWARD,
+                         _row_parts_log2=real._row_parts_log2)
     g = torch.Generator().manual_seed(5)
     for n_rows, rows_per_batch, parts_log2 in ((1024, 64, 0), (1024, 64, 1), (21, 7, 2), (5, 5, 1), (8, 1, 3)):
         blocks_per_row = 9

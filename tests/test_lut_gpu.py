@@ -130,3 +130,49 @@ def test_cached_metadata_are_plain_tensors_and_cache_invalidates(device):
     kept.add_(0)
     bs.ops.to_sparse(x, other, 16, layout_cache=cache)
     assert cache["layout_indices"] is not kept
+
+
+@pytest.mark.parametrize("n_rows,rows_per_batch,parts_log2", [(1024, 64, 0), (1024, 64, 1), (21, 7, 2), (5, 5, 1),
+                                                              (8, 1, 3), (3, 3, 0), (4099, 128, 0)])
+def test_row_work_table_of_the_device_equals_its_restatement(device, n_rows, rows_per_batch, parts_log2):
+    """``bsa_lut_row_work_table`` (keys on the device, a stable radix sort, placement by binary search) against the
+    restatement in torch, bit for bit: plain, with a sweep, with long and short rows paired, and with a bound on the
+    work that is far above the largest row."""
+    import importlib
+    from tests import helpers
+    mm = importlib.import_module("blksprs_amd.ops.matmul")
+    g = torch.Generator().manual_seed(n_rows + parts_log2)
+    blocks_per_row = 9
+    row_offsets = torch.arange(n_rows + 1, dtype=torch.int32) * blocks_per_row
+    pair_offsets = torch.cumsum(torch.randint(0, 6, (n_rows * blocks_per_row + 1,), generator=g), 0).to(torch.int32)
+    bound = 5 * blocks_per_row
+    for pair_up, sweep, max_work in ((False, 0, bound), (False, 3, bound), (True, 0, bound), (False, 32, 1000 * bound)):
+        want = helpers.expected_row_work_table(pair_offsets, row_offsets, rows_per_batch, parts_log2, pair_up,
+                                               max_work=max_work, sweep=sweep)
+        got = mm._row_work_table(pair_offsets.to(device), row_offsets.to(device), rows_per_batch, parts_log2, pair_up,
+                                 max_work=max_work, sweep=sweep)
+        assert got.dtype == torch.int32 and torch.equal(got.cpu(), want), (pair_up, sweep)
+    # many rows of equal work keep their order (the sort is stable)
+    flat = torch.arange(n_rows * blocks_per_row + 1, dtype=torch.int32) * 2
+    want = helpers.expected_row_work_table(flat, row_offsets, rows_per_batch, parts_log2, max_work=2 * blocks_per_row)
+    got = mm._row_work_table(flat.to(device), row_offsets.to(device), rows_per_batch, parts_log2,
+                             max_work=2 * blocks_per_row)
+    assert torch.equal(got.cpu(), want)
+    # no rows: an empty table, nothing launched
+    assert mm._row_work_table(torch.zeros(1, dtype=torch.int32, device=device),
+                              torch.zeros(1, dtype=torch.int32, device=device), 1, 1).numel() == 0
+
+
+@pytest.mark.parametrize("shape,density", [((3, 40, 37), 0.3), ((1, 5, 130), 0.9), ((2, 64, 64), 0.02), ((1, 1, 1), 1.0)])
+def test_block_order_of_the_device_equals_its_restatement(device, shape, density):
+    """``bsa_lut_block_order`` against the stable argsort of the same key in torch, and as a permutation."""
+    import importlib
+    from tests import helpers
+    mm = importlib.import_module("blksprs_amd.ops.matmul")
+    layout = rand_layout(shape, density, 11, ensure_rows=True)
+    coords = torch.nonzero(layout)
+    got = mm._block_order(coords.to(device), shape[1], shape[2]).cpu()
+    want = helpers.expected_block_order(coords, shape[1], shape[2])
+    assert got.dtype == torch.int32 and torch.equal(got, want)
+    assert torch.equal(torch.sort(got.long())[0], torch.arange(coords.size(0)))
+    assert mm._block_order(torch.empty((0, 3), dtype=torch.int64, device=device), 4, 4).numel() == 0
