@@ -339,38 +339,6 @@ __global__ __launch_bounds__(kOrderThreads) void attn_bwd_order_kernel(bsa_attn_
   for (int64_t r = r0 + tid; r < r1; r += kOrderThreads) emit(r0 + atomicAdd(&bins[bin_of(r)], 1), r);
 }
 
-// ---------------------------------------------------------------------------------------------------------
-// delta[b, qb, i] = sum over active output slices of rowsum(o * dO); four lanes per query row
-template <typename Tr>
-__global__ __launch_bounds__(kBwdThreads) void attn_bwd_delta_kernel(bsa_attn_args a) {
-  const int64_t row = blockIdx.x;  // b * nq + qb
-  const int tid = threadIdx.x;
-  // the dK / dV kernel that follows hands out key rows by tickets: the workgroups of an XCD start with the
-  // positions 0 .. slots - 1 of its eighth, the next one to hand out is `slots`
-  if (row == 0 && tid < 8) bwd_lists(a).kv_tickets[tid] = (int32_t)kv_slots(a.B * a.nk);
-  const int i = tid >> 2, part = tid & 3;
-  float acc = 0.f;
-  for (int64_t h = 0; h < a.nhv; ++h) {
-    const int64_t po = a.pidx_o[row * a.nhv + h];
-    if (po < 0 || po >= a.n_o_blocks) continue;
-    const char *ob = static_cast<const char *>(a.o) + po * kBlockBytes + i * 128 + part * 32;
-    const char *gb = static_cast<const char *>(a.d_o) + po * kBlockBytes + i * 128 + part * 32;
-#pragma unroll
-    for (int c = 0; c < 2; ++c) {
-      const u32x4 ov = *reinterpret_cast<const u32x4 *>(ob + 16 * c);
-      const u32x4 gv = *reinterpret_cast<const u32x4 *>(gb + 16 * c);
-#pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        acc = fmaf(Tr::widen((uint16_t)(ov[t] & 0xffffu)), Tr::widen((uint16_t)(gv[t] & 0xffffu)), acc);
-        acc = fmaf(Tr::widen((uint16_t)(ov[t] >> 16)), Tr::widen((uint16_t)(gv[t] >> 16)), acc);
-      }
-    }
-  }
-  acc += __shfl_xor(acc, 1);
-  acc += __shfl_xor(acc, 2);
-  if (part == 0) a.delta[row * kSbs + i] = acc;
-}
-
 // The work of one wave on one tile (a query block in LDS at `base`, this wave's quadrant of the 64 x 64 scores):
 // S and dP, P and dS, then dV^T += dO^T P and / or dK^T += Q^T dS.  mbits: the mask bytes of this lane's 16
 // scores, one bit each (0 when the tile has no mask block).
@@ -1266,8 +1234,11 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_q_kernel(bsa_attn_arg
   const int li = lane & 31, kg = lane >> 5;
   const int wi = wave & 1, wj = wave >> 1;
   const int64_t qpos_in_order = xcd_row();
-  if (qpos_in_order >= a.B * a.nq) return;
   const BwdLists lists = bwd_lists(a);
+  // the dK / dV kernel that follows hands out key rows by tickets: the workgroups of an XCD start with the
+  // positions 0 .. slots - 1 of its eighth, the next one to hand out is `slots`
+  if (blockIdx.x == 0 && tid < 8) lists.kv_tickets[tid] = (int32_t)kv_slots(a.B * a.nk);
+  if (qpos_in_order >= a.B * a.nq) return;
   // the workgroup's header, int i in lane i (lanes 0 .. 7 double as the record of the first tile)
   int head = -1;
   if (lane < 16) head = lists.q_head[qpos_in_order * 16 + lane];
@@ -1281,19 +1252,40 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_q_kernel(bsa_attn_arg
     pq[h] = __builtin_amdgcn_readlane(head, 11 + h);
     any = any || pq[h] >= 0;
   }
-  if (!any) return;
 
   // this wave's queries: B operands Q[i][.], dO[i][.] with i = 32 wi + li
   const int qi = 32 * wi + li;
   u32x4 qfr[NH][4], dofr[NHV][4];
 #pragma unroll
-  for (int h = 0; h < NH; ++h) load_resident(qfr[h], a.q, pq[h], a.n_q_blocks, qi, kg);
-#pragma unroll
   for (int h = 0; h < NHV; ++h) load_resident(dofr[h], a.d_o, __builtin_amdgcn_readlane(head, 13 + h), a.n_o_blocks, qi, kg);
+#pragma unroll
+  for (int h = 0; h < NH; ++h) load_resident(qfr[h], a.q, pq[h], a.n_q_blocks, qi, kg);
   // a query without any visible key has lse = -inf and P = 0 everywhere: +inf gives exp2(s - lse) = 0 for it
   const float lse_raw = a.lse[qrow * kSbs + qi];
   const float lse = lse_raw == -INFINITY ? INFINITY : lse_raw;
-  const float delta = a.delta[qrow * kSbs + qi];
+  // delta[i] = sum over the output slices of rowsum(o * dO) of the wave's queries, from the dO fragments it holds
+  // anyway and the same pieces of o: the two lanes of a query hold every other 16-byte piece of its rows.  The
+  // dK / dV kernel, which runs after this one, reads it from a.delta; it needs it for every row that has a pair,
+  // with or without a q block, so this comes before the test below.  Both key halves compute the same bits; the
+  // first writes them.
+  float delta = 0.f;
+  {
+    u32x4 ofr[NHV][4];
+#pragma unroll
+    for (int h = 0; h < NHV; ++h) load_resident(ofr[h], a.o, __builtin_amdgcn_readlane(head, 13 + h), a.n_o_blocks, qi, kg);
+#pragma unroll
+    for (int h = 0; h < NHV; ++h)
+#pragma unroll
+      for (int s4 = 0; s4 < 4; ++s4)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          delta = fmaf(Tr::widen((uint16_t)(ofr[h][s4][t] & 0xffffu)), Tr::widen((uint16_t)(dofr[h][s4][t] & 0xffffu)), delta);
+          delta = fmaf(Tr::widen((uint16_t)(ofr[h][s4][t] >> 16)), Tr::widen((uint16_t)(dofr[h][s4][t] >> 16)), delta);
+        }
+    delta = sum_across32(delta);
+    if (wj == 0 && kg == 0) a.delta[qrow * kSbs + qi] = delta;
+  }
+  if (!any) return;
 
   f32x16 dqacc[NH * 2];
 #pragma unroll
@@ -1514,9 +1506,13 @@ int launch_bwd(const bsa_attn_args &a, hipStream_t s) {
     attn_bwd_order_kernel<<<16, kOrderThreads, 0, s>>>(a);
     if (int rc = check_launch("attn_bwd_order_kernel")) return rc;
   }
+  // dQ first: its kernel also leaves delta = rowsum(o * dO) and the tickets for the dK / dV kernel
   if (qrows > 0) {
-    attn_bwd_delta_kernel<Tr><<<(unsigned)qrows, kBwdThreads, 0, s>>>(a);
-    if (int rc = check_launch("attn_bwd_delta_kernel")) return rc;
+    constexpr int lds = 2 * (NH + NHV) * kBlockBytes;
+    BSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_bwd_q_kernel<Tr, NH, NHV>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    attn_bwd_q_kernel<Tr, NH, NHV><<<(unsigned)(cdiv(qrows, 8) * 8), kBwdThreads, lds, s>>>(a);
+    if (int rc = check_launch("attn_bwd_q_kernel")) return rc;
   }
   if (krows > 0) {
     constexpr int lds = 2 * ((NH + NHV) * kBlockBytes + kStatBytes + kSbs * kSbs);
@@ -1550,13 +1546,6 @@ int launch_bwd(const bsa_attn_args &a, hipStream_t s) {
       attn_bwd_kv_kernel<Tr, NH, NHV, true, true><<<(unsigned)(cdiv(krows, 8) * 8), kBwdThreads, lds, s>>>(a);
       if (int rc = check_launch("attn_bwd_kv_kernel")) return rc;
     }
-  }
-  if (qrows > 0) {
-    constexpr int lds = 2 * (NH + NHV) * kBlockBytes;
-    BSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_bwd_q_kernel<Tr, NH, NHV>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-    attn_bwd_q_kernel<Tr, NH, NHV><<<(unsigned)(cdiv(qrows, 8) * 8), kBwdThreads, lds, s>>>(a);
-    if (int rc = check_launch("attn_bwd_q_kernel")) return rc;
   }
   return BSA_OK;
 }
