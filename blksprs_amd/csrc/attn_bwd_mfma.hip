@@ -1278,10 +1278,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_q_kernel(bsa_attn_arg
 #pragma unroll
       for (int s4 = 0; s4 < 4; ++s4)
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          delta = fmaf(Tr::widen((uint16_t)(ofr[h][s4][t] & 0xffffu)), Tr::widen((uint16_t)(dofr[h][s4][t] & 0xffffu)), delta);
-          delta = fmaf(Tr::widen((uint16_t)(ofr[h][s4][t] >> 16)), Tr::widen((uint16_t)(dofr[h][s4][t] >> 16)), delta);
-        }
+        for (int t = 0; t < 4; ++t) delta = Tr::dot2(ofr[h][s4][t], dofr[h][s4][t], delta);
     delta = sum_across32(delta);
     if (wj == 0 && kg == 0) a.delta[qrow * kSbs + qi] = delta;
   }
