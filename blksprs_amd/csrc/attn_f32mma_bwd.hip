@@ -416,18 +416,32 @@ __global__ __launch_bounds__(BwdShape<SBS>::kThreads) void attn_f32mma_dq_kernel
     Quad<Tr>::store(static_cast<E *>(a.dq) + (pq * SBS + qi) * SBS + 16 * c + 4 * grp, dq[c] * a.scale);
 }
 
-template <typename T>
-__global__ void f32mma_zero_kernel(T *p, int64_t n) {
+// dq, dk, dv (and the bias gradient) set to zero by ONE launch: the lengths one after the other
+template <typename E>
+__global__ void f32mma_zero_kernel(E *dq, int64_t n_dq, E *dk, int64_t n_dk, E *dv, int64_t n_dv, float *dbias,
+                                   int64_t n_dbias) {
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) p[i] = (T)0;
+  const int64_t total = n_dq + n_dk + n_dv + n_dbias;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+    if (i < n_dq) dq[i] = (E)0;
+    else if (i < n_dq + n_dk) dk[i - n_dq] = (E)0;
+    else if (i < n_dq + n_dk + n_dv) dv[i - n_dq - n_dk] = (E)0;
+    else dbias[i - n_dq - n_dk - n_dv] = 0.f;
+  }
 }
 
-template <typename T>
-int zero_fill(T *p, int64_t n, hipStream_t s) {
-  if (!p || n <= 0) return BSA_OK;
-  int64_t blocks = cdiv(n, (int64_t)256);
+template <typename E>
+int zero_fill(E *dq, int64_t n_dq, E *dk, int64_t n_dk, E *dv, int64_t n_dv, float *dbias, int64_t n_dbias,
+              hipStream_t s) {
+  n_dq = dq && n_dq > 0 ? n_dq : 0;
+  n_dk = dk && n_dk > 0 ? n_dk : 0;
+  n_dv = dv && n_dv > 0 ? n_dv : 0;
+  n_dbias = dbias && n_dbias > 0 ? n_dbias : 0;
+  const int64_t total = n_dq + n_dk + n_dv + n_dbias;
+  if (total == 0) return BSA_OK;
+  int64_t blocks = cdiv(total, (int64_t)256);
   if (blocks > 65536) blocks = 65536;
-  f32mma_zero_kernel<T><<<(unsigned)blocks, 256, 0, s>>>(p, n);
+  f32mma_zero_kernel<E><<<(unsigned)blocks, 256, 0, s>>>(dq, n_dq, dk, n_dk, dv, n_dv, dbias, n_dbias);
   return check_launch("f32mma_zero_kernel");
 }
 
@@ -437,10 +451,9 @@ int bwd_f32mma(const bsa_attn_args &a, hipStream_t s) {
   using S = BwdShape<SBS>;
   const int64_t bs = (int64_t)SBS * SBS;
   // blocks no workgroup reaches (inactive counterpart slices) and bias blocks outside the attention layout stay zero
-  if (int rc = zero_fill(static_cast<E *>(a.dq), a.n_q_blocks * bs, s)) return rc;
-  if (int rc = zero_fill(static_cast<E *>(a.dk), a.n_k_blocks * bs, s)) return rc;
-  if (int rc = zero_fill(static_cast<E *>(a.dv), a.n_v_blocks * bs, s)) return rc;
-  if (int rc = zero_fill(a.dbias, a.n_bias_blocks * bs, s)) return rc;
+  if (int rc = zero_fill(static_cast<E *>(a.dq), a.n_q_blocks * bs, static_cast<E *>(a.dk), a.n_k_blocks * bs,
+                         static_cast<E *>(a.dv), a.n_v_blocks * bs, a.dbias, a.n_bias_blocks * bs, s))
+    return rc;
   const int64_t qrows = a.B * a.nq, krows = a.B * a.nk;
   if (qrows > 0) {
     attn_f32mma_delta_kernel<Tr><<<(unsigned)qrows, 64, 0, s>>>(a);
