@@ -67,6 +67,14 @@ def test_bad_arguments_of_the_neighbouring_entry_points_are_rejected_on_the_host
     # byte per mask block
     assert lib.bsa_attn_bwd_scratch_bytes(2, 3, 5, 7, 11) == (2 * 32 * 7 + 68 * (2 * 3 + 2 * 5) + 64 + 11 + 15) // 16 * 16
     assert lib.bsa_attn_bwd_scratch_bytes(-1, 3, 5, 7, 11) == 0
+    # work orders built on the device: sizes, part counts, the table's length, the bound on a row's pairs
+    assert lib.bsa_lut_block_order(0, -1, 4, 4, 16, 0, 0, 0, 0) == -1 and b"number of blocks" in lib.bsa_last_error()
+    assert lib.bsa_lut_block_order(0, 4, 4, 4, 0, 0, 0, 0, 0) == -1 and b"tile size" in lib.bsa_last_error()
+    assert lib.bsa_lut_block_order(0, 0, 4, 4, 16, 0, 0, 0, 0) == 0  # nothing to order
+    assert lib.bsa_lut_row_work_table(0, 0, 8, 4, 4, 0, 10, 0, 0, 8, 0, 0, 0) == -1 and b"parts_log2" in lib.bsa_last_error()
+    assert lib.bsa_lut_row_work_table(0, 0, 9, 3, 1, 0, 10, 0, 0, 8, 0, 0, 0) == -1 and b"are needed" in lib.bsa_last_error()
+    assert lib.bsa_lut_row_work_table(0, 0, 9, 3, 1, 0, -1, 0, 0, 32, 0, 0, 0) == -1 and b"bound" in lib.bsa_last_error()
+    assert lib.bsa_lut_row_work_table(0, 0, 0, 3, 1, 0, 10, 0, 0, 0, 0, 0, 0) == 0  # no rows
     # records of the row kernel: parts_log2 in 0..3; without a table the rows are taken whole and in order
     assert lib.bsa_matmul_rows_records(0, 4, 4, 0, 0, 0, 4, 4, 0, 0, 0) == -1 and b"parts_log2" in lib.bsa_last_error()
     assert lib.bsa_matmul_rows_records(0, 8, 1, 0, 0, 0, 4, 4, 0, 0, 0) == -1 and b"work table" in lib.bsa_last_error()
