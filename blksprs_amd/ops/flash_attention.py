@@ -23,7 +23,8 @@ from ..utils.tools import (CacheHolder, INT32_INDEX_MAX, as_base_tensor, cast_fo
                            pack_layouts, prepare_layout_cache)
 from ..utils.validation import (ensure_contiguous, mask_facts_enabled, validate_binary, validate_contiguous,
                                 validate_device, validate_dimensions, validate_dtype_float, validate_shape,
-                                validate_sparsity, validate_sparsity_block_size, validate_sparsity_layout)
+                                validate_sparsity, validate_sparsity_block_size, validate_sparsity_layout,
+                                validation_enabled)
 
 
 def _select_segmented_index_dtype(n_active_blocks: int, n_blocks_col: int) -> torch.dtype:
@@ -127,21 +128,22 @@ def flash_attention_build_layout_cache(attention_layout: Tensor,
         dict: The populated layout metadata cache.
 
     """
-    validate_dimensions(attention_layout)
-    validate_contiguous(attention_layout)
-    validate_sparsity_layout(attention_layout)
-
     named = (("sparsity_layout_q", sparsity_layout_q), ("sparsity_layout_k", sparsity_layout_k),
              ("sparsity_layout_v", sparsity_layout_v), ("sparsity_layout_o", sparsity_layout_o),
              ("sparsity_layout_mask", sparsity_layout_mask), ("sparsity_layout_bias", sparsity_layout_bias))
-    given = tuple(layout for _, layout in named if layout is not None)
-    if given:
-        validate_dimensions(*given)
-        validate_contiguous(*given)
-        validate_device(attention_layout, *given)
-        validate_sparsity_layout(*given)
-    else:
-        validate_device(attention_layout)
+    checking = validation_enabled()  # one test here instead of one in every check below
+    if checking:
+        validate_dimensions(attention_layout)
+        validate_contiguous(attention_layout)
+        validate_sparsity_layout(attention_layout)
+        given = tuple(layout for _, layout in named if layout is not None)
+        if given:
+            validate_dimensions(*given)
+            validate_contiguous(*given)
+            validate_device(attention_layout, *given)
+            validate_sparsity_layout(*given)
+        else:
+            validate_device(attention_layout)
 
     n_batches, rows_q, rows_k = attention_layout.shape
     if n_seq_blocks_q is None:
@@ -171,9 +173,10 @@ def flash_attention_build_layout_cache(attention_layout: Tensor,
         "sparsity_layout_mask": (n_batches, n_seq_blocks_q, n_seq_blocks_k),
         "sparsity_layout_bias": (n_batches, n_seq_blocks_q, n_seq_blocks_k),
     }
-    for name, layout in named:
-        if layout is not None:
-            validate_shape(layout, expected[name], name)
+    if checking:
+        for name, layout in named:
+            if layout is not None:
+                validate_shape(layout, expected[name], name)
 
     layout_cache = prepare_layout_cache(
         layout_cache, "flash_attention",
@@ -521,19 +524,22 @@ def flash_attention(q: BlksprsTensor, sparsity_layout_q: Tensor,
     q, k, v, attention_layout = ensure_contiguous(q, k, v, attention_layout)
     q, k, v = cast_for_autocast(q, k, v)
 
-    validate_dimensions(q, k, v)
-    validate_contiguous(q, k, v)
-    validate_dtype_float(q, k, v)
-    validate_device(q, k, v)
-    validate_sparsity(sparsity_block_size, (q, sparsity_layout_q), (k, sparsity_layout_k), (v, sparsity_layout_v))
-    validate_sparsity_block_size(sparsity_block_size, q, k, v)
+    checking = validation_enabled()  # one test for each group of checks instead of one inside every check
+    if checking:
+        validate_dimensions(q, k, v)
+        validate_contiguous(q, k, v)
+        validate_dtype_float(q, k, v)
+        validate_device(q, k, v)
+        validate_sparsity(sparsity_block_size, (q, sparsity_layout_q), (k, sparsity_layout_k), (v, sparsity_layout_v))
+        validate_sparsity_block_size(sparsity_block_size, q, k, v)
     if sparsity_block_size > 64:
         raise ValueError("Flash Attention sparsity block size must be at most 64")
 
-    validate_dimensions(attention_layout)
-    validate_contiguous(attention_layout)
-    validate_device(attention_layout, q)
-    validate_sparsity_layout(attention_layout)
+    if checking:
+        validate_dimensions(attention_layout)
+        validate_contiguous(attention_layout)
+        validate_device(attention_layout, q)
+        validate_sparsity_layout(attention_layout)
 
     n_batches = sparsity_layout_q.size(0)
     n_seq_blocks_q = sparsity_layout_q.size(1)

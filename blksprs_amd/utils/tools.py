@@ -261,13 +261,18 @@ def prepare_layout_cache(layout_cache: LayoutCache | None, operation: str, *valu
 
 
 def _same_inputs_record(operation: str, values: tuple):
-    """What ``_same_inputs`` compares against, or ``None`` when some value is not a tensor with a version counter
-    (the full key decides then)."""
+    """What ``_same_inputs`` compares against, or ``None`` when some value is neither a tensor with a version
+    counter nor a plain number, string or ``None`` (the full key decides then)."""
     entries = []
     for v in values:
-        if not isinstance(v, Tensor) or v.is_inference():
+        if isinstance(v, Tensor):
+            if v.is_inference():
+                return None
+            entries.append((v, v._version, v.data_ptr(), v.requires_grad, v.shape))
+        elif v is None or type(v) in (int, bool, float, str):
+            entries.append((None, v, 0, False, None))  # a plain value: compared as it is
+        else:
             return None
-        entries.append((v, v._version, v.data_ptr(), v.requires_grad, v.shape))
     return operation, tuple(entries)
 
 
@@ -279,7 +284,10 @@ def _same_inputs(record, operation: str, values: tuple) -> bool:
     if record is None or record[0] != operation or len(record[1]) != len(values):
         return False
     for (tensor, version, address, requires_grad, shape), v in zip(record[1], values):
-        if (v is not tensor or v._version != version or v.data_ptr() != address or v.requires_grad != requires_grad
+        if tensor is None:  # a plain value (the recorded one sits in `version`)
+            if type(v) is not type(version) or v != version:
+                return False
+        elif (v is not tensor or v._version != version or v.data_ptr() != address or v.requires_grad != requires_grad
                 or v.shape != shape):
             return False
     return True
