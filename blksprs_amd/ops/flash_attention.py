@@ -426,17 +426,23 @@ def _fill_args(meta: "_Meta", q, k, v, bias, mask, causal_lengths) -> _capi.Attn
     return a
 
 
+def _forward_launch(q, k, v, bias, mask, causal_lengths, meta: "_Meta"):
+    """The forward launch by itself: ``(out, lse)``."""
+    B, nq, nk, nh, nhv = meta.dims
+    sbs = meta.sbs
+    out = torch.empty((meta.tables.n_sparse_blocks_o, sbs, sbs), dtype=q.dtype, device=q.device)
+    lse = torch.empty((B, nq, sbs), dtype=torch.float32, device=q.device)
+    args = _fill_args(meta, q, k, v, bias, mask, causal_lengths)
+    args.o, args.lse = _capi.ptr(out), _capi.ptr(lse)
+    with _capi.on_device(q.device):
+        _capi.call("bsa_attn_fwd", ctypes.byref(args), _capi.stream(q.device))
+    return out, lse
+
+
 class _FlashAttention(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, v, bias, mask, causal_lengths, meta: "_Meta"):
-        B, nq, nk, nh, nhv = meta.dims
-        sbs = meta.sbs
-        out = torch.empty((meta.tables.n_sparse_blocks_o, sbs, sbs), dtype=q.dtype, device=q.device)
-        lse = torch.empty((B, nq, sbs), dtype=torch.float32, device=q.device)
-        args = _fill_args(meta, q, k, v, bias, mask, causal_lengths)
-        args.o, args.lse = _capi.ptr(out), _capi.ptr(lse)
-        with _capi.on_device(q.device):
-            _capi.call("bsa_attn_fwd", ctypes.byref(args), _capi.stream(q.device))
+        out, lse = _forward_launch(q, k, v, bias, mask, causal_lengths, meta)
         # the mask and the lengths are saved like the operands (as the reference does,
         # blksprs/ops/flash_attention.py:498-501): autograd then refuses a backward pass after either was
         # changed in place
@@ -638,4 +644,9 @@ def flash_attention(q: BlksprsTensor, sparsity_layout_q: Tensor,
     meta.facts = _mask_facts(layout_cache, attention_layout, attention_mask, mask_bytes, lengths, meta.dims,
                              sparsity_block_size)
 
+    needs_grad = torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad
+                                              or (attention_bias is not None and attention_bias.requires_grad))
+    if not needs_grad:
+        # nothing to differentiate: the launch itself, without the autograd machinery around it
+        return BlksprsTensor.wrap(_forward_launch(q, k, v, attention_bias, mask_bytes, lengths, meta)[0])
     return BlksprsTensor.wrap(_FlashAttention.apply(q, k, v, attention_bias, mask_bytes, lengths, meta))
