@@ -50,6 +50,8 @@ SIGNATURES = {
     "bsa_lut_nonzero": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p]),
     "bsa_lut_csr_indices": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_void_p]),
     "bsa_lut_sorted_rows": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_void_p]),
+    "bsa_lut_pair_union": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p]),
+    "bsa_lut_pair_entries": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p]),
     "bsa_layout_matmul": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p]),
     "bsa_lut_contraction_offsets": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64,
                                             c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t,

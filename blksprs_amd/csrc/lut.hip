@@ -429,6 +429,55 @@ extern "C" int bsa_lut_csr_indices(const int64_t *packed, int64_t n, int64_t C, 
   return bsa::check_launch("csr_indices_kernel");
 }
 
+// ---- lists over pairs of neighbouring rows (the attention forward's groups of two query blocks)
+// the union of rows 2 g and 2 g + 1 of a layout of 0/1 bytes [B, R, C], as bytes [B, ceil(R / 2), C]
+__global__ __launch_bounds__(256) void pair_union_kernel(const uint8_t *__restrict__ layout, int64_t B, int64_t R,
+                                                         int64_t C, uint8_t *__restrict__ uni) {
+  const int64_t G = (R + 1) / 2;
+  const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (e >= B * G * C) return;
+  const int64_t c = e % C, g = (e / C) % G, b = e / (C * G);
+  const uint8_t first = layout[(b * R + 2 * g) * C + c];
+  const uint8_t second = 2 * g + 1 < R ? layout[(b * R + 2 * g + 1) * C + c] : (uint8_t)0;
+  uni[e] = (first | second) ? 1 : 0;
+}
+
+// entries[p] = column | first row active << 28 | second row active << 29 for the p-th active position of the union
+__global__ __launch_bounds__(256) void pair_entries_kernel(const uint8_t *__restrict__ layout,
+                                                           const int64_t *__restrict__ union_packed, int64_t B,
+                                                           int64_t R, int64_t C, int32_t *__restrict__ entries) {
+  const int64_t G = (R + 1) / 2;
+  const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (e >= B * G * C) return;
+  const int64_t p = union_packed[e];
+  if (p < 0) return;
+  const int64_t c = e % C, g = (e / C) % G, b = e / (C * G);
+  const int32_t first = layout[(b * R + 2 * g) * C + c] ? 1 : 0;
+  const int32_t second = (2 * g + 1 < R && layout[(b * R + 2 * g + 1) * C + c]) ? 1 : 0;
+  entries[p] = (int32_t)c | (first << 28) | (second << 29);
+}
+
+extern "C" int bsa_lut_pair_union(const uint8_t *layout, int64_t B, int64_t R, int64_t C, uint8_t *uni,
+                                  bsa_stream_t stream) {
+  BSA_REQUIRE(B >= 0 && R >= 0 && C >= 0, "bsa_lut_pair_union: negative size");
+  const int64_t n = B * ((R + 1) / 2) * C;
+  if (n == 0) return BSA_OK;
+  BSA_REQUIRE(layout && uni, "bsa_lut_pair_union: NULL pointer");
+  pair_union_kernel<<<grid_for(n, 256), 256, 0, bsa::as_stream(stream)>>>(layout, B, R, C, uni);
+  return bsa::check_launch("pair_union_kernel");
+}
+
+extern "C" int bsa_lut_pair_entries(const uint8_t *layout, const int64_t *union_packed, int64_t B, int64_t R,
+                                    int64_t C, int32_t *entries, bsa_stream_t stream) {
+  BSA_REQUIRE(B >= 0 && R >= 0 && C >= 0, "bsa_lut_pair_entries: negative size");
+  BSA_REQUIRE(C < (1 << 28), "bsa_lut_pair_entries: too many columns for an entry");
+  const int64_t n = B * ((R + 1) / 2) * C;
+  if (n == 0) return BSA_OK;
+  BSA_REQUIRE(layout && union_packed, "bsa_lut_pair_entries: NULL pointer");
+  pair_entries_kernel<<<grid_for(n, 256), 256, 0, bsa::as_stream(stream)>>>(layout, union_packed, B, R, C, entries);
+  return bsa::check_launch("pair_entries_kernel");
+}
+
 extern "C" int bsa_lut_sorted_rows(const int32_t *row_offsets, int64_t n_rows, int64_t C, int64_t *sorted,
                                    bsa_stream_t stream) {
   BSA_REQUIRE(n_rows >= 0 && C >= 0, "bsa_lut_sorted_rows: negative size");

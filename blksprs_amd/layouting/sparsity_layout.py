@@ -10,7 +10,7 @@ import torch
 from torch import Tensor
 
 from .. import _capi
-from ..utils.tools import _layout_bytes, as_base_tensor
+from ..utils.tools import layout_bytes, as_base_tensor
 from ..utils.validation import (validate_contiguous, validate_device, validate_dimensions, validate_dtype_supported,
                                 validate_sparsity_block_size, validate_sparsity_layout, _validation_enabled,
                                 ensure_contiguous)
@@ -93,7 +93,7 @@ def build_sparsity_layout_matmul(sparsity_layout_x: Tensor, sparsity_layout_y: T
     dev = sparsity_layout_x.device
     out = torch.empty((B, R, C), dtype=torch.bool, device=dev)
     if out.numel():
-        lx, ly = _layout_bytes(sparsity_layout_x), _layout_bytes(sparsity_layout_y)
+        lx, ly = layout_bytes(sparsity_layout_x), layout_bytes(sparsity_layout_y)
         with _capi.on_device(dev):
             _capi.call("bsa_layout_matmul", _capi.ptr(lx), _capi.ptr(ly), B, R, K, C,
                        out.view(torch.uint8).data_ptr(), _capi.stream(dev))

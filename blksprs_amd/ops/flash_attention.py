@@ -19,7 +19,7 @@ from .. import _capi
 from ..layouting.sparsity_layout import build_sparsity_layout_matmul
 from ..utils.blksprs_tensor import BlksprsTensor
 from ..utils.tools import (CacheHolder, INT32_INDEX_MAX, as_base_tensor, cast_for_autocast, csr_indices_from_packed,
-                           PackedLayout, eager_only, finalize_layout_cache, nonzero_from_packed, pack_layout,
+                           PackedLayout, eager_only, finalize_layout_cache, layout_bytes, pack_layout,
                            pack_layouts, prepare_layout_cache)
 from ..utils.validation import (ensure_contiguous, mask_facts_enabled, validate_binary, validate_contiguous,
                                 validate_device, validate_dimensions, validate_dtype_float, validate_shape,
@@ -69,15 +69,16 @@ def _build_group_lists(attention_layout: Tensor, n_batches: int, n_blocks_row: i
     ``offsets`` has ``B * ceil(rows / 2) + 1`` int32 entries.  The forward kernel gives a pair to one workgroup,
     which fetches a K / V block both query blocks need once.  These lists have no counterpart in the reference.
     """
-    even, odd, union = _group_union(attention_layout, n_batches, n_blocks_row, n_blocks_col)
+    union = _group_union(attention_layout, n_batches, n_blocks_row, n_blocks_col)
     if info is None:
         info = pack_layout(union, row_len=n_blocks_col)
-    # coordinates of the union's blocks from its scan (no read of the device: the count is known)
-    where = nonzero_from_packed(info.packed, union.shape, info.count)
-    flags = even[where[:, 0], where[:, 1], where[:, 2]].to(torch.int32) \
-        | (odd[where[:, 0], where[:, 1], where[:, 2]].to(torch.int32) << 1)
-    entries = (where[:, 2].to(torch.int32) | (flags << 28)).contiguous()
-    return as_base_tensor(info.row_offsets), as_base_tensor(entries), 2
+    entries = torch.empty(info.count, dtype=torch.int32, device=union.device)
+    if info.count:
+        lay = layout_bytes(attention_layout)
+        with _capi.on_device(union.device):
+            _capi.call("bsa_lut_pair_entries", lay.data_ptr(), info.packed.data_ptr(), n_batches, n_blocks_row,
+                       n_blocks_col, entries.data_ptr(), _capi.stream(union.device))
+    return as_base_tensor(info.row_offsets), entries, 2
 
 
 def _grouped_lists_apply(n_blocks_col, n_head_blocks, n_head_blocks_v) -> bool:
@@ -87,13 +88,16 @@ def _grouped_lists_apply(n_blocks_col, n_head_blocks, n_head_blocks_v) -> bool:
             and n_head_blocks <= 2 and n_head_blocks_v <= 2)
 
 
-def _group_union(attention_layout: Tensor, n_batches: int, n_blocks_row: int, n_blocks_col: int):
-    """``(even rows, odd rows, their union)`` of the attention layout as boolean ``(B, ceil(rows / 2), cols)``."""
-    active = attention_layout.reshape(n_batches, n_blocks_row, n_blocks_col) != 0
-    if n_blocks_row % 2:
-        active = torch.cat([active, torch.zeros_like(active[:, :1])], dim=1)
-    even, odd = active[:, 0::2], active[:, 1::2]
-    return even, odd, (even | odd).contiguous()
+def _group_union(attention_layout: Tensor, n_batches: int, n_blocks_row: int, n_blocks_col: int) -> Tensor:
+    """The union of rows ``2 g`` and ``2 g + 1`` of the attention layout, 0/1 bytes ``(B, ceil(rows / 2), cols)``
+    (``bsa_lut_pair_union``)."""
+    lay = layout_bytes(attention_layout)
+    union = torch.empty((n_batches, (n_blocks_row + 1) // 2, n_blocks_col), dtype=torch.uint8, device=lay.device)
+    if union.numel():
+        with _capi.on_device(lay.device):
+            _capi.call("bsa_lut_pair_union", lay.data_ptr(), n_batches, n_blocks_row, n_blocks_col, union.data_ptr(),
+                       _capi.stream(lay.device))
+    return union
 
 
 def flash_attention_build_layout_cache(attention_layout: Tensor,
@@ -210,7 +214,7 @@ def flash_attention_build_layout_cache(attention_layout: Tensor,
                                                                        n_head_blocks_v)
             and attention_layout.numel()):
         wanted.append(("groups", _group_union(attention_layout, int(n_batches), int(n_seq_blocks_q),
-                                              int(n_seq_blocks_k))[2], n_seq_blocks_k))
+                                              int(n_seq_blocks_k)), n_seq_blocks_k))
     scans = dict(zip((w[0] for w in wanted), pack_layouts(*((w[1], w[2]) for w in wanted)))) if wanted else {}
 
     if "key_indices" not in layout_cache:

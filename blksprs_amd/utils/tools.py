@@ -35,7 +35,7 @@ def as_base_tensor(value: Tensor) -> Tensor:
 
 # --------------------------------------------------------------------------- device LUT builders
 
-def _layout_bytes(layout: Tensor) -> Tensor:
+def layout_bytes(layout: Tensor) -> Tensor:
     """The layout as contiguous 0/1 bytes on its device (a view for bool layouts)."""
     layout = as_base_tensor(layout)
     if not layout.is_contiguous():
@@ -85,7 +85,7 @@ def pack_layouts(*specs, then=None):
     stats_dev = None
     for number, (layout, row_len) in enumerate(specs):
         _require_device(layout)
-        lay = _layout_bytes(layout)
+        lay = layout_bytes(layout)
         n = lay.numel()
         dev = lay.device
         if stats_dev is None:

@@ -107,6 +107,18 @@ int bsa_lut_sorted_rows(const int32_t *row_offsets, int64_t n_rows, int64_t C, i
                         bsa_stream_t stream);
 
 /*
+ * Lists over pairs of neighbouring rows of a layout (0/1 bytes [B, R, C]): the groups of two query blocks the
+ * attention forward kernel gives to one workgroup (bsa_attn_fwd_records takes their entries).
+ * bsa_lut_pair_union writes the union of rows 2 g and 2 g + 1 as bytes [B, ceil(R / 2), C]; scanned with
+ * bsa_lut_packed (row_len = C) it yields the groups' offsets and the reverse index union_packed, from which
+ * bsa_lut_pair_entries writes, for the p-th active position of the union, entries[p] = column |
+ * first row active << 28 | second row active << 29 (C < 2^28).  No counterpart in the reference.
+ */
+int bsa_lut_pair_union(const uint8_t *layout, int64_t B, int64_t R, int64_t C, uint8_t *uni, bsa_stream_t stream);
+int bsa_lut_pair_entries(const uint8_t *layout, const int64_t *union_packed, int64_t B, int64_t R, int64_t C,
+                         int32_t *entries, bsa_stream_t stream);
+
+/*
  * Boolean block product lo[b,i,j] = OR_k lx[b,i,k] & ly[b,k,j]:
  * build_sparsity_layout_matmul (blksprs/layouting/sparsity_layout.py:244-258).
  */
