@@ -473,7 +473,7 @@ extern "C" int bsa_lut_pair_entries(const uint8_t *layout, const int64_t *union_
   BSA_REQUIRE(C < (1 << 28), "bsa_lut_pair_entries: too many columns for an entry");
   const int64_t n = B * ((R + 1) / 2) * C;
   if (n == 0) return BSA_OK;
-  BSA_REQUIRE(layout && union_packed, "bsa_lut_pair_entries: NULL pointer");
+  BSA_REQUIRE(layout && union_packed && entries, "bsa_lut_pair_entries: NULL pointer");
   pair_entries_kernel<<<grid_for(n, 256), 256, 0, bsa::as_stream(stream)>>>(layout, union_packed, B, R, C, entries);
   return bsa::check_launch("pair_entries_kernel");
 }

@@ -75,6 +75,13 @@ def test_bad_arguments_of_the_neighbouring_entry_points_are_rejected_on_the_host
     assert lib.bsa_lut_row_work_table(0, 0, 9, 3, 1, 0, 10, 0, 0, 8, 0, 0, 0) == -1 and b"are needed" in lib.bsa_last_error()
     assert lib.bsa_lut_row_work_table(0, 0, 9, 3, 1, 0, -1, 0, 0, 32, 0, 0, 0) == -1 and b"bound" in lib.bsa_last_error()
     assert lib.bsa_lut_row_work_table(0, 0, 0, 3, 1, 0, 10, 0, 0, 0, 0, 0, 0) == 0  # no rows
+    # lists over pairs of rows: sizes, the 28 bits of a column, pointers
+    assert lib.bsa_lut_pair_union(0, 1, -2, 4, 0, 0) == -1 and b"negative size" in lib.bsa_last_error()
+    assert lib.bsa_lut_pair_union(0, 1, 2, 4, 0, 0) == -1 and b"NULL" in lib.bsa_last_error()
+    assert lib.bsa_lut_pair_union(0, 0, 2, 4, 0, 0) == 0
+    assert lib.bsa_lut_pair_entries(0, 0, 1, 2, 1 << 28, 0, 0) == -1 and b"too many columns" in lib.bsa_last_error()
+    assert lib.bsa_lut_pair_entries(0, 0, 1, 2, 4, 0, 0) == -1 and b"NULL" in lib.bsa_last_error()
+    assert lib.bsa_lut_pair_entries(0, 0, 1, 0, 4, 0, 0) == 0
     # records of the row kernel: parts_log2 in 0..3; without a table the rows are taken whole and in order
     assert lib.bsa_matmul_rows_records(0, 4, 4, 0, 0, 0, 4, 4, 0, 0, 0) == -1 and b"parts_log2" in lib.bsa_last_error()
     assert lib.bsa_matmul_rows_records(0, 8, 1, 0, 0, 0, 4, 4, 0, 0, 0) == -1 and b"work table" in lib.bsa_last_error()

@@ -176,3 +176,34 @@ def test_block_order_of_the_device_equals_its_restatement(device, shape, density
     assert got.dtype == torch.int32 and torch.equal(got, want)
     assert torch.equal(torch.sort(got.long())[0], torch.arange(coords.size(0)))
     assert mm._block_order(torch.empty((0, 3), dtype=torch.int64, device=device), 4, 4).numel() == 0
+
+
+@pytest.mark.parametrize("shape,density", [((3, 40, 37), 0.3), ((2, 5, 130), 0.9), ((2, 64, 64), 0.02), ((1, 1, 1), 1.0),
+                                           ((2, 7, 9), 0.0), ((4, 9, 300), 0.5)])
+def test_pair_lists_of_the_device_equal_their_restatement(device, shape, density):
+    """``bsa_lut_pair_union`` / ``bsa_lut_pair_entries`` through the C ABI against the same lists formed in numpy:
+    the union of rows 2 g and 2 g + 1 (a lone last row with nothing), and per active position of the union, in
+    row-major order, column | first row active << 28 | second row active << 29."""
+    from blksprs_amd import _capi
+    B, R, C = shape
+    G = (R + 1) // 2
+    layout = rand_layout(shape, density, seed=3 + sum(shape)).to(torch.uint8)
+    padded = np.zeros((B, 2 * G, C), dtype=np.uint8)
+    padded[:, :R] = layout.numpy()
+    first, second = padded[:, 0::2], padded[:, 1::2]
+    want_union = first | second
+    where = np.nonzero(want_union.reshape(-1))[0]
+    want_entries = ((where % C) | (first.reshape(-1)[where].astype(np.int64) << 28)
+                    | (second.reshape(-1)[where].astype(np.int64) << 29)).astype(np.int32)
+
+    dev_layout = layout.to(device)
+    uni = torch.full((B, G, C), 7, dtype=torch.uint8, device=device)
+    stream = torch.cuda.current_stream(device).cuda_stream
+    _capi.call("bsa_lut_pair_union", dev_layout.data_ptr(), B, R, C, uni.data_ptr(), stream)
+    assert np.array_equal(uni.cpu().numpy(), want_union)
+    packed = tools.build_packed_indices(uni)
+    entries = torch.full((max(len(where), 1),), -5, dtype=torch.int32, device=device)
+    _capi.call("bsa_lut_pair_entries", dev_layout.data_ptr(), packed.data_ptr(), B, R, C, entries.data_ptr(), stream)
+    assert np.array_equal(entries.cpu().numpy()[:len(where)], want_entries)
+    if len(where) == 0:
+        assert int(entries[0]) == -5  # nothing written
