@@ -12,7 +12,7 @@ import torch
 
 _LIB_PATH = Path(__file__).resolve().parent / "lib" / "libblksprs_amd.so"
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 F32, F16, BF16 = 0, 1, 2
 DTYPE_CODES = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
 
@@ -31,7 +31,8 @@ class AttnArgs(ctypes.Structure):
                                   "n_o_blocks", "n_mask_blocks", "n_bias_blocks")]
         + [("sbs", ctypes.c_int32), ("dtype", ctypes.c_int32), ("mask_kind", ctypes.c_int32), ("scale", c_float)]
         + [("group_offsets", c_void_p), ("group_records", c_void_p), ("group_size", ctypes.c_int32)]
-        + [("bwd_scratch", c_void_p), ("n_layout_blocks", c_int64), ("bwd_scratch_ready", c_int64)]
+        + [("bwd_scratch", c_void_p), ("n_layout_blocks", c_int64), ("bwd_scratch_ready", c_int64),
+           ("bwd_scratch_bytes", c_int64)]
     )
 
 
@@ -83,6 +84,7 @@ SIGNATURES = {
     "bsa_attn_fwd_records": (c_int, [ctypes.POINTER(AttnArgs), c_void_p, c_void_p, c_void_p]),
     "bsa_attn_mask_dead": (c_int, [c_void_p, c_int64, ctypes.c_int32, c_void_p, c_void_p]),
     "bsa_attn_bwd_scratch_bytes": (c_size_t, [c_int64, c_int64, c_int64, c_int64, c_int64]),
+    "bsa_attn_bwd_scratch_bytes_ds": (c_size_t, [c_int64, c_int64, c_int64, c_int64, c_int64]),
     "bsa_attn_fwd": (c_int, [ctypes.POINTER(AttnArgs), c_void_p]),
     "bsa_attn_bwd": (c_int, [ctypes.POINTER(AttnArgs), c_void_p]),
 }

@@ -86,9 +86,16 @@ extern "C" size_t bsa_attn_bwd_scratch_bytes(int64_t B, int64_t nq, int64_t nk, 
   return bsa::attn_bwd_scratch_bytes(B, nq, nk, n_layout_blocks, n_mask_blocks);
 }
 
+extern "C" size_t bsa_attn_bwd_scratch_bytes_ds(int64_t B, int64_t nq, int64_t nk, int64_t n_layout_blocks,
+                                                int64_t n_mask_blocks) {
+  if (B < 0 || nq < 0 || nk < 0 || n_layout_blocks < 0 || n_mask_blocks < 0) return 0;
+  return bsa::attn_bwd_scratch_bytes_ds(B, nq, nk, n_layout_blocks, n_mask_blocks);
+}
+
 extern "C" int bsa_attn_bwd(const bsa_attn_args *args, bsa_stream_t stream) {
   if (int rc = check_args("bsa_attn_bwd", args, true)) return rc;
   BSA_REQUIRE(args->bwd_scratch == nullptr || args->n_layout_blocks >= 0, "bsa_attn_bwd: negative n_layout_blocks");
+  BSA_REQUIRE(args->bwd_scratch_bytes >= 0, "bsa_attn_bwd: negative bwd_scratch_bytes");
   BSA_REQUIRE((reinterpret_cast<uintptr_t>(args->bwd_scratch) & 15) == 0, "bsa_attn_bwd: bwd_scratch must be 16-byte aligned");
   hipStream_t s = bsa::as_stream(stream);
   int rc = bsa::attn_bwd_mfma(*args, s);

@@ -167,7 +167,7 @@ struct BwdRecord {
   int32_t pb[2];   // packed indices of its O / dO (resp. V) slices
   int32_t mask;    // mask block of the pair, -1: none
   int32_t bias;    // bias block of the pair
-  int32_t pad;
+  int32_t pair;    // position of the pair in key_indices (the same number in both lists): its block of dS
 };
 static_assert(sizeof(BwdRecord) == 32, "one record is eight int32");
 
@@ -182,7 +182,22 @@ struct BwdLists {
   int32_t *q_head, *k_head;
   int32_t *kv_tickets;             // [16]: per XCD, the next position of its eighth of the key rows to hand out
   uint8_t *mask_dead;              // [n_mask_blocks]
+  // [n_layout_blocks] blocks of 64 x 64 16-bit values, or NULL (the scratch is too small for them): dS^T of every
+  // pair (row = key, column = query), written by the dK / dV kernel for the dQ kernel
+  char *ds;
 };
+
+// bytes of the scratch without the dS blocks, and the offset at which they start when the scratch holds them
+__host__ __device__ inline size_t bwd_lists_bytes(int64_t B, int64_t nq, int64_t nk, int64_t n_layout_blocks,
+                                                  int64_t n_mask_blocks) {
+  const size_t bytes = 2 * sizeof(BwdRecord) * (size_t)n_layout_blocks + (4 + 64) * (size_t)(B * nq + B * nk) + 64 +
+                       (size_t)n_mask_blocks;
+  return (bytes + 15) & ~(size_t)15;
+}
+__host__ __device__ inline size_t bwd_ds_offset(int64_t B, int64_t nq, int64_t nk, int64_t n_layout_blocks,
+                                                int64_t n_mask_blocks) {
+  return (bwd_lists_bytes(B, nq, nk, n_layout_blocks, n_mask_blocks) + 4095) & ~(size_t)4095;
+}
 
 __host__ __device__ inline BwdLists bwd_lists(const bsa_attn_args &a) {
   BwdLists L;
@@ -194,6 +209,10 @@ __host__ __device__ inline BwdLists bwd_lists(const bsa_attn_args &a) {
   L.k_head = L.q_head + 16 * a.B * a.nq;
   L.kv_tickets = L.k_head + 16 * a.B * a.nk;
   L.mask_dead = reinterpret_cast<uint8_t *>(L.kv_tickets + 16);
+  const size_t ds_at = bwd_ds_offset(a.B, a.nq, a.nk, a.n_layout_blocks, a.n_mask_blocks);
+  const bool has_ds = a.bwd_scratch_bytes > 0 &&
+                      (size_t)a.bwd_scratch_bytes >= ds_at + (size_t)a.n_layout_blocks * kBlockBytes;
+  L.ds = has_ds ? static_cast<char *>(a.bwd_scratch) + ds_at : nullptr;
   return L;
 }
 
@@ -262,7 +281,20 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_records_kernel(bsa_attn_
       }
       r.mask = pm;
       r.bias = a.bias ? checked_index(a.pidx_bias, pair, a.n_bias_blocks) : -1;
-      r.pad = 0;
+      // the pair's position in the lists per query block: entry e itself, or where kb stands in the (ascending)
+      // list of query block qb
+      int at = e;
+      if (by_key) {
+        int lo = a.key_offsets[b * a.nq + qb], hi = a.key_offsets[b * a.nq + qb + 1];
+        const int last = hi - 1;
+        while (lo < hi) {
+          const int mid = (lo + hi) >> 1;
+          if (a.key_indices[mid] < kb) lo = mid + 1;
+          else hi = mid;
+        }
+        at = lo <= last ? lo : last;  // the two lists hold the same pairs: kb is found; never past the row
+      }
+      r.pair = at;
       out[n + __popcll(votes & ((1ull << lane) - 1))] = r;
     }
     n += __popcll(votes);
@@ -337,6 +369,33 @@ __global__ __launch_bounds__(kOrderThreads) void attn_bwd_order_kernel(bsa_attn_
   if (tid < 256) bins[tid] = before;
   __syncthreads();
   for (int64_t r = r0 + tid; r < r1; r += kOrderThreads) emit(r0 + atomicAdd(&bins[bin_of(r)], 1), r);
+}
+
+// delta[b, qb, i] = sum over the output slices of rowsum(o * dO), four lanes per query row; also the tickets of
+// the dK / dV walk.  Launched in front of that walk when the dQ kernel runs after it (dQ from the stored dS).
+template <typename Tr>
+__global__ __launch_bounds__(kBwdThreads) void attn_bwd_delta_kernel(bsa_attn_args a) {
+  const int64_t row = blockIdx.x;  // b * nq + qb
+  const int tid = threadIdx.x;
+  if (row == 0 && tid < 8) bwd_lists(a).kv_tickets[tid] = (int32_t)kv_slots(a.B * a.nk);
+  const int i = tid >> 2, part = tid & 3;
+  float acc = 0.f;
+  for (int64_t h = 0; h < a.nhv; ++h) {
+    const int64_t po = a.pidx_o[row * a.nhv + h];
+    if (po < 0 || po >= a.n_o_blocks) continue;
+    const char *ob = static_cast<const char *>(a.o) + po * kBlockBytes + i * 128 + part * 32;
+    const char *gb = static_cast<const char *>(a.d_o) + po * kBlockBytes + i * 128 + part * 32;
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      const u32x4 ov = *reinterpret_cast<const u32x4 *>(ob + 16 * c);
+      const u32x4 gv = *reinterpret_cast<const u32x4 *>(gb + 16 * c);
+#pragma unroll
+      for (int t = 0; t < 4; ++t) acc = Tr::dot2(ov[t], gv[t], acc);
+    }
+  }
+  acc += __shfl_xor(acc, 1);
+  acc += __shfl_xor(acc, 2);
+  if (part == 0) a.delta[row * kSbs + i] = acc;
 }
 
 // The work of one wave on one tile (a query block in LDS at `base`, this wave's quadrant of the 64 x 64 scores):
@@ -603,8 +662,12 @@ template <typename Tr, int NH, int NHV, bool DK, bool DV>
 __device__ __forceinline__ void kv_second_half(const KvCarry &c, const bool live, const bsa_attn_args &a, const char *base,
                                                const int64_t pb, const int wi, const int wj, const int li, const int kg,
                                                const int lane, f32x16 (&dkacc)[DK ? NH * 2 : 1],
-                                               f32x16 (&dvacc)[DV ? NHV * 2 : 1], const f32x4 *p_lds) {
+                                               f32x16 (&dvacc)[DV ? NHV * 2 : 1], const f32x4 *p_lds,
+                                               u32x4 (&ds_keep)[2]) {
   constexpr int kQRows = 0, kDoRows = NH * kBlockBytes, kStats = (NH + NHV) * kBlockBytes;
+  // ds_keep (dK team): dS of this lane's 16 scores as packed for the dK product, zeros for a quadrant without a
+  // surviving score; the caller stores it for the dQ kernel
+  if constexpr (DK) ds_keep[0] = ds_keep[1] = u32x4{0u, 0u, 0u, 0u};
   if (!live) return;
   const int col_t = 16 * ((lane >> 4) & 1);
   if constexpr (DV) {
@@ -641,6 +704,8 @@ __device__ __forceinline__ void kv_second_half(const KvCarry &c, const bool live
     for (int u = 0; u < 2; ++u)
 #pragma unroll
       for (int t = 0; t < 4; ++t) dsf[u][t] = Tr::pack2(ds[8 * u + 2 * t], ds[8 * u + 2 * t + 1]);
+    ds_keep[0] = dsf[0];
+    ds_keep[1] = dsf[1];
     staged_products_from<NH>(
         c.g0,
         [&](int h, u32x4(&f)[4]) {
@@ -960,7 +1025,7 @@ __device__ __forceinline__ void attn_bwd_kv8_walk(const bsa_attn_args &a, char *
     const int32_t *src = recs_lane + (int64_t)pos * 8;
     asm volatile("global_load_dword %0, %1, off" : "+v"(rec_in_flight) : "v"(src) : "memory");
   };
-  int qb_nxt = 0, pm_nxt = -1, pb_nxt = -1;
+  int qb_nxt = 0, pm_nxt = -1, pb_nxt = -1, pair_nxt = 0;
   // requests the tile of record `rec` (field i in lane i) of batch entry `batch` into tile buffer `buf`
   auto fetch = [&](int rec, int buf, int64_t batch) {
     const int qb = __builtin_amdgcn_readlane(rec, 0);
@@ -976,6 +1041,7 @@ __device__ __forceinline__ void attn_bwd_kv8_walk(const bsa_attn_args &a, char *
     // mask block are fetched by the dK team alone (waves 4 .. 7), the Q blocks by all eight waves.
     pm_nxt = __builtin_amdgcn_readlane(rec, 5);
     pb_nxt = __builtin_amdgcn_readlane(rec, 6);
+    pair_nxt = __builtin_amdgcn_readlane(rec, 7);
     if (wave >= 4) {
 #pragma unroll
       for (int h = 0; h < NHV; ++h) {
@@ -1027,6 +1093,20 @@ __device__ __forceinline__ void attn_bwd_kv8_walk(const bsa_attn_args &a, char *
     }
   };
 
+  // dS of the tile before (dK team), kept in registers until the next tile has started: a store issued right
+  // behind the tile's products would be waited for, with everything else in flight, at the end of that tile
+  u32x4 ds_pending[2] = {u32x4{0u, 0u, 0u, 0u}, u32x4{0u, 0u, 0u, 0u}};
+  char *ds_pending_at = nullptr;
+  auto store_pending_ds = [&]() {
+    if constexpr (DK) {
+      if (ds_pending_at) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) *reinterpret_cast<u32x4 *>(ds_pending_at + 1024 * u) = ds_pending[u];
+        ds_pending_at = nullptr;
+      }
+    }
+  };
+
   // the first block's fragments have arrived: from here on the compiler has no load of its own in flight when a
   // tile starts (see stage())
   __builtin_amdgcn_s_waitcnt(0x0F70);
@@ -1069,6 +1149,8 @@ __device__ __forceinline__ void attn_bwd_kv8_walk(const bsa_attn_args &a, char *
         const char *base = smem + buf * kBufBytes;
         const int qb = qb_nxt;
         const int64_t pm = pm_nxt, pb = pb_nxt;
+        const int pair = pair_nxt;
+        store_pending_ds();  // of the tile before: it has this whole tile to get there before the next wait
         uint32_t mbits = 0;
         if (pm >= 0) {
           const uint8_t *mp = reinterpret_cast<const uint8_t *>(base + kMask) + (32 * wi + 4 * kg) * kSbs + 32 * wj + li;
@@ -1109,7 +1191,12 @@ __device__ __forceinline__ void attn_bwd_kv8_walk(const bsa_attn_args &a, char *
         kv_first_half<Tr, NH, NHV, DK, DV>(carry, f0, live, a, base, qb, pm, pb, mbits, causal, seq_len, (int)kb, kpos,
                                            qk_scale, wi, wj, li, kg, lane, kfr, vfr, p_lds);
         __syncthreads();  // P is in LDS
-        kv_second_half<Tr, NH, NHV, DK, DV>(carry, live, a, base, pb, wi, wj, li, kg, lane, dkacc, dvacc, p_lds);
+        kv_second_half<Tr, NH, NHV, DK, DV>(carry, live, a, base, pb, wi, wj, li, kg, lane, dkacc, dvacc, p_lds, ds_pending);
+        if constexpr (DK) {
+          // dS of the pair for the dQ kernel, as the lanes hold it: quadrant (wi, wj) is 2 KiB, in it plane u (1 KiB)
+          // holds ds_pending[u] of lane l at 16 l (see frag_ds)
+          if (lists.ds) ds_pending_at = lists.ds + (int64_t)pair * kBlockBytes + (wi + 2 * wj) * 2048 + lane * 16;
+        }
 
         if (next_tile) stage(buf ^ 1);
         else {  // K / V of the next block, the record
@@ -1126,6 +1213,7 @@ __device__ __forceinline__ void attn_bwd_kv8_walk(const bsa_attn_args &a, char *
     }
 
     // ---- end of the block
+    store_pending_ds();
     if (has_next && !kv_requested) {
       // a block of fewer than two tiles: nothing was overlapped
       __syncthreads();  // R is free
@@ -1475,6 +1563,140 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_q_kernel(bsa_attn_arg
   }
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// Second operand of dQ^T += K^T dS^T from a dS block as the dK / dV kernel leaves it: quadrant (wi, wj) of the pair
+// (queries 32 wi .., keys 32 wj ..) is 2 KiB; in it, plane u (1 KiB) holds at 16 l the eight values of lane l =
+// 32 kg + key % 32 of that kernel: dS of key l % 32 and queries 32 wi + 16 u + 8 h + 4 kg + t for h = 0, 1 and
+// t = 0 .. 3.  Seen as rows of 16 values (both planes of a lane side by side), row 32 g + j holds key j and the
+// sixteen queries 8 (c / 4) + 4 g + c % 4, c = 0 .. 15.  The transposing load hands lane i of a 16-lane group column
+// i of four rows: with group g16 of a wave half on the rows of g = g16, the 32 lanes of a half cover the quadrant's
+// 32 queries, lane (i, g16) holding query 8 (i / 4) + 4 g16 + i % 4 (query_of_lane) and keys key0 .. + 3 and
+// key0 + 8 .. + 11, the same eight as frag_cols_t gives for the first operand.
+__device__ static inline u32x4 frag_ds(const char *blob, int wi, int wj, int key0, int lane) {
+  const int s = lane & 15, g16 = (lane >> 4) & 1;
+  const int row = 32 * g16 + key0 + (s >> 2);
+  const char *p0 = blob + (wi + 2 * wj) * 2048 + ((s & 3) >> 1) * 1024 + row * 16 + (s & 1) * 8;
+  const char *p1 = p0 + 8 * 16;
+  const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4 *)p0);
+  const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4 *)p1);
+  const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+  return u32x4{l2[0], l2[1], h2[0], h2[1]};
+}
+__device__ static inline int query_of_lane(int lane) { return 8 * ((lane & 15) >> 2) + 4 * ((lane >> 4) & 1) + (lane & 3); }
+
+// dQ of one query block from the dS^T blocks the dK / dV kernel has written: dQ^T += K^T dS^T, one product per
+// pair and no scores.  Wave (wi, wj) owns queries 32 wi .. + 31 and the head-dimension columns 32 NH wj .. + 32 NH - 1
+// (of the NH slices: slice wj with two slices, half of the slice with one) and contracts over all 64 keys of every
+// tile, so no wave needs another's sums.  A tile is the pair's K slices and its dS^T block, both copied
+// asynchronously into LDS and both read with the transposing load (the contraction runs over the keys, the rows
+// of both).  Every pair of the list is multiplied: quadrants without a surviving score hold zeros.
+template <typename Tr, int NH>
+__global__ __launch_bounds__(kBwdThreads, 3) void attn_bwd_dq_kernel(bsa_attn_args a) {
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  constexpr int kKRows = 0, kDsRows = NH * kBlockBytes;
+  constexpr int kBufBytes = (NH + 1) * kBlockBytes;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = first_lane(tid >> 6);
+  const int kg = lane >> 5;
+  const int wi = wave & 1, wj = wave >> 1;
+  const int64_t qpos_in_order = xcd_row();
+  const BwdLists lists = bwd_lists(a);
+  if (qpos_in_order >= a.B * a.nq) return;
+  int head = -1;
+  if (lane < 16) head = lists.q_head[qpos_in_order * 16 + lane];
+  // this wave's NH column blocks of 32: block n is columns 32 (NH wj + n) of the head dimension, that is slice
+  // (NH wj + n) / 2, half (NH wj + n) % 2
+  const int first_block = NH * wj;
+  bool any = false;
+#pragma unroll
+  for (int h = 0; h < NH; ++h) any = any || __builtin_amdgcn_readlane(head, 11 + h) >= 0;
+  if (!any) return;
+
+  f32x16 dqacc[NH];
+#pragma unroll
+  for (int n = 0; n < NH; ++n)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) dqacc[n][r] = 0.f;
+
+  const int k_begin = __builtin_amdgcn_readlane(head, 9), k_end = __builtin_amdgcn_readlane(head, 10);
+  if (k_begin < k_end) {
+    const int32_t *recs = reinterpret_cast<const int32_t *>(lists.key_rec);
+    auto load_record = [&](int pos) -> int {
+      int v = -1;
+      if (lane < 8) v = recs[(int64_t)pos * 8 + lane];
+      return v;
+    };
+    auto clamp_e = [&](int e) { return e < k_end ? e : k_end - 1; };
+    auto fetch = [&](int rec, int buf) {
+      char *base = smem + buf * kBufBytes;
+#pragma unroll
+      for (int h = 0; h < NH; ++h) {
+        const int pk = __builtin_amdgcn_readlane(rec, 1 + h);
+        copy_block(static_cast<const char *>(a.k) + (int64_t)(pk >= 0 ? pk : 0) * kBlockBytes, pk >= 0,
+                   base + kKRows + h * kBlockBytes, wave, lane, tid);
+      }
+      // the dS block as it lies, 2 KiB per wave
+      const int pair = __builtin_amdgcn_readlane(rec, 7);
+      copy_2k_to_lds(lists.ds + (int64_t)pair * kBlockBytes + wave * 2048, lane * 16, base + kDsRows + wave * 2048);
+    };
+
+    int rec = load_record(clamp_e(k_begin + 1));
+    fetch(head, 0);
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+
+    const int col_t = 16 * ((lane >> 4) & 1);
+    for (int e = k_begin; e < k_end; ++e) {
+      const int buf = (e - k_begin) & 1;
+      const char *base = smem + buf * kBufBytes;
+      const bool more = e + 1 < k_end;
+      if (more) fetch(rec, buf ^ 1);
+      rec = load_record(clamp_e(e + 2));
+
+      // dS^T as the second operand: query 32 wi + query_of_lane, keys 16 u + 4 kg .. + 3 and + 8 .. + 11
+      u32x4 dsf[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) dsf[u] = frag_ds(base + kDsRows, wi, u >> 1, 16 * (u & 1) + 4 * kg, lane);
+      // stage n: column block first_block + n of K^T against all four key steps
+      staged_products<NH>(
+          [&](int n, u32x4(&f)[4]) {
+            const int blk = first_block + n;
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+              f[u] = frag_cols_t(base + kKRows + (blk >> 1) * kBlockBytes, 16 * u + 4 * kg, 32 * (blk & 1) + col_t, lane);
+          },
+          [&](int n, u32x4(&f)[4]) {
+#pragma unroll
+            for (int u = 0; u < 4; ++u) dqacc[n] = Tr::mfma(f[u], dsf[u], dqacc[n]);
+          });
+
+      // the copies of the next tile have landed (vmcnt(0): the record of the tile after it, requested right
+      // behind them, as well)
+      if (more) __builtin_amdgcn_s_waitcnt(0x0F70);
+      __syncthreads();
+    }
+  }
+
+  // ---- scale, store: register 4 q + t of block n = column 32 (first_block + n) + 8 q + 4 kg + t ----
+  const int qi = 32 * wi + query_of_lane(lane);
+#pragma unroll
+  for (int n = 0; n < NH; ++n) {
+    const int blk = first_block + n;
+    const int64_t pq = __builtin_amdgcn_readlane(head, 11 + (blk >> 1));
+    if (pq < 0) continue;
+    char *op = static_cast<char *>(a.dq) + pq * kBlockBytes + qi * 128 + 64 * (blk & 1) + kg * 8;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const f32x16 &acc = dqacc[n];
+      u32x2 w;
+      w[0] = Tr::pack2(acc[4 * q] * a.scale, acc[4 * q + 1] * a.scale);
+      w[1] = Tr::pack2(acc[4 * q + 2] * a.scale, acc[4 * q + 3] * a.scale);
+      *reinterpret_cast<u32x2 *>(op + 16 * q) = w;
+    }
+  }
+}
+
 __global__ void fill_zero_f32_kernel(float *p, int64_t n) {
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) p[i] = 0.f;
@@ -1503,8 +1725,14 @@ int launch_bwd(const bsa_attn_args &a, hipStream_t s) {
     attn_bwd_order_kernel<<<16, kOrderThreads, 0, s>>>(a);
     if (int rc = check_launch("attn_bwd_order_kernel")) return rc;
   }
-  // dQ first: its kernel also leaves delta = rowsum(o * dO) and the tickets for the dK / dV kernel
-  if (qrows > 0) {
+  // With room for the dS blocks in the scratch: delta and the tickets first, then the dK / dV walk, which leaves
+  // dS^T of every pair behind, then dQ = dS K as a product of its own.  Without: the dQ kernel forms the scores
+  // and dS of its pairs a second time; it runs first and leaves delta and the tickets for the walk.
+  const bool from_ds = kEightWaves && kKvWalk && qrows > 0 && krows > 0 && bwd_lists(a).ds != nullptr;
+  if (from_ds) {
+    attn_bwd_delta_kernel<Tr><<<(unsigned)qrows, kBwdThreads, 0, s>>>(a);
+    if (int rc = check_launch("attn_bwd_delta_kernel")) return rc;
+  } else if (qrows > 0) {
     constexpr int lds = 2 * (NH + NHV) * kBlockBytes;
     BSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_bwd_q_kernel<Tr, NH, NHV>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, lds));
@@ -1522,6 +1750,13 @@ int launch_bwd(const bsa_attn_args &a, hipStream_t s) {
                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds_walk));
       attn_bwd_kv8_walk_kernel<Tr, NH, NHV><<<(unsigned)(kv_slots(krows) * 8), kKv8Threads, lds_walk, s>>>(a);
       if (int rc = check_launch("attn_bwd_kv8_walk_kernel")) return rc;
+      if (from_ds) {
+        constexpr int lds_dq = 2 * (NH + 1) * kBlockBytes;
+        BSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_bwd_dq_kernel<Tr, NH>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, lds_dq));
+        attn_bwd_dq_kernel<Tr, NH><<<(unsigned)(cdiv(qrows, 8) * 8), kBwdThreads, lds_dq, s>>>(a);
+        if (int rc = check_launch("attn_bwd_dq_kernel")) return rc;
+      }
     } else if (kEightWaves) {
       constexpr int lds8 = lds > 65536 ? lds : 65536;  // the tile buffers; at the end, the partial sums of both teams
       BSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_bwd_kv8_kernel<Tr, NH, NHV>),
@@ -1565,9 +1800,11 @@ int attn_mask_dead(const void *mask, int64_t n_mask_blocks, uint8_t *dead, hipSt
 }
 
 size_t attn_bwd_scratch_bytes(int64_t B, int64_t nq, int64_t nk, int64_t n_layout_blocks, int64_t n_mask_blocks) {
-  const size_t bytes = 2 * sizeof(BwdRecord) * (size_t)n_layout_blocks + (4 + 64) * (size_t)(B * nq + B * nk) + 64 +
-                       (size_t)n_mask_blocks;
-  return (bytes + 15) & ~(size_t)15;
+  return bwd_lists_bytes(B, nq, nk, n_layout_blocks, n_mask_blocks);
+}
+
+size_t attn_bwd_scratch_bytes_ds(int64_t B, int64_t nq, int64_t nk, int64_t n_layout_blocks, int64_t n_mask_blocks) {
+  return bwd_ds_offset(B, nq, nk, n_layout_blocks, n_mask_blocks) + (size_t)n_layout_blocks * kBlockBytes;
 }
 
 int attn_bwd_mfma(const bsa_attn_args &a, hipStream_t s) {

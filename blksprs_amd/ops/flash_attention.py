@@ -26,6 +26,10 @@ from ..utils.validation import (ensure_contiguous, mask_facts_enabled, validate_
                                 validate_sparsity, validate_sparsity_block_size, validate_sparsity_layout,
                                 validation_enabled)
 
+# The backward keeps dS of every pair of the attention layout (8 KiB per active block, in a scratch tensor that
+# lives for the call, or with the facts of a mask) when that takes at most this many bytes; above it, dS is
+# formed twice, as the reference does (blksprs/ops/flash_attention.py:1228-1480).
+KEPT_DS_LIMIT_BYTES = 4 << 30
 
 def _select_segmented_index_dtype(n_active_blocks: int, n_blocks_col: int) -> torch.dtype:
     """int32 unless the number of active blocks or the largest column id needs more."""
@@ -470,6 +474,11 @@ class _FlashAttention(torch.autograd.Function):
         n_layout_blocks = meta.tables.key_indices_i32.numel()
         n_mask_blocks = mask.size(0) if mask is not None else 0
         size = max(_capi.load().bsa_attn_bwd_scratch_bytes(B, nq, nk, n_layout_blocks, n_mask_blocks), 16)
+        # With room for dS of every pair (one block per active block of the attention layout) the dK / dV kernel
+        # leaves it behind and dQ = dS K is a product of its own; beyond the limit dS is formed a second time.
+        if (meta.sbs == 64 and q.dtype in (torch.bfloat16, torch.float16) and nh <= 2 and nhv <= 2
+                and n_layout_blocks * 64 * 64 * 2 <= KEPT_DS_LIMIT_BYTES):
+            size = _capi.load().bsa_attn_bwd_scratch_bytes_ds(B, nq, nk, n_layout_blocks, n_mask_blocks)
         stream = _capi.stream(q.device)
         facts = meta.facts
         # the records depend on the layouts and on the values of the mask and of the causal lengths only: a
@@ -478,7 +487,7 @@ class _FlashAttention(torch.autograd.Function):
         args.bwd_scratch_ready = 1 if scratch is not None and scratch.numel() == size else 0
         if not args.bwd_scratch_ready:
             scratch = torch.empty(size, dtype=torch.uint8, device=q.device)
-        args.bwd_scratch, args.n_layout_blocks = scratch.data_ptr(), n_layout_blocks
+        args.bwd_scratch, args.n_layout_blocks, args.bwd_scratch_bytes = scratch.data_ptr(), n_layout_blocks, size
         with _capi.on_device(q.device):
             _capi.call("bsa_attn_bwd", ctypes.byref(args), stream)
         if facts is not None and not args.bwd_scratch_ready and not torch.cuda.is_current_stream_capturing():

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define BSA_ABI_VERSION 1
+#define BSA_ABI_VERSION 2
 
 /* error codes */
 #define BSA_OK 0
@@ -379,6 +379,13 @@ typedef struct bsa_attn_args {
    * which its dK / dV kernel hands key rows to the workgroups that stay for the launch), so two calls that
    * overlap in time (different streams) need a scratch each. */
   int64_t bwd_scratch_ready;
+  /* Size of bwd_scratch in bytes, or 0 for "bsa_attn_bwd_scratch_bytes(...) and no more".  With at least
+   * bsa_attn_bwd_scratch_bytes_ds(...) bytes the dK / dV kernel also leaves dS of every visited pair in the
+   * scratch (one 64 x 64 block of the operand type per active block of the attention layout) and dQ = dS K is a
+   * product of its own; with less, the dQ kernel forms the scores and dS of its pairs a second time.  The
+   * reference recomputes (blksprs/ops/flash_attention.py:1228-1480); keeping dS trades memory for a third of the
+   * backward's matrix-core work. */
+  int64_t bwd_scratch_bytes;
 } bsa_attn_args;
 
 #define BSA_ATTN_RECORD_INTS 16
@@ -413,6 +420,10 @@ int bsa_attn_mask_dead(const void *mask, int64_t n_mask_blocks, int32_t sbs, uin
 
 /* Size in bytes of bsa_attn_args.bwd_scratch for these sizes (16-byte aligned buffer). */
 size_t bsa_attn_bwd_scratch_bytes(int64_t B, int64_t nq, int64_t nk, int64_t n_layout_blocks, int64_t n_mask_blocks);
+/* The same with room for the dS blocks (see bsa_attn_args.bwd_scratch_bytes): the lists, padded to a multiple of
+ * 4096 bytes, then n_layout_blocks * 8192 bytes. */
+size_t bsa_attn_bwd_scratch_bytes_ds(int64_t B, int64_t nq, int64_t nk, int64_t n_layout_blocks,
+                                     int64_t n_mask_blocks);
 
 /*
  * dq, dk, dv (and dbias) from the saved lse.  Replaces
