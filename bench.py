@@ -633,7 +633,7 @@ def attention_workload(dev, backward):
     return dict(step=step, flops=flops, alg_bytes=alg_bytes, dtype="bf16", bound="mfma", cpu_baseline=cpu_baseline,
                 check=check, executed_flops=flops * live_pairs / nnz,
                 kernel="attn_fwd_mfma_kernel" if not backward else
-                "attn_fwd_mfma_kernel + attn_bwd_q_kernel + attn_bwd_kv8_walk_kernel (one step; the mask_dead / records / order kernels ran once, in the warm-up)",
+                "attn_fwd_mfma_kernel + attn_bwd_delta_kernel + attn_bwd_kv8_walk_kernel + attn_bwd_dq_kernel (one step; the mask_dead / records / order kernels ran once, in the warm-up)",
                 config={"workload": "c4_flash_attention_bf16" + ("_fwd_bwd" if backward else "_fwd"),
                         "batch_heads": BH, "seq": n * sbs, "head_dim": nh * sbs, "sparsity_block_size": sbs,
                         "layout_blocks": nnz, "mask": "explicit causal blocks"})

@@ -254,6 +254,16 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_records_kernel(bsa_attn_
   const bool causal = a.causal_lengths != nullptr;
   const int64_t seq_len = causal ? a.causal_lengths[b] : 0;
   const int begin = offsets[row], end = offsets[row + 1];
+  // does some score of the pair survive?  pm: its mask block
+  auto pair_live = [&](int64_t qb, int64_t kb, int32_t &pm) -> bool {
+    pm = -1;
+    if (causal && (kb > qb || qb * kSbs >= seq_len || kb * kSbs >= seq_len)) return false;
+    if (a.mask) {
+      pm = checked_index(a.pidx_mask, (b * a.nq + qb) * a.nk + kb, a.n_mask_blocks);
+      if (pm >= 0 && L.mask_dead[pm]) return false;
+    }
+    return true;
+  };
   int n = begin;
   for (int e0 = begin; e0 < end; e0 += 64) {
     const int e = e0 + lane;
@@ -261,12 +271,8 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_records_kernel(bsa_attn_
     const int64_t other = live ? indices[e] : 0;
     const int64_t qb = by_key ? other : mine, kb = by_key ? mine : other;
     const int64_t pair = (b * a.nq + qb) * a.nk + kb;
-    if (live && causal && (kb > qb || qb * kSbs >= seq_len || kb * kSbs >= seq_len)) live = false;
     int32_t pm = -1;
-    if (live && a.mask) {
-      pm = checked_index(a.pidx_mask, pair, a.n_mask_blocks);
-      if (pm >= 0 && L.mask_dead[pm]) live = false;
-    }
+    if (live) live = pair_live(qb, kb, pm);
     const unsigned long long votes = __ballot(live);
     if (live) {
       BwdRecord r;
@@ -281,18 +287,16 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_records_kernel(bsa_attn_
       }
       r.mask = pm;
       r.bias = a.bias ? checked_index(a.pidx_bias, pair, a.n_bias_blocks) : -1;
-      // the pair's position in the lists per query block: entry e itself, or where kb stands in the (ascending)
-      // list of query block qb
-      int at = e;
+      // the pair's position in the list of its query block as written here (without the dead pairs): where this
+      // record goes, or, from the side of the key block, the row's start plus the live pairs in front of kb
+      int at = n + __popcll(votes & ((1ull << lane) - 1));
       if (by_key) {
-        int lo = a.key_offsets[b * a.nq + qb], hi = a.key_offsets[b * a.nq + qb + 1];
-        const int last = hi - 1;
-        while (lo < hi) {
-          const int mid = (lo + hi) >> 1;
-          if (a.key_indices[mid] < kb) lo = mid + 1;
-          else hi = mid;
+        const int q_begin = a.key_offsets[b * a.nq + qb], q_end = a.key_offsets[b * a.nq + qb + 1];
+        at = q_begin;
+        for (int i = q_begin; i < q_end && a.key_indices[i] < kb; ++i) {
+          int32_t ignored;
+          at += pair_live(qb, a.key_indices[i], ignored) ? 1 : 0;
         }
-        at = lo <= last ? lo : last;  // the two lists hold the same pairs: kb is found; never past the row
       }
       r.pair = at;
       out[n + __popcll(votes & ((1ull << lane) - 1))] = r;
@@ -1150,7 +1154,6 @@ __device__ __forceinline__ void attn_bwd_kv8_walk(const bsa_attn_args &a, char *
         const int qb = qb_nxt;
         const int64_t pm = pm_nxt, pb = pb_nxt;
         const int pair = pair_nxt;
-        store_pending_ds();  // of the tile before: it has this whole tile to get there before the next wait
         uint32_t mbits = 0;
         if (pm >= 0) {
           const uint8_t *mp = reinterpret_cast<const uint8_t *>(base + kMask) + (32 * wi + 4 * kg) * kSbs + 32 * wj + li;
@@ -1187,6 +1190,9 @@ __device__ __forceinline__ void attn_bwd_kv8_walk(const bsa_attn_args &a, char *
         request_record((!more && next_tile) ? (q_begin_next + 1 < q_end_next ? q_begin_next + 1 : q_end_next - 1)
                                             : clamp_e(e + 2));
 
+        // dS of the tile before: behind the requests for the next tile, and with this whole tile to get there
+        // before the next wait
+        store_pending_ds();
         KvCarry carry;
         kv_first_half<Tr, NH, NHV, DK, DV>(carry, f0, live, a, base, qb, pm, pb, mbits, causal, seq_len, (int)kb, kpos,
                                            qk_scale, wi, wj, li, kg, lane, kfr, vfr, p_lds);
@@ -1584,17 +1590,25 @@ __device__ static inline u32x4 frag_ds(const char *blob, int wi, int wj, int key
 }
 __device__ static inline int query_of_lane(int lane) { return 8 * ((lane & 15) >> 2) + 4 * ((lane >> 4) & 1) + (lane & 3); }
 
-// dQ of one query block from the dS^T blocks the dK / dV kernel has written: dQ^T += K^T dS^T, one product per
-// pair and no scores.  Wave (wi, wj) owns queries 32 wi .. + 31 and the head-dimension columns 32 NH wj .. + 32 NH - 1
-// (of the NH slices: slice wj with two slices, half of the slice with one) and contracts over all 64 keys of every
-// tile, so no wave needs another's sums.  A tile is the pair's K slices and its dS^T block, both copied
-// asynchronously into LDS and both read with the transposing load (the contraction runs over the keys, the rows
-// of both).  Every pair of the list is multiplied: quadrants without a surviving score hold zeros.
+// dQ of one query block from the dS blocks the dK / dV kernel has written: dQ^T += K^T dS^T, one product per pair
+// and no scores.  Wave (wi, wj) owns queries 32 wi .. + 31 (in the order of query_of_lane) and the head-dimension
+// columns 32 NH wj .. + 32 NH - 1 (slice wj with two slices, half of the slice with one) and contracts over all 64
+// keys of every tile, so no wave needs another's sums.  The dS block of the e-th pair of the list is block e of
+// the scratch region (the records are numbered that way), so its address needs no record.  A tile is the K slices
+// and the dS block of a pair, 8 KiB each, copied asynchronously into LDS; there is ONE buffer for the K slices
+// (their copies are requested when the products of the tile before are done, and waited for) and two for dS
+// (the block of the next tile, which comes from memory, is requested one tile ahead).  What hides the latency of
+// the copies is the number of workgroups per compute unit that the small buffers allow, each at another point of
+// its list: the kernel's time is that of its copies (without the products it runs as long; without the copies in
+// a third of the time).  Measured on configuration 4 of the benchmark: two buffers for the whole tile and three
+// workgroups per compute unit 215 microseconds; a ring of five dS blocks with two waves copying dS and two K, two
+// workgroups, 238; one buffer, five workgroups, 198; with the second dS buffer 195.  Every pair of the list is
+// multiplied: quadrants without a surviving score hold zeros.
+constexpr int kDqWorkgroupsPerCu = 5;
 template <typename Tr, int NH>
-__global__ __launch_bounds__(kBwdThreads, 3) void attn_bwd_dq_kernel(bsa_attn_args a) {
+__global__ __launch_bounds__(kBwdThreads, kDqWorkgroupsPerCu) void attn_bwd_dq_kernel(bsa_attn_args a) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  constexpr int kKRows = 0, kDsRows = NH * kBlockBytes;
-  constexpr int kBufBytes = (NH + 1) * kBlockBytes;
+  constexpr int kDsRows = NH * kBlockBytes;
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = first_lane(tid >> 6);
@@ -1622,59 +1636,66 @@ __global__ __launch_bounds__(kBwdThreads, 3) void attn_bwd_dq_kernel(bsa_attn_ar
   const int k_begin = __builtin_amdgcn_readlane(head, 9), k_end = __builtin_amdgcn_readlane(head, 10);
   if (k_begin < k_end) {
     const int32_t *recs = reinterpret_cast<const int32_t *>(lists.key_rec);
-    auto load_record = [&](int pos) -> int {
-      int v = -1;
-      if (lane < 8) v = recs[(int64_t)pos * 8 + lane];
-      return v;
+    // eight records at a time, field f of the j-th in lane 8 j + f (two lines of the list, which come from memory:
+    // requested eight tiles before their first use)
+    auto load_records = [&](int first) -> int {
+      int pos = first + (lane >> 3);
+      pos = pos < k_end ? pos : k_end - 1;
+      return recs[(int64_t)pos * 8 + (lane & 7)];
     };
-    auto clamp_e = [&](int e) { return e < k_end ? e : k_end - 1; };
-    auto fetch = [&](int rec, int buf) {
-      char *base = smem + buf * kBufBytes;
+    // the K slices of the tile of record j of `chunk`, a quarter of every block per wave, into the one K buffer
+    auto fetch_k = [&](int chunk, int j) {
 #pragma unroll
       for (int h = 0; h < NH; ++h) {
-        const int pk = __builtin_amdgcn_readlane(rec, 1 + h);
+        const int pk = __builtin_amdgcn_readlane(chunk, 8 * j + 1 + h);
         copy_block(static_cast<const char *>(a.k) + (int64_t)(pk >= 0 ? pk : 0) * kBlockBytes, pk >= 0,
-                   base + kKRows + h * kBlockBytes, wave, lane, tid);
+                   smem + h * kBlockBytes, wave, lane, tid);
       }
-      // the dS block as it lies, 2 KiB per wave
-      const int pair = __builtin_amdgcn_readlane(rec, 7);
-      copy_2k_to_lds(lists.ds + (int64_t)pair * kBlockBytes + wave * 2048, lane * 16, base + kDsRows + wave * 2048);
+    };
+    // the dS block of list entry e (it comes from memory: one tile ahead, into the other of two buffers)
+    auto fetch_ds = [&](int e) {
+      copy_2k_to_lds(lists.ds + (int64_t)e * kBlockBytes + wave * 2048, lane * 16,
+                     smem + kDsRows + first_lane((e - k_begin) & 1) * kBlockBytes + wave * 2048);
     };
 
-    int rec = load_record(clamp_e(k_begin + 1));
-    fetch(head, 0);
-    __builtin_amdgcn_s_waitcnt(0x0F70);
-    __syncthreads();
-
     const int col_t = 16 * ((lane >> 4) & 1);
+    int chunk = load_records(k_begin), chunk_next = chunk;
+    fetch_ds(k_begin);
     for (int e = k_begin; e < k_end; ++e) {
-      const int buf = (e - k_begin) & 1;
-      const char *base = smem + buf * kBufBytes;
-      const bool more = e + 1 < k_end;
-      if (more) fetch(rec, buf ^ 1);
-      rec = load_record(clamp_e(e + 2));
+      const int j = (e - k_begin) & 7;
+      if (j == 0 && e != k_begin) chunk = chunk_next;
+      // the header holds the first record, so the first tile does not wait for the list
+      if (e == k_begin) fetch_k(head, 0);
+      else fetch_k(chunk, j);
+      // this tile's copies have landed; the next tile's dS block (two loads, the youngest) may stay in flight
+      if (e + 1 < k_end) {
+        fetch_ds(e + 1);
+        __builtin_amdgcn_s_waitcnt(0x0F72);
+      } else {
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+      }
+      __syncthreads();
+      // the next eight records: in flight behind this tile's products
+      if (j == 0 && e + 8 < k_end) chunk_next = load_records(e + 8);
+      const char *ds_tile = smem + kDsRows + ((e - k_begin) & 1) * kBlockBytes;
 
       // dS^T as the second operand: query 32 wi + query_of_lane, keys 16 u + 4 kg .. + 3 and + 8 .. + 11
       u32x4 dsf[4];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) dsf[u] = frag_ds(base + kDsRows, wi, u >> 1, 16 * (u & 1) + 4 * kg, lane);
+      for (int u = 0; u < 4; ++u) dsf[u] = frag_ds(ds_tile, wi, u >> 1, 16 * (u & 1) + 4 * kg, lane);
       // stage n: column block first_block + n of K^T against all four key steps
       staged_products<NH>(
           [&](int n, u32x4(&f)[4]) {
             const int blk = first_block + n;
 #pragma unroll
             for (int u = 0; u < 4; ++u)
-              f[u] = frag_cols_t(base + kKRows + (blk >> 1) * kBlockBytes, 16 * u + 4 * kg, 32 * (blk & 1) + col_t, lane);
+              f[u] = frag_cols_t(smem + (blk >> 1) * kBlockBytes, 16 * u + 4 * kg, 32 * (blk & 1) + col_t, lane);
           },
           [&](int n, u32x4(&f)[4]) {
 #pragma unroll
             for (int u = 0; u < 4; ++u) dqacc[n] = Tr::mfma(f[u], dsf[u], dqacc[n]);
           });
-
-      // the copies of the next tile have landed (vmcnt(0): the record of the tile after it, requested right
-      // behind them, as well)
-      if (more) __builtin_amdgcn_s_waitcnt(0x0F70);
-      __syncthreads();
+      __syncthreads();  // the buffer is free
     }
   }
 
@@ -1751,7 +1772,7 @@ int launch_bwd(const bsa_attn_args &a, hipStream_t s) {
       attn_bwd_kv8_walk_kernel<Tr, NH, NHV><<<(unsigned)(kv_slots(krows) * 8), kKv8Threads, lds_walk, s>>>(a);
       if (int rc = check_launch("attn_bwd_kv8_walk_kernel")) return rc;
       if (from_ds) {
-        constexpr int lds_dq = 2 * (NH + 1) * kBlockBytes;
+        constexpr int lds_dq = (NH + 2) * kBlockBytes;
         BSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_bwd_dq_kernel<Tr, NH>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, lds_dq));
         attn_bwd_dq_kernel<Tr, NH><<<(unsigned)(cdiv(qrows, 8) * 8), kBwdThreads, lds_dq, s>>>(a);

@@ -69,6 +69,7 @@ def _run_case(device, dtype, sbs, B, nq, nk, nh, nhv, density, seed, use_mask=Fa
     assert_close(vd.grad, v64.grad, gtol, "dV " + tag)
     if bias is not None:
         assert_close(bd.grad, b64.grad, gtol, "dBias " + tag)
+    return qd.grad, kd.grad, vd.grad
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
@@ -116,6 +117,24 @@ def test_dk_dv_of_more_key_blocks_than_workgroups(device, dtype, use_mask, use_b
     B, nq, nk = (3, 90, 90) if use_causal else (4, 12, 100)  # the native causal predicate wants a square layout
     _run_case(device, dtype, 64, B, nq, nk, nh, nhv, 0.08, seed=23, use_mask=use_mask, use_bias=use_bias,
               use_causal=use_causal)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("use_mask,use_bias,use_causal,nh,nhv", [(False, False, False, 2, 2), (True, True, False, 1, 2),
+                                                               (False, False, True, 2, 1), (True, False, True, 1, 1)])
+def test_backward_without_room_for_ds_forms_it_twice(device, dtype, use_mask, use_bias, use_causal, nh, nhv, monkeypatch):
+    """With room in the scratch the dK / dV kernel leaves dS of every pair behind and dQ = dS K is a product of its
+    own (the path every other backward test of 64 x 64 16-bit blocks takes); without, the dQ kernel forms the scores
+    and dS a second time.  Both against the oracle, and the two against each other."""
+    import importlib
+    fa = importlib.import_module("blksprs_amd.ops.flash_attention")
+    B, nq, nk = (2, 24, 24) if use_causal else (2, 12, 40)
+    kwargs = dict(seed=31, use_mask=use_mask, use_bias=use_bias, use_causal=use_causal)
+    kept = _run_case(device, dtype, 64, B, nq, nk, nh, nhv, 0.3, **kwargs)
+    monkeypatch.setattr(fa, "KEPT_DS_LIMIT_BYTES", 0)
+    twice = _run_case(device, dtype, 64, B, nq, nk, nh, nhv, 0.3, **kwargs)
+    for name, a, b in zip(("dQ", "dK", "dV"), kept, twice):
+        assert_close(a, b.double(), 1e-2, f"{name}, dS kept against dS formed twice")
 
 
 def test_bigbird_layout_with_causal_mask_head_dim_128(device):
