@@ -21,15 +21,10 @@ from ..utils.blksprs_tensor import BlksprsTensor
 from ..utils.tools import (CacheHolder, INT32_INDEX_MAX, as_base_tensor, cast_for_autocast, csr_indices_from_packed,
                            PackedLayout, eager_only, finalize_layout_cache, layout_bytes, pack_layout,
                            pack_layouts, prepare_layout_cache)
-from ..utils.validation import (ensure_contiguous, mask_facts_enabled, validate_binary, validate_contiguous,
+from ..utils.validation import (ensure_contiguous, kept_ds_limit, mask_facts_enabled, validate_binary, validate_contiguous,
                                 validate_device, validate_dimensions, validate_dtype_float, validate_shape,
                                 validate_sparsity, validate_sparsity_block_size, validate_sparsity_layout,
                                 validation_enabled)
-
-# The backward keeps dS of every pair of the attention layout (8 KiB per active block, in a scratch tensor that
-# lives for the call, or with the facts of a mask) when that takes at most this many bytes; above it, dS is
-# formed twice, as the reference does (blksprs/ops/flash_attention.py:1228-1480).
-KEPT_DS_LIMIT_BYTES = 4 << 30
 
 def _select_segmented_index_dtype(n_active_blocks: int, n_blocks_col: int) -> torch.dtype:
     """int32 unless the number of active blocks or the largest column id needs more."""
@@ -475,9 +470,10 @@ class _FlashAttention(torch.autograd.Function):
         n_mask_blocks = mask.size(0) if mask is not None else 0
         size = max(_capi.load().bsa_attn_bwd_scratch_bytes(B, nq, nk, n_layout_blocks, n_mask_blocks), 16)
         # With room for dS of every pair (one block per active block of the attention layout) the dK / dV kernel
-        # leaves it behind and dQ = dS K is a product of its own; beyond the limit dS is formed a second time.
+        # leaves it behind and dQ = dS K is a product of its own; beyond the limit (set_kept_ds_limit) dS is formed a
+        # second time, as the reference does (blksprs/ops/flash_attention.py:1228-1480).
         if (meta.sbs == 64 and q.dtype in (torch.bfloat16, torch.float16) and nh <= 2 and nhv <= 2
-                and n_layout_blocks * 64 * 64 * 2 <= KEPT_DS_LIMIT_BYTES):
+                and n_layout_blocks * 64 * 64 * 2 <= kept_ds_limit()):
             size = _capi.load().bsa_attn_bwd_scratch_bytes_ds(B, nq, nk, n_layout_blocks, n_mask_blocks)
         stream = _capi.stream(q.device)
         facts = meta.facts

@@ -65,6 +65,22 @@ def enable_mask_facts() -> None:
     _state.mask_facts = True
 
 
+_kept_ds_limit = 4 << 30
+
+
+def kept_ds_limit() -> int:
+    return _kept_ds_limit
+
+
+def set_kept_ds_limit(n_bytes: int) -> None:
+    """The backward of ``flash_attention`` on 64 x 64 16-bit blocks keeps dS of every pair in a scratch tensor
+    (8 KiB per active block of the attention layout; with it dQ costs one matrix product per pair instead of three)
+    when that takes at most ``n_bytes`` (default 4 GiB, for the whole process); 0: never, dS is formed twice, as
+    the reference does (blksprs/ops/flash_attention.py:1228-1480)."""
+    global _kept_ds_limit
+    _kept_ds_limit = int(n_bytes)
+
+
 def _check(fn):
     """Turns ``fn`` into a no-op while validation is disabled."""
 

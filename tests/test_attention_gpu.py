@@ -126,12 +126,11 @@ def test_backward_without_room_for_ds_forms_it_twice(device, dtype, use_mask, us
     """With room in the scratch the dK / dV kernel leaves dS of every pair behind and dQ = dS K is a product of its
     own (the path every other backward test of 64 x 64 16-bit blocks takes); without, the dQ kernel forms the scores
     and dS a second time.  Both against the oracle, and the two against each other."""
-    import importlib
-    fa = importlib.import_module("blksprs_amd.ops.flash_attention")
+    from blksprs_amd.utils import validation
     B, nq, nk = (2, 24, 24) if use_causal else (2, 12, 40)
     kwargs = dict(seed=31, use_mask=use_mask, use_bias=use_bias, use_causal=use_causal)
     kept = _run_case(device, dtype, 64, B, nq, nk, nh, nhv, 0.3, **kwargs)
-    monkeypatch.setattr(fa, "KEPT_DS_LIMIT_BYTES", 0)
+    monkeypatch.setattr(validation, "_kept_ds_limit", 0)
     twice = _run_case(device, dtype, 64, B, nq, nk, nh, nhv, 0.3, **kwargs)
     for name, a, b in zip(("dQ", "dK", "dV"), kept, twice):
         assert_close(a, b.double(), 1e-2, f"{name}, dS kept against dS formed twice")
