@@ -263,3 +263,19 @@ def test_library_operators_are_registered_with_shape_functions():
         xf = torch.empty((5, 32, 32), device="meta")
         assert ops.softmax_fused_forward(xf, table, 6, 32).shape == xf.shape
         assert ops.softmax_fused_backward(xf, xf, table, 6, 32).dtype == torch.float32
+
+
+def test_the_limit_on_kept_ds_is_a_process_wide_setting():
+    """``bs.utils.set_kept_ds_limit`` is what ``flash_attention``'s backward asks (through ``kept_ds_limit``) before it
+    requests room for dS; 0 turns the kept dS off."""
+    import blksprs_amd as bs
+    from blksprs_amd.utils import validation
+    before = validation.kept_ds_limit()
+    try:
+        assert before == 4 << 30
+        bs.utils.set_kept_ds_limit(0)
+        assert validation.kept_ds_limit() == 0
+        bs.utils.set_kept_ds_limit(1 << 20)
+        assert validation.kept_ds_limit() == 1 << 20
+    finally:
+        bs.utils.set_kept_ds_limit(before)
