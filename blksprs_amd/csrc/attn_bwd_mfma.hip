@@ -1254,37 +1254,44 @@ __device__ __forceinline__ void attn_bwd_kv8_walk(const bsa_attn_args &a, char *
     if constexpr (DK) reduce_partner(dkacc, reduce_lds, wi == 1, wj, lane);
     if constexpr (DV) reduce_partner(dvacc, reduce_lds, wi == 1, wj, lane);
     const int t_after = first_lane(mailbox[0]);
-    if (wi == 0) {
-      // lane: key 32 wj + li; register 4 q + t of half db: column 32 db + 8 q + 4 kg + t
+    // The sums leave as whole rows: the waves that hold them (lane: key 32 wj + li; register 4 q + t of half db:
+    // column 32 db + 8 q + 4 kg + t, eight bytes of a row per lane and store) write the rounded block into this
+    // team's part of R, as rows of 128 bytes with the 16-byte chunks swizzled by the row, and all four waves of the
+    // team store it from there, 16 rows each, eight lanes to a row: whole lines per instruction, past the caches.
+    // (Stores of eight bytes per lane straight from the registers are written to memory as partial lines, twice
+    // the bytes, and are waited for with the copies of the next tile.)
+    {
+      constexpr int kOut = DK ? NH : NHV;
+      char *rows_lds = reinterpret_cast<char *>(reduce_lds);
+      __syncthreads();  // the partial sums have been read
+      if (wi == 0) {
+        const int row = 32 * wj + li;
+        const float factor = DK ? a.scale : 1.f;
 #pragma unroll
-      for (int h = 0; h < (DK ? NH : 0); ++h) {
-        if (pk[h] < 0) continue;
-        char *op = static_cast<char *>(a.dk) + pk[h] * kBlockBytes + (32 * wj + li) * 128 + kg * 8;
+        for (int h = 0; h < kOut; ++h)
 #pragma unroll
-        for (int db = 0; db < 2; ++db)
+          for (int db = 0; db < 2; ++db)
 #pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const f32x16 &acc = dkacc[2 * h + db];
-            u32x2 w;
-            w[0] = Tr::pack2(acc[4 * q] * a.scale, acc[4 * q + 1] * a.scale);
-            w[1] = Tr::pack2(acc[4 * q + 2] * a.scale, acc[4 * q + 3] * a.scale);
-            *reinterpret_cast<u32x2 *>(op + 64 * db + 16 * q) = w;
-          }
+            for (int q = 0; q < 4; ++q) {
+              const f32x16 &acc = DK ? dkacc[DK ? 2 * h + db : 0] : dvacc[DV ? 2 * h + db : 0];
+              u32x2 w;
+              w[0] = Tr::pack2(acc[4 * q] * factor, acc[4 * q + 1] * factor);
+              w[1] = Tr::pack2(acc[4 * q + 2] * factor, acc[4 * q + 3] * factor);
+              *reinterpret_cast<u32x2 *>(rows_lds + h * kBlockBytes + row * 128 + (((4 * db + q) ^ (row & 7)) << 4) + 8 * kg) = w;
+            }
       }
+      __syncthreads();
 #pragma unroll
-      for (int h = 0; h < (DV ? NHV : 0); ++h) {
-        if (pv[h] < 0) continue;
-        char *op = static_cast<char *>(a.dv) + pv[h] * kBlockBytes + (32 * wj + li) * 128 + kg * 8;
+      for (int h = 0; h < kOut; ++h) {
+        const int64_t p = DK ? pk[DK ? h : 0] : pv[DV ? h : 0];
+        if (p < 0) continue;
+        char *out = static_cast<char *>(DK ? a.dk : a.dv) + p * kBlockBytes;
 #pragma unroll
-        for (int db = 0; db < 2; ++db)
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const f32x16 &acc = dvacc[2 * h + db];
-            u32x2 w;
-            w[0] = Tr::pack2(acc[4 * q], acc[4 * q + 1]);
-            w[1] = Tr::pack2(acc[4 * q + 2], acc[4 * q + 3]);
-            *reinterpret_cast<u32x2 *>(op + 64 * db + 16 * q) = w;
-          }
+        for (int i = 0; i < 2; ++i) {
+          const int r = 16 * quad + 8 * i + (lane >> 3), c = lane & 7;
+          const u32x4 v = *reinterpret_cast<const u32x4 *>(rows_lds + h * kBlockBytes + r * 128 + ((c ^ (r & 7)) << 4));
+          __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(out + r * 128 + c * 16));
+        }
       }
     }
     if (!has_next) break;
