@@ -1720,21 +1720,34 @@ __global__ __launch_bounds__(kBwdThreads, kDqWorkgroupsPerCu) void attn_bwd_dq_k
     }
   }
 
-  // ---- scale, store: register 4 q + t of block n = column 32 (first_block + n) + 8 q + 4 kg + t ----
+  // ---- scale, round, store.  Register 4 q + t of block n is column 32 (first_block + n) + 8 q + 4 kg + t of the
+  // lane's query: eight bytes of a row at a time.  The rounded block goes through LDS (rows of 128 bytes, chunks
+  // swizzled by the row; the tile buffers are free) and leaves as whole rows, 16 per wave, eight lanes to a row,
+  // past the caches: half the bytes written of stores straight from the registers. ----
   const int qi = 32 * wi + query_of_lane(lane);
 #pragma unroll
   for (int n = 0; n < NH; ++n) {
     const int blk = first_block + n;
-    const int64_t pq = __builtin_amdgcn_readlane(head, 11 + (blk >> 1));
-    if (pq < 0) continue;
-    char *op = static_cast<char *>(a.dq) + pq * kBlockBytes + qi * 128 + 64 * (blk & 1) + kg * 8;
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const f32x16 &acc = dqacc[n];
       u32x2 w;
       w[0] = Tr::pack2(acc[4 * q] * a.scale, acc[4 * q + 1] * a.scale);
       w[1] = Tr::pack2(acc[4 * q + 2] * a.scale, acc[4 * q + 3] * a.scale);
-      *reinterpret_cast<u32x2 *>(op + 16 * q) = w;
+      *reinterpret_cast<u32x2 *>(smem + (blk >> 1) * kBlockBytes + qi * 128 + (((4 * (blk & 1) + q) ^ (qi & 7)) << 4) + 8 * kg) = w;
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int h = 0; h < NH; ++h) {
+    const int64_t pq = __builtin_amdgcn_readlane(head, 11 + h);
+    if (pq < 0) continue;
+    char *out = static_cast<char *>(a.dq) + pq * kBlockBytes;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int r = 16 * wave + 8 * i + (lane >> 3), c = lane & 7;
+      const u32x4 v = *reinterpret_cast<const u32x4 *>(smem + h * kBlockBytes + r * 128 + ((c ^ (r & 7)) << 4));
+      __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(out + r * 128 + c * 16));
     }
   }
 }
