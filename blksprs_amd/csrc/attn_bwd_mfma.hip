@@ -154,6 +154,36 @@ __device__ inline void reduce_partner(f32x16 (&acc)[N], float *lds, bool writer,
   }
 }
 
+// The same sum, shared out between the two waves of a pair: of the accumulators 2 h and 2 h + 1 (the two column
+// halves of slice h) each wave gives one away and adds what it gets to the other, so both move and add half as
+// much and both end with a finished half.  The caller has put the half it keeps into the EVEN accumulators (the
+// wave with partner bit 1 swaps its pairs first), so that one copy of these loops serves both waves.
+// Layout [slot][giver][h][r / 4][lane][r % 4].
+template <int N>
+__device__ inline void exchange_odd_for_even(f32x16 (&acc)[N], float *lds, int giver, int slot, int lane) {
+  static_assert(N % 2 == 0, "pairs of accumulators");
+  constexpr int kPerWave = (N / 2) * 16 * 64;
+  f32x4 *give = reinterpret_cast<f32x4 *>(lds + (size_t)(slot * 2 + giver) * kPerWave) + lane;
+  const f32x4 *take = reinterpret_cast<const f32x4 *>(lds + (size_t)(slot * 2 + (1 - giver)) * kPerWave) + lane;
+  __syncthreads();  // the tile buffers are free
+#pragma unroll
+  for (int h = 0; h < N / 2; ++h)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const f32x16 &out = acc[2 * h + 1];
+      give[(h * 4 + q) * 64] = f32x4{out[4 * q], out[4 * q + 1], out[4 * q + 2], out[4 * q + 3]};
+    }
+  __syncthreads();
+#pragma unroll
+  for (int h = 0; h < N / 2; ++h)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const f32x4 v = take[(h * 4 + q) * 64];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) acc[2 * h][4 * q + t] += v[t];
+    }
+}
+
 // ---------------------------------------------------------------------------------------------------------
 // Records of the pairs that can contribute.  A (query block, key block) pair whose mask block masks every score,
 // or that the causal predicate rules out as a whole, has P = dS = 0.  Which pairs those are depends on the mask's
@@ -1251,11 +1281,30 @@ __device__ __forceinline__ void attn_bwd_kv8_walk(const bsa_attn_args &a, char *
     }
     if (tid == 0) mailbox[0] = drawn;  // published by the barriers of the sum
     // ---- add the two query halves, scale, store
-    if constexpr (DK) reduce_partner(dkacc, reduce_lds, wi == 1, wj, lane);
-    if constexpr (DV) reduce_partner(dvacc, reduce_lds, wi == 1, wj, lane);
+    // wave wi keeps column half wi of every slice: it moves that half into the even accumulators
+    if (wi == 1) {
+      if constexpr (DK) {
+#pragma unroll
+        for (int h = 0; h < NH; ++h) {
+          const f32x16 t = dkacc[2 * h];
+          dkacc[2 * h] = dkacc[2 * h + 1];
+          dkacc[2 * h + 1] = t;
+        }
+      }
+      if constexpr (DV) {
+#pragma unroll
+        for (int h = 0; h < NHV; ++h) {
+          const f32x16 t = dvacc[2 * h];
+          dvacc[2 * h] = dvacc[2 * h + 1];
+          dvacc[2 * h + 1] = t;
+        }
+      }
+    }
+    if constexpr (DK) exchange_odd_for_even(dkacc, reduce_lds, wi, wj, lane);
+    if constexpr (DV) exchange_odd_for_even(dvacc, reduce_lds, wi, wj, lane);
     const int t_after = first_lane(mailbox[0]);
-    // The sums leave as whole rows: the waves that hold them (lane: key 32 wj + li; register 4 q + t of half db:
-    // column 32 db + 8 q + 4 kg + t, eight bytes of a row per lane and store) write the rounded block into this
+    // The sums leave as whole rows: every wave holds, for its key 32 wj + li, the column half db = wi of each slice
+    // (register 4 q + t: column 32 db + 8 q + 4 kg + t, eight bytes of a row per lane) and writes it, rounded, into this
     // team's part of R, as rows of 128 bytes with the 16-byte chunks swizzled by the row, and all four waves of the
     // team store it from there, 16 rows each, eight lanes to a row: whole lines per instruction, past the caches.
     // (Stores of eight bytes per lane straight from the registers are written to memory as partial lines, twice
@@ -1264,21 +1313,19 @@ __device__ __forceinline__ void attn_bwd_kv8_walk(const bsa_attn_args &a, char *
       constexpr int kOut = DK ? NH : NHV;
       char *rows_lds = reinterpret_cast<char *>(reduce_lds);
       __syncthreads();  // the partial sums have been read
-      if (wi == 0) {
+      {
         const int row = 32 * wj + li;
         const float factor = DK ? a.scale : 1.f;
 #pragma unroll
         for (int h = 0; h < kOut; ++h)
 #pragma unroll
-          for (int db = 0; db < 2; ++db)
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-              const f32x16 &acc = DK ? dkacc[DK ? 2 * h + db : 0] : dvacc[DV ? 2 * h + db : 0];
-              u32x2 w;
-              w[0] = Tr::pack2(acc[4 * q] * factor, acc[4 * q + 1] * factor);
-              w[1] = Tr::pack2(acc[4 * q + 2] * factor, acc[4 * q + 3] * factor);
-              *reinterpret_cast<u32x2 *>(rows_lds + h * kBlockBytes + row * 128 + (((4 * db + q) ^ (row & 7)) << 4) + 8 * kg) = w;
-            }
+          for (int q = 0; q < 4; ++q) {
+            const f32x16 &acc = DK ? dkacc[DK ? 2 * h : 0] : dvacc[DV ? 2 * h : 0];  // column half wi
+            u32x2 w;
+            w[0] = Tr::pack2(acc[4 * q] * factor, acc[4 * q + 1] * factor);
+            w[1] = Tr::pack2(acc[4 * q + 2] * factor, acc[4 * q + 3] * factor);
+            *reinterpret_cast<u32x2 *>(rows_lds + h * kBlockBytes + row * 128 + (((4 * wi + q) ^ (row & 7)) << 4) + 8 * kg) = w;
+          }
       }
       __syncthreads();
 #pragma unroll
