@@ -466,11 +466,13 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
   // bit they would buy is rounded away with the other fifteen when the quotient becomes a 16-bit value
   l_i = sum_across32(l_i);
   const float inv_l = (l_i != 0.f) ? 1.f / l_i : 0.f;
+  // A lane holds eight bytes of a row at a time (register 4 q + t of half db: column 32 db + 8 q + 4 kg + t).  The
+  // wave writes its 32 rounded rows into LDS (the V tiles are free: every wave has passed the last tile's barrier),
+  // 128 bytes per row with the 16-byte chunks swizzled by the row, and stores them from there, eight lanes to a
+  // row: whole lines per instruction, past the caches.  Rows and chunks are the wave's own, so no barrier.
+  char *rows_lds = lds_v + (wave >> 1) * NHV * kBlockBytes;
 #pragma unroll
-  for (int h = 0; h < NHV; ++h) {
-    const int64_t po = a.pidx_o[row * NHV + h];
-    if (po < 0 || po >= a.n_o_blocks) continue;
-    char *op = static_cast<char *>(a.o) + po * kBlockBytes + qi * 128 + kg * 8;
+  for (int h = 0; h < NHV; ++h)
 #pragma unroll
     for (int db = 0; db < 2; ++db)
 #pragma unroll
@@ -481,8 +483,19 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
         u32x2 w;
         w[0] = Tr::pack2(v[0], v[1]);
         w[1] = Tr::pack2(v[2], v[3]);
-        *reinterpret_cast<u32x2 *>(op + 64 * db + 16 * q) = w;
+        *reinterpret_cast<u32x2 *>(rows_lds + h * kBlockBytes + qi * 128 + (((4 * db + q) ^ (qi & 7)) << 4) + 8 * kg) = w;
       }
+#pragma unroll
+  for (int h = 0; h < NHV; ++h) {
+    const int64_t po = a.pidx_o[row * NHV + h];
+    if (po < 0 || po >= a.n_o_blocks) continue;
+    char *out = static_cast<char *>(a.o) + po * kBlockBytes;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = 32 * (wave & 1) + 8 * i + (lane >> 3), c = lane & 7;
+      const u32x4 v = *reinterpret_cast<const u32x4 *>(rows_lds + h * kBlockBytes + r * 128 + ((c ^ (r & 7)) << 4));
+      __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(out + r * 128 + c * 16));
+    }
   }
   if (kg == 0) a.lse[row * kSbs + qi] = (l_i != 0.f) ? m_i + log2f(l_i) : -INFINITY;
 }
