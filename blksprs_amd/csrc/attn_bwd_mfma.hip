@@ -421,7 +421,8 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_delta_kernel(bsa_attn_ar
     const char *gb = static_cast<const char *>(a.d_o) + po * kBlockBytes + i * 128 + part * 32;
 #pragma unroll
     for (int c = 0; c < 2; ++c) {
-      const u32x4 ov = *reinterpret_cast<const u32x4 *>(ob + 16 * c);
+      // o is read here and nowhere else in the backward; dO is read again by the walk that follows: o goes past the caches
+      const u32x4 ov = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(ob + 16 * c));
       const u32x4 gv = *reinterpret_cast<const u32x4 *>(gb + 16 * c);
 #pragma unroll
       for (int t = 0; t < 4; ++t) acc = Tr::dot2(ov[t], gv[t], acc);
