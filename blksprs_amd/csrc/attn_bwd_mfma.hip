@@ -1609,10 +1609,13 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_q_kernel(bsa_attn_arg
   // ---- add the two key halves, scale, store ----
   reduce_partner(dqacc, reinterpret_cast<float *>(smem), wj == 1, wi, lane);
   if (wj == 1) return;
+  // The wave's 32 rounded rows pass through LDS behind the partial sums (rows of 128 bytes, chunks swizzled by the
+  // row) and leave as whole lines, eight lanes to a row, past the caches; rows and chunks are the wave's own: no
+  // barrier.
+  char *rows_lds = smem + NH * 2 * 2 * 16 * 64 * 4;
+  static_assert(NH * 2 * 2 * 16 * 64 * 4 + NH * kBlockBytes <= 2 * kBufBytes, "the rows fit behind the partial sums");
 #pragma unroll
-  for (int h = 0; h < NH; ++h) {
-    if (pq[h] < 0) continue;
-    char *op = static_cast<char *>(a.dq) + pq[h] * kBlockBytes + qi * 128 + kg * 8;
+  for (int h = 0; h < NH; ++h)
 #pragma unroll
     for (int db = 0; db < 2; ++db)
 #pragma unroll
@@ -1621,8 +1624,18 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_q_kernel(bsa_attn_arg
         u32x2 w;
         w[0] = Tr::pack2(acc[4 * q] * a.scale, acc[4 * q + 1] * a.scale);
         w[1] = Tr::pack2(acc[4 * q + 2] * a.scale, acc[4 * q + 3] * a.scale);
-        *reinterpret_cast<u32x2 *>(op + 64 * db + 16 * q) = w;
+        *reinterpret_cast<u32x2 *>(rows_lds + h * kBlockBytes + qi * 128 + (((4 * db + q) ^ (qi & 7)) << 4) + 8 * kg) = w;
       }
+#pragma unroll
+  for (int h = 0; h < NH; ++h) {
+    if (pq[h] < 0) continue;
+    char *out = static_cast<char *>(a.dq) + pq[h] * kBlockBytes;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = 32 * wi + 8 * i + (lane >> 3), c = lane & 7;
+      const u32x4 v = *reinterpret_cast<const u32x4 *>(rows_lds + h * kBlockBytes + r * 128 + ((c ^ (r & 7)) << 4));
+      __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(out + r * 128 + c * 16));
+    }
   }
 }
 
