@@ -1305,15 +1305,16 @@ __device__ __forceinline__ void attn_bwd_kv8_walk(const bsa_attn_args &a, char *
     if constexpr (DV) exchange_odd_for_even(dvacc, reduce_lds, wi, wj, lane);
     const int t_after = first_lane(mailbox[0]);
     // The sums leave as whole rows: every wave holds, for its key 32 wj + li, the column half db = wi of each slice
-    // (register 4 q + t: column 32 db + 8 q + 4 kg + t, eight bytes of a row per lane) and writes it, rounded, into this
-    // team's part of R, as rows of 128 bytes with the 16-byte chunks swizzled by the row, and all four waves of the
+    // (register 4 q + t: column 32 db + 8 q + 4 kg + t, eight bytes of a row per lane) and writes it, rounded, into LDS, as rows of 128 bytes with the 16-byte chunks swizzled by the row, and all four waves of the
     // team store it from there, 16 rows each, eight lanes to a row: whole lines per instruction, past the caches.
     // (Stores of eight bytes per lane straight from the registers are written to memory as partial lines, twice
     // the bytes, and are waited for with the copies of the next tile.)
     {
       constexpr int kOut = DK ? NH : NHV;
-      char *rows_lds = reinterpret_cast<char *>(reduce_lds);
-      __syncthreads();  // the partial sums have been read
+      // in the tile buffer that the block's last tile has left free (the other one may hold the first tile of the
+      // next block): the partial sums in R may still be read by the partner, and need no barrier of their own
+      char *rows_lds = smem + first_lane(buf ^ 1) * kBufBytes + (DK ? 0 : NH * kBlockBytes);
+      static_assert((NH + NHV) * kBlockBytes <= kBufBytes, "both teams' rows fit a tile buffer");
       {
         const int row = 32 * wj + li;
         const float factor = DK ? a.scale : 1.f;
