@@ -12,7 +12,7 @@ import torch
 
 _LIB_PATH = Path(__file__).resolve().parent / "lib" / "libblksprs_amd.so"
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 F32, F16, BF16 = 0, 1, 2
 DTYPE_CODES = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
 
@@ -32,7 +32,7 @@ class AttnArgs(ctypes.Structure):
         + [("sbs", ctypes.c_int32), ("dtype", ctypes.c_int32), ("mask_kind", ctypes.c_int32), ("scale", c_float)]
         + [("group_offsets", c_void_p), ("group_records", c_void_p), ("group_size", ctypes.c_int32)]
         + [("bwd_scratch", c_void_p), ("n_layout_blocks", c_int64), ("bwd_scratch_ready", c_int64),
-           ("bwd_scratch_bytes", c_int64)]
+           ("bwd_scratch_bytes", c_int64), ("bwd_ds", c_void_p), ("bwd_ds_bytes", c_int64)]
     )
 
 
@@ -43,6 +43,7 @@ ROWS_RECORD_INTS = 128  # BSA_ROWS_RECORD_INTS
 SIGNATURES = {
     "bsa_abi_version": (c_int, []),
     "bsa_last_error": (ctypes.c_char_p, []),
+    "bsa_build_info": (ctypes.c_char_p, []),
     "bsa_lut_workspace_bytes": (c_size_t, [c_int64]),
     "bsa_lut_packed": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                c_size_t, c_void_p]),
@@ -84,7 +85,7 @@ SIGNATURES = {
     "bsa_attn_fwd_records": (c_int, [ctypes.POINTER(AttnArgs), c_void_p, c_void_p, c_void_p]),
     "bsa_attn_mask_dead": (c_int, [c_void_p, c_int64, ctypes.c_int32, c_void_p, c_void_p]),
     "bsa_attn_bwd_scratch_bytes": (c_size_t, [c_int64, c_int64, c_int64, c_int64, c_int64]),
-    "bsa_attn_bwd_scratch_bytes_ds": (c_size_t, [c_int64, c_int64, c_int64, c_int64, c_int64]),
+    "bsa_attn_bwd_ds_bytes": (c_size_t, [c_int64, ctypes.c_int32]),
     "bsa_attn_fwd": (c_int, [ctypes.POINTER(AttnArgs), c_void_p]),
     "bsa_attn_bwd": (c_int, [ctypes.POINTER(AttnArgs), c_void_p]),
 }

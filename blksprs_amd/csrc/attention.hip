@@ -86,10 +86,9 @@ extern "C" size_t bsa_attn_bwd_scratch_bytes(int64_t B, int64_t nq, int64_t nk, 
   return bsa::attn_bwd_scratch_bytes(B, nq, nk, n_layout_blocks, n_mask_blocks);
 }
 
-extern "C" size_t bsa_attn_bwd_scratch_bytes_ds(int64_t B, int64_t nq, int64_t nk, int64_t n_layout_blocks,
-                                                int64_t n_mask_blocks) {
-  if (B < 0 || nq < 0 || nk < 0 || n_layout_blocks < 0 || n_mask_blocks < 0) return 0;
-  return bsa::attn_bwd_scratch_bytes_ds(B, nq, nk, n_layout_blocks, n_mask_blocks);
+extern "C" size_t bsa_attn_bwd_ds_bytes(int64_t n_layout_blocks, int32_t sbs) {
+  if (n_layout_blocks < 0 || sbs != 64) return 0;
+  return bsa::attn_bwd_ds_bytes(n_layout_blocks);
 }
 
 extern "C" int bsa_attn_bwd(const bsa_attn_args *args, bsa_stream_t stream) {
@@ -97,6 +96,13 @@ extern "C" int bsa_attn_bwd(const bsa_attn_args *args, bsa_stream_t stream) {
   BSA_REQUIRE(args->bwd_scratch == nullptr || args->n_layout_blocks >= 0, "bsa_attn_bwd: negative n_layout_blocks");
   BSA_REQUIRE(args->bwd_scratch_bytes >= 0, "bsa_attn_bwd: negative bwd_scratch_bytes");
   BSA_REQUIRE((reinterpret_cast<uintptr_t>(args->bwd_scratch) & 15) == 0, "bsa_attn_bwd: bwd_scratch must be 16-byte aligned");
+  BSA_REQUIRE(args->bwd_ds_bytes >= 0, "bsa_attn_bwd: negative bwd_ds_bytes");
+  BSA_REQUIRE((reinterpret_cast<uintptr_t>(args->bwd_ds) & 15) == 0, "bsa_attn_bwd: bwd_ds must be 16-byte aligned");
+  if (args->bwd_scratch != nullptr && args->bwd_scratch_bytes > 0) {
+    const size_t need = bsa::attn_bwd_scratch_bytes(args->B, args->nq, args->nk, args->n_layout_blocks, args->n_mask_blocks);
+    BSA_REQUIRE((size_t)args->bwd_scratch_bytes >= need, "bsa_attn_bwd: bwd_scratch holds %lld bytes, %zu are needed",
+                (long long)args->bwd_scratch_bytes, need);
+  }
   hipStream_t s = bsa::as_stream(stream);
   int rc = bsa::attn_bwd_mfma(*args, s);
   if (rc == 1) rc = bsa::attn_bwd_f32mma(*args, s);

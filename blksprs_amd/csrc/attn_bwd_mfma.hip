@@ -26,6 +26,7 @@
 //
 // The two waves that share a half of the stationary block hold partial sums over the two halves of the streamed
 // blocks; they are added through LDS once, at the end.  No atomics, fixed summation order.
+#include <atomic>
 #include <type_traits>
 
 #include "attn_mfma_common.h"
@@ -37,15 +38,6 @@ using namespace mfma;
 
 constexpr int kBwdThreads = 256;
 constexpr int kStatBytes = 2 * kSbs * 4;  // lse and delta of the 64 queries of a tile
-// dK and dV in one pass over the query blocks (one workgroup per CU) or in two passes (two workgroups per CU,
-// scores computed twice): measured equal within 3 % on the BigBird configuration; one pass reads less
-constexpr bool kSplitKeyPass = false;
-// dK and dV by two teams of four waves in one workgroup of eight (the default); the two switches above
-// choose among the four-wave kernels otherwise
-constexpr bool kEightWaves = true;
-// the eight-wave kernel by workgroups that stay for the whole launch and walk key block after key block
-constexpr bool kKvWalk = true;
-
 // One 64 x 64 16-bit block, global -> LDS, by the NW (4 or 8) waves of a workgroup: wave w copies rows
 // (64 / NW) w .. with asynchronous 1 KiB copies (eight rows each); lane l supplies the chunk that belongs at
 // position l of the KiB, which is where the chunk swizzle is applied.  An inactive block becomes zeros.
@@ -212,23 +204,18 @@ struct BwdLists {
   int32_t *q_head, *k_head;
   int32_t *kv_tickets;             // [16]: per XCD, the next position of its eighth of the key rows to hand out
   uint8_t *mask_dead;              // [n_mask_blocks]
-  // [n_layout_blocks] blocks of 64 x 64 16-bit values, or NULL (the scratch is too small for them): dS^T of every
+  // [n_layout_blocks] blocks of 64 x 64 16-bit values, or NULL (the caller brought no room for them): dS^T of every
   // pair (row = key, column = query), written by the dK / dV kernel for the dQ kernel
   char *ds;
 };
 
-// bytes of the scratch without the dS blocks, and the offset at which they start when the scratch holds them
+// bytes of the scratch (the dS blocks have a buffer of their own, bsa_attn_args.bwd_ds)
 __host__ __device__ inline size_t bwd_lists_bytes(int64_t B, int64_t nq, int64_t nk, int64_t n_layout_blocks,
                                                   int64_t n_mask_blocks) {
   const size_t bytes = 2 * sizeof(BwdRecord) * (size_t)n_layout_blocks + (4 + 64) * (size_t)(B * nq + B * nk) + 64 +
                        (size_t)n_mask_blocks;
   return (bytes + 15) & ~(size_t)15;
 }
-__host__ __device__ inline size_t bwd_ds_offset(int64_t B, int64_t nq, int64_t nk, int64_t n_layout_blocks,
-                                                int64_t n_mask_blocks) {
-  return (bwd_lists_bytes(B, nq, nk, n_layout_blocks, n_mask_blocks) + 4095) & ~(size_t)4095;
-}
-
 __host__ __device__ inline BwdLists bwd_lists(const bsa_attn_args &a) {
   BwdLists L;
   L.key_rec = static_cast<BwdRecord *>(a.bwd_scratch);
@@ -239,10 +226,8 @@ __host__ __device__ inline BwdLists bwd_lists(const bsa_attn_args &a) {
   L.k_head = L.q_head + 16 * a.B * a.nq;
   L.kv_tickets = L.k_head + 16 * a.B * a.nk;
   L.mask_dead = reinterpret_cast<uint8_t *>(L.kv_tickets + 16);
-  const size_t ds_at = bwd_ds_offset(a.B, a.nq, a.nk, a.n_layout_blocks, a.n_mask_blocks);
-  const bool has_ds = a.bwd_scratch_bytes > 0 &&
-                      (size_t)a.bwd_scratch_bytes >= ds_at + (size_t)a.n_layout_blocks * kBlockBytes;
-  L.ds = has_ds ? static_cast<char *>(a.bwd_scratch) + ds_at : nullptr;
+  const bool has_ds = a.bwd_ds != nullptr && a.bwd_ds_bytes >= a.n_layout_blocks * (int64_t)kBlockBytes;
+  L.ds = has_ds ? static_cast<char *>(a.bwd_ds) : nullptr;
   return L;
 }
 
@@ -431,132 +416,6 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_delta_kernel(bsa_attn_ar
   acc += __shfl_xor(acc, 1);
   acc += __shfl_xor(acc, 2);
   if (part == 0) a.delta[row * kSbs + i] = acc;
-}
-
-// The work of one wave on one tile (a query block in LDS at `base`, this wave's quadrant of the 64 x 64 scores):
-// S and dP, P and dS, then dV^T += dO^T P and / or dK^T += Q^T dS.  mbits: the mask bytes of this lane's 16
-// scores, one bit each (0 when the tile has no mask block).
-template <typename Tr, int NH, int NHV, bool DK, bool DV>
-__device__ __forceinline__ void kv_tile(const bsa_attn_args &a, const char *base, const int qb, const int64_t pm,
-                                        const int64_t pb, const uint32_t mbits, const bool causal, const int seq_len,
-                                        const int kb, const int kpos, const float qk_scale, const int wi, const int wj,
-                                        const int li, const int kg, const int lane, const u32x4 (&kfr)[NH][4],
-                                        const u32x4 (&vfr)[NHV][4], f32x16 (&dkacc)[DK ? NH * 2 : 1],
-                                        f32x16 (&dvacc)[DV ? NHV * 2 : 1]) {
-  constexpr int kQRows = 0, kDoRows = NH * kBlockBytes, kStats = (NH + NHV) * kBlockBytes;
-  // A quadrant whose every score is masked has P = dS = 0: nothing to add, nothing to compute.
-  bool live = true;
-  if (pm >= 0) live = !__all(mbits == 0xffffu);
-  if (causal) {
-    const int k_first = (int)kb * kSbs + 32 * wj, q_first = qb * kSbs + 32 * wi;
-    if (k_first > q_first + 31 || q_first >= seq_len || k_first >= seq_len) live = false;
-  }
-  if (live) {
-    // ---- S and dP of this wave's quadrant ----
-    f32x16 sacc, dpacc;
-  #pragma unroll
-    for (int r = 0; r < 16; ++r) sacc[r] = dpacc[r] = 0.f;
-    staged_products<NH + (DK ? NHV : 0)>(
-        [&](int k, u32x4(&f)[4]) {
-          const char *src = base + (k < NH ? kQRows + k * kBlockBytes : kDoRows + (k - NH) * kBlockBytes);
-  #pragma unroll
-          for (int s = 0; s < 4; ++s) f[s] = frag_rows(src, 32 * wi + li, 2 * s + kg);
-        },
-        [&](int k, u32x4(&f)[4]) {
-  #pragma unroll
-          for (int s = 0; s < 4; ++s) {
-            if (k < NH) sacc = Tr::mfma(f[s], kfr[k < NH ? k : 0][s], sacc);
-            else dpacc = Tr::mfma(f[s], vfr[k < NH ? 0 : k - NH][s], dpacc);
-          }
-        });
-
-    // ---- P and dS; element r: query 32 wi + 8 (r / 4) + 4 kg + r % 4 ----
-    const float *stats = reinterpret_cast<const float *>(base + kStats);
-    // the bias elements are read where they are used: a bias is rare, its registers are not
-    uint32_t bias_c[16];
-    if (pb >= 0) {
-      const uint16_t *bp = static_cast<const uint16_t *>(a.bias) + pb * (kSbs * kSbs) +
-                           (32 * wi + 4 * kg) * kSbs + 32 * wj + li;
-  #pragma unroll
-      for (int r = 0; r < 16; ++r) bias_c[r] = bp[(8 * (r >> 2) + (r & 3)) * kSbs];
-    }
-    float p[16], ds[16];
-    // Most tiles have no bias, no mask block and lie where the causal predicate holds for every score: they
-    // take the plain path.  The conditions are the same for the whole wave.
-    auto probabilities = [&](auto plain_tag) {
-      constexpr bool kPlain = decltype(plain_tag)::value;
-  #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int i0 = 32 * wi + 8 * q + 4 * kg;
-        const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(stats + i0);
-        const f32x4 del4 = *reinterpret_cast<const f32x4 *>(stats + kSbs + i0);
-  #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          const int r = 4 * q + t;
-          float s = sacc[r] * qk_scale;
-          if constexpr (!kPlain) {
-            if (pb >= 0) s = s + Tr::widen((uint16_t)bias_c[r]) * kLog2e;
-            if (causal) {
-              const int qpos = qb * kSbs + i0 + t;
-              s = (kpos > qpos || qpos >= seq_len || kpos >= seq_len) ? -INFINITY : s;
-            }
-            if (pm >= 0) s = ((mbits >> r) & 1u) ? -INFINITY : s;
-          }
-          p[r] = __builtin_amdgcn_exp2f(s - lse4[t]);
-          ds[r] = p[r] * (dpacc[r] - del4[t]);
-        }
-      }
-    };
-    bool plain = pb < 0 && pm < 0;
-    if (causal) {
-      // every key of the quadrant at or before every query of it, and all of them inside the sequence
-      const int k_last = (int)kb * kSbs + 32 * wj + 31, q_first = qb * kSbs + 32 * wi;
-      plain = plain && k_last <= q_first && q_first + 31 < seq_len;
-    }
-    if (plain) probabilities(std::true_type{});
-    else probabilities(std::false_type{});
-    if (DK && a.dbias != nullptr && pb >= 0) {
-      // every (query block, key block) pair is visited once, so this is a plain store
-      float *dbp = a.dbias + pb * (kSbs * kSbs) + (32 * wi + 4 * kg) * kSbs + 32 * wj + li;
-  #pragma unroll
-      for (int r = 0; r < 16; ++r) dbp[(8 * (r >> 2) + (r & 3)) * kSbs] = ds[r];
-    }
-    u32x4 pf[2], dsf[2];
-  #pragma unroll
-    for (int u = 0; u < 2; ++u)
-  #pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        pf[u][t] = Tr::pack2(p[8 * u + 2 * t], p[8 * u + 2 * t + 1]);
-        dsf[u][t] = Tr::pack2(ds[8 * u + 2 * t], ds[8 * u + 2 * t + 1]);
-      }
-
-    // ---- dV^T += dO^T P, dK^T += Q^T dS over this wave's 32 queries ----
-    const int col_t = 16 * ((lane >> 4) & 1);
-    if constexpr (DV) {
-      staged_products<NHV>(
-          [&](int h, u32x4(&f)[4]) {
-  #pragma unroll
-            for (int i = 0; i < 4; ++i)
-              f[i] = frag_cols_t(base + kDoRows + h * kBlockBytes, 32 * wi + 16 * (i & 1) + 4 * kg, 32 * (i >> 1) + col_t, lane);
-          },
-          [&](int h, u32x4(&f)[4]) {
-  #pragma unroll
-            for (int i = 0; i < 4; ++i) dvacc[2 * h + (i >> 1)] = Tr::mfma(f[i], pf[i & 1], dvacc[2 * h + (i >> 1)]);
-          });
-    }
-    if constexpr (DK) {
-      staged_products<NH>(
-          [&](int h, u32x4(&f)[4]) {
-  #pragma unroll
-            for (int i = 0; i < 4; ++i)
-              f[i] = frag_cols_t(base + kQRows + h * kBlockBytes, 32 * wi + 16 * (i & 1) + 4 * kg, 32 * (i >> 1) + col_t, lane);
-          },
-          [&](int h, u32x4(&f)[4]) {
-  #pragma unroll
-            for (int i = 0; i < 4; ++i) dkacc[2 * h + (i >> 1)] = Tr::mfma(f[i], dsf[i & 1], dkacc[2 * h + (i >> 1)]);
-          });
-    }
-  }  // live
 }
 
 // A tile with the work split between the two teams of the eight-wave kernel: the dV team (DV) computes S and P,
@@ -753,213 +612,6 @@ __device__ __forceinline__ void kv_second_half(const KvCarry &c, const bool live
           for (int i = 0; i < 4; ++i) dkacc[2 * h + (i >> 1)] = Tr::mfma(f[i], dsf[i & 1], dkacc[2 * h + (i >> 1)]);
         });
   }
-}
-
-// ---------------------------------------------------------------------------------------------------------
-// dK and dBias (DK) and / or dV (DV) of one key block.  The two are launched as separate passes: each then fits
-// two workgroups per CU (the combined kernel needs more than 256 registers per lane), which more than pays
-// for computing the scores twice.
-//
-// The body serves two kernels.  With NW = 4 the four waves of a workgroup each own a quadrant and compute
-// whatever DK / DV ask for.  With NW = 8 the workgroup has two teams of four waves, one running the body for dV
-// and one for dK (and dBias): `wave` (0 .. 7) says which rows of a tile the wave copies, `quad` which quadrant it
-// computes; both teams walk the same list, copy every tile together and meet at the same barriers, so neither
-// may leave early on its own (JOINT: leave only if there is nothing to do for either).
-template <typename Tr, int NH, int NHV, bool DK, bool DV, int NW>
-__device__ __forceinline__ void attn_bwd_kv_body(const bsa_attn_args &a, char *smem, float *reduce_lds, int wave,
-                                                 int quad) {
-  constexpr bool JOINT = NW == 8;
-  constexpr int kQRows = 0, kDoRows = NH * kBlockBytes, kStats = (NH + NHV) * kBlockBytes,
-                kMask = kStats + kStatBytes;  // the tile's mask block, row-major bytes
-  constexpr int kBufBytes = kMask + kSbs * kSbs;
-
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int li = lane & 31, kg = lane >> 5;
-  const int wi = quad & 1, wj = quad >> 1;  // query half and key half of this wave's quadrant
-  const int64_t kpos_in_order = xcd_row();
-  if (kpos_in_order >= a.B * a.nk) return;
-  const BwdLists lists = bwd_lists(a);
-  // the workgroup's header, int i in lane i (lanes 0 .. 7 double as the record of the first tile)
-  int head = -1;
-  if (lane < 16) head = lists.k_head[kpos_in_order * 16 + lane];
-  const int64_t krow = __builtin_amdgcn_readlane(head, 8);
-  const int64_t b = krow / a.nk, kb = krow % a.nk;
-
-  int64_t pk[NH], pv[NHV];
-  bool any = (DK || JOINT) && a.dbias != nullptr;
-#pragma unroll
-  for (int h = 0; h < NH; ++h) {
-    pk[h] = __builtin_amdgcn_readlane(head, 11 + h);
-    any = any || ((DK || JOINT) && pk[h] >= 0);
-  }
-#pragma unroll
-  for (int h = 0; h < NHV; ++h) {
-    pv[h] = __builtin_amdgcn_readlane(head, 13 + h);
-    any = any || ((DV || JOINT) && pv[h] >= 0);
-  }
-  if (!any) return;
-
-  // this wave's keys: B operands K[j][.], V[j][.] with j = 32 wj + li
-  u32x4 kfr[NH][4], vfr[NHV][4];
-#pragma unroll
-  for (int h = 0; h < NH; ++h) load_resident(kfr[h], a.k, pk[h], a.n_k_blocks, 32 * wj + li, kg);
-  if constexpr (DK) {
-#pragma unroll
-    for (int h = 0; h < NHV; ++h) load_resident(vfr[h], a.v, pv[h], a.n_v_blocks, 32 * wj + li, kg);
-  }
-
-  // accumulators [slice][column half db]: D[m = d][n = j]
-  f32x16 dkacc[DK ? NH * 2 : 1], dvacc[DV ? NHV * 2 : 1];
-  if constexpr (DK) {
-#pragma unroll
-    for (int n = 0; n < NH * 2; ++n)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) dkacc[n][r] = 0.f;
-  }
-  if constexpr (DV) {
-#pragma unroll
-    for (int n = 0; n < NHV * 2; ++n)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) dvacc[n][r] = 0.f;
-  }
-
-  const float qk_scale = a.scale * kLog2e;
-  const bool causal = a.causal_lengths != nullptr;
-  int seq_len = 0;
-  if (causal) {
-    const int64_t len = a.causal_lengths[b];
-    seq_len = len < 0 ? 0 : (len > 0x7fffffffLL ? 0x7fffffff : (int)len);
-  }
-  const int kpos = (int)kb * kSbs + 32 * wj + li;
-
-  const int q_begin = __builtin_amdgcn_readlane(head, 9), q_end = __builtin_amdgcn_readlane(head, 10);
-  if (q_begin < q_end) {
-    // the record of a list entry, field i in lane i: one 32-byte load, two tiles before the tile is used
-    const int32_t *recs = reinterpret_cast<const int32_t *>(lists.query_rec);
-    auto load_record = [&](int pos) -> int {
-      int v = -1;
-      if (lane < 8) v = recs[(int64_t)pos * 8 + lane];
-      return v;
-    };
-    auto clamp_e = [&](int e) { return e < q_end ? e : q_end - 1; };
-
-    // registers of the tile in flight (the blocks themselves go straight to LDS)
-    float stat = 0.f;           // thread t < 64: lse of query t; 64 <= t < 128: delta of query t - 64
-    int qb_nxt, pm_nxt, pb_nxt;
-
-    auto fetch = [&](int rec, int buf) {
-      const int qb = __builtin_amdgcn_readlane(rec, 0);
-      qb_nxt = qb;
-      char *base = smem + buf * kBufBytes;
-#pragma unroll
-      for (int h = 0; h < NH; ++h) {
-        const int pq = __builtin_amdgcn_readlane(rec, 1 + h);
-        copy_block<NW>(static_cast<const char *>(a.q) + (int64_t)(pq >= 0 ? pq : 0) * kBlockBytes, pq >= 0,
-                       base + kQRows + h * kBlockBytes, wave, lane, tid);
-      }
-#pragma unroll
-      for (int h = 0; h < NHV; ++h) {
-        const int po = __builtin_amdgcn_readlane(rec, 3 + h);
-        copy_block<NW>(static_cast<const char *>(a.d_o) + (int64_t)(po >= 0 ? po : 0) * kBlockBytes, po >= 0,
-                       base + kDoRows + h * kBlockBytes, wave, lane, tid);
-      }
-      const int64_t qrow = b * a.nq + qb;
-      if (tid < 64) stat = a.lse[qrow * kSbs + tid];
-      else if (tid < 128) stat = a.delta[qrow * kSbs + tid - 64];
-      pm_nxt = __builtin_amdgcn_readlane(rec, 5);
-      pb_nxt = __builtin_amdgcn_readlane(rec, 6);
-      // the mask block goes to LDS as it is: wave w copies its rows 16 w .. + 15 (1 KiB)
-      if (pm_nxt >= 0 && wave < 4)
-        copy_1k_to_lds(static_cast<const char *>(a.mask) + (int64_t)pm_nxt * (kSbs * kSbs) + wave * 1024, lane * 16,
-                       base + kMask + wave * 1024);
-    };
-    // the statistics of the tile go to LDS through a register; then every copy of this wave has to have landed
-    auto stage = [&](int buf) {
-      char *base = smem + buf * kBufBytes;
-      // a query without any visible key has lse = -inf and P = 0 everywhere: +inf gives exp2(s - lse) = 0 for it
-      // without a test per score
-      if (tid < 128) reinterpret_cast<float *>(base + kStats)[tid] = (tid < 64 && stat == -INFINITY) ? INFINITY : stat;
-      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-    };
-
-    // `rec` is the record of the tile after the one in flight
-    int rec;
-    {
-      rec = load_record(clamp_e(q_begin + 1));
-      fetch(head, 0);
-      stage(0);
-      __syncthreads();
-    }
-
-    for (int e = q_begin; e < q_end; ++e) {
-      const int buf = (e - q_begin) & 1;
-      const char *base = smem + buf * kBufBytes;
-      // facts and per-element inputs of tile e, before the fetch of tile e+1 replaces them
-      const int qb = qb_nxt;
-      const int64_t pm = pm_nxt, pb = pb_nxt;
-      // mask bytes (0 or 1) of this lane's 16 elements -> one bit each; element r: query
-      // 32 wi + 8 (r / 4) + 4 kg + r % 4, key 32 wj + li
-      uint32_t mbits = 0;
-      if (pm >= 0) {
-        const uint8_t *mp = reinterpret_cast<const uint8_t *>(base + kMask) + (32 * wi + 4 * kg) * kSbs + 32 * wj + li;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) mbits |= (uint32_t)mp[(8 * (r >> 2) + (r & 3)) * kSbs] << r;
-      }
-      const bool more = e + 1 < q_end;
-      if (more) fetch(rec, buf ^ 1);
-      rec = load_record(clamp_e(e + 2));
-
-      kv_tile<Tr, NH, NHV, DK, DV>(a, base, qb, pm, pb, mbits, causal, seq_len, (int)kb, kpos, qk_scale, wi, wj, li, kg,
-                                   lane, kfr, vfr, dkacc, dvacc);
-
-      // ---- tile e+1 into the other buffer; the barrier also ends the reads of tile e ----
-      if (more) stage(buf ^ 1);
-      __syncthreads();
-    }
-  }
-
-  // ---- add the two query halves, scale, store ----
-  if constexpr (DK) reduce_partner(dkacc, reduce_lds, wi == 1, wj, lane);
-  if constexpr (DV) reduce_partner(dvacc, reduce_lds, wi == 1, wj, lane);
-  if (wi == 1) return;
-  // lane: key 32 wj + li; register 4 q + t of half db: column 32 db + 8 q + 4 kg + t
-#pragma unroll
-  for (int h = 0; h < (DK ? NH : 0); ++h) {
-    if (pk[h] < 0) continue;
-    char *op = static_cast<char *>(a.dk) + pk[h] * kBlockBytes + (32 * wj + li) * 128 + kg * 8;
-#pragma unroll
-    for (int db = 0; db < 2; ++db)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const f32x16 &acc = dkacc[2 * h + db];
-        u32x2 w;
-        w[0] = Tr::pack2(acc[4 * q] * a.scale, acc[4 * q + 1] * a.scale);
-        w[1] = Tr::pack2(acc[4 * q + 2] * a.scale, acc[4 * q + 3] * a.scale);
-        *reinterpret_cast<u32x2 *>(op + 64 * db + 16 * q) = w;
-      }
-  }
-#pragma unroll
-  for (int h = 0; h < (DV ? NHV : 0); ++h) {
-    if (pv[h] < 0) continue;
-    char *op = static_cast<char *>(a.dv) + pv[h] * kBlockBytes + (32 * wj + li) * 128 + kg * 8;
-#pragma unroll
-    for (int db = 0; db < 2; ++db)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const f32x16 &acc = dvacc[2 * h + db];
-        u32x2 w;
-        w[0] = Tr::pack2(acc[4 * q], acc[4 * q + 1]);
-        w[1] = Tr::pack2(acc[4 * q + 2], acc[4 * q + 3]);
-        *reinterpret_cast<u32x2 *>(op + 64 * db + 16 * q) = w;
-      }
-  }
-}
-
-template <typename Tr, int NH, int NHV, bool DK, bool DV>
-__global__ __launch_bounds__(kBwdThreads, (DK &&DV) ? 1 : 2) void attn_bwd_kv_kernel(bsa_attn_args a) {
-  extern __shared__ __attribute__((aligned(1024))) char smem[];
-  const int wave = first_lane((int)threadIdx.x >> 6);
-  attn_bwd_kv_body<Tr, NH, NHV, DK, DV, 4>(a, smem, reinterpret_cast<float *>(smem), wave, wave);
 }
 
 // dK / dV with eight waves (two teams, as below) by workgroups that stay for the whole launch and walk one key
@@ -1355,16 +1007,6 @@ __device__ __forceinline__ void attn_bwd_kv8_walk(const bsa_attn_args &a, char *
 // Eight waves: waves 0 .. 3 accumulate dV, waves 4 .. 7 dK and dBias, two waves per SIMD.  Each team fits 256
 // registers per lane, which the two sets of accumulators in one wave do not; the tile is fetched once for both.
 constexpr int kKv8Threads = 512;
-template <typename Tr, int NH, int NHV>
-__global__ __launch_bounds__(kKv8Threads, 1) void attn_bwd_kv8_kernel(bsa_attn_args a) {
-  extern __shared__ __attribute__((aligned(1024))) char smem[];
-  const int wave = first_lane((int)threadIdx.x >> 6);
-  // the partial sums of a team take 2 * (slices * 2) * 16 * 64 floats
-  float *reduce_lds = reinterpret_cast<float *>(smem) + (wave >> 2) * (2 * (NH > NHV ? NH : NHV) * 2 * 16 * 64);
-  if (wave < 4) attn_bwd_kv_body<Tr, NH, NHV, false, true, 8>(a, smem, reduce_lds, wave, wave & 3);
-  else attn_bwd_kv_body<Tr, NH, NHV, true, false, 8>(a, smem, reduce_lds, wave, wave & 3);
-}
-
 template <typename Tr, int NH, int NHV>
 __global__ __launch_bounds__(kKv8Threads, 1) void attn_bwd_kv8_walk_kernel(bsa_attn_args a) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -1819,6 +1461,40 @@ __global__ void fill_zero_f32_kernel(float *p, int64_t n) {
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) p[i] = 0.f;
 }
 
+// The kernels that ask for more than 64 KiB of LDS say so once per process and device: the attribute belongs to
+// the loaded code object of a device, so the calls are made the first time a launch runs on it.
+constexpr int kMaxDevices = 64;
+template <typename Tr, int NH, int NHV>
+int set_lds_attributes(int lds_q, int lds_walk, int lds_dq) {
+  static std::atomic<bool> done[kMaxDevices];
+  int dev = 0;
+  BSA_HIP(hipGetDevice(&dev));
+  const bool tracked = dev >= 0 && dev < kMaxDevices;
+  if (tracked && done[dev].load(std::memory_order_acquire)) return BSA_OK;
+  BSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_bwd_q_kernel<Tr, NH, NHV>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, lds_q));
+  BSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_bwd_kv8_walk_kernel<Tr, NH, NHV>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, lds_walk));
+  BSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_bwd_dq_kernel<Tr, NH>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, lds_dq));
+  if (tracked) done[dev].store(true, std::memory_order_release);
+  return BSA_OK;
+}
+
+__global__ void fill_zero_u32x4_kernel(u32x4 *p, int64_t n) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) p[i] = u32x4{0u, 0u, 0u, 0u};
+}
+
+int zero_blocks(void *p, int64_t n_blocks, hipStream_t s) {
+  if (n_blocks <= 0 || p == nullptr) return BSA_OK;
+  const int64_t n = n_blocks * (kBlockBytes / 16);
+  int64_t blocks = cdiv(n, 1024);
+  if (blocks > 65536) blocks = 65536;
+  fill_zero_u32x4_kernel<<<(unsigned)blocks, 256, 0, s>>>(static_cast<u32x4 *>(p), n);
+  return check_launch("fill_zero_u32x4_kernel");
+}
+
 template <typename Tr, int NH, int NHV>
 int launch_bwd(const bsa_attn_args &a, hipStream_t s) {
   const int64_t qrows = a.B * a.nq, krows = a.B * a.nk;
@@ -1830,7 +1506,22 @@ int launch_bwd(const bsa_attn_args &a, hipStream_t s) {
     fill_zero_f32_kernel<<<(unsigned)blocks, 256, 0, s>>>(a.dbias, n);
     if (int rc = check_launch("fill_zero_f32_kernel")) return rc;
   }
-  if (qrows + krows > 0 && !a.bwd_scratch_ready) {
+  if (qrows == 0 || krows == 0) {
+    // no query or no key: no pair, every gradient is zero (the walk's tickets are set by the kernels of the query
+    // side, which have nothing to launch here)
+    if (int rc = zero_blocks(a.dq, a.n_q_blocks, s)) return rc;
+    if (int rc = zero_blocks(a.dk, a.n_k_blocks, s)) return rc;
+    return zero_blocks(a.dv, a.n_v_blocks, s);
+  }
+  constexpr int lds_q = 2 * (NH + NHV) * kBlockBytes;
+  // tile buffers, the region of the next block's K / V and of the partial sums of both teams, the mailbox, P of a tile
+  constexpr int kSlices = NH > NHV ? NH : NHV;
+  constexpr int lds_walk = 2 * ((NH + NHV) * kBlockBytes + kStatBytes + kSbs * kSbs) + 2 * (2 * kSlices * 2 * 16 * 64) * 4 +
+                           64 + 4 * 4 * 64 * 16;
+  static_assert((NH + NHV) * kBlockBytes <= 2 * (2 * kSlices * 2 * 16 * 64) * 4, "K and V fit the region");
+  constexpr int lds_dq = (NH + 2) * kBlockBytes;
+  if (int rc = set_lds_attributes<Tr, NH, NHV>(lds_q, lds_walk, lds_dq)) return rc;
+  if (!a.bwd_scratch_ready) {
     const BwdLists L = bwd_lists(a);
     if (a.mask != nullptr && a.n_mask_blocks > 0) {
       attn_bwd_mask_dead_kernel<<<(unsigned)cdiv(a.n_mask_blocks, 4), kBwdThreads, 0, s>>>(
@@ -1842,59 +1533,22 @@ int launch_bwd(const bsa_attn_args &a, hipStream_t s) {
     attn_bwd_order_kernel<<<16, kOrderThreads, 0, s>>>(a);
     if (int rc = check_launch("attn_bwd_order_kernel")) return rc;
   }
-  // With room for the dS blocks in the scratch: delta and the tickets first, then the dK / dV walk, which leaves
-  // dS^T of every pair behind, then dQ = dS K as a product of its own.  Without: the dQ kernel forms the scores
-  // and dS of its pairs a second time; it runs first and leaves delta and the tickets for the walk.
-  const bool from_ds = kEightWaves && kKvWalk && qrows > 0 && krows > 0 && bwd_lists(a).ds != nullptr;
+  // With room for the dS blocks: delta and the tickets first, then the dK / dV walk, which leaves dS^T of every pair
+  // behind, then dQ = dS K as a product of its own.  Without: the dQ kernel forms the scores and dS of its pairs a
+  // second time; it runs first and leaves delta and the tickets for the walk.
+  const bool from_ds = bwd_lists(a).ds != nullptr;
   if (from_ds) {
     attn_bwd_delta_kernel<Tr><<<(unsigned)qrows, kBwdThreads, 0, s>>>(a);
     if (int rc = check_launch("attn_bwd_delta_kernel")) return rc;
-  } else if (qrows > 0) {
-    constexpr int lds = 2 * (NH + NHV) * kBlockBytes;
-    BSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_bwd_q_kernel<Tr, NH, NHV>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-    attn_bwd_q_kernel<Tr, NH, NHV><<<(unsigned)(cdiv(qrows, 8) * 8), kBwdThreads, lds, s>>>(a);
+  } else {
+    attn_bwd_q_kernel<Tr, NH, NHV><<<(unsigned)(cdiv(qrows, 8) * 8), kBwdThreads, lds_q, s>>>(a);
     if (int rc = check_launch("attn_bwd_q_kernel")) return rc;
   }
-  if (krows > 0) {
-    constexpr int lds = 2 * ((NH + NHV) * kBlockBytes + kStatBytes + kSbs * kSbs);
-    if (kEightWaves && kKvWalk && qrows > 0) {
-      // tile buffers, the region of the next block's K / V and of the partial sums of both teams, the mailbox, P
-      constexpr int kSlices = NH > NHV ? NH : NHV;
-      constexpr int lds_walk = lds + 2 * (2 * kSlices * 2 * 16 * 64) * 4 + 64 + 4 * 4 * 64 * 16;  // + P of a tile
-      static_assert((NH + NHV) * kBlockBytes <= 2 * (2 * kSlices * 2 * 16 * 64) * 4, "K and V fit the region");
-      BSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_bwd_kv8_walk_kernel<Tr, NH, NHV>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds_walk));
-      attn_bwd_kv8_walk_kernel<Tr, NH, NHV><<<(unsigned)(kv_slots(krows) * 8), kKv8Threads, lds_walk, s>>>(a);
-      if (int rc = check_launch("attn_bwd_kv8_walk_kernel")) return rc;
-      if (from_ds) {
-        constexpr int lds_dq = (NH + 2) * kBlockBytes;
-        BSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_bwd_dq_kernel<Tr, NH>),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, lds_dq));
-        attn_bwd_dq_kernel<Tr, NH><<<(unsigned)(cdiv(qrows, 8) * 8), kBwdThreads, lds_dq, s>>>(a);
-        if (int rc = check_launch("attn_bwd_dq_kernel")) return rc;
-      }
-    } else if (kEightWaves) {
-      constexpr int lds8 = lds > 65536 ? lds : 65536;  // the tile buffers; at the end, the partial sums of both teams
-      BSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_bwd_kv8_kernel<Tr, NH, NHV>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds8));
-      attn_bwd_kv8_kernel<Tr, NH, NHV><<<(unsigned)(cdiv(krows, 8) * 8), kKv8Threads, lds8, s>>>(a);
-      if (int rc = check_launch("attn_bwd_kv8_kernel")) return rc;
-    } else if (kSplitKeyPass) {
-      BSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_bwd_kv_kernel<Tr, NH, NHV, true, false>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-      BSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_bwd_kv_kernel<Tr, NH, NHV, false, true>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-      attn_bwd_kv_kernel<Tr, NH, NHV, false, true><<<(unsigned)(cdiv(krows, 8) * 8), kBwdThreads, lds, s>>>(a);
-      if (int rc = check_launch("attn_bwd_kv_kernel (dV)")) return rc;
-      attn_bwd_kv_kernel<Tr, NH, NHV, true, false><<<(unsigned)(cdiv(krows, 8) * 8), kBwdThreads, lds, s>>>(a);
-      if (int rc = check_launch("attn_bwd_kv_kernel (dK)")) return rc;
-    } else {
-      BSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_bwd_kv_kernel<Tr, NH, NHV, true, true>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-      attn_bwd_kv_kernel<Tr, NH, NHV, true, true><<<(unsigned)(cdiv(krows, 8) * 8), kBwdThreads, lds, s>>>(a);
-      if (int rc = check_launch("attn_bwd_kv_kernel")) return rc;
-    }
+  attn_bwd_kv8_walk_kernel<Tr, NH, NHV><<<(unsigned)(kv_slots(krows) * 8), kKv8Threads, lds_walk, s>>>(a);
+  if (int rc = check_launch("attn_bwd_kv8_walk_kernel")) return rc;
+  if (from_ds) {
+    attn_bwd_dq_kernel<Tr, NH><<<(unsigned)(cdiv(qrows, 8) * 8), kBwdThreads, lds_dq, s>>>(a);
+    if (int rc = check_launch("attn_bwd_dq_kernel")) return rc;
   }
   return BSA_OK;
 }
@@ -1920,9 +1574,7 @@ size_t attn_bwd_scratch_bytes(int64_t B, int64_t nq, int64_t nk, int64_t n_layou
   return bwd_lists_bytes(B, nq, nk, n_layout_blocks, n_mask_blocks);
 }
 
-size_t attn_bwd_scratch_bytes_ds(int64_t B, int64_t nq, int64_t nk, int64_t n_layout_blocks, int64_t n_mask_blocks) {
-  return bwd_ds_offset(B, nq, nk, n_layout_blocks, n_mask_blocks) + (size_t)n_layout_blocks * kBlockBytes;
-}
+size_t attn_bwd_ds_bytes(int64_t n_layout_blocks) { return (size_t)n_layout_blocks * kBlockBytes; }
 
 int attn_bwd_mfma(const bsa_attn_args &a, hipStream_t s) {
   if (a.sbs != kSbs || (a.dtype != BSA_BF16 && a.dtype != BSA_F16)) return 1;

@@ -54,6 +54,6 @@ int attn_bwd_f32mma(const bsa_attn_args &a, hipStream_t s);
 int attn_bwd_mfma(const bsa_attn_args &a, hipStream_t s);
 int attn_mask_dead(const void *mask, int64_t n_mask_blocks, uint8_t *dead, hipStream_t s);
 size_t attn_bwd_scratch_bytes(int64_t B, int64_t nq, int64_t nk, int64_t n_layout_blocks, int64_t n_mask_blocks);
-size_t attn_bwd_scratch_bytes_ds(int64_t B, int64_t nq, int64_t nk, int64_t n_layout_blocks, int64_t n_mask_blocks);
+size_t attn_bwd_ds_bytes(int64_t n_layout_blocks);
 
 }  // namespace bsa

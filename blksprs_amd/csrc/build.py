@@ -22,9 +22,22 @@ FLAGS = ["-O3", "-std=c++17", "-fno-strict-aliasing", "--offload-arch=gfx950", "
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall", "-Wno-unused-function"]
 
 
+def _build_info() -> str:
+    """What ``bsa_build_info()`` returns: the compiler's own version line and the flags."""
+    try:
+        out = subprocess.run([HIPCC, "--version"], capture_output=True, text=True).stdout.splitlines()
+        version = next((line.strip() for line in out if "HIP version" in line), out[0].strip() if out else "unknown")
+        clang = next((line.strip() for line in out if "clang version" in line), "")
+    except OSError:
+        version, clang = "unknown", ""
+    text = f"hipcc: {version}; {clang}; flags: {' '.join(FLAGS)}"
+    return "".join(c for c in text if c.isprintable() and c not in '"\\')
+
+
 def _compile(src: str) -> Path:
     obj = OUT_DIR / "obj" / (Path(src).stem + ".o")
-    cmd = [HIPCC, *FLAGS, "-c", str(HERE / src), "-o", str(obj)]
+    extra = [f'-DBSA_BUILD_INFO="{_build_info()}"'] if src == "common.hip" else []
+    cmd = [HIPCC, *FLAGS, *extra, "-c", str(HERE / src), "-o", str(obj)]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     noise = "is not a recognized feature for this target"
     err = "\n".join(line for line in proc.stderr.splitlines() if noise not in line)

@@ -21,3 +21,8 @@ int fail(int code, const char *fmt, ...) {
 extern "C" int bsa_abi_version(void) { return BSA_ABI_VERSION; }
 
 extern "C" const char *bsa_last_error(void) { return bsa::error_buffer(); }
+
+#ifndef BSA_BUILD_INFO
+#define BSA_BUILD_INFO "hipcc: unknown (built without blksprs_amd/csrc/build.py)"
+#endif
+extern "C" const char *bsa_build_info(void) { return BSA_BUILD_INFO; }

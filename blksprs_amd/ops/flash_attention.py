@@ -442,6 +442,13 @@ def _forward_launch(q, k, v, bias, mask, causal_lengths, meta: "_Meta"):
     return out, lse
 
 
+def _walks_records(meta: "_Meta", dtype: torch.dtype) -> bool:
+    """Whether ``bsa_attn_bwd`` runs the kernels that build and walk records in ``bwd_scratch`` (and can keep dS)
+    for these operands: 16-bit, 64 x 64 blocks, one or two head slices each for q / k and for v / o."""
+    _, _, _, nh, nhv = meta.dims
+    return meta.sbs == 64 and dtype in (torch.bfloat16, torch.float16) and 1 <= nh <= 2 and 1 <= nhv <= 2
+
+
 class _FlashAttention(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, v, bias, mask, causal_lengths, meta: "_Meta"):
@@ -465,29 +472,38 @@ class _FlashAttention(torch.autograd.Function):
         args = _fill_args(meta, q, k, v, bias, mask, causal_lengths)
         args.o, args.d_o, args.lse, args.delta = _capi.ptr(out), _capi.ptr(grad_output), _capi.ptr(lse), _capi.ptr(delta)
         args.dq, args.dk, args.dv, args.dbias = _capi.ptr(dq), _capi.ptr(dk), _capi.ptr(dv), _capi.ptr(dbias)
-        # room for the records of the pairs that some score survives (built and used inside bsa_attn_bwd)
         n_layout_blocks = meta.tables.key_indices_i32.numel()
         n_mask_blocks = mask.size(0) if mask is not None else 0
-        size = max(_capi.load().bsa_attn_bwd_scratch_bytes(B, nq, nk, n_layout_blocks, n_mask_blocks), 16)
-        # With room for dS of every pair (one block per active block of the attention layout) the dK / dV kernel
-        # leaves it behind and dQ = dS K is a product of its own; beyond the limit (set_kept_ds_limit) dS is formed a
-        # second time, as the reference does (blksprs/ops/flash_attention.py:1228-1480).
-        if (meta.sbs == 64 and q.dtype in (torch.bfloat16, torch.float16) and nh <= 2 and nhv <= 2
-                and n_layout_blocks * 64 * 64 * 2 <= kept_ds_limit()):
-            size = _capi.load().bsa_attn_bwd_scratch_bytes_ds(B, nq, nk, n_layout_blocks, n_mask_blocks)
         stream = _capi.stream(q.device)
         facts = meta.facts
-        # the records depend on the layouts and on the values of the mask and of the causal lengths only: a
-        # later call on the same stream with the same ones reads what this call wrote
-        scratch = facts.bwd_scratch if facts is not None and facts.bwd_stream == stream else None
-        args.bwd_scratch_ready = 1 if scratch is not None and scratch.numel() == size else 0
-        if not args.bwd_scratch_ready:
-            scratch = torch.empty(size, dtype=torch.uint8, device=q.device)
-        args.bwd_scratch, args.n_layout_blocks, args.bwd_scratch_bytes = scratch.data_ptr(), n_layout_blocks, size
-        with _capi.on_device(q.device):
-            _capi.call("bsa_attn_bwd", ctypes.byref(args), stream)
-        if facts is not None and not args.bwd_scratch_ready and not torch.cuda.is_current_stream_capturing():
-            facts.bwd_scratch, facts.bwd_stream = scratch, stream
+        args.n_layout_blocks = n_layout_blocks
+        # Only the 16-bit kernels for 64 x 64 blocks and at most two head slices walk records in a scratch (the
+        # pairs that some score survives, built inside bsa_attn_bwd); the other kernel families never touch it.
+        if _walks_records(meta, q.dtype):
+            size = max(_capi.load().bsa_attn_bwd_scratch_bytes(B, nq, nk, n_layout_blocks, n_mask_blocks), 16)
+            # The records depend on the layouts and on the values of the mask and of the causal lengths only: a
+            # later call on the same stream with the same ones reads what this call wrote.  Remembered only here,
+            # where the call that ran did write them.
+            scratch = facts.bwd_scratch if facts is not None and facts.bwd_stream == stream else None
+            args.bwd_scratch_ready = 1 if scratch is not None and scratch.numel() == size else 0
+            if not args.bwd_scratch_ready:
+                scratch = torch.empty(size, dtype=torch.uint8, device=q.device)
+            args.bwd_scratch, args.bwd_scratch_bytes = scratch.data_ptr(), size
+            # With room for dS of every pair (one block per active block of the attention layout) the dK / dV kernel
+            # leaves it behind and dQ = dS K is a product of its own; beyond the limit (set_kept_ds_limit) dS is
+            # formed a second time, as the reference does (blksprs/ops/flash_attention.py:1228-1480).  dS carries
+            # nothing from one call to the next: it is taken from torch's allocator for this call alone.
+            ds_bytes = _capi.load().bsa_attn_bwd_ds_bytes(n_layout_blocks, meta.sbs)
+            if 0 < ds_bytes <= kept_ds_limit():
+                ds = torch.empty(ds_bytes, dtype=torch.uint8, device=q.device)
+                args.bwd_ds, args.bwd_ds_bytes = ds.data_ptr(), ds_bytes
+            with _capi.on_device(q.device):
+                _capi.call("bsa_attn_bwd", ctypes.byref(args), stream)
+            if facts is not None and not args.bwd_scratch_ready and not torch.cuda.is_current_stream_capturing():
+                facts.bwd_scratch, facts.bwd_stream = scratch, stream
+        else:
+            with _capi.on_device(q.device):
+                _capi.call("bsa_attn_bwd", ctypes.byref(args), stream)
         grad_bias = dbias.to(bias.dtype) if meta.has_bias else None
         return dq, dk, dv, grad_bias, None, None, None
 

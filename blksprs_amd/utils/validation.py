@@ -73,10 +73,12 @@ def kept_ds_limit() -> int:
 
 
 def set_kept_ds_limit(n_bytes: int) -> None:
-    """The backward of ``flash_attention`` on 64 x 64 16-bit blocks keeps dS of every pair in a scratch tensor
-    (8 KiB per active block of the attention layout; with it dQ costs one matrix product per pair instead of three)
-    when that takes at most ``n_bytes`` (default 4 GiB, for the whole process); 0: never, dS is formed twice, as
-    the reference does (blksprs/ops/flash_attention.py:1228-1480)."""
+    """The backward of ``flash_attention`` on 64 x 64 16-bit blocks keeps dS of every pair in a buffer that lives
+    for that one backward call (8 KiB per active block of the attention layout, taken from torch's allocator and
+    returned to it when the call is queued; with it dQ costs one matrix product per pair instead of three) when the
+    buffer of that call takes at most ``n_bytes`` (default 4 GiB; the limit is per call and the setting is shared
+    by all threads); 0: never, dS is formed twice, as the reference does
+    (blksprs/ops/flash_attention.py:1228-1480)."""
     global _kept_ds_limit
     _kept_ds_limit = int(n_bytes)
 

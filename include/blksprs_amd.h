@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define BSA_ABI_VERSION 2
+#define BSA_ABI_VERSION 3
 
 /* error codes */
 #define BSA_OK 0
@@ -43,6 +43,10 @@ typedef void *bsa_stream_t; /* hipStream_t */
 
 int bsa_abi_version(void);
 const char *bsa_last_error(void);
+/* One line naming the compiler the library was built with ("hipcc: <version line of hipcc --version>; flags: ...").
+ * Some kernels place their own waits for memory around loads the compiler does not see; a red bit-identity test
+ * after a toolchain change is read next to this line.  No counterpart in the reference. */
+const char *bsa_build_info(void);
 
 /* ------------------------------------------------------------------ LUTs */
 
@@ -379,13 +383,17 @@ typedef struct bsa_attn_args {
    * which its dK / dV kernel hands key rows to the workgroups that stay for the launch), so two calls that
    * overlap in time (different streams) need a scratch each. */
   int64_t bwd_scratch_ready;
-  /* Size of bwd_scratch in bytes, or 0 for "bsa_attn_bwd_scratch_bytes(...) and no more".  With at least
-   * bsa_attn_bwd_scratch_bytes_ds(...) bytes the dK / dV kernel also leaves dS of every visited pair in the
-   * scratch (one 64 x 64 block of the operand type per active block of the attention layout) and dQ = dS K is a
-   * product of its own; with less, the dQ kernel forms the scores and dS of its pairs a second time.  The
-   * reference recomputes (blksprs/ops/flash_attention.py:1228-1480); keeping dS trades memory for a third of the
-   * backward's matrix-core work. */
+  /* Size of bwd_scratch in bytes (checked against bsa_attn_bwd_scratch_bytes(...)), or 0 for "large enough". */
   int64_t bwd_scratch_bytes;
+  /* Optional room for dS, bsa_attn_bwd_ds_bytes(...) bytes (16-byte aligned), used by the 16-bit kernels for 64 x 64
+   * blocks only: the dK / dV kernel then leaves dS of every visited pair there (one 64 x 64 block of the operand
+   * type per active block of the attention layout) and dQ = dS K is a product of its own.  NULL or fewer bytes: the
+   * dQ kernel forms the scores and dS of its pairs a second time, as the reference does
+   * (blksprs/ops/flash_attention.py:1228-1480); keeping dS trades memory for a third of the backward's matrix-core
+   * work.  Nothing in it is read after the call returns its work to the stream: it carries nothing from one call
+   * to the next and may be handed to other work that follows on the same stream. */
+  void *bwd_ds;
+  int64_t bwd_ds_bytes;
 } bsa_attn_args;
 
 #define BSA_ATTN_RECORD_INTS 16
@@ -420,10 +428,9 @@ int bsa_attn_mask_dead(const void *mask, int64_t n_mask_blocks, int32_t sbs, uin
 
 /* Size in bytes of bsa_attn_args.bwd_scratch for these sizes (16-byte aligned buffer). */
 size_t bsa_attn_bwd_scratch_bytes(int64_t B, int64_t nq, int64_t nk, int64_t n_layout_blocks, int64_t n_mask_blocks);
-/* The same with room for the dS blocks (see bsa_attn_args.bwd_scratch_bytes): the lists, padded to a multiple of
- * 4096 bytes, then n_layout_blocks * 8192 bytes. */
-size_t bsa_attn_bwd_scratch_bytes_ds(int64_t B, int64_t nq, int64_t nk, int64_t n_layout_blocks,
-                                     int64_t n_mask_blocks);
+/* Size in bytes of bsa_attn_args.bwd_ds for an attention layout of n_layout_blocks active blocks:
+ * n_layout_blocks * 8192 for sbs 64, 0 for the block sizes whose kernels do not keep dS. */
+size_t bsa_attn_bwd_ds_bytes(int64_t n_layout_blocks, int32_t sbs);
 
 /*
  * dq, dk, dv (and dbias) from the saved lse.  Replaces
