@@ -297,7 +297,9 @@ def matmul_workload(name, B, n, sbs, dtype, density, ensure_rows, value_scale, d
 
     dt_name = {torch.bfloat16: "bf16", torch.float16: "f16", torch.float32: "f32"}[dtype]
     if backward:
-        kernel = "matmul_mfma_kernel (two launches: dX with y read transposed, dY with x read transposed)"
+        kernel = ("matmul_lines_kernel (two launches: dX by rows of dO, dY by its columns)"
+                  if sbs == 64 and dtype != torch.float32 else
+                  "matmul_mfma_kernel (two launches: dX with y read transposed, dY with x read transposed)")
     elif sbs > 16:
         kernel = "matmul_rows_kernel" if sbs == 64 and dtype != torch.float32 else "matmul_mfma_kernel"
     else:
@@ -773,7 +775,7 @@ def make_workload(name, dev):
 CONFIGS = ["a1", "a1bwd", "c1", "c2", "c2bwd", "c3", "c3bwd", "c4", "c4bwd", "c5", "t1", "l1", "r1", "r2", "p1", "v1", "v2"]
 # the configurations a default run times behind the headline one, with fewer steps (their roofline objects ride
 # along in the same JSON line so that they are timed by whoever runs the script, not quoted from elsewhere)
-COMPANIONS = ["c4", "c4bwd", "c3", "c5"]
+COMPANIONS = ["c2bwd", "c4", "c4bwd", "c3", "c5"]
 
 
 def measure(config, dev, steps, warmup, scratch):

@@ -36,6 +36,19 @@ class AttnArgs(ctypes.Structure):
     )
 
 
+class LinesArgs(ctypes.Structure):
+    """Mirror of ``struct bsa_lines_args``."""
+
+    _fields_ = (
+        [(n, c_void_p) for n in ("streamed", "priv", "out", "pidx_streamed", "pidx_private", "pidx_out",
+                                 "part_table")]
+        + [(n, c_int64) for n in ("n_batches", "lines_per_batch", "n_streamed", "n_outputs")]
+        + [("streamed_strides", c_int64 * 3), ("out_strides", c_int64 * 3), ("private_strides", c_int64 * 3)]
+        + [(n, c_int64) for n in ("nnz_streamed", "nnz_private", "nnz_out")]
+        + [("error", c_void_p)]
+    )
+
+
 ATTN_RECORD_INTS = 16  # BSA_ATTN_RECORD_INTS
 ROWS_RECORD_INTS = 128  # BSA_ROWS_RECORD_INTS
 
@@ -63,6 +76,8 @@ SIGNATURES = {
     "bsa_to_sparse": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_int, c_void_p]),
     "bsa_to_dense": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int, c_int,
                              c_uint64, c_void_p]),
+    "bsa_matmul_lines_parts": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p]),
+    "bsa_matmul_lines": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p]),
     "bsa_transpose_blocks": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
                                      c_int, c_int, c_void_p]),
     "bsa_layout_from_dense": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_int, c_int, c_void_p]),

@@ -322,14 +322,17 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_records_kernel(bsa_attn_
 }
 
 // Workgroup g of a main kernel runs on XCD g % 8, and every XCD is given a contiguous eighth of the rows, so that
-// the blocks in flight on one L2 belong to the same batch entries.  Inside its eighth an XCD takes the rows with
-// the most live pairs first when its longest row has more than four times the mean (a row that every query
-// attends to can be a hundred times longer than the others and must not be the last to start).  Workgroups 0 .. 7 order the query rows, 8 .. 15 the key rows, by a
-// counting sort on min(pairs, 255); rows of equal count come in no fixed order, which changes no result.  What
-// is written per position is the 64-byte header of the workgroup that takes it.
+// the blocks in flight on one L2 belong to the same batch entries.  Inside its eighth an XCD takes first the few
+// rows with more than four times the mean number of live pairs (a row that every query attends to can be a hundred
+// times longer than the others and must not be the last to start), then all the others, both groups in their
+// natural order: neighbouring rows share most of the blocks they stream (a local window of +-w blocks has 2 w of
+// its 2 w + 1 tiles in common with the next row's), and rows handed out one after the other are in flight together,
+// so those tiles are fetched from memory once and found in the L2 afterwards.  (Ordering all rows by length
+// scatters the neighbours over the launch: on a window + global + random layout the dK / dV walk then fetched twice
+// the bytes.)  The order is a stable partition, the same on every run.  Workgroups 0 .. 7 order the query rows,
+// 8 .. 15 the key rows.  What is written per position is the 64-byte header of the workgroup that takes it.
 constexpr int kOrderThreads = 1024;
 __global__ __launch_bounds__(kOrderThreads) void attn_bwd_order_kernel(bsa_attn_args a) {
-  __shared__ int bins[256];
   const BwdLists L = bwd_lists(a);
   const bool by_key = blockIdx.x >= 8;
   const int64_t rows = by_key ? a.B * a.nk : a.B * a.nq;
@@ -355,39 +358,49 @@ __global__ __launch_bounds__(kOrderThreads) void attn_bwd_order_kernel(bsa_attn_
   };
   const int64_t chunk = (rows + 7) / 8;  // = gridDim.x / 8 of the main kernels
   const int64_t r0 = (int64_t)(blockIdx.x & 7) * chunk, r1 = r0 + chunk < rows ? r0 + chunk : rows;
-  const int tid = threadIdx.x;
-  __shared__ int longest;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   __shared__ unsigned long long total;
-  if (tid < 256) bins[tid] = 0;
+  __shared__ int n_long;
+  __shared__ int wave_long[kOrderThreads / 64];
   if (tid == 0) {
-    longest = 0;
     total = 0;
+    n_long = 0;
   }
   __syncthreads();
-  auto bin_of = [&](int64_t r) {
-    const int n = ends[r] - offsets[r];
-    return 255 - (n < 255 ? n : 255);
-  };
-  for (int64_t r = r0 + tid; r < r1; r += kOrderThreads) {
-    const int n = ends[r] - offsets[r];
-    atomicAdd(&bins[bin_of(r)], 1);
-    atomicMax(&longest, n);
-    atomicAdd(&total, (unsigned long long)n);
-  }
+  unsigned long long mine = 0;
+  for (int64_t r = r0 + tid; r < r1; r += kOrderThreads) mine += (unsigned long long)(ends[r] - offsets[r]);
+  if (mine) atomicAdd(&total, mine);
   __syncthreads();
-  // rows of similar length stay in their natural order, which keeps neighbours (who share blocks) together
-  if ((unsigned long long)longest * (unsigned long long)(r1 - r0) <= 4ull * total) {
+  const unsigned long long sum = total, count = r0 < r1 ? (unsigned long long)(r1 - r0) : 0ull;
+  auto is_long = [&](int64_t r) { return (unsigned long long)(ends[r] - offsets[r]) * count > 4ull * sum; };
+  int mine_long = 0;
+  for (int64_t r = r0 + tid; r < r1; r += kOrderThreads) mine_long += is_long(r) ? 1 : 0;
+  if (mine_long) atomicAdd(&n_long, mine_long);
+  __syncthreads();
+  const int64_t longs = n_long;
+  if (longs == 0) {
     for (int64_t r = r0 + tid; r < r1; r += kOrderThreads) emit(r, r);
     return;
   }
-  // exclusive prefix sum of the 256 bins: thread t adds up the bins before its own
-  int before = 0;
-  if (tid < 256)
-    for (int i = 0; i < tid; ++i) before += bins[i];
-  __syncthreads();
-  if (tid < 256) bins[tid] = before;
-  __syncthreads();
-  for (int64_t r = r0 + tid; r < r1; r += kOrderThreads) emit(r0 + atomicAdd(&bins[bin_of(r)], 1), r);
+  // stable partition, 1024 rows at a time: the long rows of the tile go behind the long rows before it, the others
+  // behind all long rows and the other rows before them
+  int64_t long_done = 0;
+  for (int64_t base = r0; base < r1; base += kOrderThreads) {
+    const int64_t r = base + tid;
+    const bool valid = r < r1;
+    const bool lng = valid && is_long(r);
+    const unsigned long long votes = __ballot(lng);
+    if (lane == 0) wave_long[wave] = __popcll(votes);
+    __syncthreads();
+    int before = __popcll(votes & ((1ull << lane) - 1)), in_tile = 0;
+    for (int w = 0; w < kOrderThreads / 64; ++w) {
+      before += w < wave ? wave_long[w] : 0;
+      in_tile += wave_long[w];
+    }
+    if (valid) emit(lng ? r0 + long_done + before : r0 + longs + (base - r0 - long_done) + (tid - before), r);
+    long_done += in_tile;
+    __syncthreads();  // wave_long is written again
+  }
 }
 
 // delta[b, qb, i] = sum over the output slices of rowsum(o * dO), four lanes per query row; also the tickets of

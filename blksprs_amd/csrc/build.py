@@ -15,7 +15,7 @@ from pathlib import Path
 HERE = Path(__file__).resolve().parent
 OUT_DIR = HERE.parent / "lib"
 LIB = OUT_DIR / "libblksprs_amd.so"
-SOURCES = ["common.hip", "lut.hip", "lut_order.hip", "convert.hip", "softmax.hip", "matmul.hip", "matmul_rows.hip", "row_wise.hip",
+SOURCES = ["common.hip", "lut.hip", "lut_order.hip", "convert.hip", "softmax.hip", "matmul.hip", "matmul_rows.hip", "matmul_lines.hip", "row_wise.hip",
            "attention.hip", "attn_generic.hip", "attn_mfma.hip", "attn_bwd_mfma.hip", "attn_f32mma.hip", "attn_f32mma_bwd.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["-O3", "-std=c++17", "-fno-strict-aliasing", "--offload-arch=gfx950", "-fPIC",

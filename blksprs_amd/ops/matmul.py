@@ -7,6 +7,7 @@ and is computed by ``bsa_matmul``.  The backward pass reads the saved operands
 transposed inside the kernel instead of materialising transposed copies.
 """
 
+import ctypes
 import os
 
 import torch
@@ -44,6 +45,75 @@ def _launch_rows(x: Tensor, y: Tensor, plan: "_Plan", sbs: int) -> Tensor:
                        plan.pair_offsets.data_ptr(), _capi.ptr(plan.pairs),
                        _capi.ptr(plan.row_records), plan.row_records.size(0), plan.row_items, n_out,
                        x.size(0), y.size(0), sbs, _capi.DTYPE_CODES[x.dtype], _capi.stream(x.device))
+    return out
+
+
+_MAX_LINE_BLOCKS = 512  # blocks per line that the line kernel's lists in LDS hold
+
+
+def _lines_args(plan: "_Plan", shapes, which: str, streamed: Tensor | None, private: Tensor | None,
+                out: Tensor | None, part_table: Tensor | None) -> _capi.LinesArgs:
+    """Argument block of the line kernel for dX = dO Y^T (``which == "x"``: lines are the block rows of x) or
+    dY = X^T dO (``"y"``: the block columns of y).  The streamed operand is dO in both."""
+    (B, R, K), (_, _, C) = shapes
+    a = _capi.LinesArgs()
+    a.n_batches = B
+    a.pidx_streamed = _capi.ptr(plan.packed_o)
+    a.nnz_streamed = plan.n_out
+    if which == "x":
+        a.lines_per_batch, a.n_streamed, a.n_outputs = R, C, K
+        a.streamed_strides[:] = (R * C, C, 1)
+        a.pidx_out, a.out_strides[:] = _capi.ptr(plan.packed_x), (R * K, K, 1)
+        a.pidx_private, a.private_strides[:] = _capi.ptr(plan.packed_y), (K * C, C, 1)
+        a.nnz_out, a.nnz_private = plan.n_x, plan.n_y
+    else:
+        a.lines_per_batch, a.n_streamed, a.n_outputs = C, R, K
+        a.streamed_strides[:] = (R * C, 1, C)
+        a.pidx_out, a.out_strides[:] = _capi.ptr(plan.packed_y), (K * C, 1, C)
+        a.pidx_private, a.private_strides[:] = _capi.ptr(plan.packed_x), (R * K, 1, K)
+        a.nnz_out, a.nnz_private = plan.n_y, plan.n_x
+    a.streamed, a.priv, a.out = _capi.ptr(streamed), _capi.ptr(private), _capi.ptr(out)
+    a.part_table = _capi.ptr(part_table)
+    a.error = _capi.ptr(plan.lines_error)
+    return a
+
+
+def _lines_apply(plan: "_Plan", shapes, sbs: int, dtype: torch.dtype) -> bool:
+    """Whether the two backward products run on the line kernel: 16-bit operands, 64 x 64 blocks, lines of dO and
+    of the output of at most 512 blocks either way."""
+    (B, R, K), (_, _, C) = shapes
+    return (sbs == 64 and dtype in (torch.float16, torch.bfloat16) and max(R, C, K) <= _MAX_LINE_BLOCKS
+            and B * max(R, C) < 2 ** 31 - 1)
+
+
+def _lines_parts(plan: "_Plan", shapes) -> tuple[Tensor, Tensor]:
+    """The part tables of the two backward products (``bsa_matmul_lines_parts``), built once per plan on the
+    device; nothing is read back."""
+    if plan.grad_lines is None:
+        device = plan.packed_o.device
+        plan.lines_error = torch.zeros(32, dtype=torch.int32, device=device)
+        built = []
+        for which in ("x", "y"):
+            a = _lines_args(plan, shapes, which, None, None, None, None)
+            n_lines = a.n_batches * a.lines_per_batch
+            scratch = torch.empty(4 * n_lines + 2, dtype=torch.int32, device=device)
+            table = torch.empty(1 + a.nnz_out // 16 + n_lines, dtype=torch.int32, device=device)
+            with _capi.on_device(device):
+                _capi.call("bsa_matmul_lines_parts", ctypes.byref(a), scratch.data_ptr(), table.data_ptr(),
+                           _capi.stream(device))
+            built.append(table)
+        plan.grad_lines = tuple(built)
+    return plan.grad_lines
+
+
+def _launch_lines(plan: "_Plan", shapes, which: str, streamed: Tensor, private: Tensor, n_out: int, sbs: int) -> Tensor:
+    out = torch.empty((n_out, sbs, sbs), dtype=streamed.dtype, device=streamed.device)
+    if n_out:
+        table = _lines_parts(plan, shapes)[0 if which == "x" else 1]
+        a = _lines_args(plan, shapes, which, streamed, private, out, table)
+        with _capi.on_device(streamed.device):
+            _capi.call("bsa_matmul_lines", ctypes.byref(a), int(which == "y"), sbs, _capi.DTYPE_CODES[streamed.dtype],
+                       _capi.stream(streamed.device))
     return out
 
 
@@ -158,7 +228,7 @@ class _Plan:
     with.  Nothing writes to its tensors after they are built."""
 
     __slots__ = ("pair_offsets", "pairs", "block_order", "n_out", "n_x", "n_y", "row_records", "row_items",
-                 "packed_x", "packed_y", "packed_o", "grad_lists")
+                 "packed_x", "packed_y", "packed_o", "grad_lists", "grad_lines", "lines_error")
 
     def __init__(self, cache: dict):
         self.pair_offsets, self.pairs = cache["contraction_offsets"], cache["contraction_pairs"]
@@ -168,7 +238,8 @@ class _Plan:
                                           cache["n_sparse_blocks_y"])
         self.packed_x, self.packed_y, self.packed_o = (cache["packed_indices_x"], cache["packed_indices_y"],
                                                        cache["packed_indices_o"])
-        self.grad_lists = None
+        self.grad_lists = None  # contraction lists of the two backward products (tile kernel)
+        self.grad_lines = self.lines_error = None  # part offsets of the two backward products (line kernel)
 
 
 def _backward_lists(plan: _Plan, shape_x, shape_y):
@@ -188,10 +259,16 @@ def _backward_lists(plan: _Plan, shape_x, shape_y):
 
 
 def _publish_backward_lists(layout_cache: dict, plan: _Plan) -> None:
-    """Shows the plan's backward lists under the cache's own keys, while the cache still belongs to the plan."""
-    if layout_cache.get("plan") is plan and "grad_x_pair_offsets" not in layout_cache:
+    """Shows the plan's backward tables under the cache's own keys, while the cache still belongs to the plan."""
+    if layout_cache.get("plan") is not plan:
+        return
+    if plan.grad_lists is not None and "grad_x_pair_offsets" not in layout_cache:
         (layout_cache["grad_x_pair_offsets"], layout_cache["grad_x_pairs"], layout_cache["grad_y_pair_offsets"],
          layout_cache["grad_y_pairs"]) = plan.grad_lists
+        finalize_layout_cache(layout_cache)
+    if plan.grad_lines is not None and "grad_x_part_table" not in layout_cache:
+        layout_cache["grad_x_part_table"], layout_cache["grad_y_part_table"] = plan.grad_lines
+        layout_cache["grad_lines_error"] = plan.lines_error
         finalize_layout_cache(layout_cache)
 
 
@@ -220,9 +297,18 @@ class _Matmul(torch.autograd.Function):
         x, y = ctx.saved_tensors
         sbs = ctx.sparsity_block_size
         plan = ctx.plan
+        grad_x = grad_y = None
+        if _lines_apply(plan, ctx.shapes, sbs, x.dtype):
+            # by lines of dO (row i for dX, column j for dY), each streamed through LDS once
+            _lines_parts(plan, ctx.shapes)
+            _publish_backward_lists(ctx.layout_cache, plan)
+            if ctx.needs_input_grad[0]:
+                grad_x = _launch_lines(plan, ctx.shapes, "x", grad_output, y, x.size(0), sbs)
+            if ctx.needs_input_grad[1]:
+                grad_y = _launch_lines(plan, ctx.shapes, "y", grad_output, x, y.size(0), sbs)
+            return grad_x, grad_y, None, None, None, None
         gx_off, gx_pairs, gy_off, gy_pairs = _backward_lists(plan, *ctx.shapes)
         _publish_backward_lists(ctx.layout_cache, plan)
-        grad_x = grad_y = None
         if ctx.needs_input_grad[0]:
             grad_x = _launch(grad_output, y, gx_off, gx_pairs, None, x.size(0), sbs, False, True)
         if ctx.needs_input_grad[1]:
@@ -343,9 +429,10 @@ def matmul(x: BlksprsTensor, sparsity_layout_x: Tensor,
         return BlksprsTensor.wrap(_forward(x, y, layout_cache["plan"], sparsity_block_size))
     shape_x, shape_y = tuple(sparsity_layout_x.shape), tuple(sparsity_layout_y.shape)
     plan = layout_cache["plan"]
-    if plan.grad_lists is None:
+    if plan.grad_lists is None and not _lines_apply(plan, (shape_x, shape_y), sparsity_block_size, x.dtype):
         # the lists of the two backward products are built with the first forward pass that will need them, so
-        # that no backward pass waits for the device
+        # that no backward pass waits for the device (the line kernel needs no lists, and its part offsets are
+        # built without a read by the host)
         _backward_lists(plan, shape_x, shape_y)
         _publish_backward_lists(layout_cache, plan)
     return BlksprsTensor.wrap(_Matmul.apply(x, y, layout_cache, shape_x, shape_y, sparsity_block_size))

@@ -311,6 +311,51 @@ int bsa_matmul_rows(const void *x, const void *y, void *out, const int32_t *pair
                     int64_t nnz_o, int64_t nnz_x, int64_t nnz_y, int sbs, int dtype, bsa_stream_t stream);
 
 /*
+ * The two backward products of bsa_matmul for 16-bit operands and 64 x 64 blocks, dX = dO Y^T and dY = X^T dO
+ * (blksprs/ops/matmul.py:130-145), by LINES: a line is a block row of dX resp. a block column of dY.  All output
+ * blocks of a line need the same line of dO (the streamed operand: row i resp. column j of dO) and each pairs it
+ * with its own blocks of the other operand (the private operand: Y(k, j) resp. X(i, k)).  One workgroup takes up
+ * to 16 output blocks of a line, keeps their accumulators in registers for the whole line and streams the line
+ * of dO through LDS once, so dO is read once per launch.  No lists are needed: the kernel finds its blocks in the
+ * reverse indices (-1: inactive) of the three layouts, addressed through strides so that one kernel serves rows
+ * and columns:
+ *   streamed block t of line (b, l):  pidx_streamed[b * streamed_strides[0] + l * streamed_strides[1] + t * streamed_strides[2]]
+ *   output block u of line (b, l):    pidx_out[b * out_strides[0] + l * out_strides[1] + u * out_strides[2]]
+ *   private block of (u, t):          pidx_private[b * private_strides[0] + u * private_strides[1] + t * private_strides[2]]
+ * with t < n_streamed, u < n_outputs (at most 512 each).  dX: lines are the rows of x's layout (B, R, K), streamed =
+ * dO with the output layout (B, R, C): strides (R C, C, 1); out = dX: (R K, K, 1); private = y (B, K, C):
+ * (K C, C, 1); contract_rows = 0 (the columns of both blocks are contracted).  dY: lines are the columns of y's
+ * layout, streamed = dO: (R C, 1, C); out = dY: (K C, 1, C); private = x: (R K, 1, K); contract_rows = 1.
+ * Every active output block is written (zeros without a pair); the products of a block are added in ascending
+ * order of t, in fp32, and rounded once.
+ * part_table (int32 [1 + nnz_out / 16 + n_batches * lines_per_batch]) is written by bsa_matmul_lines_parts from
+ * the same argument block (it reads pidx_out and the sizes only; scratch: 4 * lines + 2 int32): [0] = the
+ * number of parts (a part = up to 16 output blocks of a line: ceil(blocks / 16) parts per line), then one entry
+ * line << 6 | part per part in the order in which workgroups take them: batch entry by batch entry, inside a
+ * batch entry first the parts of more than 8 blocks, then the others, each group in the order of the lines
+ * (workgroups that run side by side then do about the same work and walk the streamed operand in step).  It
+ * depends on the output's layout only.
+ * error: NULL, or 32 int32 on the device, zero before the launch: [0] becomes 1 if one of the kernel's bounded
+ * waits between the waves of a workgroup ran out (the results are then wrong; it never does unless the device
+ * loses a wave), and the other entries then hold what the first such wave saw (its wave number, which wait, the
+ * streamed block it waited for, its copying duty, the line's length, the workgroup, the eight waves' positions
+ * and the first ten slots' announcements, the line and part, its output blocks): for the library's own tests.
+ */
+typedef struct bsa_lines_args {
+  const void *streamed, *priv; /* blocks of the streamed and of the private operand */
+  void *out;
+  const int64_t *pidx_streamed, *pidx_private, *pidx_out;
+  const int32_t *part_table;
+  int64_t n_batches, lines_per_batch, n_streamed, n_outputs;
+  int64_t streamed_strides[3], out_strides[3], private_strides[3];
+  int64_t nnz_streamed, nnz_private, nnz_out;
+  int32_t *error;
+} bsa_lines_args;
+
+int bsa_matmul_lines_parts(const bsa_lines_args *args, int32_t *scratch, int32_t *part_table, bsa_stream_t stream);
+int bsa_matmul_lines(const bsa_lines_args *args, int contract_rows, int sbs, int dtype, bsa_stream_t stream);
+
+/*
  * Block gather with element transposition: out[o] = transpose(blocks[packed[(b * R + r) * C + c]]) with
  * (b, r, c) = coords[o] (int64 [nnz_out, 3], the non-zero coordinates of the OUTPUT layout, shape (B, R, C));
  * `packed` is an int64 table over the output layout that names the source block of every position (-1 or

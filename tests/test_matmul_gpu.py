@@ -77,10 +77,15 @@ def test_backward_matches_autograd_of_the_oracle(device, dtype, sbs):
     assert_close(xg.grad, x64.grad, tol, f"dX {dtype} sbs={sbs}")
     assert_close(yg.grad, y64.grad, tol, f"dY {dtype} sbs={sbs}")
     # a second step reuses the forward and backward lists
-    offsets = cache["grad_x_pair_offsets"]
+    # (16-bit operands with 64 x 64 blocks run by lines of dO and keep part offsets instead of pair lists)
+    key = "grad_x_part_table" if "grad_x_part_table" in cache else "grad_x_pair_offsets"
+    assert (key == "grad_x_part_table") == (sbs == 64 and dtype != torch.float32)
+    offsets = cache[key]
     xg.grad = None
     bs.ops.matmul(xg, lxd, yg, lyd, lod, sbs, layout_cache=cache).backward(go.to(device))
-    assert cache["grad_x_pair_offsets"] is offsets
+    assert cache[key] is offsets
+    if key == "grad_x_part_table":
+        assert int(cache["grad_lines_error"][0].item()) == 0
     assert_close(xg.grad, x64.grad, tol, "dX second step")
 
 
@@ -300,3 +305,120 @@ def test_sbs16_runs_and_pair_windows(device, dtype, trans, dims, density):
         ref.backward(go.double())
         assert_close(xd.grad, x64.grad, TOL[dtype], "dX")   # x^T-free: go @ y^T reads y transposed
         assert_close(yd.grad, y64.grad, TOL[dtype], "dY")   # x^T @ go reads x transposed
+
+
+def _tile_kernel_grads(x, y, go, lx, ly, lo, sbs):
+    """dX and dY by the tile kernel with transposed operand reads, from contraction lists of the two products."""
+    from blksprs_amd import _capi
+    from blksprs_amd.utils.tools import build_contraction_lists, pack_layout
+    B, R, K = lx.shape
+    C = ly.size(2)
+    px, py, po = pack_layout(lx), pack_layout(ly), pack_layout(lo)
+    pidx_yt = py.packed.view(B, K, C).transpose(1, 2).contiguous().view(-1)
+    pidx_xt = px.packed.view(B, R, K).transpose(1, 2).contiguous().view(-1)
+    gx, gy = build_contraction_lists((po.packed, pidx_yt, px.packed, B, R, C, K, px.count),
+                                     (pidx_xt, po.packed, py.packed, B, K, R, C, py.count))
+    dx, dy = torch.empty_like(x), torch.empty_like(y)
+    code = _capi.DTYPE_CODES[x.dtype]
+    if x.size(0):
+        _capi.call("bsa_matmul", go.data_ptr(), y.data_ptr(), dx.data_ptr(), gx.pair_offsets.data_ptr(),
+                   _capi.ptr(gx.pairs), 0, x.size(0), go.size(0), y.size(0), sbs, code, 0, 1, _capi.stream(x.device))
+    if y.size(0):
+        _capi.call("bsa_matmul", x.data_ptr(), go.data_ptr(), dy.data_ptr(), gy.pair_offsets.data_ptr(),
+                   _capi.ptr(gy.pairs), 0, y.size(0), x.size(0), go.size(0), sbs, code, 1, 0, _capi.stream(x.device))
+    return dx, dy
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("dims,dx,dy,do", [
+    ((2, 4, 6, 5), 0.5, 0.5, 0.8),      # a few blocks per line: waves without an output block, short lines
+    ((2, 3, 40, 70), 0.9, 0.5, 0.9),    # rows of x with more than 16 blocks (several parts), lines of dO of more than 64
+    ((1, 70, 20, 3), 0.6, 0.95, 1.0),   # columns of dO of more than 64 blocks, columns of y with more than 16 blocks
+    ((3, 9, 7, 11), 0.3, 0.3, 0.5),     # rows without blocks, output blocks without a pair
+    ((1, 2, 17, 130), 1.0, 1.0, 1.0),   # dense: 17 output blocks per row (parts of 16 and 1), three segments of dO
+])
+def test_backward_by_lines_matches_the_tile_kernel_and_the_oracle(device, dtype, dims, dx, dy, do):
+    """16-bit operands with 64 x 64 blocks take the line kernel in the backward pass: dX by rows of dO, dY by its
+    columns, each line streamed through a ring in LDS that eight waves fill and drain at their own pace.  Held to
+    the tile kernel (same products, same order of accumulation inside a block) at the tolerance of the type, to
+    autograd of the oracle, and to itself (a second run gives the same bits, whatever the waves' timing)."""
+    B, R, K, C = dims
+    sbs = 64
+    lx = rand_layout((B, R, K), dx, seed=11)
+    ly = rand_layout((B, K, C), dy, seed=12)
+    lo = rand_layout((B, R, C), do, seed=13)
+    if dx < 0.5:
+        lx[0, 0] = False
+        ly[0, :, 0] = False
+    x = rand_blocks(int(lx.sum()), sbs, dtype, 14, 1.0 / math.sqrt(K * sbs))
+    y = rand_blocks(int(ly.sum()), sbs, dtype, 15)
+    go = rand_blocks(int(lo.sum()), sbs, dtype, 16, 1.0 / math.sqrt(C * sbs))
+    lxd, lyd, lod = lx.to(device), ly.to(device), lo.to(device)
+    cache = {}
+    runs = []
+    for _ in range(2):
+        xg, yg = x.to(device).requires_grad_(True), y.to(device).requires_grad_(True)
+        bs.ops.matmul(xg, lxd, yg, lyd, lod, sbs, layout_cache=cache).backward(go.to(device))
+        runs.append((xg.grad, yg.grad))
+    assert "grad_x_part_table" in cache and int(cache["grad_lines_error"][0].item()) == 0
+    assert torch.equal(runs[0][0], runs[1][0]) and torch.equal(runs[0][1], runs[1][1])
+    tile_dx, tile_dy = _tile_kernel_grads(x.to(device), y.to(device), go.to(device), lxd, lyd, lod, sbs)
+    assert_close(runs[0][0], tile_dx.double(), 1e-2, "dX by lines against the tile kernel")
+    assert_close(runs[0][1], tile_dy.double(), 1e-2, "dY by lines against the tile kernel")
+    x64, y64 = x.double().requires_grad_(True), y.double().requires_grad_(True)
+    ref = orc.matmul(x64, lx.numpy(), y64, ly.numpy(), lo.numpy(), sbs, acc_dtype=torch.float64)
+    ref.backward(go.double())
+    assert_close(runs[0][0], x64.grad, 2e-2, "dX by lines against the oracle")
+    assert_close(runs[0][1], y64.grad, 2e-2, "dY by lines against the oracle")
+    # the part tables, bit for bit: per batch entry first the parts of more than 8 output blocks, then the others,
+    # each group in the order of the lines
+    def expected_table(counts_per_batch):
+        entries = []
+        for b, counts in enumerate(counts_per_batch):
+            longs, shorts = [], []
+            for l, n in enumerate(counts):
+                line = b * len(counts) + l
+                for p in range((n + 15) // 16):
+                    (longs if min(16, n - 16 * p) > 8 else shorts).append(line << 6 | p)
+            entries += longs + shorts
+        return [len(entries)] + entries
+
+    want_x = expected_table(lx.sum(-1).tolist())
+    want_y = expected_table(ly.sum(1).tolist())
+    assert cache["grad_x_part_table"].cpu().tolist()[:len(want_x)] == want_x
+    assert cache["grad_y_part_table"].cpu().tolist()[:len(want_y)] == want_y
+
+
+def test_full_size_config2_gradients_sampled_against_the_oracle(device):
+    """Config 2 at full size, backward: dX and dY of one batch entry against autograd of the oracle; linearity in
+    the upstream gradient (dO -> 2 dO doubles both, bit for bit); a second run gives the same bits."""
+    B, n, sbs = 16, 64, 64
+    lx = rand_layout((B, n, n), 0.25, seed=0)
+    ly = rand_layout((B, n, n), 0.25, seed=1)
+    lo = torch.from_numpy(orc.layout_matmul(lx.numpy(), ly.numpy()))
+    g = torch.Generator().manual_seed(2)
+    x = (torch.randn((int(lx.sum()), sbs, sbs), generator=g) / 64.0).to(torch.bfloat16)
+    y = torch.randn((int(ly.sum()), sbs, sbs), generator=g).to(torch.bfloat16)
+    go = (torch.randn((int(lo.sum()), sbs, sbs), generator=g) / 64.0).to(torch.bfloat16)
+    lxd, lyd, lod = lx.to(device), ly.to(device), lo.to(device)
+    cache = {}
+
+    def grads(scale):
+        xg, yg = x.to(device).requires_grad_(True), y.to(device).requires_grad_(True)
+        bs.ops.matmul(xg, lxd, yg, lyd, lod, sbs, layout_cache=cache).backward(go.to(device) * scale)
+        return xg.grad, yg.grad
+
+    dx, dy = grads(1)
+    again = grads(1)
+    assert torch.equal(dx, again[0]) and torch.equal(dy, again[1])
+    doubled = grads(2)
+    assert torch.equal(doubled[0], dx * 2) and torch.equal(doubled[1], dy * 2)
+    assert int(cache["grad_lines_error"][0].item()) == 0
+    b = 5
+    sl = lambda lay, t: t[int(lay[:b].sum()):int(lay[:b + 1].sum())]
+    x64, y64 = sl(lx, x).double().requires_grad_(True), sl(ly, y).double().requires_grad_(True)
+    ref = orc.matmul(x64, lx[b:b + 1].numpy(), y64, ly[b:b + 1].numpy(), lo[b:b + 1].numpy(), sbs,
+                     acc_dtype=torch.float64)
+    ref.backward(sl(lo, go).double())
+    assert_close(sl(lx, dx), x64.grad, 2e-2, "config 2 dX, batch 5")
+    assert_close(sl(ly, dy), y64.grad, 2e-2, "config 2 dY, batch 5")

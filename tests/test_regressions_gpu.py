@@ -263,3 +263,47 @@ def test_readme_sequence_with_compiled_matmul(device):
     allowed = la[0].repeat_interleave(sbs, 0).repeat_interleave(sbs, 1)
     scores = (qd @ kd.transpose(-1, -2) / math.sqrt(hd)).masked_fill(~allowed, float("-inf"))
     assert_close(dense, torch.softmax(scores, -1) @ vd, 1e-4, "README attention")
+
+
+@pytest.mark.parametrize("limit", [0, 4 << 30])
+def test_attention_backward_of_16_bit_blocks_after_an_fp32_backward_on_the_same_cache(device, limit, monkeypatch):
+    """Only the 16-bit kernels for 64 x 64 blocks write records into the backward's scratch.  An fp32 backward on the
+    same cache and mask must leave nothing behind that a later bf16 backward would take for records: the bf16 call
+    announces ``bwd_scratch_ready == 0`` and gives the bits of a fresh cache; the call after it may reuse its own."""
+    from blksprs_amd import _capi
+    from blksprs_amd.utils import validation
+    monkeypatch.setattr(validation, "_kept_ds_limit", limit)
+    sbs, B, n = 64, 2, 6
+    la = rand_layout((B, n, n), 0.6, 1, ensure_rows=True).to(device)
+    lmask = (la.cpu() & rand_layout((B, n, n), 0.7, 2)).to(device)
+    mask = (torch.rand((int(lmask.sum()), sbs, sbs), generator=torch.Generator().manual_seed(3)) < 0.3).to(device)
+    full = torch.ones((B, n, 1), dtype=torch.bool, device=device)
+    q, k, v, go = (rand_blocks(B * n, sbs, torch.float32, s).to(device) for s in (4, 5, 6, 7))
+
+    def grads(dtype, cache):
+        leaves = [t.to(dtype).requires_grad_(True) for t in (q, k, v)]
+        out = bs.ops.flash_attention(leaves[0], full, leaves[1], full, leaves[2], full, la, sbs, attention_mask=mask,
+                                     sparsity_layout_mask=lmask, layout_cache=cache)
+        return torch.autograd.grad(out, leaves, go.to(dtype))
+
+    expected = grads(torch.bfloat16, {})
+    seen = []
+    real_call = _capi.call
+
+    def spy(name, *args):
+        if name == "bsa_attn_bwd":
+            block = args[0]._obj
+            seen.append((block.dtype, block.bwd_scratch_ready, block.bwd_ds_bytes))
+        return real_call(name, *args)
+
+    monkeypatch.setattr(_capi, "call", spy)
+    shared = {}
+    grads(torch.float32, shared)
+    grads(torch.float32, shared)
+    first = grads(torch.bfloat16, shared)
+    second = grads(torch.bfloat16, shared)
+    torch.cuda.synchronize()
+    assert [s[:2] for s in seen] == [(_capi.F32, 0), (_capi.F32, 0), (_capi.BF16, 0), (_capi.BF16, 1)]
+    assert all((s[2] > 0) == (limit > 0 and s[0] == _capi.BF16) for s in seen)
+    for got in (first, second):
+        assert all(torch.equal(a, b) for a, b in zip(got, expected))
