@@ -53,25 +53,28 @@ constexpr int kDenseRows = 4;  // divides every sbs
 __global__ __launch_bounds__(256) void to_dense_kernel(const u32x4_t *__restrict__ blocks,
                                                        const int64_t *__restrict__ packed,
                                                        u32x4_t *__restrict__ dense, int64_t nnz, int64_t C,
-                                                       int64_t dense_row_vecs, int vec_per_row_log2, int sbs_log2,
-                                                       u32x4_t fill) {
+                                                       int64_t dense_row_vecs, int64_t row_groups,
+                                                       int vec_per_row_log2, int sbs_log2, u32x4_t fill) {
   const int64_t col_vec = (int64_t)blockIdx.y * 256 + threadIdx.x;
   if (col_vec >= dense_row_vecs) return;
-  const int64_t row0 = (int64_t)blockIdx.x * kDenseRows;  // b * R * sbs + row
   const int64_t c = col_vec >> vec_per_row_log2;
   const int64_t q = col_vec & (((int64_t)1 << vec_per_row_log2) - 1);
-  const int64_t e0 = row0 & (((int64_t)1 << sbs_log2) - 1);
-  const int64_t br = row0 >> sbs_log2;  // b * R + r
-  const int64_t idx = packed[br * C + c];
-  const bool active = idx >= 0 && idx < nnz;
-  u32x4_t v[kDenseRows];
+  // a launch holds fewer than 2^32 threads: beyond 2^23 groups of rows a workgroup takes several
+  for (int64_t group = blockIdx.x; group < row_groups; group += gridDim.x) {
+    const int64_t row0 = group * kDenseRows;  // b * R * sbs + row
+    const int64_t e0 = row0 & (((int64_t)1 << sbs_log2) - 1);
+    const int64_t br = row0 >> sbs_log2;  // b * R + r
+    const int64_t idx = packed[br * C + c];
+    const bool active = idx >= 0 && idx < nnz;
+    u32x4_t v[kDenseRows];
 #pragma unroll
-  for (int i = 0; i < kDenseRows; ++i) {
-    v[i] = fill;
-    if (active) v[i] = blocks[(((idx << sbs_log2) + e0 + i) << vec_per_row_log2) + q];
+    for (int i = 0; i < kDenseRows; ++i) {
+      v[i] = fill;
+      if (active) v[i] = blocks[(((idx << sbs_log2) + e0 + i) << vec_per_row_log2) + q];
+    }
+#pragma unroll
+    for (int i = 0; i < kDenseRows; ++i) __builtin_nontemporal_store(v[i], dense + (row0 + i) * dense_row_vecs + col_vec);
   }
-#pragma unroll
-  for (int i = 0; i < kDenseRows; ++i) __builtin_nontemporal_store(v[i], dense + (row0 + i) * dense_row_vecs + col_vec);
 }
 
 // layout[b][r][c] = 1 if the sbs x sbs block (r, c) of dense[b] holds an element != 0.  One workgroup owns
@@ -283,9 +286,13 @@ extern "C" int bsa_to_dense(const void *blocks, const int64_t *packed, void *den
   const int64_t dense_row_vecs = C * vec_per_row;
   const int64_t row_groups = B * R * sbs / kDenseRows;
   const int64_t col_groups = bsa::cdiv(dense_row_vecs, 256);
-  BSA_REQUIRE(row_groups < 0x7fffffffLL && col_groups <= 65535, "bsa_to_dense: dense array too large for one launch");
-  to_dense_kernel<<<dim3((unsigned)row_groups, (unsigned)col_groups), 256, 0, bsa::as_stream(stream)>>>(
-      static_cast<const u32x4_t *>(blocks), packed, static_cast<u32x4_t *>(dense), nnz, C, dense_row_vecs,
+  BSA_REQUIRE(col_groups <= 65535, "bsa_to_dense: dense rows too long for one launch");
+  // fewer than 2^32 threads per launch (HIP refuses more): the workgroups of a column stride over the rows
+  int64_t grid_rows = ((int64_t)1 << 23) / col_groups;
+  if (grid_rows < 1) grid_rows = 1;
+  if (grid_rows > row_groups) grid_rows = row_groups;
+  to_dense_kernel<<<dim3((unsigned)grid_rows, (unsigned)col_groups), 256, 0, bsa::as_stream(stream)>>>(
+      static_cast<const u32x4_t *>(blocks), packed, static_cast<u32x4_t *>(dense), nnz, C, dense_row_vecs, row_groups,
       ilog2(vec_per_row), ilog2(sbs), fill);
   return bsa::check_launch("to_dense_kernel");
 }
@@ -324,7 +331,7 @@ extern "C" int bsa_transpose_blocks(const void *blocks, const int64_t *coords, c
   BSA_REQUIRE(coords && packed && out && (nnz_in == 0 || blocks), "bsa_transpose_blocks: NULL pointer");
   const int tiles = sbs <= 64 ? 1 : sbs / 64;
   const int64_t grid = nnz_out * tiles * tiles;
-  BSA_REQUIRE(grid < 0x7fffffffLL, "bsa_transpose_blocks: too many tiles");
+  BSA_REQUIRE(grid < ((int64_t)1 << 24), "bsa_transpose_blocks: too many tiles for one launch (2^24 at most)");
   hipStream_t s = bsa::as_stream(stream);
   if (elem_size == 2 && sbs >= 64 && aligned16(blocks) && aligned16(out)) {
     transpose_blocks16_kernel<<<(unsigned)grid, 256, 0, s>>>(static_cast<const uint16_t *>(blocks), coords, packed,
