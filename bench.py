@@ -40,32 +40,122 @@ PEAK_HBM_GBS = 8000.0
 PEAK_MFMA_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}
 
 
-# HBM bytes per launch of the dominant kernel: FETCH_SIZE and WRITE_SIZE (KiB per dispatch) from the rocprofv3
-# --pmc runs summarised under profiles/ (one file per kernel and configuration), scaled by what the same
-# counters read for a plain copy kernel of known size (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).  FETCH_SIZE counts
-# what leaves an L2, so reads served by the memory-side cache are included.  Not re-measured by this script.
-TRAFFIC_KIB = {  # config: (FETCH_SIZE, WRITE_SIZE)
-    "c1": (616.2, 476.0),
-    "c2": (338582.0, 514960.1),
-    "c3": (148153.3, 296259.0),
-    "c4": (238469.4, 133139.0),
-    "c5": (28438.4, 143960.0),
-    "c3bwd": (369125.1, 296130.4),
-    "a1": (38057.2, 4160.0),
-    "v1": (66312.1, 129576.0),
-    "v2": (66851.5, 524499.4),
-    "t1": (67086.4, 129576.0),
-    "l1": (262170.4, 68.6),
-    "r1": (64865.6, 8192.0),
-    "r2": (66875.5, 129576.0),
-}
+# HBM bytes per step: FETCH_SIZE and WRITE_SIZE (KiB per dispatch, summed over the kernels of one step) from the
+# rocprofv3 --pmc runs summarised under profiles/ (one text file per configuration; the figures this script uses
+# are collected in profiles/traffic.json, which `bench.py --summarise DIR --config X` writes from rocprofv3's output
+# together with the text summary), scaled by what the same counters read for a plain copy kernel of known size
+# (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).  FETCH_SIZE counts what leaves an L2, so reads served by the memory-side
+# cache are included.  Not re-measured by a timing run of this script.
+TRAFFIC_FILE = ROOT / "profiles" / "traffic.json"
+FETCH_SCALE, WRITE_SCALE = 2.0, 1.0
 
 
 def traffic_bytes(config):
-    if config not in TRAFFIC_KIB:
+    try:
+        entry = json.loads(TRAFFIC_FILE.read_text()).get(config)
+    except (OSError, ValueError):
         return None
-    fetch, write = TRAFFIC_KIB[config]
-    return int((2.0 * fetch + 1.0 * write) * 1024)
+    if not entry or entry.get("fetch_kib") is None or entry.get("write_kib") is None:
+        return None
+    return int((FETCH_SCALE * entry["fetch_kib"] + WRITE_SCALE * entry["write_kib"]) * 1024)
+
+
+# file stem of the summary of a configuration under profiles/: the kernel(s) and the workload
+PROFILE_STEMS = {
+    "c1": "matmul_mfma_kernel_c1_fp32_matmul",
+    "c2": "matmul_rows_kernel_c2_bf16_matmul",
+    "c2bwd": "matmul_lines_kernel_c2bwd_bf16_matmul_backward",
+    "c3": "softmax_fwd_kernel_c3_fp32_softmax",
+    "c3bwd": "softmax_bwd_kernel_c3bwd_fp32_softmax_backward",
+    "c4": "attn_fwd_mfma_kernel_c4_bf16_attention_forward",
+    "c4cl": "attn_fwd_mfma_kernel_c4cl_bf16_attention_forward_causal_lengths",
+    "c4bwd": "attn_kernels_c4_bf16_attention_forward_backward",
+    "c5": "matmul_small16_kernel_c5_fp16_sbs16",
+    "a1": "attn_f32mma_kernels_a1_fp32_reference_benchmark",
+    "a1bwd": "attn_f32mma_kernels_a1bwd_fp32_reference_benchmark_backward",
+    "m32": "matmul_mfma_kernel_m32_bf16_sbs32",
+    "m128": "matmul_mfma_kernel_m128_bf16_sbs128",
+    "mf32": "matmul_mfma_kernel_mf32_fp32_sbs64",
+    "v1": "to_sparse_kernel_v1_bf16_to_sparse",
+    "v2": "to_dense_kernel_v2_bf16_to_dense",
+    "t1": "transpose_blocks16_kernel_t1_bf16_transpose",
+    "l1": "layout_from_dense_kernel_l1_bf16_build_sparsity_layout",
+    "r1": "row_reduce_kernel_r1_bf16_row_wise_sum",
+    "r2": "row_add_kernel_r2_bf16_row_wise_add",
+}
+# kernels of this library by a piece of their name (rocprofv3 reports everything the process launches)
+LIBRARY_KERNELS = ("matmul_", "softmax_", "attn_", "to_sparse", "to_dense", "transpose_blocks", "layout_from_dense",
+                   "row_reduce", "row_add", "lines_", "rows_records", "lut_", "packed", "records_kernel")
+
+
+def summarise_profile(directory, config, note):
+    """Turns rocprofv3's output for one configuration into the text summary under profiles/ and the entry of
+    profiles/traffic.json.  ``directory`` holds one sub-directory per run of the SAME command (`python3 bench.py
+    --config X --steps S --warmup W --no-cpu-baseline`): ``trace`` (--kernel-trace --stats) and any number of
+    counter runs (--pmc ...), among them FETCH_SIZE and WRITE_SIZE; each sub-directory may hold a file ``command``
+    with the full command line, which is quoted.  Durations are averages over all dispatches, counters medians
+    per dispatch (the first dispatches of a run may do one-off work)."""
+    import collections
+    import glob
+    import sqlite3
+    import statistics
+
+    directory = Path(directory)
+    lines = [f"# configuration {config} of bench.py: rocprofv3 (ROCm 7.2) on one MI355X, one run per counter set, "
+             f"each run the full command shown; durations in microseconds, counters are medians per dispatch.",
+             f"# FETCH_SIZE / WRITE_SIZE are in KiB as reported; calibration against a plain copy kernel of known "
+             f"size: FETCH_SIZE x {FETCH_SCALE}, WRITE_SIZE x {WRITE_SCALE} give bytes."]
+    if note:
+        lines.append("# " + note)
+    step_kernels, counters = {}, collections.defaultdict(dict)
+    for sub in sorted((p for p in directory.iterdir() if p.is_dir()), key=lambda p: (p.name != "trace", p.name)):
+        dbs = sorted(glob.glob(str(sub / "**" / "*_results.db"), recursive=True))
+        if not dbs:
+            continue
+        command = (sub / "command").read_text().strip() if (sub / "command").exists() else f"(run {sub.name})"
+        lines.append("# " + command)
+        cur = sqlite3.connect(dbs[0]).cursor()
+        if sub.name == "trace":
+            rows = cur.execute("select name, count(*), avg(duration), min(duration), max(duration) from kernels "
+                               "group by name order by sum(duration) desc").fetchall()
+            for name, n, avg, lo, hi in rows:
+                if any(k in name for k in LIBRARY_KERNELS):
+                    step_kernels[name] = {"n": n, "avg_us": round(avg / 1e3, 1)}
+                    lines.append(f"  kern {name[:110]:110s} n={n} avg={avg / 1e3:.1f}us min={lo / 1e3:.1f} max={hi / 1e3:.1f}")
+        else:
+            raw = cur.execute("select kernel_name, counter_name, value from counters_collection").fetchall()
+            grouped = collections.defaultdict(list)
+            for kernel, counter, value in raw:
+                grouped[(kernel, counter)].append(value)
+            per_kernel = collections.defaultdict(dict)
+            for (kernel, counter), values in grouped.items():
+                if any(k in kernel for k in LIBRARY_KERNELS):
+                    per_kernel[kernel][counter] = round(statistics.median(values), 1)
+                    counters[kernel][counter] = per_kernel[kernel][counter]
+            for kernel in sorted(per_kernel):
+                lines.append(f"  pmc {kernel[:110]:110s} {per_kernel[kernel]}")
+    # the kernels of a step: those that ran about once per step or more (one-off table builders ran a few times)
+    most = max((k["n"] for k in step_kernels.values()), default=0)
+    per_step = {name: k for name, k in step_kernels.items() if k["n"] * 4 >= most}
+    fetch = sum(counters[name].get("FETCH_SIZE", 0.0) for name in per_step if name in counters)
+    write = sum(counters[name].get("WRITE_SIZE", 0.0) for name in per_step if name in counters)
+    have = any("FETCH_SIZE" in counters[name] for name in per_step if name in counters)
+    lines.append(f"# kernels of one step: {len(per_step)}; sum of their average durations "
+                 f"{sum(k['avg_us'] for k in per_step.values()):.1f} us; FETCH_SIZE {fetch:.1f} KiB + WRITE_SIZE "
+                 f"{write:.1f} KiB per step = {(FETCH_SCALE * fetch + WRITE_SCALE * write) * 1024 / 1e6:.1f} MB")
+    stem = PROFILE_STEMS.get(config, config)
+    out = ROOT / "profiles" / (stem + ".txt")
+    out.parent.mkdir(exist_ok=True)
+    out.write_text("\n".join(lines) + "\n")
+    try:
+        table = json.loads(TRAFFIC_FILE.read_text())
+    except (OSError, ValueError):
+        table = {}
+    table[config] = {"profile": out.name, "fetch_kib": round(fetch, 1) if have else None,
+                     "write_kib": round(write, 1) if have else None,
+                     "kernels": {name[:100]: {**k, **counters.get(name, {})} for name, k in per_step.items()}}
+    TRAFFIC_FILE.write_text(json.dumps(table, indent=1, sort_keys=True) + "\n")
+    print(f"wrote {out} and {TRAFFIC_FILE}")
 
 
 def log(*a):
@@ -304,7 +394,10 @@ def matmul_workload(name, B, n, sbs, dtype, density, ensure_rows, value_scale, d
         kernel = "matmul_rows_kernel" if sbs == 64 and dtype != torch.float32 else "matmul_mfma_kernel"
     else:
         kernel = "matmul_small16_kernel" if dtype != torch.float32 else "matmul_small_kernel"
-    return dict(step=step, flops=flops, alg_bytes=alg_bytes, dtype=dt_name, bound="hbm", cpu_baseline=cpu_baseline,
+    # 172 FLOP per byte at sbs 64 and 25 % density: below the balance of the 16-bit matrix cores (312 FLOP/B), above
+    # that of the fp32 ones (20 FLOP/B): fp32 products of large problems are bound by the fp32 matrix-core peak
+    bound = "mfma" if dtype == torch.float32 and sbs >= 32 and B * n * sbs >= 16 * 4096 else "hbm"
+    return dict(step=step, flops=flops, alg_bytes=alg_bytes, dtype=dt_name, bound=bound, cpu_baseline=cpu_baseline,
                 check=check, kernel=kernel,
                 config={"workload": name, "B": B, "M": n * sbs, "K": n * sbs, "N": n * sbs,
                         "sparsity_block_size": sbs, "density": density, "nnz_x": nnz_x, "nnz_y": nnz_y,
@@ -563,7 +656,7 @@ def movement_workload(dev, which):
                         "sparsity_block_size": sbs, "active_blocks": nnz})
 
 
-def attention_workload(dev, backward):
+def attention_workload(dev, backward, native_causal=False):
     import blksprs_amd as bs
     from oracle import blksprs_oracle as orc
 
@@ -585,11 +678,17 @@ def attention_workload(dev, backward):
     cache = {}
     if backward:
         q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
-    bs.ops.flash_attention(q, full, k, full, v, full, lad, sbs, attention_mask=mask, sparsity_layout_mask=lmd,
-                           layout_cache=cache)
+    # the same causal attention two ways (blksprs/ops/flash_attention.py:1128-1142): an explicit mask tensor (the
+    # headline), or the native predicate on causal_lengths, without any mask tensor
+    lengths = torch.full((BH,), n * sbs, dtype=torch.int64, device=dev)
+    if native_causal:
+        mask_args = dict(causal_lengths=lengths)
+    else:
+        mask_args = dict(attention_mask=mask, sparsity_layout_mask=lmd)
+    bs.ops.flash_attention(q, full, k, full, v, full, lad, sbs, layout_cache=cache, **mask_args)
     fwd_flops = nnz * 4.0 * sbs * sbs * (nh * sbs)
     flops = fwd_flops * (3.5 if backward else 1.0)
-    alg_bytes = 4 * BH * n * nh * sbs * sbs * 2 + int(lmask.sum()) * sbs * sbs
+    alg_bytes = 4 * BH * n * nh * sbs * sbs * 2 + (0 if native_causal else int(lmask.sum()) * sbs * sbs)
     # pairs in which some score survives the mask: the others are in the layout (and in the metric's flop count,
     # which follows the reference, whose kernels visit them) but the kernels here neither fetch nor compute them
     live_pairs = int((la & torch.ones((n, n), dtype=torch.bool).tril()).sum())
@@ -598,8 +697,7 @@ def attention_workload(dev, backward):
     bs.utils.disable_validation()
 
     def step():
-        o = bs.ops.flash_attention(q, full, k, full, v, full, lad, sbs, attention_mask=mask,
-                                   sparsity_layout_mask=lmd, layout_cache=cache)
+        o = bs.ops.flash_attention(q, full, k, full, v, full, lad, sbs, layout_cache=cache, **mask_args)
         if backward:
             q.grad = k.grad = v.grad = None
             o.backward(d_o)
@@ -610,8 +708,12 @@ def attention_workload(dev, backward):
         cnt = int(lmask[:1].sum())
         fl = full[:1].cpu().numpy()
         leaves = [t[:n * nh].detach().float().cpu().requires_grad_(backward) for t in (q, k, v)]
-        want = orc.flash_attention(leaves[0], fl, leaves[1], fl, leaves[2], fl, la[:1].numpy(), sbs,
-                                   mask=mask[:cnt].cpu(), layout_mask=lmask[:1].numpy())
+        if native_causal:
+            want = orc.flash_attention(leaves[0], fl, leaves[1], fl, leaves[2], fl, la[:1].numpy(), sbs,
+                                       causal_lengths=lengths[:1].cpu())
+        else:
+            want = orc.flash_attention(leaves[0], fl, leaves[1], fl, leaves[2], fl, la[:1].numpy(), sbs,
+                                       mask=mask[:cnt].cpu(), layout_mask=lmask[:1].numpy())
         close = lambda got, ref: bool(torch.allclose(got[:n * nh].detach().float().cpu(), ref, rtol=2e-2, atol=2e-2))
         ok = close(step(), want.detach())
         if backward:
@@ -636,9 +738,11 @@ def attention_workload(dev, backward):
                 check=check, executed_flops=flops * live_pairs / nnz,
                 kernel="attn_fwd_mfma_kernel" if not backward else
                 "attn_fwd_mfma_kernel + attn_bwd_delta_kernel + attn_bwd_kv8_walk_kernel + attn_bwd_dq_kernel (one step; the mask_dead / records / order kernels ran once, in the warm-up)",
-                config={"workload": "c4_flash_attention_bf16" + ("_fwd_bwd" if backward else "_fwd"),
+                config={"workload": "c4_flash_attention_bf16" + ("_fwd_bwd" if backward else "_fwd")
+                        + ("_causal_lengths" if native_causal else ""),
                         "batch_heads": BH, "seq": n * sbs, "head_dim": nh * sbs, "sparsity_block_size": sbs,
-                        "layout_blocks": nnz, "mask": "explicit causal blocks"})
+                        "layout_blocks": nnz,
+                        "mask": "native causal predicate (causal_lengths)" if native_causal else "explicit causal blocks"})
 
 
 def reference_attention_benchmark(dev, m=2048, backward=False):
@@ -741,6 +845,17 @@ def make_workload(name, dev):
     if name == "c2bwd":
         return matmul_workload("c2_matmul_bf16_backward", 16, 64, 64, torch.bfloat16, 0.25, False, 1.0 / 64.0, dev,
                                16, backward=True, check_batch=3)
+    # the C2 problem (4096^3, 25 % density, product layout) off the one shape the row kernel takes: other block
+    # sizes and fp32 run on the tile kernel (blksprs/ops/matmul.py:148-253 serves every dtype and block size)
+    if name == "m32":
+        return matmul_workload("c2_problem_bf16_sbs32", 16, 128, 32, torch.bfloat16, 0.25, False, 1.0 / 64.0, dev, 4,
+                               check_batch=3)
+    if name == "m128":
+        return matmul_workload("c2_problem_bf16_sbs128", 16, 32, 128, torch.bfloat16, 0.25, False, 1.0 / 64.0, dev, 4,
+                               check_batch=3)
+    if name == "mf32":
+        return matmul_workload("c2_problem_fp32_sbs64", 16, 64, 64, torch.float32, 0.25, False, 1.0 / 64.0, dev, 4,
+                               check_batch=3)
     if name == "c3":
         return softmax_workload(dev)
     if name == "c3bwd":
@@ -749,6 +864,10 @@ def make_workload(name, dev):
         return attention_workload(dev, backward=False)
     if name == "c4bwd":
         return attention_workload(dev, backward=True)
+    if name == "c4cl":
+        return attention_workload(dev, backward=False, native_causal=True)
+    if name == "c4clbwd":
+        return attention_workload(dev, backward=True, native_causal=True)
     if name == "a1":
         return reference_attention_benchmark(dev)
     if name == "a1bwd":
@@ -772,10 +891,10 @@ def make_workload(name, dev):
     raise SystemExit(f"unknown config {name}")
 
 
-CONFIGS = ["a1", "a1bwd", "c1", "c2", "c2bwd", "c3", "c3bwd", "c4", "c4bwd", "c5", "t1", "l1", "r1", "r2", "p1", "v1", "v2"]
+CONFIGS = ["a1", "a1bwd", "c1", "c2", "c2bwd", "c3", "c3bwd", "c4", "c4bwd", "c4cl", "c4clbwd", "c5", "m32", "m128", "mf32", "t1", "l1", "r1", "r2", "p1", "v1", "v2"]
 # the configurations a default run times behind the headline one, with fewer steps (their roofline objects ride
 # along in the same JSON line so that they are timed by whoever runs the script, not quoted from elsewhere)
-COMPANIONS = ["c2bwd", "c4", "c4bwd", "c3", "c5"]
+COMPANIONS = ["c2bwd", "c4", "c4cl", "c4bwd", "c3", "c5"]
 
 
 def measure(config, dev, steps, warmup, scratch):
@@ -849,6 +968,14 @@ def measured_ceilings(dev):
     dst = torch.empty_like(src)
     ms = timed(lambda: dst.copy_(src), 10)
     out["copy_2gib_read_plus_write_gbs"] = round(2.0 * src.numel() / (ms * 1e-3) / 1e9, 1)
+    # one direction at a time over the same 2 GiB: a kernel that only reads (this library's layout builder: every
+    # byte once, one byte written per 8 KiB read) and one that only writes (torch's fill)
+    import blksprs_amd as bs
+    dense = src.view(torch.bfloat16).view(16, 8192, 8192)
+    ms = timed(lambda: bs.layouting.build_sparsity_layout(dense, 64), 10)
+    out["read_2gib_gbs"] = round(src.numel() / (ms * 1e-3) / 1e9, 1)
+    ms = timed(lambda: dst.zero_(), 10)
+    out["write_2gib_gbs"] = round(dst.numel() / (ms * 1e-3) / 1e9, 1)
     return out
 
 
@@ -860,7 +987,16 @@ def main():
     ap.add_argument("--config", default=None, choices=CONFIGS,
                     help="one configuration only; without it: c2 as the headline, then " + ", ".join(COMPANIONS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--summarise", default=None, metavar="DIR",
+                    help="no timing: write the summary under profiles/ (and the entry of profiles/traffic.json) of "
+                         "--config from rocprofv3's output in DIR (sub-directories trace, fetch, write, ...)")
+    ap.add_argument("--note", default="", help="a line of text for the summary written by --summarise")
     args = ap.parse_args()
+    if args.summarise:
+        if not args.config:
+            raise SystemExit("--summarise needs --config")
+        summarise_profile(args.summarise, args.config, args.note)
+        return
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         raise SystemExit("bench.py measures one GPU: the block-sparse path has no cross-GPU step in this build "
                          "(it would shard on the batch dimension with no collective); run with --gpus 1")

@@ -759,9 +759,12 @@ __device__ __forceinline__ void attn_bwd_kv8_walk(const bsa_attn_args &a, char *
   // knows of makes it wait for everything in flight (vmcnt(0)) at the next join, the copies included, which would
   // put the whole latency of the next tile in front of this tile's products.  Called on the straight path only (a
   // request in a branch of its own would let the compiler move the register at the join, with the load in flight);
-  // when there is no next tile the record is the last valid one and the value is not used.
+  // when there is no next tile the value is not used: the record is then the last valid one, or the header of a next
+  // key block without tiles, whose record fields are -1 (clamped: query block -1 of batch entry 0 would be a read in
+  // front of the array).
   auto request_stat = [&](int rec, int64_t batch) {
-    const int64_t qrow = batch * a.nq + __builtin_amdgcn_readlane(rec, 0);
+    const int qb_of_rec = __builtin_amdgcn_readlane(rec, 0);
+    const int64_t qrow = batch * a.nq + (qb_of_rec < 0 ? 0 : qb_of_rec);
     const float *src = (wave == 5 ? a.delta : a.lse) + qrow * kSbs + lane;
     asm volatile("global_load_dword %0, %1, off" : "+v"(stat) : "v"(src) : "memory");
   };

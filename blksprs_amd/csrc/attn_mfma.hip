@@ -363,7 +363,11 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_mfma_kernel(bsa_attn_
           }
           cc = 1.f;
         }
-        if (causal) {
+        // most tiles lie where the predicate holds for every score of the wave's 32 rows (every key of the tile at or
+        // before the wave's first query, and the wave's last query inside the sequence): one test for the wave
+        // skips the selects
+        const int q_wave_first = (int)qb * kSbs + 32 * (wave & 1);
+        if (causal && (kb * kSbs + kSbs - 1 > q_wave_first || q_wave_first + 31 >= seq_len)) {
           const int kbase = kb * kSbs + 4 * kg;
           const bool row_off = qpos >= seq_len;
   #pragma unroll

@@ -1,6 +1,6 @@
 """Operations on compressed block-sparse tensors (the MI355X compute path)."""
 
-from . import library, misc
+from . import misc
 from .conversion import from_blksprs, to_blksprs, to_dense, to_dense_shaped, to_sparse, to_sparse_shaped
 from .flash_attention import flash_attention, flash_attention_build_layout_cache
 from .matmul import matmul
@@ -11,7 +11,6 @@ __all__ = [
     "flash_attention",
     "flash_attention_build_layout_cache",
     "from_blksprs",
-    "library",
     "matmul",
     "misc",
     "softmax",

@@ -10,6 +10,7 @@ reference are not part of this package.
 
 import ctypes
 import math
+import threading
 from numbers import Real
 
 import torch
@@ -248,6 +249,9 @@ def flash_attention_build_layout_cache(attention_layout: Tensor,
     return finalize_layout_cache(layout_cache)
 
 
+_LENGTHS_SEEN = threading.local()
+
+
 def _normalise_causal_lengths(causal_lengths: Tensor | None, n_batches: int, q_length: int, k_length: int,
                               device: torch.device) -> Tensor | None:
     if causal_lengths is None:
@@ -262,9 +266,17 @@ def _normalise_causal_lengths(causal_lengths: Tensor | None, n_batches: int, q_l
         raise TypeError("causal_lengths must use an integral dtype")
     validate_device(causal_lengths, torch.empty(0, device=device))
     validate_shape(causal_lengths, (n_batches,), "causal_lengths")
-    if torch.any(causal_lengths < 0) or torch.any(causal_lengths > q_length):
-        raise ValueError(f"causal_lengths values must be between zero and {q_length}")
-    return ensure_contiguous(causal_lengths.to(dtype=torch.int64))
+    # The range check reads the device (two waits of the host): its verdict on one tensor is remembered, per
+    # thread, for as long as the tensor's version counter says that nothing was written to it in place (the
+    # reference checks on every call, blksprs/ops/flash_attention.py:239-241; a write through .data goes unseen,
+    # as for the facts kept per mask).
+    seen = getattr(_LENGTHS_SEEN, "last", None)
+    key = (causal_lengths._version, int(q_length)) if not torch.is_inference(causal_lengths) else None
+    if seen is None or seen[0] is not causal_lengths or seen[1] != key or key is None:
+        if torch.any(causal_lengths < 0) or torch.any(causal_lengths > q_length):
+            raise ValueError(f"causal_lengths values must be between zero and {q_length}")
+        _LENGTHS_SEEN.last = (causal_lengths, key, ensure_contiguous(causal_lengths.to(dtype=torch.int64)))
+    return _LENGTHS_SEEN.last[2]
 
 
 def _as_index(t: Tensor | None, dtype: torch.dtype) -> Tensor | None:

@@ -9,6 +9,7 @@ transposed inside the kernel instead of materialising transposed copies.
 
 import ctypes
 import os
+import warnings
 
 import torch
 from torch import Tensor
@@ -145,6 +146,21 @@ _L2_BYTES = 4 << 20  # one XCD's L2
 _MAX_PART_BLOCKS = 64  # a workgroup of the row kernel takes at most this many output blocks (one mask bit each)
 
 
+def _measurement_knob(name: str, default: int, lowest: int, highest: int) -> int:
+    """An integer from the environment for measurements of the row kernel's work order, clamped to its legal
+    range; a value that is not a number is ignored with a warning (a value left over in the environment must not
+    turn every product into an error)."""
+    raw = os.environ.get(name)
+    if raw is None:
+        return default
+    try:
+        value = int(raw)
+    except ValueError:
+        warnings.warn(f"{name}={raw!r} is not an integer: ignored")
+        return default
+    return min(max(value, lowest), highest)
+
+
 def _row_parts_log2(n_rows: int, rows_per_batch: int, n_cols: int, n_blocks_y: int, n_blocks_o: int,
                     block_bytes: int) -> int | None:
     """Into how many runs (as log2) the row kernel cuts the output blocks of a row; ``None`` when a row does not
@@ -160,9 +176,7 @@ def _row_parts_log2(n_rows: int, rows_per_batch: int, n_cols: int, n_blocks_y: i
     y_bytes_per_entry = n_blocks_y * block_bytes // batches
     blocks_per_row = n_blocks_o // max(n_rows, 1)
     parts_log2 = 1 if y_bytes_per_entry > 4 * _L2_BYTES and blocks_per_row >= 32 else 0
-    forced = os.environ.get("BLKSPRS_AMD_ROW_PARTS_LOG2")  # for measurements
-    if forced is not None:
-        parts_log2 = int(forced)
+    parts_log2 = _measurement_knob("BLKSPRS_AMD_ROW_PARTS_LOG2", parts_log2, 0, 3)
     while parts_log2 <= 3 and -(-n_cols // (1 << parts_log2)) > _MAX_PART_BLOCKS:
         parts_log2 += 1
     return parts_log2 if parts_log2 <= 3 else None
@@ -359,8 +373,8 @@ def matmul_build_layout_cache(layout_cache: dict | None, sparsity_layout_x: Tens
                 # workgroup, no tail of short rows), measured no faster on configuration 2: compute units differ
                 # in speed by +-12 % on equal work, which the hardware's hand-out of many small items evens out
                 # and a static split does not.  Kept switchable for measurements.
-                pair_up = (B * R << parts_log2) >= 1024 and os.environ.get("BLKSPRS_AMD_ROW_PAIRS", "0") == "1"
-                sweep = int(os.environ.get("BLKSPRS_AMD_ROW_SWEEP", _CUS_PER_XCD))  # 0: every part upward
+                pair_up = (B * R << parts_log2) >= 1024 and _measurement_knob("BLKSPRS_AMD_ROW_PAIRS", 0, 0, 1) == 1
+                sweep = _measurement_knob("BLKSPRS_AMD_ROW_SWEEP", _CUS_PER_XCD, 0, 1 << 20)  # 0: every part upward
                 table = _row_work_table(lists.pair_offsets, info_o.row_offsets, R, parts_log2, pair_up,
                                         max_work=K * C, sweep=0 if pair_up else sweep)
                 layout_cache["row_parts_log2"], layout_cache["row_work_table"] = parts_log2, table

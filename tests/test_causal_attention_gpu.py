@@ -77,3 +77,23 @@ def test_window_layout_and_mask_give_local_attention(device):
         scores = (q[b, :length] @ k[b, :length].T) / sbs ** 0.5
         want = torch.softmax(scores.masked_fill(banned, float("-inf")), -1) @ v[b, :length]
         torch.testing.assert_close(out[b, :length], want, rtol=2e-5, atol=2e-5)
+
+
+def test_range_check_of_causal_lengths_follows_changes_in_place(device):
+    """The range check of ``causal_lengths`` (blksprs/ops/flash_attention.py:239-241) reads the device; its verdict
+    on one tensor is remembered while the tensor's version counter stands still, and a change in place is checked
+    again: a tensor that was valid and is then given a length beyond the sequence is refused."""
+    sbs, n = 16, 3
+    layout = torch.ones((1, n, 1), dtype=torch.bool, device=device)
+    attention = torch.ones((1, n, n), dtype=torch.bool, device=device)
+    q = torch.randn((n, sbs, sbs), device=device)
+    lengths = torch.tensor([n * sbs], device=device)
+    call = lambda: bs.ops.flash_attention(q, layout, q, layout, q, layout, attention, sbs, causal_lengths=lengths)
+    first = call()
+    assert torch.equal(call(), first)
+    lengths.add_(1)
+    with pytest.raises(ValueError, match="between zero and"):
+        call()
+    lengths.sub_(2 * sbs)
+    shorter = call()
+    assert torch.all(shorter[n - 1] == 0) and not torch.equal(shorter, first)

@@ -240,31 +240,6 @@ def test_row_work_table_holds_every_part_once_and_keeps_eighths_together():
     assert paired[0::8].tolist() == [4, 0, 3, 1, 2]
 
 
-def test_library_operators_are_registered_with_shape_functions():
-    """The launchers are torch.library operators of the namespace blksprs_amd (the reference registers its own
-    as blksprs::..., blksprs/ops/matmul.py:70): their schemas mutate nothing and their shape functions run on
-    fake tensors, without a device."""
-    from torch._subclasses.fake_tensor import FakeTensorMode
-    ops = torch.ops.blksprs_amd
-    for name in ("matmul_forward", "to_sparse_forward", "to_dense_forward", "softmax_fused_forward",
-                 "softmax_fused_backward"):
-        schema = getattr(ops, name).default._schema
-        assert not schema.is_mutable and len(schema.returns) == 1, name
-    with FakeTensorMode():
-        x = torch.empty((5, 32, 32), dtype=torch.float16, device="meta")
-        y = torch.empty((7, 32, 32), dtype=torch.float16, device="meta")
-        table = torch.empty((9, 2), dtype=torch.int32, device="meta")
-        layout = torch.empty((2, 3, 4), dtype=torch.bool, device="meta")
-        out = ops.matmul_forward(x, y, table, table, 3, 32, False, True)
-        assert out.shape == (3, 32, 32) and out.dtype == torch.float16
-        dense = torch.empty((2, 96, 128), dtype=torch.float16, device="meta")
-        assert ops.to_sparse_forward(dense, table, 32, 5).shape == (5, 32, 32)
-        assert ops.to_dense_forward(x, layout, table, 32, 0.0).shape == (2, 96, 128)
-        xf = torch.empty((5, 32, 32), device="meta")
-        assert ops.softmax_fused_forward(xf, table, 6, 32).shape == xf.shape
-        assert ops.softmax_fused_backward(xf, xf, table, 6, 32).dtype == torch.float32
-
-
 def test_the_limit_on_kept_ds_is_a_process_wide_setting():
     """``bs.utils.set_kept_ds_limit`` is what ``flash_attention``'s backward asks (through ``kept_ds_limit``) before it
     requests room for dS; 0 turns the kept dS off."""
@@ -279,3 +254,23 @@ def test_the_limit_on_kept_ds_is_a_process_wide_setting():
         assert validation.kept_ds_limit() == 1 << 20
     finally:
         bs.utils.set_kept_ds_limit(before)
+
+
+def test_measurement_knobs_are_clamped_and_malformed_values_ignored(monkeypatch):
+    """The environment variables that steer the row kernel's work order for measurements are clamped to their legal
+    range, and a value that is no integer is ignored with a warning instead of failing every product."""
+    import importlib
+    import warnings
+    mm = importlib.import_module("blksprs_amd.ops.matmul")
+    monkeypatch.setenv("BLKSPRS_AMD_ROW_PARTS_LOG2", "-1")
+    assert mm._measurement_knob("BLKSPRS_AMD_ROW_PARTS_LOG2", 1, 0, 3) == 0
+    monkeypatch.setenv("BLKSPRS_AMD_ROW_PARTS_LOG2", "9")
+    assert mm._measurement_knob("BLKSPRS_AMD_ROW_PARTS_LOG2", 1, 0, 3) == 3
+    assert mm._row_parts_log2(1024, 64, 64, 16384, 64512, 8192) == 3
+    monkeypatch.setenv("BLKSPRS_AMD_ROW_PARTS_LOG2", "two")
+    with warnings.catch_warnings(record=True) as caught:
+        warnings.simplefilter("always")
+        assert mm._measurement_knob("BLKSPRS_AMD_ROW_PARTS_LOG2", 1, 0, 3) == 1
+    assert any("not an integer" in str(w.message) for w in caught)
+    monkeypatch.delenv("BLKSPRS_AMD_ROW_PARTS_LOG2")
+    assert mm._measurement_knob("BLKSPRS_AMD_ROW_PARTS_LOG2", 1, 0, 3) == 1

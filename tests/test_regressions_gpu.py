@@ -307,3 +307,30 @@ def test_attention_backward_of_16_bit_blocks_after_an_fp32_backward_on_the_same_
     assert all((s[2] > 0) == (limit > 0 and s[0] == _capi.BF16) for s in seen)
     for got in (first, second):
         assert all(torch.equal(a, b) for a, b in zip(got, expected))
+
+
+def test_operators_under_torch_compile_run_eagerly_with_eager_results(device):
+    """The public operators run eagerly: a compiled caller leaves its graph at each of them and resumes behind it,
+    with the results of eager mode.  ``fullgraph=True`` either gives the same results (torch then treats the
+    operator, which is marked ``torch.compiler.disable``, as an opaque call) or refuses the caller with an error
+    that names the graph break; it never gives other numbers.  (The reference registers its launchers with
+    ``torch.library.triton_op`` and traces through them; here the lookup tables are built and the kernels launched
+    outside any trace.)"""
+    import torch._dynamo
+    sbs = 32
+    layout = rand_layout((2, 3, 3), 0.7, 5, ensure_rows=True).to(device)
+    x = rand_blocks(int(layout.sum()), sbs, torch.float32, 6).to(device)
+
+    def caller(t):
+        return bs.ops.softmax(t * 2.0, layout, sbs) + 1.0
+
+    torch._dynamo.reset()
+    eager = caller(x)
+    assert torch.allclose(torch.compile(caller)(x), eager, rtol=1e-6, atol=1e-6)
+    try:
+        whole = torch.compile(caller, fullgraph=True)(x)
+    except Exception as error:  # the error class differs between torch versions
+        assert any(word in str(error).lower() for word in ("graph break", "fullgraph", "disable")), error
+    else:
+        assert torch.allclose(whole, eager, rtol=1e-6, atol=1e-6)
+    torch._dynamo.reset()

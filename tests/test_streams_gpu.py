@@ -90,30 +90,3 @@ def test_warm_operators_replay_from_a_graph(device):
                 assert torch.equal(a, b)
     finally:
         bs.utils.enable_validation()
-
-
-def test_library_operators_give_what_the_wrappers_give(device):
-    """torch.ops.blksprs_amd.* are the launchers behind the public wrappers, fed from the wrappers' caches."""
-    sbs = 64
-    lx, ly, lo, x, y = _problem(device)
-    ops = torch.ops.blksprs_amd
-    cache = {}
-    expected = bs.ops.matmul(x, lx, y, ly, lo, sbs, layout_cache=cache)
-    got = ops.matmul_forward(x, y, cache["contraction_offsets"], cache["contraction_pairs"],
-                             cache["n_sparse_blocks"], sbs, False, False)
-    assert torch.equal(got, expected)
-    cache = {}
-    dense = bs.ops.to_dense(x, lx, sbs, layout_cache=cache)
-    assert torch.equal(ops.to_dense_forward(x, lx, cache["packed_indices"], sbs, 0.0), dense)
-    cache = {}
-    sparse = bs.ops.to_sparse(dense, lx, sbs, layout_cache=cache)
-    assert torch.equal(ops.to_sparse_forward(dense, cache["layout_indices"], sbs, cache["n_sparse_blocks"]), sparse)
-    cache = {}
-    xf = x.float()
-    soft = bs.ops.softmax(xf, lx, sbs, layout_cache=cache)
-    n_rows = cache["row_offsets"].numel() - 1
-    assert torch.equal(ops.softmax_fused_forward(xf, cache["row_offsets"], n_rows, sbs), soft)
-    g = torch.randn_like(soft)
-    xr = xf.clone().requires_grad_(True)
-    bs.ops.softmax(xr, lx, sbs, layout_cache=cache).backward(g)
-    assert torch.equal(ops.softmax_fused_backward(g, soft, cache["row_offsets"], n_rows, sbs), xr.grad)
