@@ -88,7 +88,7 @@ LIBRARY_KERNELS = ("matmul_", "softmax_", "attn_", "to_sparse", "to_dense", "tra
                    "row_reduce", "row_add", "lines_", "rows_records", "lut_", "packed", "records_kernel")
 
 
-def summarise_profile(directory, config, note):
+def summarise_profile(directory, config, note, side_name=None):
     """Turns rocprofv3's output for one configuration into the text summary under profiles/ and the entry of
     profiles/traffic.json.  ``directory`` holds one sub-directory per run of the SAME command (`python3 bench.py
     --config X --steps S --warmup W --no-cpu-baseline`): ``trace`` (--kernel-trace --stats) and any number of
@@ -143,9 +143,13 @@ def summarise_profile(directory, config, note):
     lines.append(f"# kernels of one step: {len(per_step)}; sum of their average durations "
                  f"{sum(k['avg_us'] for k in per_step.values()):.1f} us; FETCH_SIZE {fetch:.1f} KiB + WRITE_SIZE "
                  f"{write:.1f} KiB per step = {(FETCH_SCALE * fetch + WRITE_SCALE * write) * 1024 / 1e6:.1f} MB")
-    stem = PROFILE_STEMS.get(config, config)
+    stem = side_name or PROFILE_STEMS.get(config, config)
     out = ROOT / "profiles" / (stem + ".txt")
     out.parent.mkdir(exist_ok=True)
+    if side_name:  # a side experiment (runs that differ in an option): the runs as they are, no totals, no table entry
+        out.write_text("\n".join(lines[:-1]) + "\n")
+        print(f"wrote {out}")
+        return
     out.write_text("\n".join(lines) + "\n")
     try:
         table = json.loads(TRAFFIC_FILE.read_text())
@@ -338,6 +342,15 @@ def matmul_workload(name, B, n, sbs, dtype, density, ensure_rows, value_scale, d
         f"algorithmic bytes={alg_bytes / 1e6:.1f}MB; first call {first_ms:.2f} ms, lookup tables of a fresh cache "
         f"{lut_ms:.2f} ms with {lut_syncs} host syncs")
 
+    generations = ROW_GENERATIONS if not backward and cache["plan"].row_records is not None else None
+    if generations is not None:
+        # measurement only: the launch ends after the first entries of every XCD's list (32 compute units per XCD
+        # take 32 entries at a time; entry k of XCD c sits at position 8 k + c), the rest of the output is not
+        # computed, so the result is not checked and the rates of the line mean nothing: the counters per launch do
+        plan = cache["plan"]
+        plan.row_records = plan.row_records[:256 * generations * plan.row_items]
+        log(f"[{name}] row kernel limited to {plan.row_records.size(0)} of its work table's entries")
+
     bs.utils.disable_validation()
     if backward:
         xg, yg = x.requires_grad_(True), y.requires_grad_(True)
@@ -397,6 +410,8 @@ def matmul_workload(name, B, n, sbs, dtype, density, ensure_rows, value_scale, d
     # 172 FLOP per byte at sbs 64 and 25 % density: below the balance of the 16-bit matrix cores (312 FLOP/B), above
     # that of the fp32 ones (20 FLOP/B): fp32 products of large problems are bound by the fp32 matrix-core peak
     bound = "mfma" if dtype == torch.float32 and sbs >= 32 and B * n * sbs >= 16 * 4096 else "hbm"
+    if generations is not None:
+        check = lambda: None
     return dict(step=step, flops=flops, alg_bytes=alg_bytes, dtype=dt_name, bound=bound, cpu_baseline=cpu_baseline,
                 check=check, kernel=kernel,
                 config={"workload": name, "B": B, "M": n * sbs, "K": n * sbs, "N": n * sbs,
@@ -897,6 +912,9 @@ CONFIGS = ["a1", "a1bwd", "c1", "c2", "c2bwd", "c3", "c3bwd", "c4", "c4bwd", "c4
 COMPANIONS = ["c2bwd", "c4", "c4cl", "c4bwd", "c3", "c5"]
 
 
+ROW_GENERATIONS = None  # --row-generations
+
+
 def measure(config, dev, steps, warmup, scratch):
     """Builds the workload, checks a sample against the oracle, times it.  Returns (workload, result dict)."""
     import blksprs_amd as bs
@@ -990,18 +1008,26 @@ def main():
     ap.add_argument("--summarise", default=None, metavar="DIR",
                     help="no timing: write the summary under profiles/ (and the entry of profiles/traffic.json) of "
                          "--config from rocprofv3's output in DIR (sub-directories trace, fetch, write, ...)")
+    ap.add_argument("--row-generations", type=int, default=None, metavar="G",
+                    help="measurement of the row kernel's memory traffic: launch only the first 32 G entries of every "
+                         "XCD's work list (forward matmul configurations on the row kernel; result unchecked)")
+    ap.add_argument("--summary-name", default=None, metavar="STEM",
+                    help="with --summarise: write profiles/STEM.txt (the runs of a side experiment as they are) and "
+                         "leave profiles/traffic.json alone")
     ap.add_argument("--note", default="", help="a line of text for the summary written by --summarise")
     args = ap.parse_args()
     if args.summarise:
         if not args.config:
             raise SystemExit("--summarise needs --config")
-        summarise_profile(args.summarise, args.config, args.note)
+        summarise_profile(args.summarise, args.config, args.note, args.summary_name)
         return
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         raise SystemExit("bench.py measures one GPU: the block-sparse path has no cross-GPU step in this build "
                          "(it would shard on the batch dimension with no collective); run with --gpus 1")
     if not torch.cuda.is_available():
         raise SystemExit("bench.py needs a GPU (the product has no CPU path)")
+    global ROW_GENERATIONS
+    ROW_GENERATIONS = args.row_generations
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     scratch = torch.empty(FLUSH_BYTES, dtype=torch.uint8, device=dev)

@@ -104,3 +104,28 @@ def test_bad_arguments_of_the_neighbouring_entry_points_are_rejected_on_the_host
     assert lib.bsa_attn_mask_dead(0, 1, 32, 0, 0) == -1 and b"64 x 64" in lib.bsa_last_error()
     assert lib.bsa_attn_mask_dead(0, 1, 64, 0, 0) == -1 and b"NULL" in lib.bsa_last_error()
     assert lib.bsa_attn_mask_dead(0, 0, 64, 0, 0) == 0
+
+
+def test_bad_arguments_of_the_line_kernel_are_rejected_on_the_host():
+    """bsa_matmul_lines / bsa_matmul_lines_parts check their argument block before anything is launched."""
+    import ctypes
+    lib = _capi.load()
+    a = _capi.LinesArgs()
+    assert lib.bsa_matmul_lines(None, 0, 64, _capi.BF16, 0) == -1 and b"NULL argument block" in lib.bsa_last_error()
+    a.n_batches, a.lines_per_batch, a.n_streamed, a.n_outputs = 1, 1, 513, 4
+    assert lib.bsa_matmul_lines(ctypes.byref(a), 0, 64, _capi.BF16, 0) == -1
+    assert b"at most 512 streamed blocks" in lib.bsa_last_error()
+    a.n_streamed, a.n_outputs = 4, 600
+    assert lib.bsa_matmul_lines(ctypes.byref(a), 0, 64, _capi.BF16, 0) == -1
+    assert b"at most 512 output blocks" in lib.bsa_last_error()
+    a.n_outputs = 4
+    assert lib.bsa_matmul_lines(ctypes.byref(a), 0, 32, _capi.BF16, 0) == -1 and b"sbs must be 64" in lib.bsa_last_error()
+    assert lib.bsa_matmul_lines(ctypes.byref(a), 0, 64, _capi.F32, 0) == -1 and b"fp16 or bf16" in lib.bsa_last_error()
+    a.nnz_out = -1
+    assert lib.bsa_matmul_lines(ctypes.byref(a), 0, 64, _capi.BF16, 0) == -1 and b"negative block count" in lib.bsa_last_error()
+    a.nnz_out = 0
+    assert lib.bsa_matmul_lines(ctypes.byref(a), 1, 64, _capi.BF16, 0) == 0  # no output block: nothing to do
+    assert lib.bsa_matmul_lines_parts(ctypes.byref(a), 0, 0, 0) == -1 and b"NULL pointer" in lib.bsa_last_error()
+    # the argument block mirrors the header: 7 pointers, 4 + 9 + 3 int64, one pointer
+    assert ctypes.sizeof(_capi.LinesArgs) == 7 * 8 + 4 * 8 + 9 * 8 + 3 * 8 + 8
+    assert _capi.LinesArgs.error.offset == 23 * 8 and _capi.LinesArgs.streamed_strides.offset == 11 * 8
