@@ -252,15 +252,14 @@ __device__ inline int32_t checked_index(const int64_t *table, int64_t at, int64_
   return (v >= 0 && v < n) ? (int32_t)v : -1;
 }
 
-// one wave per query block row, then one per key block row
-__global__ __launch_bounds__(kBwdThreads) void attn_bwd_records_kernel(bsa_attn_args a) {
+// One wave per query block row (by_key false), in a second launch one per key block row (by_key true): the lists
+// per key block name every pair by its position in the finished list of its query block.
+__global__ __launch_bounds__(kBwdThreads) void attn_bwd_records_kernel(bsa_attn_args a, bool by_key) {
   const int64_t w = ((int64_t)blockIdx.x * kBwdThreads + threadIdx.x) >> 6;
-  const int64_t qrows = a.B * a.nq, krows = a.B * a.nk;
-  if (w >= qrows + krows) return;
+  if (w >= (by_key ? a.B * a.nk : a.B * a.nq)) return;
   const int lane = threadIdx.x & 63;
   const BwdLists L = bwd_lists(a);
-  const bool by_key = w >= qrows;
-  const int64_t row = by_key ? w - qrows : w;
+  const int64_t row = w;
   const int64_t per_batch = by_key ? a.nk : a.nq;
   const int64_t b = row / per_batch, mine = row % per_batch;
   const int32_t *offsets = by_key ? a.query_offsets : a.key_offsets;
@@ -302,16 +301,20 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_records_kernel(bsa_attn_
       }
       r.mask = pm;
       r.bias = a.bias ? checked_index(a.pidx_bias, pair, a.n_bias_blocks) : -1;
-      // the pair's position in the list of its query block as written here (without the dead pairs): where this
-      // record goes, or, from the side of the key block, the row's start plus the live pairs in front of kb
+      // the pair's position in the list of its query block as written by the first launch (without the dead
+      // pairs): where this record goes, or, from the side of the key block, where the query block's list, which is
+      // sorted by key block, holds this key block (a pair is live from both sides or from neither)
       int at = n + __popcll(votes & ((1ull << lane) - 1));
       if (by_key) {
-        const int q_begin = a.key_offsets[b * a.nq + qb], q_end = a.key_offsets[b * a.nq + qb + 1];
-        at = q_begin;
-        for (int i = q_begin; i < q_end && a.key_indices[i] < kb; ++i) {
-          int32_t ignored;
-          at += pair_live(qb, a.key_indices[i], ignored) ? 1 : 0;
+        const int64_t qrow = b * a.nq + qb;
+        int lo = a.key_offsets[qrow], hi = L.key_end[qrow];
+        while (lo < hi) {
+          const int mid = lo + ((hi - lo) >> 1);
+          if (L.key_rec[mid].other < (int32_t)kb) lo = mid + 1;
+          else hi = mid;
         }
+        // lists that do not match each other must not turn into a position outside the dS blocks
+        at = lo < a.n_layout_blocks ? lo : (int)a.n_layout_blocks - 1;
       }
       r.pair = at;
       out[n + __popcll(votes & ((1ull << lane) - 1))] = r;
@@ -1544,7 +1547,9 @@ int launch_bwd(const bsa_attn_args &a, hipStream_t s) {
           static_cast<const u32x4 *>(a.mask), L.mask_dead, a.n_mask_blocks);
       if (int rc = check_launch("attn_bwd_mask_dead_kernel")) return rc;
     }
-    attn_bwd_records_kernel<<<(unsigned)cdiv(qrows + krows, 4), kBwdThreads, 0, s>>>(a);
+    attn_bwd_records_kernel<<<(unsigned)cdiv(qrows, 4), kBwdThreads, 0, s>>>(a, false);
+    if (int rc = check_launch("attn_bwd_records_kernel")) return rc;
+    attn_bwd_records_kernel<<<(unsigned)cdiv(krows, 4), kBwdThreads, 0, s>>>(a, true);
     if (int rc = check_launch("attn_bwd_records_kernel")) return rc;
     attn_bwd_order_kernel<<<16, kOrderThreads, 0, s>>>(a);
     if (int rc = check_launch("attn_bwd_order_kernel")) return rc;

@@ -326,6 +326,9 @@ class _Tables:
             setattr(self, name, cache.get(name))
 
 
+_PRUNE_AT_ONCE_BLOCKS = 32768  # active blocks of the attention layout from which dead pairs are listed at once
+
+
 class _MaskFacts:
     """What one mask tensor (and one tensor of causal lengths) adds to the layout metadata.
 
@@ -357,7 +360,11 @@ def _mask_facts(layout_cache: dict, attention_layout: Tensor, mask: Tensor | Non
     """The facts for this mask in ``layout_cache``, renewed when another mask (or another version) arrives.
 
     The forward lists without dead pairs are built when a mask is seen for the second time in a row: a caller
-    that brings a new mask with every call never pays for lists it would use once.
+    that brings a new mask with every call never pays for lists it would use once.  On a layout of
+    ``_PRUNE_AT_ONCE_BLOCKS`` active blocks or more they are built at the first sighting: there the pass over the
+    mask and the new lists cost about what the forward call saves by them (measured on 110 000 blocks of which 46 %
+    are dead: 0.14 ms for the lists, 0.12 ms saved per call), so a mask that is used once loses nothing and a mask
+    that is used again gains from its first call on.
     """
     if not mask_facts_enabled():
         return None
@@ -371,7 +378,9 @@ def _mask_facts(layout_cache: dict, attention_layout: Tensor, mask: Tensor | Non
         facts = holder.cache["facts"] = _MaskFacts(key, (mask, lengths))
     facts.sightings += 1
     has_mask = mask_bytes is not None and mask_bytes.size(0) > 0
-    if (facts.sightings == 2 and facts.group_offsets is None and (has_mask or lengths is not None)
+    at_once = "key_indices_i32" in layout_cache and layout_cache["key_indices_i32"].numel() >= _PRUNE_AT_ONCE_BLOCKS
+    if (facts.sightings >= (1 if at_once else 2) and facts.group_offsets is None
+            and (has_mask or lengths is not None)
             and "group_offsets" in layout_cache and not torch.cuda.is_current_stream_capturing()):
         B, nq, nk, nh, nhv = dims
         device = attention_layout.device

@@ -519,6 +519,46 @@ def test_lists_kept_per_mask_follow_the_mask(device, use_causal):
         assert_close(a, b, 2e-2, name)
 
 
+def test_dead_pairs_listed_at_the_first_sighting_on_a_large_layout(device, monkeypatch):
+    """From a threshold of active blocks on, the forward lists without dead pairs are built at the first call with
+    a mask (here the threshold is lowered to the test's size): same bits as with lists built at the second call,
+    forward and backward, and the first call already walks the shorter lists."""
+    import sys
+    fa = sys.modules["blksprs_amd.ops.flash_attention"]  # the package attribute of that name is the function
+    g = torch.Generator().manual_seed(31)
+    B, n, nh, sbs = 2, 8, 2, 64
+    la = orc.random_layout((B, n, n), 0.7, g, ensure_rows=True).to(device)
+    full = torch.ones((B, n, nh), dtype=torch.bool, device=device)
+    q, k, v = (rand_blocks(B * n * nh, sbs, torch.bfloat16, s).to(device) for s in (1, 2, 3))
+    go = rand_blocks(B * n * nh, sbs, torch.bfloat16, 4).to(device)
+    n_mask = int(la.sum())
+    gm = torch.Generator().manual_seed(5)
+    mask = torch.rand((n_mask, sbs, sbs), generator=gm) < 0.3
+    mask[torch.rand(n_mask, generator=gm) < 0.5] = True  # dead pairs
+    mask = mask.to(device)
+
+    def run(cache):
+        qq, kk, vv = (t.clone().requires_grad_(True) for t in (q, k, v))
+        out = bs.ops.flash_attention(qq, full, kk, full, vv, full, la, sbs, attention_mask=mask,
+                                     sparsity_layout_mask=la, layout_cache=cache)
+        out.backward(go)
+        return out.detach(), qq.grad, kk.grad, vv.grad
+
+    late = {}
+    reference = run(late)
+    assert late["mask_facts"].cache["facts"].group_offsets is None
+    monkeypatch.setattr(fa, "_PRUNE_AT_ONCE_BLOCKS", 1)
+    early = {}
+    first = run(early)
+    facts = early["mask_facts"].cache["facts"]
+    assert facts.group_offsets is not None and int(facts.group_offsets[-1]) < int(early["group_offsets"][-1])
+    for a, b in zip(first, reference):
+        assert torch.equal(a, b)
+    for a, b in zip(run(early), reference):
+        assert torch.equal(a, b)
+    assert early["mask_facts"].cache["facts"] is facts
+
+
 def test_a_mask_that_masks_everything_leaves_empty_lists(device):
     """Every mask block masks everything: from the second call on the forward's lists are empty.  Output and
     gradients are zeros, as on the first call."""
