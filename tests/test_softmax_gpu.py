@@ -31,8 +31,8 @@ def test_forward_and_backward(device, sbs, shape, density, flag_fused):
 
 
 def test_rows_sum_to_one_at_config3_size(device):
-    """Config 3 at full size (B=32, 2048x2048, sbs 64, causal + 10 %): every element row sums to 1, and a
-    sample of batches matches the oracle."""
+    """Config 3 at full size (B=32, 2048x2048, sbs 64, causal + 10 %): every element row sums to 1, and three
+    batch entries (first, middle, last) match the oracle, forward and backward; a second run gives the same bits."""
     B, n, sbs = 32, 32, 64
     g = torch.Generator().manual_seed(0)
     tri = torch.tril(torch.ones((n, n), dtype=torch.bool))
@@ -43,8 +43,19 @@ def test_rows_sum_to_one_at_config3_size(device):
     dense = bs.ops.to_dense(out, layout.to(device), sbs)
     sums = dense.sum(dim=-1)
     assert torch.allclose(sums, torch.ones_like(sums), atol=1e-5)
-    first = int(layout[0].sum())
-    assert_close(out[:first], orc.softmax(x[:first], layout[:1].numpy(), sbs), TOL, "batch 0")
+    # forward and backward of the first, a middle and the last batch entry against the oracle
+    starts = torch.cumsum(layout.reshape(B, -1).sum(dim=1), 0).tolist()
+    gout = torch.randn((nnz, sbs, sbs), generator=g)
+    xd = x.to(device).requires_grad_(True)
+    od = bs.ops.softmax(xd, layout.to(device), sbs)
+    assert torch.equal(od.detach(), out)
+    od.backward(gout.to(device))
+    for b in (0, B // 2, B - 1):
+        lo, hi = (starts[b - 1] if b else 0), starts[b]
+        lb = layout[b:b + 1].numpy()
+        want = orc.softmax(x[lo:hi], lb, sbs)
+        assert_close(out[lo:hi], want, TOL, f"batch {b}")
+        assert_close(xd.grad[lo:hi], orc.softmax_backward(gout[lo:hi], want, lb, sbs), TOL, f"batch {b} backward")
 
 
 def test_non_contiguous_gradient_and_extremes(device):
