@@ -81,10 +81,11 @@ def _lines_args(plan: "_Plan", shapes, which: str, streamed: Tensor | None, priv
 
 def _lines_apply(plan: "_Plan", shapes, sbs: int, dtype: torch.dtype) -> bool:
     """Whether the two backward products run on the line kernel: 16-bit operands, 64 x 64 blocks, lines of dO and
-    of the output of at most 512 blocks either way."""
+    of the output of at most 512 blocks either way, fewer than 2^25 lines (an entry of the part table holds the line
+    in 25 bits); everything else takes the tile kernel."""
     (B, R, K), (_, _, C) = shapes
     return (sbs == 64 and dtype in (torch.float16, torch.bfloat16) and max(R, C, K) <= _MAX_LINE_BLOCKS
-            and B * max(R, C) < 2 ** 31 - 1)
+            and B * max(R, C) < 2 ** 25)
 
 
 def _lines_parts(plan: "_Plan", shapes) -> tuple[Tensor, Tensor]:

@@ -274,3 +274,17 @@ def test_measurement_knobs_are_clamped_and_malformed_values_ignored(monkeypatch)
     assert any("not an integer" in str(w.message) for w in caught)
     monkeypatch.delenv("BLKSPRS_AMD_ROW_PARTS_LOG2")
     assert mm._measurement_knob("BLKSPRS_AMD_ROW_PARTS_LOG2", 1, 0, 3) == 1
+
+
+def test_line_kernel_is_chosen_within_its_limits_only():
+    """The backward products take the line kernel for 16-bit operands at sbs 64 when no line of either layout has
+    more than 512 blocks and there are fewer than 2^25 lines (the part table holds the line in 25 bits and
+    bsa_matmul_lines_parts refuses more); everything else takes the tile kernel."""
+    import importlib
+    mm = importlib.import_module("blksprs_amd.ops.matmul")
+    ok = lambda B, R, K, C, sbs=64, dt=torch.bfloat16: mm._lines_apply(None, ((B, R, K), (B, K, C)), sbs, dt)
+    assert ok(16, 64, 64, 64) and ok(1, 512, 512, 512) and ok(2, 4, 6, 5, dt=torch.float16)
+    assert not ok(16, 64, 64, 64, sbs=32) and not ok(16, 64, 64, 64, dt=torch.float32)
+    assert not ok(1, 513, 8, 8) and not ok(1, 8, 513, 8) and not ok(1, 8, 8, 513)
+    assert ok((1 << 25) // 512 - 1, 512, 8, 8) and not ok((1 << 25) // 512, 512, 8, 8)
+    assert not ok((1 << 25) // 512, 8, 8, 512)
