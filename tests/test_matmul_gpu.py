@@ -422,3 +422,38 @@ def test_full_size_config2_gradients_sampled_against_the_oracle(device):
     ref.backward(sl(lo, go).double())
     assert_close(sl(lx, dx), x64.grad, 2e-2, "config 2 dX, batch 5")
     assert_close(sl(ly, dy), y64.grad, 2e-2, "config 2 dY, batch 5")
+
+
+def test_line_kernel_through_the_c_abi_without_an_error_record(device):
+    """bsa_matmul_lines_parts + bsa_matmul_lines called directly, with ``error`` NULL (allowed: the bounded waits
+    then leave no record) and with part tables built in scratch of exactly the documented size: the same bits as
+    the operator's backward pass, for dX and dY; an argument block without output blocks launches nothing."""
+    import ctypes
+    import sys
+    from blksprs_amd import _capi
+    mm = sys.modules["blksprs_amd.ops.matmul"]
+    B, R, K, C, sbs = 2, 5, 19, 37, 64
+    lx, ly, lo = rand_layout((B, R, K), 0.8, seed=41), rand_layout((B, K, C), 0.5, seed=42), rand_layout((B, R, C), 0.7, seed=43)
+    x = rand_blocks(int(lx.sum()), sbs, torch.bfloat16, 44, 1.0 / math.sqrt(K * sbs)).to(device)
+    y = rand_blocks(int(ly.sum()), sbs, torch.bfloat16, 45).to(device)
+    go = rand_blocks(int(lo.sum()), sbs, torch.bfloat16, 46, 1.0 / math.sqrt(C * sbs)).to(device)
+    lxd, lyd, lod = lx.to(device), ly.to(device), lo.to(device)
+    cache = {}
+    xg, yg = x.clone().requires_grad_(True), y.clone().requires_grad_(True)
+    bs.ops.matmul(xg, lxd, yg, lyd, lod, sbs, layout_cache=cache).backward(go)
+    plan = cache["plan"]
+    shapes = ((B, R, K), (B, K, C))
+    for which, private, want in (("x", y, xg.grad), ("y", x, yg.grad)):
+        out = torch.full(want.shape, float("nan"), dtype=torch.bfloat16, device=device)
+        n_lines = B * (R if which == "x" else C)
+        scratch = torch.empty(4 * n_lines + 2, dtype=torch.int32, device=device)
+        table = torch.full((1 + want.size(0) // 16 + n_lines,), -7, dtype=torch.int32, device=device)
+        a = mm._lines_args(plan, shapes, which, go, private, out, table)
+        a.error = 0
+        _capi.call("bsa_matmul_lines_parts", ctypes.byref(a), scratch.data_ptr(), table.data_ptr(), _capi.stream(device))
+        _capi.call("bsa_matmul_lines", ctypes.byref(a), int(which == "y"), sbs, _capi.BF16, _capi.stream(device))
+        assert torch.equal(out, want), which
+        assert int(table[0]) <= table.numel() - 1
+        nothing = mm._lines_args(plan, shapes, which, go, private, None, table)
+        nothing.nnz_out, nothing.error = 0, 0
+        _capi.call("bsa_matmul_lines", ctypes.byref(nothing), int(which == "y"), sbs, _capi.BF16, _capi.stream(device))
